@@ -1,0 +1,320 @@
+"""Pins the arithmetic oracles (scores, AdamW commit, replay commit, cycle
+machine, pack) against independent float64 closed forms, brute force and the
+identities the reference's own tests assert."""
+import math
+
+import pytest
+import torch
+
+from oracle import adamw as A
+from oracle import fused_step as F
+from oracle import kernels as OK
+from oracle import replay as R
+from oracle import scores as S
+from oracle import select as SEL
+
+
+def _f64_scores(w, m, v, g, b1, b2, eps, wd, bc1, bc2, adams=False):
+    w, m, v, g = (t.double() for t in (w, m, v, g))
+    m_new = b1 * m + (1 - b1) * g
+    if adams:
+        v_new = b2 * m * m + (1 - b2) * g * g
+        v0 = b2 * m * m
+        bc1 = bc2 = 1.0
+    else:
+        v_new = b2 * v + (1 - b2) * g * g
+        v0 = b2 * v
+    ug = (m_new / bc1) / ((v_new / bc2).sqrt() + eps)
+    u0 = (b1 * m / bc1) / ((v0 / bc2).sqrt() + eps)
+    return {"abs_g": g.abs(), "abs_m": m.abs(), "update": wd * w + ug,
+            "coi": (ug - u0).abs()}
+
+
+def _state(n, seed):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(n, generator=g), torch.randn(n, generator=g) * 0.1,
+            torch.rand(n, generator=g) * 0.1 + 1e-4, torch.randn(n, generator=g))
+
+
+@pytest.mark.parametrize("opt", ["adamw", "adams"])
+def test_scores_vs_f64(opt):
+    b1, b2, eps, wd, step = 0.9, 0.95, 1e-8, 1e-2, 7
+    bc1, bc2 = 1 - b1 ** step, 1 - b2 ** step
+    w, m, v, g = _state(513, 3)
+    ref = _f64_scores(w, m, v, g, b1, b2, eps, wd, bc1, bc2, adams=opt == "adams")
+    for name in S.FORMULAS:
+        out = S.get_formula(name)(w, m, v, g, b1, b2, eps, wd, bc1, bc2,
+                                  optimizer=opt)
+        torch.testing.assert_close(out.double(), ref[name], rtol=1e-5,
+                                   atol=2e-6 if name == "coi" else 1e-7)
+        if opt == "adams":   # replay-side substitution gives the same thing
+            out2 = S.score_formula(name, w, m, v, g, b1, b2, eps, wd, bc1, bc2,
+                                   "adams", update_includes_wd=True)
+            assert torch.equal(out, out2)
+    with pytest.raises(ValueError) as ei:
+        S.get_formula("nope")
+    assert "nope" in str(ei.value) and "abs_g" in str(ei.value)
+    u = S.update(w, m, v, g, b1, b2, eps, wd, bc1, bc2, update_includes_wd=False)
+    torch.testing.assert_close(u.double(), ref["update"] - wd * w.double(),
+                               rtol=1e-5, atol=1e-7) if opt == "adamw" else None
+
+
+def _f64_adamw(p, g, m, v, lr, b1, b2, eps, wd, step):
+    p, g, m, v = (t.double() for t in (p, g, m, v))
+    m2 = b1 * m + (1 - b1) * g
+    v2 = b2 * v + (1 - b2) * g * g
+    upd = wd * p + (m2 / (1 - b1 ** step)) / ((v2 / (1 - b2 ** step)).sqrt() + eps)
+    return p - lr * upd, m2, v2, upd
+
+
+def test_grad_correct_vs_f64_and_fused_knobs():
+    n = 3000
+    lr, b1, b2, eps, wd, step = 1e-3, 0.9, 0.95, 1e-8, 0.1, 5
+    p, m, v, g = _state(n, 11)
+    mask = (torch.rand(n, generator=torch.Generator().manual_seed(1)) < 0.3).to(torch.uint8)
+    # sparse step vs f64 with g' = where(mask, g, 0)
+    pp, gg, mm, vv = p.clone(), g.clone(), m.clone(), v.clone()
+    A.adamw_grad_correct(pp, gg, mm, vv, lr, b1, b2, eps, wd, step, mask=mask)
+    rp, rm, rv, _ = _f64_adamw(p, torch.where(mask > 0, g, torch.zeros(())), m, v,
+                               lr, b1, b2, eps, wd, step)
+    torch.testing.assert_close(pp.double(), rp, rtol=1e-5, atol=1e-7)
+    torch.testing.assert_close(mm.double(), rm, rtol=1e-5, atol=1e-7)
+    torch.testing.assert_close(vv.double(), rv, rtol=1e-4, atol=1e-6)
+    assert torch.equal(gg, g)          # untouched without clear/fold
+    # fused coeff/clear/fold == standalone 3-pass sequence, bitwise
+    # (tests/test_kernels_gpu.py:227-268)
+    p1, g1, m1, v1 = p.clone(), g.clone(), m.clone(), v.clone()
+    A.adamw_grad_correct(p1, g1, m1, v1, lr, b1, b2, eps, wd, step, mask=mask,
+                         coeff=0.37, clear=True, fold=True, interval=4.0)
+    p2, g2, m2, v2 = p.clone(), g.clone(), m.clone(), v.clone()
+    g2 = torch.where(mask > 0, g2 * 0.37, g2)
+    A.adamw_grad_correct(p2, g2, m2, v2, lr, b1, b2, eps, wd, step, mask=mask)
+    g2[mask > 0] = 0.0
+    g2 /= 4.0
+    for a, b in ((p1, p2), (g1, g2), (m1, m2), (v1, v2)):
+        assert torch.equal(a, b)
+    # full step: score lands in grad, commit is mask-blind
+    for name in S.FORMULAS:
+        p3, g3, m3, v3 = p.clone(), g.clone(), m.clone(), v.clone()
+        A.adamw_grad_correct(p3, g3, m3, v3, lr, b1, b2, eps, wd, step,
+                             emit_score=name)
+        rp, rm, rv, _ = _f64_adamw(p, g, m, v, lr, b1, b2, eps, wd, step)
+        torch.testing.assert_close(p3.double(), rp, rtol=1e-5, atol=1e-7)
+        ref = _f64_scores(p, m, v, g, b1, b2, eps, wd, 1 - b1 ** step, 1 - b2 ** step)
+        # coi subtracts two O(1) directions: tolerance at operand scale
+        torch.testing.assert_close(g3.double(), ref[name], rtol=1e-5,
+                                   atol=2e-6 if name == "coi" else 1e-7)
+    # dual-lr: p == w - where(mask, lr, lr*s) * score(update); m/v mask-blind
+    p4, g4, m4, v4 = p.clone(), g.clone(), m.clone(), v.clone()
+    A.adamw_grad_correct(p4, g4, m4, v4, lr, b1, b2, eps, wd, step, mask=mask,
+                         emit_score="update", inactive_lr_scale=0.25)
+    p5, g5, m5, v5 = p.clone(), g.clone(), m.clone(), v.clone()
+    A.adamw_grad_correct(p5, g5, m5, v5, lr, b1, b2, eps, wd, step, emit_score="update")
+    assert torch.equal(m4, m5) and torch.equal(v4, v5) and torch.equal(g4, g5)
+    assert torch.equal(p4, p - torch.where(mask > 0, lr, lr * 0.25) * g4)
+    p6 = p.clone()
+    A.adamw_grad_correct(p6, g.clone(), m.clone(), v.clone(), lr, b1, b2, eps, wd,
+                         step, mask=mask, emit_score="update", inactive_lr_scale=0.0)
+    assert torch.equal(p6[mask == 0], p[mask == 0])
+
+
+def test_knob_refusals():
+    z = torch.zeros(4)
+    mk = torch.ones(4, dtype=torch.uint8)
+    for kw, sub in (
+            (dict(coeff=0.5), "requires a sparse step"),
+            (dict(mask=mk, emit_score="update"), "masked-commit full step"),
+            (dict(mask=mk, inactive_lr_scale=0.5), "requires a full step"),
+            (dict(mask=mk, emit_score="update", inactive_lr_scale=float("nan")),
+             "inactive_lr_scale"),
+            (dict(emit_score="bogus"), "no _grad_correct_kernel branch")):
+        with pytest.raises(ValueError) as ei:
+            A.adamw_grad_correct(z.clone(), z.clone(), z.clone(), z.clone(), 1e-3,
+                                 0.9, 0.95, 1e-8, 0.0, 1, **kw)
+        assert sub in str(ei.value)
+
+
+def test_compact_commit_equals_masked_commit_and_dir_table():
+    n_bucket, rec_start, n = 9000, 1500, 4000
+    lr, b1, b2, eps, wd, step = 1e-3, 0.9, 0.95, 1e-8, 0.1, 3
+    gen = torch.Generator().manual_seed(2)
+    buf = torch.randn(n_bucket, generator=gen)
+    mask = (torch.rand(n_bucket, generator=gen) < 0.2).to(torch.uint8)
+    idx = OK.compact_mask_u8(mask)
+    p, m, v, _ = _state(n, 5)
+    # masked path on the record's slice
+    b1_, p1, m1, v1 = buf.clone(), p.clone(), m.clone(), v.clone()
+    A.adamw_grad_correct(p1, b1_[rec_start:rec_start + n], m1, v1, lr, b1, b2, eps,
+                         wd, step, mask=mask[rec_start:rec_start + n], clear=True)
+    # compact path: pack first, then merge-join commit
+    b2_, p2, m2, v2 = buf.clone(), p.clone(), m.clone(), v.clone()
+    vals = torch.empty(idx.numel())
+    OK.pack_selected(b2_, idx, vals, 1.0)
+    assert torch.equal(vals, buf[mask.bool()]) and bool((b2_[mask.bool()] == 0).all())
+    assert torch.equal(b2_[~mask.bool()], buf[~mask.bool()])
+    A.adamw_grad_correct_compact(p2, b2_[rec_start:rec_start + n], m2, v2, idx, vals,
+                                 rec_start, lr, b1, b2, eps, wd, step)
+    assert torch.equal(p1, p2) and torch.equal(m1, m2) and torch.equal(v1, v2)
+    assert torch.equal(b1_[rec_start:rec_start + n], b2_[rec_start:rec_start + n])
+    # dir table == brute-force lower_bound
+    tab = A.build_dir_table(idx, n_bucket)
+    il = idx.tolist()
+    for j in range(tab.numel()):
+        assert tab[j].item() == sum(1 for x in il if x < j * 1024)
+    assert A.build_dir_table(torch.empty(0, dtype=torch.int32), 5000).tolist() == [0] * 6
+
+
+def test_pack_scatter_bruteforce_and_bf16():
+    gen = torch.Generator().manual_seed(9)
+    grad = torch.randn(1000, generator=gen)
+    idx = torch.tensor([3, 17, 500, 999], dtype=torch.int32)
+    for factor in (1.0, 0.125):
+        g = grad.clone()
+        vals = torch.empty(4)
+        OK.pack_selected(g, idx, vals, factor)
+        for j, i in enumerate(idx.tolist()):
+            assert vals[j].item() == (grad[i] * factor if factor != 1.0 else grad[i]).item()
+            assert g[i].item() == 0.0
+        vb = torch.empty(4, dtype=torch.bfloat16)
+        g = grad.clone()
+        OK.pack_selected(g, idx, vb, factor)
+        assert torch.equal(vb, (grad[idx.long()] * factor).to(torch.bfloat16))
+        dst = torch.zeros(1000)
+        OK.scatter_selected(dst, idx, vals)
+        assert torch.equal(dst[idx.long()], vals) and int((dst != 0).sum()) <= 4
+    tot = torch.zeros(())
+    OK.compact_norm_sq_contribution(vals, tot)
+    assert abs(tot.item() - sum(x * x for x in vals.tolist())) < 1e-5
+    mask = torch.zeros(1000, dtype=torch.uint8)
+    mask[idx.long()] = 1
+    tot2 = torch.zeros(())
+    OK.masked_norm_sq_contribution(grad, mask, tot2)
+    assert abs(tot2.item() - sum(grad[i].item() ** 2 for i in idx.tolist())) < 1e-5
+    pl = OK.mask_layout_pack(grad, mask, 1.0, slices=2)
+    assert [x.numel() for x in pl] == [2, 2] and torch.equal(torch.cat(pl), grad[mask.bool()])
+
+
+def _f64_replay(q, m, v, w, lr, wd, b1, b2, bc1, bc2, eps, adams, inactive=None, lr_i=None):
+    q, m, v, w = (t.double() for t in (q, m, v, w))
+    v2 = (b2 * m * m if adams else b2 * v) + (1 - b2) * q * q
+    m2 = b1 * m + (1 - b1) * q
+    upd = (m2 / bc1) / ((v2 / bc2).sqrt() + eps)
+    if inactive is None:
+        w2 = w * (1 - lr * wd) - lr * upd
+    else:
+        w2 = w - torch.where(inactive, lr_i, lr) * (wd * w + upd)
+    return m2, v2, w2, upd
+
+
+@pytest.mark.parametrize("opt", ["adamw", "adams"])
+@pytest.mark.parametrize("lr,wd,count", [(1e-3, .01, 7), (3e-4, .01, 1), (1e-3, 0.0, 100)])
+def test_replay_commit_vs_f64(opt, lr, wd, count):
+    b1, b2, eps = 0.9, 0.999, 1e-8
+    w, m, v, q = _state(2000, count)
+    bc1, bc2 = R.bc_pair(opt, count, b1, b2)
+    inactive = torch.rand(2000, generator=torch.Generator().manual_seed(3)) < 0.5
+    for ina, lri in ((None, None), (inactive, lr * 0.3)):
+        mm, vv, ww, lab = m.clone(), v.clone(), w.clone(), torch.zeros(2000)
+        R.opt_step_inplace(q, mm, vv, ww, lab, lr, wd, b1, b2, bc1, bc2, eps,
+                           optimizer=opt, inactive=ina, lr_inactive=lri)
+        rm, rv, rw, ru = _f64_replay(q, m, v, w, lr, wd, b1, b2, bc1, bc2, eps,
+                                     opt == "adams", ina, lri)
+        torch.testing.assert_close(mm.double(), rm, rtol=1e-5, atol=1e-7)
+        torch.testing.assert_close(vv.double(), rv, rtol=1e-4, atol=1e-6)
+        torch.testing.assert_close(ww.double(), rw, rtol=1e-5, atol=1e-6)
+        torch.testing.assert_close(lab.double(), (lr * ru) ** 2, rtol=1e-4, atol=1e-9)
+    with pytest.raises(ValueError):
+        R.opt_step_inplace(q, m, v, w, None, lr, wd, b1, b2, bc1, bc2, eps,
+                           inactive=inactive)
+
+
+def test_coef_dense():
+    assert R.coef_dense_for(0.0, 5.0) == 1.0
+    assert R.coef_dense_for(1.0, float("nan")) == 1.0
+    assert R.coef_dense_for(1.0, 0.5) == 1.0
+    assert R.coef_dense_for(0.3, 2.0) == 0.3 / (2.0 + 1e-6)
+
+
+def _spec_cycle(w0, m0, v0, grads, norms, lr, clip, t0, k, T, b1, b2, eps, wd,
+                fold=False):
+    """From-spec float64-free double loop (shape of
+    tests/test_replay_cycle.py:141-223), abs_g score, adamw."""
+    def adam(w, m, v, q, count):
+        m = b1 * m + (1 - b1) * q
+        v = b2 * v + (1 - b2) * q * q
+        upd = (m / (1 - b1 ** count)) / (torch.sqrt(v / (1 - b2 ** count)) + eps)
+        return w * (1 - lr * wd) - lr * upd, m, v
+    ws, ms, vs = w0.clone(), m0.clone(), v0.clone()
+    res = torch.zeros_like(w0)
+    sel = SEL.select_topk_flat(grads[0].abs(), k)[0]
+    for si, gl in enumerate(grads):
+        count = t0 + si + 1
+        cd = min(1.0, clip / (norms[si] + 1e-6)) if clip > 0 else 1.0
+        g = gl / cd
+        if si % T == 0:
+            if fold and si > 0:
+                res = res / T
+            qp = g + res
+            coef = min(1.0, clip / (float(qp.norm()) + 1e-6)) if clip > 0 else 1.0
+            q = qp * coef
+            if si > 0 and si + 1 < len(grads):
+                sel = SEL.select_topk_flat(q.abs(), k)[0]
+            res = torch.zeros_like(res)
+        else:
+            coef = min(1.0, clip / (float((g * sel).norm()) + 1e-6)) if clip > 0 else 1.0
+            q = g * sel * coef
+            res = res + g * (~sel)
+        ws, ms, vs = adam(ws, ms, vs, q, count)
+    return ws, sel, res
+
+
+@pytest.mark.parametrize("T,fold", [(1, False), (4, False), (4, True), (3, False)])
+def test_group_replay_vs_spec(T, fold):
+    n, W, t0 = 5000, 9, 10
+    b1, b2, eps, wd, lr, clip = 0.9, 0.95, 1e-8, 0.1, 5e-5, 0.3
+    gen = torch.Generator().manual_seed(2026)
+    w0 = torch.randn(n, generator=gen) * 0.02
+    m0 = torch.randn(n, generator=gen) * 1e-3
+    v0 = torch.rand(n, generator=gen) * 1e-6
+    grads = [torch.randn(n, generator=gen) * 1e-2 for _ in range(W)]
+    norms = [float(g.norm()) for g in grads]
+    k = SEL.replay_k(n, 10.0)
+    entries = [{"a": 0, "n": 3000, "b1": b1, "b2": b2, "eps": eps, "wd": wd},
+               {"a": 3000, "n": 2000, "b1": b1, "b2": b2, "eps": eps, "wd": wd}]
+    cfg = R.Config("abs_g", 10.0, T, fold=fold)
+    sel0 = SEL.select_topk_flat(grads[0].abs(), k)[0]
+    metas = [{"clip_grad": clip, "grad_norm": norms[i], "lr": lr} for i in range(W)]
+    out = R.group_replay(entries, w0, m0, v0, [sel0], [cfg], grads, metas, t0)[0]
+    ws, sel, res = _spec_cycle(w0, m0, v0, grads, norms, lr, clip, t0, k, T, b1, b2,
+                               eps, wd, fold)
+    assert torch.equal(out["sel"], sel)
+    torch.testing.assert_close(out["w"], ws, rtol=1e-5, atol=1e-7)
+    torch.testing.assert_close(out["res"], res, rtol=1e-5, atol=1e-9)
+    if T == 1:   # every step a boundary: residual never survives a step
+        assert float(out["res"].abs().max()) == 0.0
+
+
+def test_fused_step_end_state_invariant():
+    """buf[idx]==0 and buf[~mask]==(g+r)[~mask] bitwise
+    (tests/test_plugins_unit.py:785-837)."""
+    n = 1 << 14
+    gen = torch.Generator().manual_seed(0)
+    segs = [dict(start=0, n=10000, lr=1e-4, b1=0.9, b2=0.95, eps=1e-8, wd=0.1),
+            dict(start=10000, n=n - 10000, lr=1e-4, b1=0.9, b2=0.95, eps=1e-8, wd=0.0)]
+    p = torch.randn(n, generator=gen) * 0.02
+    m, v, r = torch.zeros(n), torch.zeros(n), torch.zeros(n)
+    for step in range(1, 4):
+        g = (torch.randn(n, generator=gen) * 1e-3).to(torch.bfloat16)
+        before = r + g.float()
+        p0, m0, v0 = p.clone(), m.clone(), v.clone()
+        idx, vals, mask, th = F.fused_sparse_step(g, r, p, m, v, segs, step,
+                                                  ratio_percent=1.0,
+                                                  values_dtype=torch.bfloat16)
+        assert idx.numel() == SEL.k_for(n, 1.0) == int(mask.sum())
+        assert bool((r[mask] == 0).all()) and torch.equal(r[~mask], before[~mask])
+        assert torch.equal(vals, before[mask].to(torch.bfloat16))
+        gq = torch.where(mask, before.to(torch.bfloat16).float(), torch.zeros(()))
+        rp, rm, rv, _ = _f64_adamw(p0[:10000], gq[:10000], m0[:10000], v0[:10000],
+                                   1e-4, 0.9, 0.95, 1e-8, 0.1, step)
+        torch.testing.assert_close(p[:10000].double(), rp, rtol=1e-5, atol=1e-7)
+        torch.testing.assert_close(m[:10000].double(), rm, rtol=1e-5, atol=1e-9)

@@ -1,0 +1,165 @@
+"""Pins the selection oracle against the reference's known-answer vectors
+(tests/golden/select_kats.json), torch.kthvalue, and a stable sort."""
+import json
+import os
+
+import pytest
+import torch
+
+from oracle import kernels as OK
+from oracle import select as SEL
+
+KATS = json.load(open(os.path.join(os.path.dirname(__file__), "golden",
+                                   "select_kats.json")))
+
+
+def _f(x):
+    return float(x)
+
+
+def adversarial(n, gen):
+    """Tie-heavy families of tests/test_replay_fused.py:2059-2074 (shape of
+    the data, regenerated here with our own generator)."""
+    plateau = torch.ones(n)
+    plateau[: int(0.4 * n)] = 2.0
+    npos = max(8, n // 1000)
+    zh = torch.zeros(n)
+    zh[:npos] = torch.rand(npos, generator=gen) + 0.5
+    return {
+        "all-equal": torch.full((n,), 1.0),
+        "boundary-plateau": plateau,
+        "quantized": torch.rand(n, generator=gen).mul(1000).round().div(1000),
+        "zero-heavy": zh,
+        "uniform": torch.rand(n, generator=gen) + 1e-6,
+    }
+
+
+def sort_topk_mask(t, k):
+    """Independent statement of the contract: stable descending sort, the
+    first k win (ties therefore go to the lowest index)."""
+    order = torch.sort(t, descending=True, stable=True).indices
+    m = torch.zeros(t.numel(), dtype=torch.bool)
+    m[order[:k]] = True
+    return m
+
+
+@pytest.mark.parametrize("kat", KATS["tie_fill"], ids=lambda k: k["name"])
+def test_tie_fill_kats(kat):
+    t = torch.tensor(kat["t"], dtype=torch.float32)
+    mask, th = SEL.select_topk_flat(t, kat["k"])
+    assert mask.to(torch.int64).tolist() == kat["mask"]
+    assert th == kat["thresh"]
+
+
+@pytest.mark.parametrize("kat", KATS["rejections"])
+def test_rejections(kat):
+    t = torch.tensor([_f(x) for x in kat["t"]], dtype=torch.float32)
+    with pytest.raises(ValueError) as ei:
+        SEL.select_topk_flat(t, kat["k"])
+    assert kat["substr"] in str(ei.value)
+
+
+def test_injected_tie_layer_random():
+    g = torch.Generator().manual_seed(8)
+    t = torch.rand(200, generator=g)
+    k = 50
+    v = float(torch.kthvalue(t, t.numel() - k + 1).values)
+    t[100:160] = v
+    mask, th = SEL.select_topk_flat(t, k)
+    assert th == v
+    assert torch.equal(mask, sort_topk_mask(t, k))
+    t7 = torch.rand(7, generator=g)
+    mask, th = SEL.select_topk_flat(t7, 7)
+    assert bool(mask.all()) and th == float(t7.min())
+
+
+def test_exact_k_equals_stable_sort_on_adversarial_sets():
+    gen = torch.Generator().manual_seed(20260912)
+    n = 20000
+    for name, sc in adversarial(n, gen).items():
+        for k in sorted({1, n // 100, 3 * n // 10, n - 1, n, 10, 80}):
+            mask, th = SEL.select_topk_flat(sc, k)
+            assert int(mask.sum()) == k
+            assert th == float(torch.kthvalue(sc, n - k + 1).values), name
+            assert torch.equal(mask, sort_topk_mask(sc, k)), (name, k)
+
+
+def test_threshold_is_kthvalue_all_distributions():
+    """Distribution families of tests/test_xp_capability.py:61-91."""
+    N = 4097
+    g = torch.Generator().manual_seed(1234)
+    ds = [torch.randn(N, generator=g) * 1e-3,
+          (torch.randn(N, generator=g) * 1e3).round() / 1e3,
+          torch.randn(N, generator=g).exp() * torch.sign(torch.randn(N, generator=g)),
+          torch.full((N,), 0.5),
+          torch.randn(N, generator=g) * 1e-3,
+          torch.randn(N, generator=g) * 1e-3]
+    ds[4][::3] = 0.0
+    ds[5][::7] *= 1e30
+    for x in ds:
+        views = [x[:N // 2].contiguous(), x[N // 2:].contiguous()]
+        for k in (1, 2, N // 10, N // 2, N - 1, N):
+            ref = torch.kthvalue(x.abs(), N - k + 1).values.item()
+            assert SEL.select_threshold_views(views, k) == ref
+            th, masks = SEL.select_masks_histogram(views, k, mode="exact")
+            te, me = SEL.select_masks_exact_kthvalue(views, k)
+            assert th == ref == te
+            for gv, m, m2 in zip(views, masks, me):
+                assert torch.equal(m, (gv.abs() >= ref).to(torch.uint8))
+                assert torch.equal(m, m2)
+            assert sum(int(m.sum()) for m in masks) >= k
+
+
+def test_balanced_closed_form_and_edges():
+    g = torch.Generator().manual_seed(5)
+    views = [torch.randn(40001, generator=g), torch.full((7,), 0.25),
+             torch.randn(65536, generator=g) * 3, torch.randn(100009, generator=g)]
+    n_total = sum(v.numel() for v in views)
+    k = SEL.k_for(n_total, 5.0)
+    th, masks = SEL.select_masks_histogram(views, k, mode="balanced")
+    bits = torch.tensor(th, dtype=torch.float32).view(torch.int32).item()
+    assert bits & 0xFFFF == 0
+    # brute-force restatement of the integer closed form
+    keys = torch.cat([SEL.abs_bit_top(v)[::8] for v in views]).tolist()
+    keys.sort()
+    n_s = len(keys)
+    r = max(1, round(n_s * (n_total - k + 1) / n_total))
+    b = keys[r - 1]              # smallest bin whose cumulative count >= r
+    assert bits >> 16 == b
+    n_sel = sum(int(m.sum()) for m in masks)
+    n_exact = sum(int(m.sum()) for m in SEL.select_masks_histogram(views, k)[1])
+    assert abs(n_sel - n_exact) / n_total < 0.005
+    th_f, m_f = SEL.select_masks_histogram(views, k, mode="fast")
+    bits_f = torch.tensor(th_f, dtype=torch.float32).view(torch.int32).item()
+    assert bits_f & 0x7FFFF == 0
+    # replay twin with p_off = 0 is the same mask
+    flat = torch.cat(views).abs()
+    ent, off = [], 0
+    for v in views:
+        ent.append({"a": off, "n": v.numel(), "p_off": 0})
+        off += v.numel()
+    m2, t2 = SEL.shard_select_balanced(flat, k, ent)
+    assert t2 == th and torch.equal(m2.to(torch.uint8), torch.cat(masks))
+
+
+@pytest.mark.parametrize("kat", KATS["k_for"])
+def test_k_formulas(kat):
+    assert SEL.k_for(kat["n"], kat["ratio"]) == kat["k"]
+    assert SEL.replay_k(kat["n"], kat["ratio"]) == kat["k"]
+
+
+def test_k_bankers_rounding():
+    assert SEL.k_for(250, 1.0) == 2      # 2.5 -> 2
+    assert SEL.k_for(350, 1.0) == 4      # 3.5 -> 4
+    assert SEL.k_for(10, 0.001) == 1     # floor at 1
+
+
+def test_compact_mask_kats():
+    for kat in KATS["compact_mask"]:
+        m = torch.tensor(kat["mask"], dtype=torch.uint8)
+        idx = OK.compact_mask_u8(m)
+        assert idx.dtype == torch.int32 and idx.tolist() == kat["idx"]
+        assert int(torch.searchsorted(idx, m.numel() // 2)) == kat["split_at_mid"]
+    g = torch.Generator().manual_seed(4)
+    m = (torch.rand(300000, generator=g) < 0.4).to(torch.uint8)
+    assert OK.compact_mask_u8(m).tolist() == [i for i, b in enumerate(m.tolist()) if b]
