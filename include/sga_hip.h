@@ -1,0 +1,245 @@
+/* C ABI of libsga_hip.so -- the MI355X (gfx950) kernels behind SGA's operator
+ * boundary.  Plain device pointers, sizes, scalars and a hipStream_t passed
+ * as void*; no allocation inside except where a function says so.  Every
+ * function returns SGA_OK (0) or a negative code and never throws;
+ * sga_last_error() gives the text for the calling thread.
+ *
+ * Each entry point names the reference interface it stands behind
+ * (paths relative to wenqingqian/SGA).
+ */
+#ifndef SGA_HIP_H_
+#define SGA_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SGA_OK 0
+#define SGA_ERR_ARG (-1)
+#define SGA_ERR_LAUNCH (-2)
+#define SGA_ERR_WORKSPACE (-3)
+
+#define SGA_F32 0
+#define SGA_BF16 1
+
+/* score ids: sga/plugins/optimizer/adamw.py:75-80 (_TRITON_SCORE_MAP) */
+#define SGA_SCORE_UPDATE 0
+#define SGA_SCORE_ABS_G 1
+#define SGA_SCORE_ABS_M 2
+#define SGA_SCORE_COI 3
+
+/* grad-correct flags: constexprs of _grad_correct_kernel, adamw.py:88-106 */
+#define SGA_GC_HAS_MASK 1
+#define SGA_GC_APPLY_COEFF 2
+#define SGA_GC_CLEAR 4
+#define SGA_GC_FOLD 8
+#define SGA_GC_LR_SPLIT 16
+#define SGA_GC_ADAMS 32
+
+/* tie semantics of the exact select */
+#define SGA_TIE_ALL 0          /* |s| >= thresh, count >= k  (_histogram.py:194-200) */
+#define SGA_TIE_LOWEST_INDEX 1 /* exactly k, ascending index (replay.py:559-572)    */
+
+/* replay commit flags: constexprs of _k_adam, replay_kernels.py:163-168 */
+#define SGA_RP_HAS_LAB 1
+#define SGA_RP_ADAMS 2
+#define SGA_RP_SPLIT 4
+
+int sga_version(void);
+const char* sga_last_error(void);
+
+/* Per-segment hyper-parameters of a flat bucket (one ParamRecord each:
+ * sga/plugins/optimizer/__init__.py:20-60).  All floats are the fp32
+ * roundings of the Python doubles; om1 = f32(1-beta1), bc = f32(1-beta^step). */
+typedef struct sga_segment {
+  int64_t start;
+  int64_t n;
+  float lr, beta1, om1, beta2, om2, eps, wd, bc1, bc2;
+  float pad_;
+} sga_segment;
+
+/* Result block written on the device by the select entry points. */
+typedef struct sga_select_result {
+  uint32_t thresh_bits; /* fp32 pattern of the k-th largest |score|        */
+  uint32_t need;        /* ties to take at thresh (lowest index first)     */
+  uint32_t n_gt;        /* count of |score| >  thresh                      */
+  uint32_t n_eq;        /* count of |score| == thresh                      */
+  uint32_t n_selected;  /* coordinates selected under the tie mode         */
+  uint32_t nonfinite;   /* NaN/Inf lanes seen (selection is undefined > 0) */
+  uint32_t status;      /* 0 ok; 1 k out of range; 2 fast path fell back   */
+  uint32_t path;        /* 0 radix passes, 1 sampled bracket               */
+} sga_select_result;
+
+/* ---- scheme-agnostic masked ops (sga/kernels.py) ------------------------ */
+
+/* dst[idx[i]] = src[i]            -- scatter_selected, kernels.py:145-163 */
+int sga_scatter_selected(float* dst, const int32_t* idx, const float* src,
+                         int64_t k, int64_t n_dst, void* stream);
+
+/* values[i] = grad[idx[i]]*factor; grad[idx[i]] = 0
+ *                                 -- pack_selected, kernels.py:166-187.
+ * values_dtype SGA_F32 or SGA_BF16 (round-to-nearest-even of the product). */
+int sga_pack_selected(float* grad, const int32_t* idx, void* values,
+                      int values_dtype, float factor, int64_t k,
+                      int64_t n_grad, void* stream);
+
+/* total[0] += sum(values^2), two-stage, fixed order
+ *                 -- compact_norm_sq_contribution, kernels.py:252-268.
+ * partials: workspace of sga_norm_partials(k) floats. */
+int64_t sga_norm_partials(int64_t n);
+int sga_compact_norm_sq(const float* values, int64_t k, float* partials,
+                        float* total, void* stream);
+
+/* total[0] += sum(grad[mask]^2)
+ *                 -- masked_norm_sq_contribution, kernels.py:284-302.
+ * Deterministic two-stage reduction (the reference uses a float atomic). */
+int sga_masked_norm_sq(const float* grad, const uint8_t* mask, int64_t n,
+                       float* partials, float* total, void* stream);
+
+/* block gather / scatter  -- gather_selected_blocks / scatter_selected_blocks,
+ * kernels.py:190-249 */
+int sga_gather_selected_blocks(const float* grad, const uint8_t* mask,
+                               const int32_t* block_idx, float* values,
+                               int64_t kb, int x, float factor, int64_t n_grad,
+                               void* stream);
+int sga_scatter_selected_blocks(float* dst, const uint8_t* mask,
+                                const int32_t* block_idx, const float* src,
+                                int64_t kb, int x, int64_t n_dst, void* stream);
+
+/* ---- support: mask -> sorted int32 idx (sga/support.py:57-99) ----------- */
+
+/* Phase 1: per-chunk set-byte counts + total.  chunk_counts has
+ * sga_mask_chunks(n) uint32 entries and is turned into exclusive offsets;
+ * total[0] (device, int64) receives k. */
+int64_t sga_mask_chunks(int64_t n);
+int sga_mask_count(const uint8_t* mask, int64_t n, uint32_t* chunk_counts,
+                   int64_t* total, void* stream);
+/* Phase 2: idx_out[..k) = ascending positions of the non-zero bytes. */
+int sga_mask_fill(const uint8_t* mask, int64_t n, const uint32_t* chunk_offsets,
+                  int32_t* idx_out, int64_t idx_capacity, void* stream);
+
+/* ---- residual-aware AdamW (sga/plugins/optimizer/adamw.py) -------------- */
+
+/* adamw_grad_correct / _grad_correct_kernel, adamw.py:88-213, 502-634.
+ * emit_mode -1 = sparse step, 0..3 = full step writing that score into g.
+ * flags: SGA_GC_*.  interval is the fold divisor (fp32 division). */
+int sga_adamw_grad_correct(float* p, float* g, float* m, float* v,
+                           const uint8_t* mask, int64_t n, float lr,
+                           float beta1, float om1, float beta2, float om2,
+                           float eps, float wd, float bc1, float bc2,
+                           float coeff, float interval, float lr_inactive,
+                           int emit_mode, int flags, void* stream);
+
+/* adamw_grad_correct_compact, adamw.py:217-322, 637-792: the commit reads its
+ * gradient from the bucket-level sorted (idx, values) by merge-join.
+ * flags: SGA_GC_APPLY_COEFF | SGA_GC_FOLD.  dir_table may be NULL. */
+int sga_adamw_grad_correct_compact(float* p, float* g, float* m, float* v,
+                                   const int32_t* idx, const void* values,
+                                   int values_dtype, int64_t rec_start,
+                                   int64_t n, int64_t k_total, float lr,
+                                   float beta1, float om1, float beta2,
+                                   float om2, float eps, float wd, float bc1,
+                                   float bc2, float coeff, float interval,
+                                   int flags, const int32_t* dir_table,
+                                   int64_t n_table, void* stream);
+
+/* build_dir_table, adamw.py:325-349, 472-499:
+ * table[j] = lower_bound(idx, j*1024), j < n_table. */
+int sga_build_dir_table(const int32_t* idx, int64_t k, int32_t* table,
+                        int64_t n_table, void* stream);
+
+/* ---- exact top-k selection --------------------------------------------- */
+
+/* Workspace for every select entry point over n elements. */
+size_t sga_select_workspace_bytes(int64_t n);
+
+/* select_topk_flat / shard_select (replay.py:538-572, replay_fused.py:290-402)
+ * and select_masks_histogram(mode="exact") (_histogram.py:161-201) on one
+ * contiguous fp32 score array (sign is stripped).  Writes mask_out[n] (0/1)
+ * and *result (device).  Runs entirely on the stream, no host sync. */
+int sga_select_topk(const float* score, int64_t n, int64_t k, int tie_mode,
+                    uint8_t* mask_out, sga_select_result* result, void* ws,
+                    size_t ws_bytes, void* stream);
+
+/* The same select over several disjoint runs (the online plugin's per-param
+ * views, _histogram.py:97-112): begin, then per radix level one hist call per
+ * run followed by one scan; then count per run, tile scan, mask per run.
+ * tile_base is the run's first chunk index: runs are laid out back to back
+ * in chunk space, each starting on a fresh 1024-element chunk. */
+int sga_sel_begin(int64_t k, void* ws, size_t ws_bytes, void* stream);
+int sga_sel_hist(const float* score, int64_t n, int level, void* ws,
+                 size_t ws_bytes, void* stream);
+int sga_sel_scan(int level, void* ws, size_t ws_bytes, void* stream);
+int sga_sel_count(const float* score, int64_t n, int64_t tile_base, void* ws,
+                  size_t ws_bytes, void* stream);
+int sga_sel_tile_scan(int64_t n_tiles, int tie_mode, void* ws, size_t ws_bytes,
+                      void* stream);
+int sga_sel_mask(const float* score, int64_t n, int64_t tile_base,
+                 int tie_mode, uint8_t* mask_out, void* ws, size_t ws_bytes,
+                 void* stream);
+int sga_sel_result(sga_select_result* result, void* ws, size_t ws_bytes,
+                   void* stream);
+
+/* Balanced / fast histogram select (_histogram.py:115-123, 203-216): the
+ * histogram over a stride subsample, mask = top-bits >= crossing bin.
+ * hist is int64[nbins] on the device and is ACCUMULATED into. */
+int sga_hist_topbits(const float* score, int64_t n, int shift, int stride,
+                     int phase, int64_t* hist, int nbins, uint32_t* nonfinite,
+                     void* stream);
+int sga_mask_topbits_ge(const float* score, int64_t n, int shift, int32_t bin,
+                        uint8_t* mask_out, void* stream);
+
+/* replay_kernels.py:372-414 building blocks with the same outputs. */
+int sga_cand_extract_count(const float* score, int64_t n, int32_t bin,
+                           uint32_t* chunk_counts, int64_t* total,
+                           void* stream);
+int sga_cand_extract_fill(const float* score, int64_t n, int32_t bin,
+                          const uint32_t* chunk_offsets, float* cand,
+                          int64_t cand_capacity, void* stream);
+int sga_gt_eq(const float* score, int64_t n, float thresh, uint8_t* gt,
+              uint8_t* eq, int32_t* counts2, void* stream);
+
+/* ---- score formulas and replay commit (sga/replay_kernels.py) ----------- */
+
+/* formula(name): out = score(w,m,v,g); absolute != 0 stores |score|.
+ * scores.py:147-269 / replay_kernels.py:109-160.  adams != 0 substitutes
+ * v := m*m and bc := 1 (replay.py:486-505). */
+int sga_score_formula(int score_id, const float* w, const float* m,
+                      const float* v, const float* g, float* out, int64_t n,
+                      float beta1, float om1, float beta2, float om2, float wd,
+                      float bc1, float bc2, float eps, int absolute, int adams,
+                      void* stream);
+
+/* opt_step_inplace / _k_adam, replay_kernels.py:163-216, 330-369 and
+ * replay.py:674-744.  flags: SGA_RP_*. */
+int sga_opt_step_inplace(const float* q, float* m, float* v, float* w,
+                         float* lab, const uint8_t* inactive, int64_t n,
+                         float beta1, float om1, float beta2, float om2,
+                         float bc1, float bc2, float eps, float omlwd,
+                         float neglr, float lr2, float lr, float lr_inactive,
+                         float wd, int flags, void* stream);
+
+/* ---- fused per-rank sparse step ----------------------------------------- */
+
+/* One pass pair over a flat bucket: buf = resid + g; score; exact top-k
+ * (lowest-index ties); idx/values pack; resid <- buf with selected coords
+ * zeroed; sparse AdamW commit on p/m/v (engine order: engine.py:416-604,
+ * pack kernels.py:166-187, commit adamw.py:637-724).
+ * g_dtype / values_dtype: SGA_F32 | SGA_BF16.  mask_out may be NULL.
+ * idx_out / values_out need room for k entries.  segs is a DEVICE array. */
+size_t sga_fused_workspace_bytes(int64_t n);
+int sga_fused_sparse_step(const void* g, int g_dtype, float* resid, float* p,
+                          float* m, float* v, int64_t n, int64_t k,
+                          const sga_segment* segs, int n_segs, int score_id,
+                          int32_t* idx_out, void* values_out, int values_dtype,
+                          uint8_t* mask_out, float factor, float coeff,
+                          int fast, sga_select_result* result, void* ws,
+                          size_t ws_bytes, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SGA_HIP_H_ */

@@ -1,0 +1,96 @@
+// Shared AdamW arithmetic.  Every operation is a separately rounded IEEE fp32
+// op (translation units are built with -ffp-contract=off); FMAs appear only
+// where written explicitly.
+#pragma once
+#include "common.hpp"
+
+namespace sga {
+
+struct Hyper {
+  float lr, b1, om1, b2, om2, eps, wd, bc1, bc2;
+};
+
+struct Commit {
+  float m_new, v_new, u, upd;
+};
+
+#ifdef __HIPCC__
+__device__ __forceinline__ Hyper hyper_of(const sga_segment& s) {
+  Hyper h;
+  h.lr = s.lr; h.b1 = s.beta1; h.om1 = s.om1; h.b2 = s.beta2; h.om2 = s.om2;
+  h.eps = s.eps; h.wd = s.wd; h.bc1 = s.bc1; h.bc2 = s.bc2;
+  return h;
+}
+
+// Online commit chain (torch elementwise ops, one rounding each):
+//   sa = m*b1 + g*(1-b1)          sb = v*b2 + (g*(1-b2))*g
+//   m' = sa                        v' = sb
+//   u  = (sa/bc1) / (sqrt(sb/bc2) + eps)      upd = wd*p + u
+__device__ __forceinline__ Commit adamw_commit(float p, float g, float m, float v,
+                                               const Hyper& h) {
+  Commit c;
+  const float sa = m * h.b1 + g * h.om1;
+  const float sb = v * h.b2 + (g * h.om2) * g;
+  c.m_new = sa;
+  c.v_new = sb;
+  const float mh = __fdiv_rn(sa, h.bc1);
+  const float vh = __fdiv_rn(sb, h.bc2);
+  const float den = __fsqrt_rn(vh) + h.eps;
+  c.u = __fdiv_rn(mh, den);
+  c.upd = h.wd * p + c.u;
+  return c;
+}
+
+// U(0): the direction the same commit would take with a zero gradient.
+__device__ __forceinline__ float coi_u0(float m, float v, const Hyper& h) {
+  const float num = __fdiv_rn(m * h.b1, h.bc1);
+  const float den = __fsqrt_rn(__fdiv_rn(v * h.b2, h.bc2)) + h.eps;
+  return __fdiv_rn(num, den);
+}
+
+// Signed registry score.  SCORE: 0 update, 1 g, 2 m, 3 coi (already >= 0).
+template <int SCORE>
+__device__ __forceinline__ float score_value(float q, float p, float m, float v, const Hyper& h) {
+  if (SCORE == SGA_SCORE_ABS_G) return fabsf(q);
+  if (SCORE == SGA_SCORE_ABS_M) return fabsf(m);
+  const Commit c = adamw_commit(p, q, m, v, h);
+  if (SCORE == SGA_SCORE_UPDATE) return c.upd;
+  return fabsf(c.u - coi_u0(m, v, h));
+}
+template <int SCORE>
+__device__ __forceinline__ uint32_t score_key(float q, float p, float m, float v, const Hyper& h) {
+  return abs_key(score_value<SCORE>(q, p, m, v, h));
+}
+
+// Segment cursor: segments tile [0, n) in ascending order.
+struct SegCursor {
+  const sga_segment* segs;
+  int n_segs;
+  int64_t lo, hi;
+  Hyper h;
+  __device__ __forceinline__ void init(const sga_segment* s, int ns) {
+    segs = s; n_segs = ns; lo = 1; hi = 0;
+  }
+  __device__ __forceinline__ void seek(int64_t i) {
+    if (i >= lo && i < hi) return;
+    int a = 0, b = n_segs - 1;
+    while (a < b) {                      // last segment with start <= i
+      const int mid = (a + b + 1) >> 1;
+      if (segs[mid].start <= i) a = mid; else b = mid - 1;
+    }
+    lo = segs[a].start;
+    hi = lo + segs[a].n;
+    h = hyper_of(segs[a]);
+  }
+};
+#endif
+
+static inline Hyper mk_hyper(float lr, float b1, float om1, float b2, float om2, float eps,
+                             float wd, float bc1, float bc2) {
+  Hyper h;
+  h.lr = lr; h.b1 = b1; h.om1 = om1; h.b2 = b2; h.om2 = om2; h.eps = eps;
+  h.wd = wd; h.bc1 = bc1; h.bc2 = bc2;
+  return h;
+}
+
+}  // namespace sga

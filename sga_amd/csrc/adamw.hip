@@ -1,0 +1,290 @@
+// Residual-aware AdamW commit: masked / full-step / compact (merge-join) forms.
+//
+// Arithmetic recipe: every multiply, add, divide and square root below is a
+// separately rounded IEEE fp32 operation (the translation unit is compiled
+// with -ffp-contract=off), in the order of the torch elementwise chain
+//     sa = m*b1 + g*(1-b1)            sb = v*b2 + (g*(1-b2))*g
+//     m' = sa                          v' = sb
+//     upd = wd*p + (sa/bc1) / (sqrt(sb/bc2) + eps)
+//     p'  = p - lr*upd
+// so m'/v' are bit-identical to a correctly rounded host evaluation and p'
+// differs only where the host library's sqrt is not correctly rounded.
+#include "adam_math.hpp"
+
+namespace sga {
+
+// EMIT: -1 sparse step; 0 update, 1 |g|, 2 |m|, 3 coi -> written into g.
+template <int EMIT>
+__global__ __launch_bounds__(kBlock) void k_grad_correct(
+    float* __restrict__ p, float* __restrict__ g, float* __restrict__ m,
+    float* __restrict__ v, const uint8_t* __restrict__ mask, int64_t n, Hyper h,
+    float coeff, float interval, float lr_inactive, int flags, bool vec) {
+  const bool has_mask = flags & SGA_GC_HAS_MASK;
+  const bool apply_coeff = flags & SGA_GC_APPLY_COEFF;
+  const bool clear = flags & SGA_GC_CLEAR;
+  const bool fold = flags & SGA_GC_FOLD;
+  const bool split = flags & SGA_GC_LR_SPLIT;
+  const int64_t stride = (int64_t)gridDim.x * kBlock * kVec;
+  for (int64_t i = ((int64_t)blockIdx.x * kBlock + threadIdx.x) * kVec; i < n;
+       i += stride) {
+    float pp[4], gg[4], mm[4], vv[4];
+    uint32_t mk[4] = {1, 1, 1, 1};
+    load4_f32(p, i, n, pp, vec);
+    load4_f32(g, i, n, gg, vec);
+    load4_f32(m, i, n, mm, vec);
+    load4_f32(v, i, n, vv, vec);
+    if (has_mask) load4_u8(mask, i, n, mk, vec);
+    float gout[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const bool active = mk[e] != 0;
+      const float raw = gg[e];
+      float ge = raw;
+      if (EMIT < 0 && has_mask && !active) ge = 0.0f;
+      if (apply_coeff && active) ge = ge * coeff;
+      const Commit c = adamw_commit(pp[e], ge, mm[e], vv[e], h);
+      if (EMIT == 0) gout[e] = c.upd;
+      else if (EMIT == 1) gout[e] = fabsf(ge);
+      else if (EMIT == 2) gout[e] = fabsf(mm[e]);
+      else if (EMIT == 3) gout[e] = fabsf(c.u - coi_u0(mm[e], vv[e], h));
+      else {
+        float t = (clear && active) ? 0.0f : raw;
+        if (fold) t = __fdiv_rn(t, interval);
+        gout[e] = t;
+      }
+      const float lr_a = (split && !active) ? lr_inactive : h.lr;
+      pp[e] = pp[e] - lr_a * c.upd;
+      mm[e] = c.m_new;
+      vv[e] = c.v_new;
+    }
+    store4_f32(m, i, n, mm, vec);
+    store4_f32(v, i, n, vv, vec);
+    if (EMIT >= 0 || clear || fold) store4_f32(g, i, n, gout, vec);
+    store4_f32(p, i, n, pp, vec);
+  }
+}
+
+// ---------------------------------------------------------------- compact
+// A workgroup owns kBlockSpan consecutive coordinates of the record.  The
+// slice [lo, hi) of the bucket's sorted idx that falls in the span is found
+// with two 64-way cooperative searches (<= 6 rounds for k < 2^31, or <= 2
+// rounds from a directory-table bracket), staged through LDS as a dense
+// (value, found-bit) span, and consumed by the same commit arithmetic.
+__device__ __forceinline__ int64_t coop_lower_bound(
+    const int32_t* __restrict__ idx, int64_t lo, int64_t hi, int64_t key) {
+  // all 64 lanes of the calling wave participate; returns the first
+  // position in [lo, hi] whose entry is >= key (hi when none).
+  while (hi - lo > 0) {
+    const int64_t width = hi - lo;
+    const int64_t step = (width + kWave - 1) / kWave;   // >= 1
+    const int64_t probe = lo + (int64_t)lane_id() * step;
+    bool less = false;
+    if (probe < hi) less = (int64_t)idx[probe] < key;
+    const uint64_t b = ballot64(less);
+    // entries are sorted, so `less` lanes form a prefix
+    const int cnt = __popcll(b);
+    if (cnt == 0) { hi = lo; break; }
+    const int64_t last_less = lo + (int64_t)(cnt - 1) * step;
+    const int64_t nlo = last_less + 1;
+    int64_t nhi = lo + (int64_t)cnt * step;
+    if (nhi > hi) nhi = hi;
+    lo = nlo;
+    hi = nhi;
+  }
+  return lo;
+}
+
+template <bool BF16>
+__global__ __launch_bounds__(kBlock) void k_grad_correct_compact(
+    float* __restrict__ p, float* __restrict__ g, float* __restrict__ m,
+    float* __restrict__ v, const int32_t* __restrict__ idx,
+    const void* __restrict__ values, int64_t rec_start, int64_t n,
+    int64_t k_total, Hyper h, float coeff, float interval, int flags,
+    const int32_t* __restrict__ table, int64_t n_table, bool vec) {
+  __shared__ float s_val[kBlockSpan];
+  __shared__ uint32_t s_found[kBlockSpan / 32];
+  __shared__ int64_t s_bounds[2];
+  const bool apply_coeff = flags & SGA_GC_APPLY_COEFF;
+  const bool fold = flags & SGA_GC_FOLD;
+  const int64_t n_spans = cdiv64(n, kBlockSpan);
+  for (int64_t span = blockIdx.x; span < n_spans; span += gridDim.x) {
+    const int64_t off0 = span * kBlockSpan;
+    const int64_t c0 = rec_start + off0;
+    int64_t c1 = c0 + kBlockSpan;
+    if (c1 > rec_start + n) c1 = rec_start + n;
+    for (int t = threadIdx.x; t < kBlockSpan; t += kBlock) s_val[t] = 0.0f;
+    if (threadIdx.x < kBlockSpan / 32) s_found[threadIdx.x] = 0u;
+    if (wave_id() < 2) {
+      const int64_t key = wave_id() == 0 ? c0 : c1;
+      int64_t lo = 0, hi = k_total;
+      if (table) {
+        const int64_t j = key >> 10;
+        if (j < n_table) {
+          lo = table[j];
+          hi = lo + (key & 1023);
+          if (hi > k_total) hi = k_total;
+          if (lo > k_total) lo = k_total;
+        }
+      }
+      const int64_t r = coop_lower_bound(idx, lo, hi, key);
+      if (lane_id() == 0) s_bounds[wave_id()] = r;
+    }
+    __syncthreads();
+    const int64_t lo = s_bounds[0], hi = s_bounds[1];
+    for (int64_t j = lo + threadIdx.x; j < hi; j += kBlock) {
+      const int64_t t = (int64_t)idx[j] - c0;
+      if (t >= 0 && t < kBlockSpan) {
+        float x = BF16 ? bf16_to_f32(reinterpret_cast<const uint16_t*>(values)[j])
+                       : reinterpret_cast<const float*>(values)[j];
+        s_val[t] = x;
+        atomicOr(&s_found[t >> 5], 1u << (t & 31));
+      }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int it = 0; it < kChunkIters; ++it) {
+      const int t0 = it * (kBlock * kVec) + threadIdx.x * kVec;
+      const int64_t i = off0 + t0;
+      if (i < n) {
+        float pp[4], mm[4], vv[4], raw[4] = {0, 0, 0, 0};
+        load4_f32(p, i, n, pp, vec);
+        load4_f32(m, i, n, mm, vec);
+        load4_f32(v, i, n, vv, vec);
+        if (fold) load4_f32(g, i, n, raw, vec);
+        const uint32_t fw = s_found[t0 >> 5] >> (t0 & 31);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const bool found = (fw >> e) & 1u;
+          float ge = s_val[t0 + e];
+          if (apply_coeff && found) ge = ge * coeff;
+          const Commit c = adamw_commit(pp[e], ge, mm[e], vv[e], h);
+          pp[e] = pp[e] - h.lr * c.upd;
+          mm[e] = c.m_new;
+          vv[e] = c.v_new;
+          if (fold && !found) raw[e] = __fdiv_rn(raw[e], interval);
+        }
+        store4_f32(m, i, n, mm, vec);
+        store4_f32(v, i, n, vv, vec);
+        if (fold) store4_f32(g, i, n, raw, vec);
+        store4_f32(p, i, n, pp, vec);
+      }
+    }
+    __syncthreads();
+  }
+}
+
+__global__ __launch_bounds__(kBlock) void k_dir_table(
+    const int32_t* __restrict__ idx, int64_t k, int32_t* __restrict__ table,
+    int64_t n_table) {
+  for (int64_t j = (int64_t)blockIdx.x * kBlock + threadIdx.x; j < n_table;
+       j += (int64_t)gridDim.x * kBlock) {
+    const int64_t key = j * 1024;
+    int64_t a = 0, b = k;
+    while (a < b) {
+      const int64_t mid = a + (b - a) / 2;
+      if ((int64_t)idx[mid] < key) a = mid + 1; else b = mid;
+    }
+    table[j] = (int32_t)a;
+  }
+}
+
+}  // namespace sga
+
+using namespace sga;
+
+extern "C" int sga_adamw_grad_correct(float* p, float* g, float* m, float* v,
+                                      const uint8_t* mask, int64_t n, float lr,
+                                      float beta1, float om1, float beta2,
+                                      float om2, float eps, float wd, float bc1,
+                                      float bc2, float coeff, float interval,
+                                      float lr_inactive, int emit_mode,
+                                      int flags, void* stream) {
+  if (n == 0) return SGA_OK;
+  if (!p || !g || !m || !v || n < 0 || emit_mode < -1 || emit_mode > 3) {
+    set_error("sga_adamw_grad_correct: bad argument (n=%lld emit_mode=%d)",
+              (long long)n, emit_mode);
+    return SGA_ERR_ARG;
+  }
+  if ((flags & SGA_GC_HAS_MASK) && !mask) {
+    set_error("sga_adamw_grad_correct: HAS_MASK without a mask pointer");
+    return SGA_ERR_ARG;
+  }
+  if ((flags & (SGA_GC_APPLY_COEFF | SGA_GC_CLEAR | SGA_GC_FOLD)) &&
+      (emit_mode >= 0 || !(flags & SGA_GC_HAS_MASK))) {
+    set_error("sga_adamw_grad_correct: coeff/clear/fold need a sparse step with a mask");
+    return SGA_ERR_ARG;
+  }
+  if ((flags & SGA_GC_LR_SPLIT) && (emit_mode < 0 || !(flags & SGA_GC_HAS_MASK))) {
+    set_error("sga_adamw_grad_correct: LR_SPLIT needs a full step with a mask");
+    return SGA_ERR_ARG;
+  }
+  if (flags & SGA_GC_ADAMS) {
+    set_error("sga_adamw_grad_correct: the AdamS recursion is not built");
+    return SGA_ERR_ARG;
+  }
+  const Hyper h = mk_hyper(lr, beta1, om1, beta2, om2, eps, wd, bc1, bc2);
+  const bool vec = aligned4(p, 4) && aligned4(g, 4) && aligned4(m, 4) &&
+                   aligned4(v, 4) && aligned4(mask, 1);
+  dim3 grid(stream_grid(n, (int64_t)kBlock * kVec)), block(kBlock);
+  hipStream_t st = (hipStream_t)stream;
+#define SGA_GC_LAUNCH(E)                                                       \
+  hipLaunchKernelGGL((k_grad_correct<E>), grid, block, 0, st, p, g, m, v, mask, \
+                     n, h, coeff, interval, lr_inactive, flags, vec)
+  switch (emit_mode) {
+    case -1: SGA_GC_LAUNCH(-1); break;
+    case 0: SGA_GC_LAUNCH(0); break;
+    case 1: SGA_GC_LAUNCH(1); break;
+    case 2: SGA_GC_LAUNCH(2); break;
+    default: SGA_GC_LAUNCH(3); break;
+  }
+#undef SGA_GC_LAUNCH
+  return check_launch("sga_adamw_grad_correct");
+}
+
+extern "C" int sga_adamw_grad_correct_compact(
+    float* p, float* g, float* m, float* v, const int32_t* idx,
+    const void* values, int values_dtype, int64_t rec_start, int64_t n,
+    int64_t k_total, float lr, float beta1, float om1, float beta2, float om2,
+    float eps, float wd, float bc1, float bc2, float coeff, float interval,
+    int flags, const int32_t* dir_table, int64_t n_table, void* stream) {
+  if (n == 0) return SGA_OK;
+  if (!p || !m || !v || n < 0 || k_total < 0 || rec_start < 0 ||
+      (k_total > 0 && (!idx || !values)) ||
+      ((flags & SGA_GC_FOLD) && !g) ||
+      (values_dtype != SGA_F32 && values_dtype != SGA_BF16)) {
+    set_error("sga_adamw_grad_correct_compact: bad argument");
+    return SGA_ERR_ARG;
+  }
+  if (k_total + 1024 >= (1ll << 31) || rec_start + n + 1024 >= (1ll << 31)) {
+    set_error("sga_adamw_grad_correct_compact: offsets must stay < 2^31 (k_total=%lld, rec_start+n=%lld)",
+              (long long)k_total, (long long)(rec_start + n));
+    return SGA_ERR_ARG;
+  }
+  if (dir_table && n_table < ((rec_start + n - 1) >> 10) + 2) {
+    set_error("sga_adamw_grad_correct_compact: dir_table has %lld entries, needs >= %lld",
+              (long long)n_table, (long long)(((rec_start + n - 1) >> 10) + 2));
+    return SGA_ERR_ARG;
+  }
+  const Hyper h = mk_hyper(lr, beta1, om1, beta2, om2, eps, wd, bc1, bc2);
+  const bool vec = aligned4(p, 4) && aligned4(g, 4) && aligned4(m, 4) && aligned4(v, 4);
+  dim3 grid(stream_grid(n, kBlockSpan)), block(kBlock);
+  hipStream_t st = (hipStream_t)stream;
+  if (values_dtype == SGA_BF16)
+    hipLaunchKernelGGL((k_grad_correct_compact<true>), grid, block, 0, st, p, g, m, v, idx, values, rec_start, n, k_total, h, coeff, interval, flags, dir_table, n_table, vec);
+  else
+    hipLaunchKernelGGL((k_grad_correct_compact<false>), grid, block, 0, st, p, g, m, v, idx, values, rec_start, n, k_total, h, coeff, interval, flags, dir_table, n_table, vec);
+  return check_launch("sga_adamw_grad_correct_compact");
+}
+
+extern "C" int sga_build_dir_table(const int32_t* idx, int64_t k, int32_t* table,
+                                   int64_t n_table, void* stream) {
+  if (n_table == 0) return SGA_OK;
+  if (!table || n_table < 0 || k < 0 || (k > 0 && !idx) ||
+      (n_table - 1) * 1024 >= (1ll << 31)) {
+    set_error("sga_build_dir_table: bad argument ((n_table-1)*1024 must stay < 2^31)");
+    return SGA_ERR_ARG;
+  }
+  hipLaunchKernelGGL(k_dir_table, dim3(stream_grid(n_table, kBlock)),
+                     dim3(kBlock), 0, (hipStream_t)stream, idx, k, table, n_table);
+  return check_launch("sga_build_dir_table");
+}

@@ -1,0 +1,160 @@
+// Shared device/host helpers for the gfx950 (CDNA4, wave64) kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/sga_hip.h"
+
+namespace sga {
+
+constexpr int kWave = 64;
+constexpr int kBlock = 256;            // 4 waves per workgroup
+constexpr int kVec = 4;                // 128-bit fp32 vectors
+constexpr int kChunkIters = 4;         // vectors per lane per chunk
+constexpr int kChunk = kWave * kVec * kChunkIters;   // 1024 elements / wave
+constexpr int kChunksPerBlock = kBlock / kWave;      // 4
+constexpr int kBlockSpan = kChunk * kChunksPerBlock; // 4096 elements / block
+
+void set_error(const char* fmt, ...);
+int check_launch(const char* what);
+
+__host__ __device__ static inline int64_t cdiv64(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+// Grid for streaming kernels that loop grid-stride: enough workgroups to fill
+// 256 CUs several times over, never more than the work needs.
+static inline unsigned stream_grid(int64_t n_items, int64_t items_per_block,
+                                   int64_t max_blocks = 256 * 16) {
+  int64_t b = cdiv64(n_items, items_per_block);
+  if (b < 1) b = 1;
+  if (b > max_blocks) b = max_blocks;
+  return (unsigned)b;
+}
+
+// True when p is aligned for 4-element vector access of `elem` bytes each.
+static inline bool aligned4(const void* p, int elem) {
+  return p == nullptr || (reinterpret_cast<uintptr_t>(p) % (4 * (size_t)elem)) == 0;
+}
+
+#ifdef __HIPCC__
+
+__device__ __forceinline__ uint32_t f2u(float x) { return __float_as_uint(x); }
+__device__ __forceinline__ float u2f(uint32_t x) { return __uint_as_float(x); }
+__device__ __forceinline__ uint32_t abs_key(float x) {
+  return __float_as_uint(x) & 0x7FFFFFFFu;
+}
+
+// bf16 <-> fp32, round-to-nearest-even, NaN -> quiet NaN (torch's rule).
+__device__ __forceinline__ float bf16_to_f32(uint16_t h) {
+  return __uint_as_float(((uint32_t)h) << 16);
+}
+__device__ __forceinline__ uint16_t f32_to_bf16(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7FFFFFFFu) > 0x7F800000u) return 0x7FC0;
+  u += 0x7FFFu + ((u >> 16) & 1u);
+  return (uint16_t)(u >> 16);
+}
+
+__device__ __forceinline__ int lane_id() { return threadIdx.x & (kWave - 1); }
+__device__ __forceinline__ int wave_id() { return threadIdx.x >> 6; }
+
+// Number of set bits of `mask` strictly below the calling lane.
+__device__ __forceinline__ uint32_t lanes_below(uint64_t mask) {
+  return __builtin_amdgcn_mbcnt_hi((uint32_t)(mask >> 32),
+                                   __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0u));
+}
+
+__device__ __forceinline__ uint64_t ballot64(bool p) { return __ballot(p); }
+
+template <typename T>
+__device__ __forceinline__ T wave_sum(T v) {
+#pragma unroll
+  for (int o = kWave / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
+  return v;
+}
+
+// Inclusive scan across the 64 lanes of a wave.
+__device__ __forceinline__ uint32_t wave_incl_scan(uint32_t v) {
+  const int l = lane_id();
+#pragma unroll
+  for (int o = 1; o < kWave; o <<= 1) {
+    uint32_t t = __shfl_up(v, o, kWave);
+    if (l >= o) v += t;
+  }
+  return v;
+}
+
+struct alignas(16) F4 { float x, y, z, w; };
+struct alignas(8) H4 { uint16_t x, y, z, w; };
+struct alignas(16) U4 { uint32_t x, y, z, w; };
+struct alignas(4) B4 { uint8_t x, y, z, w; };
+
+__device__ __forceinline__ F4 ld4(const float* p) {
+  return *reinterpret_cast<const F4*>(p);
+}
+__device__ __forceinline__ void st4(float* p, const F4& v) {
+  *reinterpret_cast<F4*>(p) = v;
+}
+
+// Load 4 consecutive elements starting at i (i % 4 == 0 relative to a
+// 16-byte aligned base) with a scalar tail when fewer than 4 remain.
+__device__ __forceinline__ void load4_f32(const float* base, int64_t i,
+                                          int64_t n, float out[4],
+                                          bool vec = true) {
+  if (vec && i + 4 <= n) {
+    F4 v = ld4(base + i);
+    out[0] = v.x; out[1] = v.y; out[2] = v.z; out[3] = v.w;
+  } else {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) out[e] = (i + e < n) ? base[i + e] : 0.0f;
+  }
+}
+__device__ __forceinline__ void load4_bf16(const uint16_t* base, int64_t i,
+                                           int64_t n, float out[4],
+                                           bool vec = true) {
+  if (vec && i + 4 <= n) {
+    H4 v = *reinterpret_cast<const H4*>(base + i);
+    out[0] = bf16_to_f32(v.x); out[1] = bf16_to_f32(v.y);
+    out[2] = bf16_to_f32(v.z); out[3] = bf16_to_f32(v.w);
+  } else {
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+      out[e] = (i + e < n) ? bf16_to_f32(base[i + e]) : 0.0f;
+  }
+}
+__device__ __forceinline__ void load4_u8(const uint8_t* base, int64_t i,
+                                         int64_t n, uint32_t out[4],
+                                         bool vec = true) {
+  if (vec && i + 4 <= n) {
+    B4 v = *reinterpret_cast<const B4*>(base + i);
+    out[0] = v.x; out[1] = v.y; out[2] = v.z; out[3] = v.w;
+  } else {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) out[e] = (i + e < n) ? base[i + e] : 0u;
+  }
+}
+__device__ __forceinline__ void store4_f32(float* base, int64_t i, int64_t n,
+                                           const float v[4], bool vec = true) {
+  if (vec && i + 4 <= n) {
+    F4 t{v[0], v[1], v[2], v[3]};
+    st4(base + i, t);
+  } else {
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+      if (i + e < n) base[i + e] = v[e];
+  }
+}
+__device__ __forceinline__ void store4_u8(uint8_t* base, int64_t i, int64_t n,
+                                          const uint32_t v[4], bool vec = true) {
+  if (vec && i + 4 <= n) {
+    B4 t{(uint8_t)v[0], (uint8_t)v[1], (uint8_t)v[2], (uint8_t)v[3]};
+    *reinterpret_cast<B4*>(base + i) = t;
+  } else {
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+      if (i + e < n) base[i + e] = (uint8_t)v[e];
+  }
+}
+
+#endif  // __HIPCC__
+
+}  // namespace sga

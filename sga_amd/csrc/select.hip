@@ -1,0 +1,323 @@
+// Exact top-k selection entry points over fp32 score arrays, plus the
+// histogram / candidate / compare building blocks of the replay select.
+#include "select_impl.hpp"
+
+namespace sga {
+int exclusive_scan_u32(uint32_t* data, int64_t n, int64_t* total, hipStream_t st);
+int64_t scan_scratch_entries(int64_t n);
+
+// int64 histogram of (|x| bits >> shift) over a strided subsample; bins in
+// LDS when they fit (4097 coarse bins), otherwise straight to global.
+__global__ __launch_bounds__(kBlock) void k_hist_topbits(
+    const float* __restrict__ x, int64_t n, int shift, int stride, int phase,
+    unsigned long long* __restrict__ hist, int nbins, uint32_t* __restrict__ nonfinite) {
+  extern __shared__ uint32_t s_h[];
+  for (int b = threadIdx.x; b < nbins; b += kBlock) s_h[b] = 0u;
+  __syncthreads();
+  const int64_t n_s = n <= phase ? 0 : (n - phase + stride - 1) / stride;
+  uint32_t nf = 0;
+  const int64_t step = (int64_t)gridDim.x * kBlock;
+  for (int64_t base = (int64_t)blockIdx.x * kBlock; base < n_s; base += step) {
+    const int64_t j = base + threadIdx.x;
+    const bool ok = j < n_s;
+    uint32_t key = 0;
+    if (ok) key = abs_key(x[phase + j * stride]);
+    nf += (ok && key >= 0x7F800000u);
+    uint32_t bin = key >> shift;
+    if (bin >= (uint32_t)nbins) bin = nbins - 1;
+    lds_hist_add(s_h, bin, ok);
+  }
+  __syncthreads();
+  for (int b = threadIdx.x; b < nbins; b += kBlock) {
+    const uint32_t c = s_h[b];
+    if (c) atomicAdd(&hist[b], (unsigned long long)c);
+  }
+  nf = wave_sum(nf);
+  if (lane_id() == 0 && nf && nonfinite) atomicAdd(nonfinite, nf);
+}
+
+__global__ __launch_bounds__(kBlock) void k_mask_topbits_ge(
+    const float* __restrict__ x, int64_t n, int shift, uint32_t bin,
+    uint8_t* __restrict__ mask, bool vec) {
+  const int64_t stride = (int64_t)gridDim.x * kBlock * kVec;
+  for (int64_t i = ((int64_t)blockIdx.x * kBlock + threadIdx.x) * kVec; i < n; i += stride) {
+    float v[4];
+    load4_f32(x, i, n, v, vec);
+    uint32_t mk[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) mk[e] = (abs_key(v[e]) >> shift) >= bin;
+    store4_u8(mask, i, n, mk, vec);
+  }
+}
+
+// Candidates of one top-16 bin, in ascending index order (two sweeps).
+__global__ __launch_bounds__(kBlock) void k_cand_count(
+    const float* __restrict__ x, int64_t n, uint32_t bin, uint32_t* __restrict__ counts,
+    int64_t n_chunks, bool vec) {
+  const int64_t wstride = (int64_t)gridDim.x * kChunksPerBlock;
+  for (int64_t c = (int64_t)blockIdx.x * kChunksPerBlock + wave_id(); c < n_chunks; c += wstride) {
+    uint32_t cnt = 0;
+#pragma unroll
+    for (int it = 0; it < kChunkIters; ++it) {
+      const int64_t i = c * kChunk + it * (kWave * kVec) + lane_id() * kVec;
+      float v[4] = {0, 0, 0, 0};
+      if (i < n) load4_f32(x, i, n, v, vec);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) cnt += (i + e < n && (abs_key(v[e]) >> 16) == bin);
+    }
+    cnt = wave_sum(cnt);
+    if (lane_id() == 0) counts[c] = cnt;
+  }
+}
+
+__global__ __launch_bounds__(kBlock) void k_cand_fill(
+    const float* __restrict__ x, int64_t n, uint32_t bin, const uint32_t* __restrict__ offsets,
+    float* __restrict__ cand, int64_t cap, int64_t n_chunks, bool vec) {
+  const int64_t wstride = (int64_t)gridDim.x * kChunksPerBlock;
+  for (int64_t c = (int64_t)blockIdx.x * kChunksPerBlock + wave_id(); c < n_chunks; c += wstride) {
+    uint32_t run = offsets[c];
+#pragma unroll
+    for (int it = 0; it < kChunkIters; ++it) {
+      const int64_t i = c * kChunk + it * (kWave * kVec) + lane_id() * kVec;
+      float v[4] = {0, 0, 0, 0};
+      if (i < n) load4_f32(x, i, n, v, vec);
+      bool hit[4];
+      uint32_t mine = 0;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        hit[e] = i + e < n && (abs_key(v[e]) >> 16) == bin;
+        mine += hit[e];
+      }
+      const uint32_t incl = wave_incl_scan(mine);
+      uint32_t pos = run + incl - mine;
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        if (hit[e]) {
+          if ((int64_t)pos < cap) cand[pos] = v[e];
+          ++pos;
+        }
+      run += __shfl(incl, kWave - 1, kWave);
+    }
+  }
+}
+
+__global__ __launch_bounds__(kBlock) void k_gt_eq(
+    const float* __restrict__ x, int64_t n, float thresh, uint8_t* __restrict__ gt,
+    uint8_t* __restrict__ eq, int32_t* __restrict__ counts, bool vec) {
+  uint32_t cg = 0, ce = 0;
+  const int64_t stride = (int64_t)gridDim.x * kBlock * kVec;
+  for (int64_t i = ((int64_t)blockIdx.x * kBlock + threadIdx.x) * kVec; i < n; i += stride) {
+    float v[4];
+    load4_f32(x, i, n, v, vec);
+    uint32_t g4[4], e4[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const bool ok = i + e < n;
+      g4[e] = ok && v[e] > thresh;
+      e4[e] = ok && v[e] == thresh;
+      cg += g4[e];
+      ce += e4[e];
+    }
+    store4_u8(gt, i, n, g4, vec);
+    store4_u8(eq, i, n, e4, vec);
+  }
+  cg = wave_sum(cg);
+  ce = wave_sum(ce);
+  if (lane_id() == 0) {
+    if (cg) atomicAdd(&counts[0], (int32_t)cg);
+    if (ce) atomicAdd(&counts[1], (int32_t)ce);
+  }
+}
+
+__global__ void k_zero_i32(int32_t* p, int n) {
+  for (int i = threadIdx.x; i < n; i += blockDim.x) p[i] = 0;
+}
+
+}  // namespace sga
+
+using namespace sga;
+
+extern "C" size_t sga_select_workspace_bytes(int64_t n) { return sel_ws_bytes(n < 0 ? 0 : n); }
+
+static int carve(void* ws, size_t bytes, int64_t tiles, SelWorkspace* w, const char* who) {
+  if (!sel_ws_carve(ws, bytes, tiles, w)) {
+    set_error("%s: workspace missing, misaligned (16 B) or too small for %lld chunks "
+              "(size it with sga_select_workspace_bytes)", who, (long long)tiles);
+    return SGA_ERR_WORKSPACE;
+  }
+  return SGA_OK;
+}
+
+extern "C" int sga_sel_begin(int64_t k, void* ws, size_t ws_bytes, void* stream) {
+  SelWorkspace w;
+  if (int rc = carve(ws, ws_bytes, 0, &w, "sga_sel_begin")) return rc;
+  if (k < 1 || k >= (1ll << 31)) {
+    set_error("sga_sel_begin: k=%lld out of range", (long long)k);
+    return SGA_ERR_ARG;
+  }
+  launch_begin((uint32_t)k, w, (hipStream_t)stream);
+  return check_launch("sga_sel_begin");
+}
+
+extern "C" int sga_sel_hist(const float* score, int64_t n, int level, void* ws,
+                            size_t ws_bytes, void* stream) {
+  if (n == 0) return SGA_OK;
+  SelWorkspace w;
+  if (int rc = carve(ws, ws_bytes, 0, &w, "sga_sel_hist")) return rc;
+  if (!score || n < 0 || n >= (1ll << 31) || level < 0 || level > 2) {
+    set_error("sga_sel_hist: bad argument");
+    return SGA_ERR_ARG;
+  }
+  SrcF32 src{score, aligned4(score, 4)};
+  launch_level_hist(src, n, level, w, (hipStream_t)stream);
+  return check_launch("sga_sel_hist");
+}
+
+extern "C" int sga_sel_scan(int level, void* ws, size_t ws_bytes, void* stream) {
+  SelWorkspace w;
+  if (int rc = carve(ws, ws_bytes, 0, &w, "sga_sel_scan")) return rc;
+  if (level < 0 || level > 2) { set_error("sga_sel_scan: bad level"); return SGA_ERR_ARG; }
+  launch_level_scan(level, w, (hipStream_t)stream);
+  return check_launch("sga_sel_scan");
+}
+
+extern "C" int sga_sel_count(const float* score, int64_t n, int64_t tile_base, void* ws,
+                             size_t ws_bytes, void* stream) {
+  if (n == 0) return SGA_OK;
+  SelWorkspace w;
+  if (int rc = carve(ws, ws_bytes, tile_base + cdiv64(n, kChunk), &w, "sga_sel_count")) return rc;
+  if (!score || n < 0 || tile_base < 0) { set_error("sga_sel_count: bad argument"); return SGA_ERR_ARG; }
+  SrcF32 src{score, aligned4(score, 4)};
+  launch_tile_count(src, n, tile_base, w, (hipStream_t)stream);
+  return check_launch("sga_sel_count");
+}
+
+extern "C" int sga_sel_tile_scan(int64_t n_tiles, int tie_mode, void* ws, size_t ws_bytes,
+                                 void* stream) {
+  SelWorkspace w;
+  if (int rc = carve(ws, ws_bytes, n_tiles, &w, "sga_sel_tile_scan")) return rc;
+  if (n_tiles < 1 || cdiv64(n_tiles, kTileScanSpan) > kMaxTileBlocks) {
+    set_error("sga_sel_tile_scan: n_tiles=%lld out of range", (long long)n_tiles);
+    return SGA_ERR_ARG;
+  }
+  launch_tile_scan(n_tiles, tie_mode == SGA_TIE_ALL, w, (hipStream_t)stream);
+  return check_launch("sga_sel_tile_scan");
+}
+
+extern "C" int sga_sel_mask(const float* score, int64_t n, int64_t tile_base, int tie_mode,
+                            uint8_t* mask_out, void* ws, size_t ws_bytes, void* stream) {
+  if (n == 0) return SGA_OK;
+  SelWorkspace w;
+  if (int rc = carve(ws, ws_bytes, tile_base + cdiv64(n, kChunk), &w, "sga_sel_mask")) return rc;
+  if (!score || !mask_out || n < 0 || tile_base < 0) { set_error("sga_sel_mask: bad argument"); return SGA_ERR_ARG; }
+  SrcF32 src{score, aligned4(score, 4)};
+  const int64_t nc = cdiv64(n, kChunk);
+  hipLaunchKernelGGL((k_write_mask<SrcF32>), dim3(stream_grid(nc, kChunksPerBlock)), dim3(kBlock), 0,
+                     (hipStream_t)stream, src, n, tile_base, tie_mode == SGA_TIE_ALL, w.st,
+                     w.tile_gt, w.tile_eq, mask_out, aligned4(mask_out, 1));
+  return check_launch("sga_sel_mask");
+}
+
+extern "C" int sga_sel_result(sga_select_result* result, void* ws, size_t ws_bytes, void* stream) {
+  SelWorkspace w;
+  if (int rc = carve(ws, ws_bytes, 0, &w, "sga_sel_result")) return rc;
+  if (!result) { set_error("sga_sel_result: null result"); return SGA_ERR_ARG; }
+  hipLaunchKernelGGL(k_sel_result, dim3(1), dim3(1), 0, (hipStream_t)stream, w.st, result);
+  return check_launch("sga_sel_result");
+}
+
+extern "C" int sga_select_topk(const float* score, int64_t n, int64_t k, int tie_mode,
+                               uint8_t* mask_out, sga_select_result* result, void* ws,
+                               size_t ws_bytes, void* stream) {
+  if (!score || !mask_out || n < 1 || n >= (1ll << 31) || k < 1 || k > n) {
+    set_error("sga_select_topk: bad argument (n=%lld k=%lld; need 1 <= k <= n < 2^31)",
+              (long long)n, (long long)k);
+    return SGA_ERR_ARG;
+  }
+  int rc;
+  if ((rc = sga_sel_begin(k, ws, ws_bytes, stream))) return rc;
+  for (int level = 0; level < 3; ++level) {
+    if ((rc = sga_sel_hist(score, n, level, ws, ws_bytes, stream))) return rc;
+    if ((rc = sga_sel_scan(level, ws, ws_bytes, stream))) return rc;
+  }
+  if ((rc = sga_sel_count(score, n, 0, ws, ws_bytes, stream))) return rc;
+  if ((rc = sga_sel_tile_scan(cdiv64(n, kChunk), tie_mode, ws, ws_bytes, stream))) return rc;
+  if ((rc = sga_sel_mask(score, n, 0, tie_mode, mask_out, ws, ws_bytes, stream))) return rc;
+  if (result && (rc = sga_sel_result(result, ws, ws_bytes, stream))) return rc;
+  return SGA_OK;
+}
+
+extern "C" int sga_hist_topbits(const float* score, int64_t n, int shift, int stride, int phase,
+                                int64_t* hist, int nbins, uint32_t* nonfinite, void* stream) {
+  if (n == 0) return SGA_OK;
+  if (!score || !hist || n < 0 || shift < 1 || shift > 30 || stride < 1 || phase < 0 ||
+      phase >= stride || nbins < 1 || nbins > 32769 || nbins < (int)((0x7FFFFFFFu >> shift) + 1)) {
+    set_error("sga_hist_topbits: bad argument (shift=%d stride=%d phase=%d nbins=%d)", shift,
+              stride, phase, nbins);
+    return SGA_ERR_ARG;
+  }
+  const int64_t n_s = n <= phase ? 0 : (n - phase + stride - 1) / stride;
+  if (n_s == 0) return SGA_OK;
+  hipLaunchKernelGGL(k_hist_topbits, dim3(stream_grid(n_s, (int64_t)kBlock * 16, 256 * 2)),
+                     dim3(kBlock), (size_t)nbins * 4, (hipStream_t)stream, score, n, shift, stride,
+                     phase, reinterpret_cast<unsigned long long*>(hist), nbins, nonfinite);
+  return check_launch("sga_hist_topbits");
+}
+
+extern "C" int sga_mask_topbits_ge(const float* score, int64_t n, int shift, int32_t bin,
+                                   uint8_t* mask_out, void* stream) {
+  if (n == 0) return SGA_OK;
+  if (!score || !mask_out || n < 0 || shift < 1 || shift > 30 || bin < 0) {
+    set_error("sga_mask_topbits_ge: bad argument");
+    return SGA_ERR_ARG;
+  }
+  hipLaunchKernelGGL(k_mask_topbits_ge, dim3(stream_grid(n, (int64_t)kBlock * kVec)), dim3(kBlock),
+                     0, (hipStream_t)stream, score, n, shift, (uint32_t)bin, mask_out,
+                     aligned4(score, 4) && aligned4(mask_out, 1));
+  return check_launch("sga_mask_topbits_ge");
+}
+
+extern "C" int sga_cand_extract_count(const float* score, int64_t n, int32_t bin,
+                                      uint32_t* chunk_counts, int64_t* total, void* stream) {
+  if (!total || n < 0 || n >= (1ll << 31) || bin < 0 || (n > 0 && (!score || !chunk_counts))) {
+    set_error("sga_cand_extract_count: bad argument");
+    return SGA_ERR_ARG;
+  }
+  const int64_t nc = cdiv64(n, kChunk);
+  hipStream_t st = (hipStream_t)stream;
+  if (nc > 0)
+    hipLaunchKernelGGL(k_cand_count, dim3(stream_grid(nc, kChunksPerBlock)), dim3(kBlock), 0, st,
+                       score, n, (uint32_t)bin, chunk_counts, nc, aligned4(score, 4));
+  if (int rc = exclusive_scan_u32(chunk_counts, nc, total, st)) return rc;
+  return check_launch("sga_cand_extract_count");
+}
+
+extern "C" int sga_cand_extract_fill(const float* score, int64_t n, int32_t bin,
+                                     const uint32_t* chunk_offsets, float* cand,
+                                     int64_t cand_capacity, void* stream) {
+  if (n == 0 || cand_capacity == 0) return SGA_OK;
+  if (!score || !chunk_offsets || !cand || n < 0 || bin < 0) {
+    set_error("sga_cand_extract_fill: bad argument");
+    return SGA_ERR_ARG;
+  }
+  const int64_t nc = cdiv64(n, kChunk);
+  hipLaunchKernelGGL(k_cand_fill, dim3(stream_grid(nc, kChunksPerBlock)), dim3(kBlock), 0,
+                     (hipStream_t)stream, score, n, (uint32_t)bin, chunk_offsets, cand,
+                     cand_capacity, nc, aligned4(score, 4));
+  return check_launch("sga_cand_extract_fill");
+}
+
+extern "C" int sga_gt_eq(const float* score, int64_t n, float thresh, uint8_t* gt, uint8_t* eq,
+                         int32_t* counts2, void* stream) {
+  if (!counts2 || n < 0 || (n > 0 && (!score || !gt || !eq))) {
+    set_error("sga_gt_eq: bad argument");
+    return SGA_ERR_ARG;
+  }
+  hipStream_t st = (hipStream_t)stream;
+  hipLaunchKernelGGL(k_zero_i32, dim3(1), dim3(64), 0, st, counts2, 2);
+  if (n > 0)
+    hipLaunchKernelGGL(k_gt_eq, dim3(stream_grid(n, (int64_t)kBlock * kVec * 4, 256 * 8)),
+                       dim3(kBlock), 0, st, score, n, thresh, gt, eq, counts2,
+                       aligned4(score, 4) && aligned4(gt, 1) && aligned4(eq, 1));
+  return check_launch("sga_gt_eq");
+}

@@ -1,0 +1,520 @@
+// Exact k-th-largest select over 31-bit magnitude keys, templated on where
+// the keys come from (a score array, raw key buffers, or a fused g+residual
+// expression).  Non-negative fp32 values order like their integer patterns,
+// so the k-th largest key is found by a three-level radix descent
+// (12 + 12 + 7 bits) over LDS-privatised histograms, followed by an ordered
+// per-chunk count so that ties at the threshold can be granted in ascending
+// index order without any float compare ambiguity.
+#pragma once
+#include "common.hpp"
+
+namespace sga {
+
+constexpr int kL0Bits = 12, kL1Bits = 12, kL2Bits = 7;
+constexpr int kL0Shift = 19, kL1Shift = 7;
+constexpr int kBinsBig = 4096, kBinsSmall = 128;
+constexpr int kTileScanPer = 16;
+constexpr int kTileScanSpan = kBlock * kTileScanPer;  // 4096 tiles / workgroup
+constexpr int kMaxTileBlocks = 1024;                  // covers n < 2^32
+
+struct SelState {
+  uint32_t k;
+  uint32_t prefix;
+  uint32_t krem;
+  uint32_t thresh_bits;
+  uint32_t need;
+  uint32_t n_gt;
+  uint32_t n_eq;
+  uint32_t nonfinite;
+  uint32_t status;
+  uint32_t total;
+  uint32_t n_selected;
+  uint32_t path;
+  // sampled-bracket path
+  uint32_t t_lo;        // candidates are keys in [t_lo, t_hi)
+  uint32_t t_hi;
+  uint32_t n_hi;        // keys >= t_hi
+  uint32_t cand_count;  // keys in the bracket (may exceed capacity)
+  uint32_t cand_cap;
+  uint32_t bracket_ok;
+  uint32_t sample_n;
+  uint32_t pad_[13];
+};
+static_assert(sizeof(SelState) == 128, "SelState layout");
+
+struct SelWorkspace {
+  SelState* st;
+  uint32_t* hist;      // 3 levels: [0,4096) [4096,8192) [8192,8320)
+  uint32_t* tile_gt;   // n_tiles (+ scan scratch) -> selected-count prefix
+  uint32_t* tile_eq;   // n_tiles (+ scan scratch) -> tie-count prefix
+  uint32_t* blk_gt;    // kMaxTileBlocks
+  uint32_t* blk_eq;    // kMaxTileBlocks
+  int64_t n_tiles_cap;
+};
+
+// Workspace layout: state | 3 level histograms | tile-scan block sums |
+// tile_gt[nt] | tile_eq[nt], where nt is whatever the byte size leaves room
+// for -- so every entry point can recover the carve from (ws, ws_bytes).
+constexpr size_t kSelFixedBytes =
+    256 + (size_t)(2 * kBinsBig + kBinsSmall + 64) * 4 + (size_t)kMaxTileBlocks * 4 * 2;
+
+static inline size_t sel_ws_bytes(int64_t n) {
+  const int64_t nt = cdiv64(n, kChunk) + 8;
+  size_t b = kSelFixedBytes + (size_t)nt * 4 * 2;
+  return (b + 255) & ~(size_t)255;
+}
+
+static inline bool sel_ws_carve(void* ws, size_t bytes, int64_t n_tiles_needed,
+                                SelWorkspace* out) {
+  if (!ws || bytes < kSelFixedBytes || (reinterpret_cast<uintptr_t>(ws) & 15))
+    return false;
+  const int64_t nt = (int64_t)((bytes - kSelFixedBytes) / 8);
+  if (nt < n_tiles_needed) return false;
+  char* p = reinterpret_cast<char*>(ws);
+  out->st = reinterpret_cast<SelState*>(p);
+  p += 256;
+  out->hist = reinterpret_cast<uint32_t*>(p);
+  p += (size_t)(2 * kBinsBig + kBinsSmall + 64) * 4;
+  out->blk_gt = reinterpret_cast<uint32_t*>(p);
+  p += (size_t)kMaxTileBlocks * 4;
+  out->blk_eq = reinterpret_cast<uint32_t*>(p);
+  p += (size_t)kMaxTileBlocks * 4;
+  out->tile_gt = reinterpret_cast<uint32_t*>(p);
+  p += (size_t)nt * 4;
+  out->tile_eq = reinterpret_cast<uint32_t*>(p);
+  out->n_tiles_cap = nt;
+  return true;
+}
+
+#ifdef __HIPCC__
+
+// ------------------------------------------------------------ key sources
+// A key source yields the 31-bit magnitude keys of 4 consecutive elements.
+struct SrcF32 {                 // |x| of an fp32 score array
+  const float* x;
+  bool vec;
+  __device__ __forceinline__ void load(int64_t i, int64_t n, uint32_t key[4]) const {
+    float v[4];
+    load4_f32(x, i, n, v, vec);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) key[e] = abs_key(v[e]);
+  }
+};
+
+struct SrcU32 {                 // raw keys (sample / candidate buffers)
+  const uint32_t* x;
+  __device__ __forceinline__ void load(int64_t i, int64_t n, uint32_t key[4]) const {
+    if (i + 4 <= n) {
+      U4 v = *reinterpret_cast<const U4*>(x + i);
+      key[0] = v.x; key[1] = v.y; key[2] = v.z; key[3] = v.w;
+    } else {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) key[e] = (i + e < n) ? x[i + e] : 0u;
+    }
+  }
+};
+
+// ------------------------------------------------------------- LDS histogram
+// One increment per participating lane; when many lanes of the wave hit the
+// bin of the first participating lane (zero-heavy or plateau data) they are
+// folded into a single add so same-address LDS atomics do not serialise.
+__device__ __forceinline__ void lds_hist_add(uint32_t* s_h, uint32_t bin, bool part) {
+  uint64_t act = ballot64(part);
+  if (act == 0) return;
+  const int leader = __ffsll((unsigned long long)act) - 1;
+  const uint32_t lead_bin = __shfl(bin, leader, kWave);
+  const uint64_t same = ballot64(part && bin == lead_bin);
+  const int ns = __popcll(same);
+  if (ns >= 8) {
+    if (lane_id() == leader) atomicAdd(&s_h[lead_bin], (uint32_t)ns);
+    part = part && bin != lead_bin;
+  }
+  if (part) atomicAdd(&s_h[bin], 1u);
+}
+
+template <int LEVEL>
+__device__ __forceinline__ void level_bin(uint32_t key, uint32_t prefix, bool valid,
+                                          uint32_t& bin, bool& part) {
+  if (LEVEL == 0) { bin = key >> kL0Shift; part = valid; }
+  else if (LEVEL == 1) { bin = (key >> kL1Shift) & (kBinsBig - 1); part = valid && (key >> kL0Shift) == prefix; }
+  else { bin = key & (kBinsSmall - 1); part = valid && (key >> kL1Shift) == prefix; }
+}
+
+template <class Src, int LEVEL>
+__global__ __launch_bounds__(kBlock) void k_level_hist(Src src, int64_t n,
+                                                       const SelState* __restrict__ st,
+                                                       uint32_t* __restrict__ hist) {
+  constexpr int NB = LEVEL == 2 ? kBinsSmall : kBinsBig;
+  __shared__ uint32_t s_h[NB];
+  for (int b = threadIdx.x; b < NB; b += kBlock) s_h[b] = 0u;
+  __syncthreads();
+  const uint32_t prefix = st->prefix;
+  const int64_t stride = (int64_t)gridDim.x * kBlock * kVec;
+  // uniform trip count so the wave-level ballots inside lds_hist_add are safe
+  const int64_t first = ((int64_t)blockIdx.x * kBlock) * kVec;
+  for (int64_t base = first; base < n; base += stride) {
+    const int64_t i = base + (int64_t)threadIdx.x * kVec;
+    uint32_t key[4] = {0, 0, 0, 0};
+    if (i < n) src.load(i, n, key);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      uint32_t bin; bool part;
+      level_bin<LEVEL>(key[e], prefix, i + e < n, bin, part);
+      lds_hist_add(s_h, bin, part);
+    }
+  }
+  __syncthreads();
+  for (int b = threadIdx.x; b < NB; b += kBlock) {
+    const uint32_t c = s_h[b];
+    if (c) atomicAdd(&hist[b], c);
+  }
+}
+
+// Single workgroup: find the bin where the descending cumulative count
+// crosses the remaining rank; descend one level.
+template <int LEVEL>
+__global__ __launch_bounds__(kBlock) void k_level_scan(SelState* __restrict__ st,
+                                                       const uint32_t* __restrict__ hist) {
+  constexpr int NB = LEVEL == 2 ? kBinsSmall : kBinsBig;
+  constexpr int PER = NB >= kBlock ? NB / kBlock : 1;
+  constexpr int BITS = LEVEL == 2 ? kL2Bits : 12;
+  __shared__ uint32_t s_suf[kBlock + 1];
+  const int t = threadIdx.x;
+  // read the incoming rank before any barrier: the one thread that descends
+  // overwrites st->krem after the barriers below
+  const uint32_t krem = (LEVEL == 0) ? st->k : st->krem;
+  const uint32_t pre_in = (LEVEL == 0) ? 0u : st->prefix;
+  uint32_t loc[PER];
+  uint32_t mine = 0;
+#pragma unroll
+  for (int j = 0; j < PER; ++j) {
+    const int b = t * PER + j;
+    loc[j] = (b < NB) ? hist[b] : 0u;
+    mine += loc[j];
+  }
+  // suffix sums over threads: s_suf[t] = sum of `mine` for threads >= t
+  s_suf[t] = mine;
+  if (t == 0) s_suf[kBlock] = 0u;
+  __syncthreads();
+  for (int o = 1; o < kBlock; o <<= 1) {
+    uint32_t add = (t + o < kBlock) ? s_suf[t + o] : 0u;
+    __syncthreads();
+    s_suf[t] += add;
+    __syncthreads();
+  }
+  const uint32_t total = s_suf[0];
+  if (LEVEL == 0 && t == 0) {
+    st->total = total;
+    uint32_t nf = 0;
+    for (int b = 0xFF0; b < kBinsBig; ++b) nf += hist[b];   // exponent 255
+    st->nonfinite = nf;
+    if (krem < 1 || krem > total) st->status = 1;
+  }
+  const uint32_t above_me = s_suf[t + 1];
+  if (krem >= 1 && above_me < krem && krem <= above_me + mine) {
+    uint32_t above = above_me;
+#pragma unroll
+    for (int j = PER - 1; j >= 0; --j) {
+      const int b = t * PER + j;
+      if (b < NB) {
+        if (above < krem && krem <= above + loc[j]) {
+          const uint32_t np = (pre_in << BITS) | (uint32_t)b;
+          st->prefix = np;
+          st->krem = krem - above;
+          if (LEVEL == 2) {
+            st->thresh_bits = np;
+            st->need = krem - above;
+            st->n_eq = loc[j];
+            st->n_gt = st->k - (krem - above);
+          }
+        }
+        above += loc[j];
+      }
+    }
+  }
+}
+
+static __global__ void k_sel_begin(SelState* st, uint32_t* hist, int nhist, uint32_t k) {
+  for (int i = threadIdx.x; i < nhist; i += blockDim.x) hist[i] = 0u;
+  if (threadIdx.x == 0) {
+    SelState z = {};
+    z.k = k;
+    *st = z;
+  }
+}
+
+// Per-chunk (1024 elements, one wave) counts of keys above / equal to the
+// threshold.
+template <class Src>
+__global__ __launch_bounds__(kBlock) void k_tile_count(Src src, int64_t n,
+                                                       int64_t tile_base,
+                                                       const SelState* __restrict__ st,
+                                                       uint32_t* __restrict__ tile_gt,
+                                                       uint32_t* __restrict__ tile_eq) {
+  const uint32_t T = st->thresh_bits;
+  const int64_t n_chunks = cdiv64(n, kChunk);
+  const int64_t wstride = (int64_t)gridDim.x * kChunksPerBlock;
+  for (int64_t c = (int64_t)blockIdx.x * kChunksPerBlock + wave_id(); c < n_chunks;
+       c += wstride) {
+    uint32_t cg = 0, ce = 0;
+#pragma unroll
+    for (int it = 0; it < kChunkIters; ++it) {
+      const int64_t i = c * kChunk + it * (kWave * kVec) + lane_id() * kVec;
+      uint32_t key[4] = {0, 0, 0, 0};
+      if (i < n) src.load(i, n, key);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const bool valid = i + e < n;
+        cg += (valid && key[e] > T);
+        ce += (valid && key[e] == T);
+      }
+    }
+    cg = wave_sum(cg);
+    ce = wave_sum(ce);
+    if (lane_id() == 0) {
+      tile_gt[tile_base + c] = cg;
+      tile_eq[tile_base + c] = ce;
+    }
+  }
+}
+
+// Tile scan, kernel 1: per-workgroup totals of (gt, eq).
+static __global__ __launch_bounds__(kBlock) void k_tile_sums(const uint32_t* __restrict__ tile_gt,
+                                                      const uint32_t* __restrict__ tile_eq,
+                                                      int64_t n_tiles,
+                                                      uint32_t* __restrict__ blk_gt,
+                                                      uint32_t* __restrict__ blk_eq) {
+  __shared__ uint32_t s_g[kChunksPerBlock], s_e[kChunksPerBlock];
+  const int64_t base = (int64_t)blockIdx.x * kTileScanSpan + (int64_t)threadIdx.x * kTileScanPer;
+  uint32_t g = 0, e = 0;
+#pragma unroll
+  for (int j = 0; j < kTileScanPer; ++j)
+    if (base + j < n_tiles) { g += tile_gt[base + j]; e += tile_eq[base + j]; }
+  g = wave_sum(g);
+  e = wave_sum(e);
+  if (lane_id() == 0) { s_g[wave_id()] = g; s_e[wave_id()] = e; }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    blk_gt[blockIdx.x] = s_g[0] + s_g[1] + s_g[2] + s_g[3];
+    blk_eq[blockIdx.x] = s_e[0] + s_e[1] + s_e[2] + s_e[3];
+  }
+}
+
+__device__ __forceinline__ uint32_t ties_taken(uint32_t need, uint32_t eq_before, uint32_t eq_here) {
+  if (need <= eq_before) return 0u;
+  const uint32_t left = need - eq_before;
+  return left < eq_here ? left : eq_here;
+}
+
+// Block-wide exclusive scan of one uint32 per thread (kBlock threads).
+__device__ __forceinline__ uint32_t block_excl_scan(uint32_t v, uint32_t* s_w4, uint32_t& block_total) {
+  const uint32_t incl = wave_incl_scan(v);
+  __syncthreads();
+  if (lane_id() == kWave - 1) s_w4[wave_id()] = incl;
+  __syncthreads();
+  uint32_t pre = 0;
+  for (int w = 0; w < wave_id(); ++w) pre += s_w4[w];
+  block_total = s_w4[0] + s_w4[1] + s_w4[2] + s_w4[3];
+  return pre + incl - v;
+}
+
+// Tile scan, kernel 2: tile_eq[i] <- ties before tile i; tile_gt[i] <- selected
+// coordinates before tile i (ties granted in ascending order until `need`
+// is used up; all of them when tie_all).
+static __global__ __launch_bounds__(kBlock) void k_tile_apply(uint32_t* __restrict__ tile_gt,
+                                                       uint32_t* __restrict__ tile_eq,
+                                                       int64_t n_tiles,
+                                                       const uint32_t* __restrict__ blk_gt,
+                                                       const uint32_t* __restrict__ blk_eq,
+                                                       int n_blocks, int tie_all,
+                                                       SelState* __restrict__ st) {
+  __shared__ uint32_t s_w4[kChunksPerBlock];
+  const uint32_t need = tie_all ? 0xFFFFFFFFu : st->need;
+  // prefixes of the workgroups before this one (n_blocks <= 1024 -> 4 each)
+  uint32_t be[4], bg[4];
+  uint32_t mine_e = 0;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int b = threadIdx.x * 4 + j;
+    be[j] = (b < n_blocks) ? blk_eq[b] : 0u;
+    bg[j] = (b < n_blocks) ? blk_gt[b] : 0u;
+    mine_e += be[j];
+  }
+  uint32_t tot_e;
+  uint32_t e_run = block_excl_scan(mine_e, s_w4, tot_e);
+  uint32_t sel_before = 0, eq_before = 0;   // contributions of blocks < blockIdx.x
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int b = threadIdx.x * 4 + j;
+    if (b < (int)blockIdx.x) {
+      sel_before += bg[j] + ties_taken(need, e_run, be[j]);
+      eq_before += be[j];
+    }
+    e_run += be[j];
+  }
+  uint32_t dummy;
+  __syncthreads();
+  // reduce sel_before / eq_before across the workgroup via scans' totals
+  block_excl_scan(sel_before, s_w4, dummy);
+  const uint32_t S0 = dummy;
+  __syncthreads();
+  block_excl_scan(eq_before, s_w4, dummy);
+  const uint32_t E0 = dummy;
+  __syncthreads();
+
+  const int64_t base = (int64_t)blockIdx.x * kTileScanSpan + (int64_t)threadIdx.x * kTileScanPer;
+  uint32_t g[kTileScanPer], e[kTileScanPer];
+  uint32_t my_e = 0;
+#pragma unroll
+  for (int j = 0; j < kTileScanPer; ++j) {
+    const bool ok = base + j < n_tiles;
+    g[j] = ok ? tile_gt[base + j] : 0u;
+    e[j] = ok ? tile_eq[base + j] : 0u;
+    my_e += e[j];
+  }
+  uint32_t blk_tot_e;
+  uint32_t er = E0 + block_excl_scan(my_e, s_w4, blk_tot_e);
+  uint32_t my_s = 0;
+  uint32_t ebase[kTileScanPer], scount[kTileScanPer];
+#pragma unroll
+  for (int j = 0; j < kTileScanPer; ++j) {
+    ebase[j] = er;
+    scount[j] = g[j] + ties_taken(need, er, e[j]);
+    my_s += scount[j];
+    er += e[j];
+  }
+  __syncthreads();
+  uint32_t blk_tot_s;
+  uint32_t sr = S0 + block_excl_scan(my_s, s_w4, blk_tot_s);
+#pragma unroll
+  for (int j = 0; j < kTileScanPer; ++j) {
+    if (base + j < n_tiles) {
+      tile_gt[base + j] = sr;
+      tile_eq[base + j] = ebase[j];
+    }
+    sr += scount[j];
+  }
+  if (blockIdx.x == gridDim.x - 1 && threadIdx.x == 0) st->n_selected = S0 + blk_tot_s;
+}
+
+// Ordered flags for one 256-element slab of a wave's chunk: `sel[e]` says
+// whether element e of this lane is selected; `pos` is the number of selected
+// elements before this lane's first element (within the whole array).
+struct ChunkCursor {
+  uint32_t sel_run;   // selected before the current slab
+  uint32_t eq_run;    // ties before the current slab
+};
+
+__device__ __forceinline__ void slab_select(const uint32_t key[4], const bool valid[4],
+                                            uint32_t T, uint32_t need, ChunkCursor& cur,
+                                            bool sel[4], uint32_t& pos) {
+  uint32_t my_eq = 0;
+  bool eq[4];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    eq[e] = valid[e] && key[e] == T;
+    my_eq += eq[e];
+  }
+  uint32_t eq_rank = cur.eq_run;
+  const uint64_t any_eq = ballot64(my_eq != 0);
+  if (any_eq) {
+    const uint32_t incl = wave_incl_scan(my_eq);
+    eq_rank += incl - my_eq;
+    cur.eq_run += __shfl(incl, kWave - 1, kWave);
+  }
+  uint32_t my_sel = 0;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    bool s = valid[e] && key[e] > T;
+    if (eq[e]) { s = eq_rank < need; ++eq_rank; }
+    sel[e] = s;
+    my_sel += s;
+  }
+  const uint32_t incl = wave_incl_scan(my_sel);
+  pos = cur.sel_run + incl - my_sel;
+  cur.sel_run += __shfl(incl, kWave - 1, kWave);
+}
+
+template <class Src>
+__global__ __launch_bounds__(kBlock) void k_write_mask(Src src, int64_t n, int64_t tile_base,
+                                                       int tie_all,
+                                                       const SelState* __restrict__ st,
+                                                       const uint32_t* __restrict__ tile_sel,
+                                                       const uint32_t* __restrict__ tile_eq,
+                                                       uint8_t* __restrict__ mask, bool mvec) {
+  const uint32_t T = st->thresh_bits;
+  const uint32_t need = tie_all ? 0xFFFFFFFFu : st->need;
+  const int64_t n_chunks = cdiv64(n, kChunk);
+  const int64_t wstride = (int64_t)gridDim.x * kChunksPerBlock;
+  for (int64_t c = (int64_t)blockIdx.x * kChunksPerBlock + wave_id(); c < n_chunks;
+       c += wstride) {
+    ChunkCursor cur;
+    cur.sel_run = tile_sel[tile_base + c];
+    cur.eq_run = tile_eq[tile_base + c];
+#pragma unroll
+    for (int it = 0; it < kChunkIters; ++it) {
+      const int64_t i = c * kChunk + it * (kWave * kVec) + lane_id() * kVec;
+      uint32_t key[4] = {0, 0, 0, 0};
+      if (i < n) src.load(i, n, key);
+      bool valid[4], sel[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) valid[e] = i + e < n;
+      uint32_t pos;
+      slab_select(key, valid, T, need, cur, sel, pos);
+      if (i < n) {
+        uint32_t mk[4] = {sel[0], sel[1], sel[2], sel[3]};
+        store4_u8(mask, i, n, mk, mvec);
+      }
+    }
+  }
+}
+
+static __global__ void k_sel_result(const SelState* st, sga_select_result* out) {
+  out->thresh_bits = st->thresh_bits;
+  out->need = st->need;
+  out->n_gt = st->n_gt;
+  out->n_eq = st->n_eq;
+  out->n_selected = st->n_selected;
+  out->nonfinite = st->nonfinite;
+  out->status = st->status;
+  out->path = st->path;
+}
+
+// -------------------------------------------------------------- host drivers
+template <class Src>
+static inline void launch_level_hist(Src src, int64_t n, int level,
+                                     const SelWorkspace& w, hipStream_t s) {
+  dim3 grid(stream_grid(n, (int64_t)kBlock * kVec * 4, 256 * 8)), block(kBlock);
+  if (level == 0) hipLaunchKernelGGL((k_level_hist<Src, 0>), grid, block, 0, s, src, n, w.st, w.hist);
+  else if (level == 1) hipLaunchKernelGGL((k_level_hist<Src, 1>), grid, block, 0, s, src, n, w.st, w.hist + kBinsBig);
+  else hipLaunchKernelGGL((k_level_hist<Src, 2>), grid, block, 0, s, src, n, w.st, w.hist + 2 * kBinsBig);
+}
+
+static inline void launch_level_scan(int level, const SelWorkspace& w, hipStream_t s) {
+  if (level == 0) hipLaunchKernelGGL((k_level_scan<0>), dim3(1), dim3(kBlock), 0, s, w.st, w.hist);
+  else if (level == 1) hipLaunchKernelGGL((k_level_scan<1>), dim3(1), dim3(kBlock), 0, s, w.st, w.hist + kBinsBig);
+  else hipLaunchKernelGGL((k_level_scan<2>), dim3(1), dim3(kBlock), 0, s, w.st, w.hist + 2 * kBinsBig);
+}
+
+static inline void launch_begin(uint32_t k, const SelWorkspace& w, hipStream_t s) {
+  hipLaunchKernelGGL(k_sel_begin, dim3(1), dim3(kBlock), 0, s, w.st, w.hist,
+                     2 * kBinsBig + kBinsSmall, k);
+}
+
+template <class Src>
+static inline void launch_tile_count(Src src, int64_t n, int64_t tile_base,
+                                     const SelWorkspace& w, hipStream_t s) {
+  const int64_t nc = cdiv64(n, kChunk);
+  hipLaunchKernelGGL((k_tile_count<Src>), dim3(stream_grid(nc, kChunksPerBlock)),
+                     dim3(kBlock), 0, s, src, n, tile_base, w.st, w.tile_gt, w.tile_eq);
+}
+
+static inline void launch_tile_scan(int64_t n_tiles, int tie_all,
+                                    const SelWorkspace& w, hipStream_t s) {
+  const int nb = (int)cdiv64(n_tiles, kTileScanSpan);
+  hipLaunchKernelGGL(k_tile_sums, dim3(nb), dim3(kBlock), 0, s, w.tile_gt, w.tile_eq, n_tiles, w.blk_gt, w.blk_eq);
+  hipLaunchKernelGGL(k_tile_apply, dim3(nb), dim3(kBlock), 0, s, w.tile_gt, w.tile_eq, n_tiles, w.blk_gt, w.blk_eq, nb, tie_all, w.st);
+}
+
+#endif  // __HIPCC__
+}  // namespace sga

@@ -1,0 +1,93 @@
+"""Fused per-rank sparse step over a flat bucket (engine order of
+``sga/engine.py:416-604``): score -> exact top-k -> index pack -> residual
+update -> residual-aware AdamW, as two kinds of sweeps over HBM."""
+import ctypes as C
+
+import torch
+
+from . import _lib as L
+from .scores import SCORE_MAP
+from .selection import read_result
+
+
+def k_for(n_total, ratio_percent):
+    """``sga/plugins/selection/topk.py:111-112``"""
+    return max(1, int(round(n_total * ratio_percent / 100.0)))
+
+
+class FusedSparseStep:
+    """Owns the workspace, the device segment table and the pack buffers for
+    one flat bucket of ``n`` elements.
+
+    segments: list of dicts {"start", "n", "lr", "b1", "b2", "eps", "wd"}
+    tiling [0, n) in ascending order (one per parameter tensor).
+    """
+
+    def __init__(self, n, segments, device, values_dtype=torch.bfloat16,
+                 max_k=None, want_mask=False):
+        assert 0 < n < 2 ** 31
+        off = 0
+        for s in segments:
+            if s["start"] != off or s["n"] <= 0:
+                raise ValueError("segments must tile [0, n) contiguously in order")
+            off += s["n"]
+        if off != n:
+            raise ValueError(f"segments cover {off} elements, bucket has {n}")
+        self.n, self.segments, self.device = n, segments, device
+        self.values_dtype = values_dtype
+        self.ws_bytes = int(L.raw("sga_fused_workspace_bytes", n))
+        self.ws = torch.empty(self.ws_bytes, dtype=torch.uint8, device=device)
+        self.result = torch.zeros(8, dtype=torch.int32, device=device)
+        self.max_k = max_k or n
+        self.idx = torch.empty(self.max_k, dtype=torch.int32, device=device)
+        self.values = torch.empty(self.max_k, dtype=values_dtype, device=device)
+        self.mask = (torch.empty(n, dtype=torch.uint8, device=device)
+                     if want_mask else None)
+        self._seg_host = (L.Segment * len(segments))()
+        self._seg_dev = torch.empty(C.sizeof(self._seg_host), dtype=torch.uint8,
+                                    device=device)
+        self._seg_step = None
+
+    def _upload_segments(self, step):
+        if self._seg_step == step:
+            return
+        for i, s in enumerate(self.segments):
+            e = self._seg_host[i]
+            e.start, e.n = s["start"], s["n"]
+            e.lr = L.f32(s["lr"])
+            e.beta1, e.om1 = L.f32(s["b1"]), L.f32(1.0 - s["b1"])
+            e.beta2, e.om2 = L.f32(s["b2"]), L.f32(1.0 - s["b2"])
+            e.eps, e.wd = L.f32(s["eps"]), L.f32(s["wd"])
+            e.bc1 = L.f32(1.0 - s["b1"] ** step)
+            e.bc2 = L.f32(1.0 - s["b2"] ** step)
+        host = torch.frombuffer(bytearray(bytes(self._seg_host)), dtype=torch.uint8)
+        self._seg_dev.copy_(host)
+        self._seg_step = step
+
+    def step(self, g, resid, p, m, v, step, k=None, ratio_percent=None,
+             score="abs_g", factor=1.0, coeff=1.0, fast=True):
+        """Run one fused step in place; returns (idx[:k], values[:k]) views.
+        ``self.result`` holds the device-side select result (threshold bits,
+        counts); nothing is synchronised here."""
+        n = self.n
+        for t in (g, resid, p, m, v):
+            L.require_dev(t)
+            L.require_contig(t=t)
+            assert t.numel() == n
+        if k is None:
+            k = k_for(n, ratio_percent)
+        if not (1 <= k <= min(n, self.max_k)):
+            raise ValueError(f"k={k} out of range (n={n}, max_k={self.max_k})")
+        if score not in SCORE_MAP:
+            raise ValueError(f"Unknown SGA score '{score}'. Registered: {sorted(SCORE_MAP)}")
+        self._upload_segments(step)
+        L.call("sga_fused_sparse_step", L.ptr(g), L.dtype_code(g), L.ptr(resid), L.ptr(p),
+               L.ptr(m), L.ptr(v), n, k, L.ptr(self._seg_dev), len(self.segments),
+               SCORE_MAP[score], L.ptr(self.idx), L.ptr(self.values),
+               L.dtype_code(self.values), L.ptr(self.mask), L.f32(factor), L.f32(coeff),
+               1 if fast else 0, L.ptr(self.result), L.ptr(self.ws), self.ws_bytes,
+               L.stream())
+        return self.idx[:k], self.values[:k]
+
+    def read_result(self):
+        return read_result(self.result)

@@ -1,0 +1,200 @@
+"""Top-k selection plugin on MI355X (``sga/plugins/selection/topk.py``,
+``_histogram.py``, ``_exact.py``): strict-ratio global top-k over per-param
+score views, returning per-view uint8 masks.
+
+The exact threshold is found on the device by a three-level radix descent
+over the sign-stripped fp32 patterns (no host round trip, no candidate
+gather); ``balanced`` / ``fast`` keep the reference's stride-8 subsample
+histogram and crossing-bin rule so the masks are identical to its.
+"""
+import ctypes as C
+from types import SimpleNamespace
+
+import torch
+
+from . import _lib as L
+
+_HIST_MODES = {"exact": (16, 32769, 1), "balanced": (16, 32769, 8),
+               "fast": (19, 4097, 8)}            # _histogram.py:68-72
+_CHUNK = 1024
+
+
+class SelectResult(C.Structure):
+    """struct sga_select_result"""
+    _fields_ = [(n, C.c_uint32) for n in
+                ("thresh_bits", "need", "n_gt", "n_eq", "n_selected", "nonfinite",
+                 "status", "path")]
+
+
+def read_result(res_t):
+    """Decode a device uint32[8] result block (one host sync)."""
+    r = res_t.cpu().tolist()
+    out = SimpleNamespace(thresh_bits=r[0], need=r[1], n_gt=r[2], n_eq=r[3],
+                          n_selected=r[4], nonfinite=r[5], status=r[6], path=r[7])
+    out.thresh = torch.tensor([r[0]], dtype=torch.int32).view(torch.float32).item()
+    return out
+
+
+def _bin_edge_float(b, shift):
+    bits = (b << shift) & 0x7FFFFFFF
+    return torch.tensor([bits], dtype=torch.int32).view(torch.float32).item()
+
+
+def _sampled_count(n, stride, phase=0):
+    return len(range(phase, n, stride))
+
+
+def _flat_views(views):
+    out = []
+    for g in views:
+        L.require_dev(g)
+        f = g.reshape(-1)
+        if f.dtype != torch.float32:
+            raise TypeError("selection scores must be fp32")
+        L.require_contig(view=f)
+        out.append(f)
+    return out
+
+
+def select_exact_device(views, k, tie_mode, masks=None):
+    """Exact top-k over a list of flat fp32 views; returns (result, masks).
+    Views are laid out back to back in chunk space, each on a fresh
+    1024-element chunk, so flat-index order == view order then in-view order
+    (the reference's catalog order)."""
+    views = _flat_views(views)
+    dev = views[0].device
+    bases, nt = [], 0
+    for g in views:
+        bases.append(nt)
+        nt += -(-g.numel() // _CHUNK)
+    n_total = sum(g.numel() for g in views)
+    if not (1 <= k <= n_total):
+        raise ValueError(f"k={k} > N={n_total}" if k > n_total else f"k={k} < 1")
+    ws_bytes = int(L.raw("sga_select_workspace_bytes", nt * _CHUNK))
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    res = torch.empty(8, dtype=torch.int32, device=dev)
+    st = L.stream()
+    L.call("sga_sel_begin", k, L.ptr(ws), ws_bytes, st)
+    for level in range(3):
+        for g in views:
+            L.call("sga_sel_hist", L.ptr(g), g.numel(), level, L.ptr(ws), ws_bytes, st)
+        L.call("sga_sel_scan", level, L.ptr(ws), ws_bytes, st)
+    for g, b in zip(views, bases):
+        L.call("sga_sel_count", L.ptr(g), g.numel(), b, L.ptr(ws), ws_bytes, st)
+    L.call("sga_sel_tile_scan", max(nt, 1), tie_mode, L.ptr(ws), ws_bytes, st)
+    if masks is None:
+        masks = [torch.empty(g.numel(), dtype=torch.uint8, device=dev) for g in views]
+    for g, b, m in zip(views, bases, masks):
+        L.call("sga_sel_mask", L.ptr(g), g.numel(), b, tie_mode, L.ptr(m), L.ptr(ws),
+               ws_bytes, st)
+    L.call("sga_sel_result", L.ptr(res), L.ptr(ws), ws_bytes, st)
+    return res, masks
+
+
+def select_masks_histogram(grads, k, comm_group=None, mode="exact",
+                           global_allreduce=True):
+    """``_histogram.py:161-216`` at world size 1 (no collective in this
+    build): returns (threshold, per-view uint8 masks), ties all selected."""
+    try:
+        shift, nbins, stride = _HIST_MODES[mode]
+    except KeyError:
+        raise ValueError(f"unknown histogram_mode: {mode!r}") from None
+    if mode == "exact":
+        res, masks = select_exact_device(grads, k, L.TIE_ALL)
+        return read_result(res).thresh, masks
+    views = _flat_views(grads)
+    dev = views[0].device
+    hist = torch.zeros(nbins, dtype=torch.int64, device=dev)
+    nf = torch.zeros(1, dtype=torch.int32, device=dev)
+    st = L.stream()
+    for g in views:
+        L.call("sga_hist_topbits", L.ptr(g), g.numel(), shift, stride, 0, L.ptr(hist),
+               nbins, L.ptr(nf), st)
+    n_total = sum(g.numel() for g in views)
+    n_sampled = sum(_sampled_count(g.numel(), stride) for g in views)
+    r = max(1, round(n_sampled * (n_total - k + 1) / n_total))
+    b = int(torch.searchsorted(torch.cumsum(hist, 0), r).item())
+    masks = []
+    for g in views:
+        m = torch.empty(g.numel(), dtype=torch.uint8, device=dev)
+        L.call("sga_mask_topbits_ge", L.ptr(g), g.numel(), shift, b, L.ptr(m), st)
+        masks.append(m)
+    return _bin_edge_float(b, shift), masks
+
+
+def select_masks_exact_kthvalue(grads, k, comm_group=None):
+    """``_exact.py:12-41`` at world size 1: same threshold and masks as the
+    exact histogram tier, produced by the same device select."""
+    res, masks = select_exact_device(grads, k, L.TIE_ALL)
+    return read_result(res).thresh, masks
+
+
+class HistogramSelect:
+    """``_histogram.py:254-307`` (element granularity)."""
+
+    def __init__(self, mode="exact", block_size=1, block_reduce="mean",
+                 global_allreduce=True):
+        if mode not in _HIST_MODES:
+            raise ValueError(f"unknown histogram_mode: {mode!r} "
+                             f"(expected one of {sorted(_HIST_MODES)})")
+        if (not isinstance(block_size, int) or isinstance(block_size, bool)
+                or block_size < 1 or block_size > 1024 or block_size & (block_size - 1)):
+            raise ValueError(
+                f"block_size must be a power of two in [1, 1024], got {block_size!r}")
+        if block_reduce not in ("mean", "max"):
+            raise ValueError(f"block_reduce must be 'mean' or 'max', got {block_reduce!r}")
+        if block_size != 1:
+            raise NotImplementedError("block-granular selection is not built")
+        self.mode, self.block_size = mode, block_size
+        self.block_reduce, self.global_allreduce = block_reduce, global_allreduce
+
+    def select(self, grads, k, comm_group, warmup_target=None):
+        return select_masks_histogram(grads, k, comm_group, mode=self.mode,
+                                      global_allreduce=self.global_allreduce)
+
+
+class ExactKthvalue:
+    def select(self, grads, k, comm_group, warmup_target=None):
+        return select_masks_exact_kthvalue(grads, k, comm_group)
+
+
+class TopkSelection:
+    """``selection/topk.py:59-167``; ``args`` carries the ``sga_selection_*``
+    flags (the reference reads them from its config singleton)."""
+
+    def __init__(self, args):
+        self.method = args.sga_selection_method
+        self.ratio_percent = float(args.sga_selection_ratio_percent)
+        assert 0.0 < self.ratio_percent < 100.0, (
+            f"ratio_percent must be in (0, 100), got {self.ratio_percent}")
+        if self.method == "histogram":
+            self._impl = HistogramSelect(
+                getattr(args, "sga_selection_histogram_mode", "exact"),
+                block_size=int(getattr(args, "sga_selection_block_size", 1)),
+                block_reduce=getattr(args, "sga_selection_block_reduce", "mean"),
+                global_allreduce=bool(getattr(
+                    args, "sga_selection_topk_histogram_add_global_allreduce", False)))
+        elif self.method == "exact":
+            self._impl = ExactKthvalue()
+        elif self.method == "adaptive":
+            raise NotImplementedError("the adaptive-tau controller is host control "
+                                      "logic outside this build")
+        else:
+            raise ValueError("sga_selection_method must be adaptive|exact|histogram "
+                             f"(got {self.method!r})")
+        self.last_threshold = None
+
+    @property
+    def block_size(self):
+        return getattr(self._impl, "block_size", 1)
+
+    def k_for(self, n_total):
+        return max(1, int(round(n_total * self.ratio_percent / 100.0)))
+
+    def select(self, ctx):
+        k = self.k_for(sum(g.numel() for g in ctx.grad_views))
+        thresh, masks = self._impl.select(ctx.grad_views, k,
+                                          getattr(ctx, "comm_group", None),
+                                          getattr(ctx, "warmup_target", None))
+        self.last_threshold = thresh
+        return masks

@@ -1,0 +1,81 @@
+"""CPU-side checks of the boundary: the shared library loads, exports every
+symbol declared in include/sga_hip.h, the Python table lists the same set,
+and the product refuses CPU tensors (no fallback)."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared():
+    txt = open(os.path.join(ROOT, "include", "sga_hip.h")).read()
+    txt = re.sub(r"/\*.*?\*/", "", txt, flags=re.S)
+    return sorted(set(re.findall(r"\b(sga_[a-z0-9_]+)\s*\(", txt)))
+
+
+def test_library_exports_every_declared_symbol():
+    from sga_amd import _lib as L
+    assert os.path.exists(L.LIB_PATH), "run python -m sga_amd.build"
+    lib = ctypes.CDLL(L.LIB_PATH)
+    names = _declared()
+    assert len(names) >= 30
+    for n in names:
+        assert hasattr(lib, n), f"{n} declared in sga_hip.h but not exported"
+    assert sorted(L.SIGNATURES) == names
+    assert L.load().sga_version() >= 1
+
+
+def test_struct_layouts_match_header():
+    from sga_amd import _lib as L
+    from sga_amd.selection import SelectResult
+    assert ctypes.sizeof(L.Segment) == 56
+    assert ctypes.sizeof(SelectResult) == 32
+
+
+def test_no_cpu_fallback():
+    from sga_amd import adamw, kernels, replay, support
+    z = torch.zeros(8)
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        kernels.pack_selected(z, torch.zeros(2, dtype=torch.int32), torch.zeros(2), 1.0)
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        adamw.adamw_grad_correct(z, z.clone(), z.clone(), z.clone(), 1e-3, .9, .95, 1e-8, 0., 1)
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        support.compact_mask_u8(torch.zeros(8, dtype=torch.uint8))
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        replay.select_topk_flat(z, 2)
+
+
+def test_host_refusals_before_launch():
+    from sga_amd import adamw
+    z = torch.zeros(4)
+    mk = torch.ones(4, dtype=torch.uint8)
+    for kw, sub in ((dict(coeff=0.5), "requires a sparse step"),
+                    (dict(mask=mk, emit_score="update"), "masked-commit full step"),
+                    (dict(mask=mk, inactive_lr_scale=0.5), "requires a full step"),
+                    (dict(mask=mk, emit_score="update", inactive_lr_scale=float("inf")),
+                     "inactive_lr_scale"),
+                    (dict(emit_score="bogus"), "no _grad_correct_kernel branch")):
+        with pytest.raises(ValueError) as ei:
+            adamw.adamw_grad_correct(z, z.clone(), z.clone(), z.clone(), 1e-3, .9, .95,
+                                     1e-8, 0., 1, **kw)
+        assert sub in str(ei.value)
+    from sga_amd.scores import get_score_spec, score_names
+    assert score_names() == ["abs_g", "abs_m", "coi", "update"]
+    with pytest.raises(ValueError) as ei:
+        get_score_spec("nope")
+    assert "nope" in str(ei.value) and "abs_g" in str(ei.value)
+    from sga_amd.fused_step import k_for
+    assert k_for(4194304, 1.0) == 41943 and k_for(250, 1.0) == 2
+
+
+def test_oracle_is_not_imported_by_the_product():
+    pkg = os.path.join(ROOT, "sga_amd")
+    for dp, _, fs in os.walk(pkg):
+        for f in fs:
+            if f.endswith((".py", ".hip", ".hpp")):
+                src = open(os.path.join(dp, f)).read()
+                assert "oracle" not in src.replace("# oracle", ""), f

@@ -1,0 +1,115 @@
+"""GPU parity of the fused per-rank sparse step vs the CPU oracle driver on
+the same seeded inputs: idx / mask / values / residual bit-exact, m and v
+bit-exact, p within 1e-6 relative."""
+import pytest
+import torch
+
+from oracle import fused_step as OF
+from oracle import select as SEL
+from tests.util import rel_close, student_t, sub_scale
+
+pytestmark = pytest.mark.gpu
+
+
+def _segments(sizes, wd_every=2):
+    segs, off = [], 0
+    for i, s in enumerate(sizes):
+        segs.append(dict(start=off, n=s, lr=1e-4, b1=0.9, b2=0.95, eps=1e-8,
+                         wd=0.1 if i % wd_every == 0 else 0.0))
+        off += s
+    return segs, off
+
+
+def _run(dev, sizes, steps, ratio, gdtype, vdtype, score="abs_g", seed0=0):
+    from sga_amd.fused_step import FusedSparseStep
+    segs, n = _segments(sizes)
+    gen = torch.Generator().manual_seed(1234)
+    p = torch.randn(n, generator=gen) * 0.02
+    m, v, r = torch.zeros(n), torch.zeros(n), torch.zeros(n)
+    dp, dm, dv, dr = (t.to(dev) for t in (p, m, v, r))
+    fs = FusedSparseStep(n, segs, dev, values_dtype=vdtype, want_mask=True)
+    k = SEL.k_for(n, ratio)
+    travelled = p.abs()          # |p0| + sum of |applied steps| so far
+    for step in range(1, steps + 1):
+        g = student_t(n, seed0 + step - 1).to(gdtype)
+        given = None
+        if score != "abs_g":
+            # index parity for sqrt/div scores is asserted on identical score
+            # bits: feed the device's own score to the CPU selector
+            from sga_amd.scores import SCORE_MAP, device_formula
+            buf = dr + g.to(dev).float()
+            given = torch.empty(n)
+            for s in segs:
+                a, b = s["start"], s["start"] + s["n"]
+                given[a:b] = device_formula(
+                    SCORE_MAP[score], dp[a:b], dm[a:b], dv[a:b], buf[a:b], s["b1"], s["b2"],
+                    s["eps"], s["wd"], 1 - s["b1"] ** step, 1 - s["b2"] ** step,
+                    absolute=True).cpu()
+        p_old = p.clone()
+        idx_ref, val_ref, mask_ref, th_ref = OF.fused_sparse_step(
+            g, r, p, m, v, segs, step, k=k, score=score, values_dtype=vdtype,
+            given_score=given)
+        idx, vals = fs.step(g.to(dev), dr, dp, dm, dv, step, k=k, score=score)
+        res = fs.read_result()
+        assert res.status == 0 and res.nonfinite == 0 and res.n_selected == k
+        assert res.thresh == th_ref, (step, res.thresh, th_ref)
+        assert torch.equal(idx.cpu(), idx_ref), step
+        assert torch.equal(fs.mask.cpu().bool(), mask_ref), step
+        it = torch.int16 if vdtype == torch.bfloat16 else torch.int32
+        assert torch.equal(vals.cpu().view(it), val_ref.view(it)), step
+        assert torch.equal(dr.cpu().view(torch.int32), r.view(torch.int32)), step
+        assert torch.equal(dm.cpu(), m) and torch.equal(dv.cpu(), v), step
+        # 1e-6 relative; where p' = p - lr*update cancels, relative to the
+        # operands of the subtractions applied so far (the device state is
+        # never re-synchronised from the oracle between steps)
+        travelled += (p - p_old).abs()
+        bad, worst = rel_close(dp, p, 1e-6, scale=travelled)
+        assert bad == 0, (step, worst)
+    return n, k
+
+
+def test_config1_flat_fp32_8_steps(dev):
+    """2^22 fp32 Student-t(3)x1e-3 gradients, 8 seeded steps, ratio 1 %."""
+    n, k = _run(dev, [1 << 22], 8, 1.0, torch.float32, torch.float32)
+    assert k == 41943
+
+
+def test_bf16_grads_bf16_values_multi_segment(dev):
+    _run(dev, [400_000, 1024, 300_000, 128, 170_000, 2048], 4, 1.0, torch.bfloat16,
+         torch.bfloat16)
+
+
+@pytest.mark.parametrize("ratio", [0.1, 10.0])
+def test_ratios(dev, ratio):
+    _run(dev, [1_000_003], 3, ratio, torch.bfloat16, torch.bfloat16)
+
+
+def test_ragged_unaligned_segments(dev):
+    _run(dev, [1001, 7, 2999, 64_001], 3, 1.0, torch.float32, torch.bfloat16)
+
+
+@pytest.mark.parametrize("score", ["update", "coi", "abs_m"])
+def test_adam_normalised_scores(dev, score):
+    _run(dev, [200_000, 1024, 100_000], 3, 1.0, torch.bfloat16, torch.bfloat16, score=score)
+
+
+def test_tie_heavy_gradients(dev):
+    """Quantised gradients: many equal magnitudes at the threshold; ties must
+    go to the lowest flat indices exactly like the oracle."""
+    from sga_amd.fused_step import FusedSparseStep
+    n = 500_000
+    segs, _ = _segments([n])
+    gen = torch.Generator().manual_seed(7)
+    g = (torch.randn(n, generator=gen) * 4).round() / 1024
+    p = torch.randn(n, generator=gen) * 0.02
+    m, v, r = torch.zeros(n), torch.zeros(n), torch.zeros(n)
+    dp, dm, dv, dr = (t.to(dev) for t in (p, m, v, r))
+    fs = FusedSparseStep(n, segs, dev, values_dtype=torch.float32, want_mask=True)
+    for k in (1, 5000, 250_000, n):
+        rr, pp, mm, vv = r.clone(), p.clone(), m.clone(), v.clone()
+        idx_ref, val_ref, mask_ref, th = OF.fused_sparse_step(g, rr, pp, mm, vv, segs, 1, k=k)
+        er, ep, em, ev = (t.clone() for t in (dr, dp, dm, dv))
+        idx, vals = fs.step(g.to(dev), er, ep, em, ev, 1, k=k)
+        assert fs.read_result().thresh == th
+        assert torch.equal(idx.cpu(), idx_ref) and torch.equal(vals.cpu(), val_ref)
+        assert torch.equal(er.cpu(), rr) and torch.equal(em.cpu(), mm)

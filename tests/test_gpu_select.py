@@ -1,0 +1,150 @@
+"""GPU parity of the exact top-k select (both tie semantics), the balanced /
+fast histogram tiers and the replay select building blocks vs the CPU
+oracle.  Masks, indices, counts and thresholds are bit-exact."""
+import json
+import os
+
+import pytest
+import torch
+
+from oracle import select as SEL
+from tests.test_oracle_select import adversarial
+from tests.util import adv, student_t
+
+pytestmark = pytest.mark.gpu
+KATS = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "select_kats.json")))
+
+
+@pytest.mark.parametrize("kat", KATS["tie_fill"], ids=lambda k: k["name"])
+def test_tie_fill_kats(dev, kat):
+    from sga_amd.replay import select_topk_flat
+    t = torch.tensor(kat["t"], dtype=torch.float32, device=dev)
+    mask, th = select_topk_flat(t, kat["k"])
+    assert mask.dtype == torch.bool
+    assert mask.cpu().to(torch.int64).tolist() == kat["mask"] and th == kat["thresh"]
+
+
+@pytest.mark.parametrize("kat", KATS["rejections"])
+def test_rejections(dev, kat):
+    from sga_amd.replay import select_topk_flat
+    t = torch.tensor([float(x) for x in kat["t"]], dtype=torch.float32, device=dev)
+    with pytest.raises(ValueError) as ei:
+        select_topk_flat(t, kat["k"])
+    assert kat["substr"] in str(ei.value)
+
+
+def test_adversarial_families_bitwise(dev):
+    from sga_amd.replay import select_topk_flat
+    gen = torch.Generator().manual_seed(20260912)
+    n = 200_000
+    for name, sc in adversarial(n, gen).items():
+        npos = max(8, n // 1000)
+        ks = sorted({1, n // 100, 3 * n // 10, n - 1, n})
+        if name == "zero-heavy":
+            ks = sorted(set(ks) | {max(1, npos // 2), min(n, npos * 4)})
+        sd = sc.to(dev)
+        for k in ks:
+            m_ref, t_ref = SEL.select_topk_flat(sc, k)
+            m_dev, t_dev = select_topk_flat(sd, k)
+            assert t_dev == t_ref, (name, k)
+            assert torch.equal(m_dev.cpu(), m_ref), (name, k)
+
+
+@pytest.mark.parametrize("n", [1, 5, 1023, 1024, 1025, 4097, 1_000_003])
+def test_sizes_and_random_bit_patterns(dev, n):
+    from sga_amd.replay import select_topk_flat
+    sc = adv(n, n, nonneg=True)
+    for k in sorted({1, max(1, n // 100), max(1, n // 2), n}):
+        m_ref, t_ref = SEL.select_topk_flat(sc, k)
+        m_dev, t_dev = select_topk_flat(sc.to(dev), k)
+        assert t_dev == t_ref and torch.equal(m_dev.cpu(), m_ref), (n, k)
+
+
+def test_heavy_tail_with_duplicates(dev):
+    """Stress-config shape at reduced size: heavy-tailed magnitudes with 5 %
+    duplicated values, ratios 0.01 % and 1 %."""
+    from sga_amd.replay import select_topk_flat
+    n = 3_000_000
+    sc = student_t(n, 3).abs()
+    gen = torch.Generator().manual_seed(1)
+    dup = torch.randint(0, n, (n // 20,), generator=gen)
+    sc[dup] = sc[dup.roll(1)]
+    for ratio in (0.01, 1.0):
+        k = SEL.k_for(n, ratio)
+        m_ref, t_ref = SEL.select_topk_flat(sc, k)
+        m_dev, t_dev = select_topk_flat(sc.to(dev), k)
+        assert t_dev == t_ref and torch.equal(m_dev.cpu(), m_ref)
+
+
+def test_online_ties_all_views(dev):
+    """Distribution families of the reference's xp-capability test: exact
+    histogram tier == kthvalue masks, ties all selected, over split views."""
+    from sga_amd.selection import select_masks_exact_kthvalue, select_masks_histogram
+    N = 4097
+    g = torch.Generator().manual_seed(1234)
+    ds = [torch.randn(N, generator=g) * 1e-3,
+          (torch.randn(N, generator=g) * 1e3).round() / 1e3,
+          torch.randn(N, generator=g).exp() * torch.sign(torch.randn(N, generator=g)),
+          torch.full((N,), 0.5), torch.randn(N, generator=g) * 1e-3,
+          torch.randn(N, generator=g) * 1e-3]
+    ds[4][::3] = 0.0
+    ds[5][::7] *= 1e30
+    for x in ds:
+        views = [x[:N // 2].contiguous(), x[N // 2:].contiguous()]
+        dviews = [v.to(dev) for v in views]
+        for k in (1, 2, N // 10, N // 2, N - 1, N):
+            t_ref, m_ref = SEL.select_masks_histogram(views, k, mode="exact")
+            t_dev, m_dev = select_masks_histogram(dviews, k, None, mode="exact")
+            assert t_dev == t_ref
+            for a, b in zip(m_dev, m_ref):
+                assert a.dtype == torch.uint8 and torch.equal(a.cpu(), b)
+            t_e, m_e = select_masks_exact_kthvalue(dviews, k, None)
+            assert t_e == t_ref and all(torch.equal(a.cpu(), b) for a, b in zip(m_e, m_ref))
+
+
+@pytest.mark.parametrize("mode", ["balanced", "fast"])
+def test_balanced_and_fast_tiers(dev, mode):
+    from sga_amd.selection import HistogramSelect, TopkSelection
+    from types import SimpleNamespace
+    g = torch.Generator().manual_seed(5)
+    views = [torch.randn(40001, generator=g), torch.full((7,), 0.25),
+             torch.randn(65536, generator=g) * 3, torch.randn(100009, generator=g)]
+    n_total = sum(v.numel() for v in views)
+    k = SEL.k_for(n_total, 5.0)
+    t_ref, m_ref = SEL.select_masks_histogram(views, k, mode=mode)
+    t_dev, m_dev = HistogramSelect(mode).select([v.to(dev) for v in views], k, None)
+    assert t_dev == t_ref
+    for a, b in zip(m_dev, m_ref):
+        assert torch.equal(a.cpu(), b)
+    sel = TopkSelection(SimpleNamespace(sga_selection_method="histogram",
+                                        sga_selection_ratio_percent=5.0,
+                                        sga_selection_histogram_mode=mode))
+    masks = sel.select(SimpleNamespace(grad_views=[v.to(dev) for v in views]))
+    assert sel.k_for(n_total) == k and sel.last_threshold == t_ref
+    assert all(torch.equal(a.cpu(), b) for a, b in zip(masks, m_ref))
+
+
+def test_replay_select_building_blocks(dev):
+    from sga_amd import replay_kernels as K
+    n = 250_007
+    sc = student_t(n, 4).abs()
+    sc[1000:1300] = sc[999]
+    sd = sc.to(dev)
+    hist, nf = K.hist_top16(sd)
+    assert nf == 0 and hist.dtype == torch.int64 and hist.numel() == 32769
+    top = SEL.abs_bit_top(sc)
+    assert torch.equal(hist, torch.bincount(top, minlength=32769))
+    b = int(top[999])
+    cand = K.cand_extract(sd, b)
+    assert torch.equal(cand, sc[top == b])
+    th = float(sc[999])
+    gt, eq, counts = K.gt_eq_counts(sd, th)
+    assert gt.dtype == torch.bool and torch.equal(gt.cpu(), sc > th)
+    assert torch.equal(eq.cpu(), sc == th)
+    assert counts.tolist() == [int((sc > th).sum()), int((sc == th).sum())]
+    bad = sc.clone()
+    bad[5] = float("nan")
+    bad[6] = float("inf")
+    assert K.hist_top16(bad.to(dev))[1] == 2
+    assert K.arm(True, torch.float32) and not K.arm(False, torch.float32)
+    assert K.formula("update") is not None and K.formula("nope") is None
