@@ -1,0 +1,203 @@
+#!/usr/bin/env python3
+"""Benchmark of the fused per-rank sparse step on one MI355X.
+
+One "step" = score |g+r| -> exact top-k (1 %, lowest-index ties) -> index pack
+(int32 idx + bf16 values) -> residual update -> residual-aware AdamW over the
+Llama-3.2-1B-shaped gradient set (1,235,814,400 elements, 146 tensors, bf16
+Student-t(3) gradients, fp32 p/m/v/residual) with every input resident in HBM.
+
+Prints ONE JSON line: whole-job elements/s, the roofline of the dominant
+kernel (the final sweep, timed live with HIP events on its launch stream) and
+the CPU oracle timed on a bounded sample of the same workload.
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK = 8.0e12          # MI355X HBM3E, B/s
+ALG_BYTES_STEP = 40.0      # 2*(2+4) + 4 + 24  (bf16 g, two-buffer contract)
+ALG_BYTES_FINAL = 34.0     # final sweep: read g,r,p,m,v (18) + write r,p,m,v (16)
+
+
+def student_t_dev(n, seed, dev, scale=1e-3, nu=3, chunk=1 << 26):
+    import torch
+    out = torch.empty(n, dtype=torch.bfloat16, device=dev)
+    gen = torch.Generator(device=dev).manual_seed(seed)
+    for a in range(0, n, chunk):
+        b = min(n, a + chunk)
+        z = torch.randn(b - a, generator=gen, device=dev)
+        chi = torch.zeros(b - a, device=dev)
+        for _ in range(nu):
+            chi += torch.randn(b - a, generator=gen, device=dev).pow_(2)
+        out[a:b] = (z / torch.sqrt(chi / nu) * scale).to(torch.bfloat16)
+    return out
+
+
+def cpu_baseline(sample_n, steps, ratio):
+    """Oracle (torch CPU restatement of the reference's pure-torch path) on the
+    first ``sample_n`` elements of the same tensor list."""
+    import torch
+    from oracle import fused_step as OF
+    from sga_amd.shapes import llama32_1b, segments_for
+    from tests.util import student_t
+    shapes, acc = [], 0
+    for name, n in llama32_1b()[1:]:          # layer tensors, skipping the embedding
+        if acc + n > sample_n:
+            break
+        shapes.append((name, n))
+        acc += n
+    segs, n = segments_for(shapes)
+    gen = torch.Generator().manual_seed(0)
+    p = torch.randn(n, generator=gen) * 0.02
+    m, v, r = torch.zeros(n), torch.zeros(n), torch.zeros(n)
+    grads = [student_t(n, 100 + s).to(torch.bfloat16) for s in range(steps)]
+    OF.fused_sparse_step(grads[0], r, p, m, v, segs, 1, ratio_percent=ratio,
+                         values_dtype=torch.bfloat16)             # warm-up step
+    t0 = time.perf_counter()
+    for s in range(steps):
+        OF.fused_sparse_step(grads[s], r, p, m, v, segs, s + 2, ratio_percent=ratio,
+                             values_dtype=torch.bfloat16)
+    dt = time.perf_counter() - t0
+    return {"value": n * steps / dt, "unit": "elem/s", "cores": torch.get_num_threads(),
+            "kind": "port",
+            "sample": f"{len(shapes)} layer tensors of the Llama-3.2-1B list "
+                      f"({n} elements), {steps} steps at {ratio}% after 1 warm-up step, "
+                      f"{dt:.1f} s; host cpu_count={os.cpu_count()}"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--ratio", type=float, default=1.0)
+    ap.add_argument("--score", default="abs_g")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--cpu-sample", type=int, default=1 << 27)
+    ap.add_argument("--calib", action="store_true",
+                    help="also launch one plain copy of 2^30 fp32 (k_calib_copy) so counter "
+                         "runs can be scaled against a kernel of known traffic")
+    ap.add_argument("--sweep", action="store_true",
+                    help="also time ratios 0.1/1/10 % and the update score")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs one data-parallel rank's share on ONE GPU; "
+              "there are no collectives, so --gpus must be 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from sga_amd import _lib as L
+    from sga_amd.fused_step import FusedSparseStep, k_for
+    from sga_amd.shapes import llama32_1b, segments_for
+
+    L.load()
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    segs, n = segments_for(llama32_1b())
+    gen = torch.Generator(device=dev).manual_seed(0)
+    p = torch.randn(n, generator=gen, device=dev) * 0.02
+    m = torch.zeros(n, device=dev)
+    v = torch.zeros(n, device=dev)
+    r = torch.zeros(n, device=dev)
+    grads = [student_t_dev(n, 10 + i, dev) for i in range(2)]
+    fs = FusedSparseStep(n, segs, dev, values_dtype=torch.bfloat16,
+                         max_k=k_for(n, 10.0) + 16)
+
+    def run(steps, step0, ratio, score):
+        k = k_for(n, ratio)
+        for s in range(steps):
+            fs.step(grads[(step0 + s) % 2], r, p, m, v, step0 + s + 1, k=k, score=score)
+
+    calib = None
+    if args.calib:
+        cn = 1 << 30
+        src = torch.ones(cn, device=dev)
+        dst = torch.empty(cn, device=dev)
+        ev = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
+        L.call("sga_calib_copy", L.ptr(dst), L.ptr(src), cn, L.stream())
+        ev[0].record()
+        for _ in range(5):
+            L.call("sga_calib_copy", L.ptr(dst), L.ptr(src), cn, L.stream())
+        ev[1].record()
+        torch.cuda.synchronize()
+        ms = ev[0].elapsed_time(ev[1]) / 5
+        calib = {"kernel": "k_calib_copy", "bytes": cn * 8, "avg_ms": ms,
+                 "GBps": cn * 8 / ms / 1e6}
+        del src, dst
+    run(args.warmup, 0, args.ratio, args.score)
+    torch.cuda.synchronize()
+    L.raw("sga_prof_enable", 1)
+    t0 = time.perf_counter()
+    run(args.steps, args.warmup, args.ratio, args.score)
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    tot_ms, cnt = ctypes.c_double(0), ctypes.c_int(0)
+    L.call("sga_prof_read", ctypes.byref(tot_ms), ctypes.byref(cnt))
+    L.raw("sga_prof_enable", 0)
+    res = fs.read_result()
+    assert res.status == 0 and res.n_selected == k_for(n, args.ratio), vars(res)
+
+    k = k_for(n, args.ratio)
+    final_ms = tot_ms.value / max(cnt.value, 1)
+    final_bytes = n * ALG_BYTES_FINAL + k * 6.0
+    achieved = final_bytes / (final_ms * 1e-3) if final_ms > 0 else 0.0
+    traffic = None
+    tpath = os.path.join(ROOT, "profiles", "fused_final_llama1b_traffic.json")
+    if os.path.exists(tpath):
+        try:
+            traffic = json.load(open(tpath)).get("hbm_bytes_per_launch")
+        except Exception:
+            traffic = None
+    value = n * args.steps / dt
+    out = {
+        "metric": "grad elems/s (score+top-k+resid AdamW)",
+        "value": value, "unit": "elem/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": dt / args.steps * 1e3,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "Llama-3.2-1B-shaped set, 1,235,814,400 elems / 146 tensors, "
+                               "bf16 Student-t(3) grads, fp32 p/m/v/residual, score "
+                               f"{args.score}, exact top-k {args.ratio}% (k={k}), index pack "
+                               "int32+bf16, residual-aware AdamW",
+                   "ratio_percent": args.ratio, "score": args.score, "k": k},
+        "roofline": {"bound": "hbm", "achieved": achieved / 1e9, "peak": HBM_PEAK / 1e9,
+                     "unit": "GB/s", "frac": achieved / HBM_PEAK, "traffic": traffic,
+                     "kernel": "k_fused_final", "avg_ms": final_ms,
+                     "alg_bytes_per_launch": final_bytes},
+        "step_roofline": {"alg_bytes_per_elem": ALG_BYTES_STEP,
+                          "achieved_GBps": value * ALG_BYTES_STEP / 1e9,
+                          "frac": value * ALG_BYTES_STEP / HBM_PEAK},
+        "select": {"thresh": res.thresh, "n_gt": res.n_gt, "n_eq": res.n_eq, "path": res.path},
+    }
+    if calib:
+        out["copy_calibration"] = calib
+    if args.sweep:
+        sw = []
+        step0 = args.warmup + args.steps
+        for score, ratio in (("abs_g", 0.1), ("abs_g", 10.0), ("update", 0.1),
+                             ("update", 1.0), ("update", 10.0)):
+            run(1, step0, ratio, score)
+            torch.cuda.synchronize()
+            t1 = time.perf_counter()
+            run(3, step0 + 1, ratio, score)
+            torch.cuda.synchronize()
+            d = (time.perf_counter() - t1) / 3
+            step0 += 4
+            sw.append({"score": score, "ratio_percent": ratio, "elem_per_s": n / d,
+                       "ms_per_step": d * 1e3})
+        out["sweep"] = sw
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline(args.cpu_sample, 2, args.ratio)
+    else:
+        out["cpu_baseline"] = None
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -239,6 +239,16 @@ int sga_fused_sparse_step(const void* g, int g_dtype, float* resid, float* p,
                           int fast, sga_select_result* result, void* ws,
                           size_t ws_bytes, void* stream);
 
+/* Live timing of the fused step's final sweep with HIP events recorded on the
+ * launch stream (no counterpart in the reference; used by the benchmark).
+ * enable(1) resets and arms up to 512 launches; read() waits for the recorded
+ * events and returns their summed duration in ms and their number. */
+int sga_prof_enable(int on);
+/* dst[0..n) = src[0..n), fp32, n % 4 == 0: plain copy of known size used to
+ * calibrate the HBM traffic counters (no counterpart in the reference). */
+int sga_calib_copy(float* dst, const float* src, int64_t n, void* stream);
+int sga_prof_read(double* total_ms, int* launches);
+
 #ifdef __cplusplus
 }
 #endif

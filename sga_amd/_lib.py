@@ -62,6 +62,9 @@ SIGNATURES = {
     "sga_gt_eq": (I32, [P, I64, F, P, P, P, P]),
     "sga_score_formula": (I32, [I32, P, P, P, P, P, I64] + [F] * 8 + [I32, I32, P]),
     "sga_opt_step_inplace": (I32, [P, P, P, P, P, P, I64] + [F] * 13 + [I32, P]),
+    "sga_calib_copy": (I32, [P, P, I64, P]),
+    "sga_prof_enable": (I32, [I32]),
+    "sga_prof_read": (I32, [P, P]),
     "sga_fused_workspace_bytes": (SZ, [I64]),
     "sga_fused_sparse_step": (I32, [P, I32, P, P, P, P, I64, I64, P, I32, I32, P, P,
                                     I32, P, F, F, I32, P, P, SZ, P]),

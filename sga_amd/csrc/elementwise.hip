@@ -17,6 +17,16 @@ __global__ __launch_bounds__(kBlock) void k_scatter(float* __restrict__ dst,
   }
 }
 
+// Plain 128-bit copy of known size: the yardstick the HBM traffic counters
+// and the achievable streaming bandwidth are calibrated against.
+__global__ __launch_bounds__(kBlock) void k_calib_copy(float* __restrict__ dst,
+                                                       const float* __restrict__ src,
+                                                       int64_t n4) {
+  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n4;
+       i += (int64_t)gridDim.x * kBlock)
+    reinterpret_cast<F4*>(dst)[i] = reinterpret_cast<const F4*>(src)[i];
+}
+
 // ------------------------------------------------------------------- pack
 template <bool BF16, bool SCALE>
 __global__ __launch_bounds__(kBlock) void k_pack(float* __restrict__ grad,
@@ -198,6 +208,17 @@ extern "C" int sga_scatter_selected(float* dst, const int32_t* idx,
   hipLaunchKernelGGL(k_scatter, dim3(stream_grid(k, kBlock)), dim3(kBlock), 0,
                      (hipStream_t)stream, dst, idx, src, k, n_dst);
   return check_launch("sga_scatter_selected");
+}
+
+extern "C" int sga_calib_copy(float* dst, const float* src, int64_t n, void* stream) {
+  if (!dst || !src || n < 0 || (n & 3) || !aligned4(dst, 4) || !aligned4(src, 4)) {
+    set_error("sga_calib_copy: needs 16-byte aligned buffers and n %% 4 == 0");
+    return SGA_ERR_ARG;
+  }
+  if (n == 0) return SGA_OK;
+  hipLaunchKernelGGL(k_calib_copy, dim3(stream_grid(n / 4, kBlock, 1 << 20)), dim3(kBlock), 0,
+                     (hipStream_t)stream, dst, src, n / 4);
+  return check_launch("sga_calib_copy");
 }
 
 extern "C" int sga_pack_selected(float* grad, const int32_t* idx, void* values,

@@ -234,17 +234,18 @@ extern "C" int sga_select_topk(const float* score, int64_t n, int64_t k, int tie
               (long long)n, (long long)k);
     return SGA_ERR_ARG;
   }
-  int rc;
-  if ((rc = sga_sel_begin(k, ws, ws_bytes, stream))) return rc;
-  for (int level = 0; level < 3; ++level) {
-    if ((rc = sga_sel_hist(score, n, level, ws, ws_bytes, stream))) return rc;
-    if ((rc = sga_sel_scan(level, ws, ws_bytes, stream))) return rc;
-  }
-  if ((rc = sga_sel_count(score, n, 0, ws, ws_bytes, stream))) return rc;
-  if ((rc = sga_sel_tile_scan(cdiv64(n, kChunk), tie_mode, ws, ws_bytes, stream))) return rc;
-  if ((rc = sga_sel_mask(score, n, 0, tie_mode, mask_out, ws, ws_bytes, stream))) return rc;
-  if (result && (rc = sga_sel_result(result, ws, ws_bytes, stream))) return rc;
-  return SGA_OK;
+  SelWorkspace w;
+  if (int rc = carve(ws, ws_bytes, cdiv64(n, kChunk), &w, "sga_select_topk")) return rc;
+  hipStream_t s = (hipStream_t)stream;
+  SrcF32 src{score, aligned4(score, 4)};
+  const int tie_all = tie_mode == SGA_TIE_ALL;
+  run_select(src, n, k, tie_all, true, w, s);
+  const int64_t nc = cdiv64(n, kChunk);
+  hipLaunchKernelGGL((k_write_mask<SrcF32>), dim3(stream_grid(nc, kChunksPerBlock)), dim3(kBlock), 0,
+                     s, src, n, (int64_t)0, tie_all, w.st, w.tile_gt, w.tile_eq, mask_out,
+                     aligned4(mask_out, 1));
+  if (result) hipLaunchKernelGGL(k_sel_result, dim3(1), dim3(1), 0, s, w.st, result);
+  return check_launch("sga_select_topk");
 }
 
 extern "C" int sga_hist_topbits(const float* score, int64_t n, int shift, int stride, int phase,

@@ -36,31 +36,68 @@ struct SelState {
   uint32_t n_hi;        // keys >= t_hi
   uint32_t cand_count;  // keys in the bracket (may exceed capacity)
   uint32_t cand_cap;
-  uint32_t bracket_ok;
+  uint32_t bracket_ok;  // 1: the sampled bracket holds the k-th key; radix passes skip
   uint32_t sample_n;
-  uint32_t pad_[13];
+  uint32_t overflow;    // a candidate segment ran out of room
+  uint32_t skip;        // 1: kernels driven by this state do nothing
+  uint32_t pad_[11];
 };
 static_assert(sizeof(SelState) == 128, "SelState layout");
 
 struct SelWorkspace {
-  SelState* st;
+  SelState* st;        // main state (result, bracket)
+  SelState* aux;       // scratch state of the sample / candidate selects
   uint32_t* hist;      // 3 levels: [0,4096) [4096,8192) [8192,8320)
-  uint32_t* tile_gt;   // n_tiles (+ scan scratch) -> selected-count prefix
-  uint32_t* tile_eq;   // n_tiles (+ scan scratch) -> tie-count prefix
+  uint32_t* tile_gt;   // n_tiles -> selected-count prefix
+  uint32_t* tile_eq;   // n_tiles -> tie-count prefix
   uint32_t* blk_gt;    // kMaxTileBlocks
   uint32_t* blk_eq;    // kMaxTileBlocks
   int64_t n_tiles_cap;
+  // sampled-bracket path (null / 0 when the workspace has no room for it)
+  uint32_t* sample;    // sample_cap keys
+  uint32_t* seg_cnt;   // kSegWaves (+1) counts -> offsets
+  uint32_t* seg_idx;   // kSegWaves * seg_cap
+  uint32_t* seg_key;
+  uint32_t* cand_idx;  // dense candidates
+  uint32_t* cand_key;
+  int64_t sample_cap;
+  int64_t seg_cap;     // per-wave candidate capacity
 };
 
-// Workspace layout: state | 3 level histograms | tile-scan block sums |
-// tile_gt[nt] | tile_eq[nt], where nt is whatever the byte size leaves room
-// for -- so every entry point can recover the carve from (ws, ws_bytes).
+constexpr int kSegWaves = 4096;            // persistent waves of the bracket sweep
+constexpr int64_t kFastMinN = 1 << 20;     // below this the radix passes are cheap enough
+
+static inline int64_t fast_sample_vecs(int64_t n) {
+  int64_t v = n / 1024;
+  if (v < 16384) v = 16384;
+  if (v > (1 << 20)) v = 1 << 20;
+  return v;
+}
+static inline int64_t fast_seg_cap(int64_t n) {
+  int64_t c = n / 32 / kSegWaves;
+  if (c < 64) c = 64;
+  if (c > 8192) c = 8192;
+  return c;
+}
+
+// Workspace layout: [fixed: states | level histograms | tile-scan block sums]
+// [tile_gt[nt] | tile_eq[nt]] [fast-path buffers sized from nt].  nt is
+// derived from the byte size, so every entry point recovers the same carve
+// from (ws, ws_bytes) alone.
 constexpr size_t kSelFixedBytes =
     256 + (size_t)(2 * kBinsBig + kBinsSmall + 64) * 4 + (size_t)kMaxTileBlocks * 4 * 2;
 
+static inline size_t fast_bytes_for_tiles(int64_t nt) {
+  const int64_t n = nt * kChunk;
+  if (n < kFastMinN) return 0;
+  const int64_t sc = fast_seg_cap(n);
+  return (size_t)fast_sample_vecs(n) * 16 + (size_t)(kSegWaves + 64) * 4 +
+         (size_t)kSegWaves * sc * 4 * 4 + 256;
+}
+
 static inline size_t sel_ws_bytes(int64_t n) {
   const int64_t nt = cdiv64(n, kChunk) + 8;
-  size_t b = kSelFixedBytes + (size_t)nt * 4 * 2;
+  size_t b = kSelFixedBytes + (size_t)nt * 4 * 2 + fast_bytes_for_tiles(nt);
   return (b + 255) & ~(size_t)255;
 }
 
@@ -68,10 +105,18 @@ static inline bool sel_ws_carve(void* ws, size_t bytes, int64_t n_tiles_needed,
                                 SelWorkspace* out) {
   if (!ws || bytes < kSelFixedBytes || (reinterpret_cast<uintptr_t>(ws) & 15))
     return false;
-  const int64_t nt = (int64_t)((bytes - kSelFixedBytes) / 8);
+  // largest nt whose full layout fits (layout size is monotone in nt)
+  int64_t lo = 0, hi = (int64_t)((bytes - kSelFixedBytes) / 8);
+  while (lo < hi) {
+    const int64_t mid = lo + (hi - lo + 1) / 2;
+    if (kSelFixedBytes + (size_t)mid * 8 + fast_bytes_for_tiles(mid) <= bytes) lo = mid;
+    else hi = mid - 1;
+  }
+  const int64_t nt = lo;
   if (nt < n_tiles_needed) return false;
   char* p = reinterpret_cast<char*>(ws);
   out->st = reinterpret_cast<SelState*>(p);
+  out->aux = reinterpret_cast<SelState*>(p + 128);
   p += 256;
   out->hist = reinterpret_cast<uint32_t*>(p);
   p += (size_t)(2 * kBinsBig + kBinsSmall + 64) * 4;
@@ -82,7 +127,26 @@ static inline bool sel_ws_carve(void* ws, size_t bytes, int64_t n_tiles_needed,
   out->tile_gt = reinterpret_cast<uint32_t*>(p);
   p += (size_t)nt * 4;
   out->tile_eq = reinterpret_cast<uint32_t*>(p);
+  p += (size_t)nt * 4;
   out->n_tiles_cap = nt;
+  out->sample = nullptr;
+  out->sample_cap = 0;
+  out->seg_cap = 0;
+  if (fast_bytes_for_tiles(nt) > 0) {
+    const int64_t n = nt * kChunk;
+    p = reinterpret_cast<char*>((reinterpret_cast<uintptr_t>(p) + 255) & ~(uintptr_t)255);
+    out->sample_cap = fast_sample_vecs(n) * 4;
+    out->seg_cap = fast_seg_cap(n);
+    out->sample = reinterpret_cast<uint32_t*>(p);
+    p += (size_t)out->sample_cap * 4;
+    out->seg_cnt = reinterpret_cast<uint32_t*>(p);
+    p += (size_t)(kSegWaves + 64) * 4;
+    const size_t seg_bytes = (size_t)kSegWaves * out->seg_cap * 4;
+    out->seg_idx = reinterpret_cast<uint32_t*>(p); p += seg_bytes;
+    out->seg_key = reinterpret_cast<uint32_t*>(p); p += seg_bytes;
+    out->cand_idx = reinterpret_cast<uint32_t*>(p); p += seg_bytes;
+    out->cand_key = reinterpret_cast<uint32_t*>(p);
+  }
   return true;
 }
 
@@ -140,12 +204,17 @@ __device__ __forceinline__ void level_bin(uint32_t key, uint32_t prefix, bool va
   else { bin = key & (kBinsSmall - 1); part = valid && (key >> kL1Shift) == prefix; }
 }
 
+// n_dev (optional) caps n with a count produced on the device; a state whose
+// `skip` flag is set turns the kernel into a no-op.
 template <class Src, int LEVEL>
 __global__ __launch_bounds__(kBlock) void k_level_hist(Src src, int64_t n,
+                                                       const uint32_t* __restrict__ n_dev,
                                                        const SelState* __restrict__ st,
                                                        uint32_t* __restrict__ hist) {
   constexpr int NB = LEVEL == 2 ? kBinsSmall : kBinsBig;
   __shared__ uint32_t s_h[NB];
+  if (st->skip) return;
+  if (n_dev && (int64_t)*n_dev < n) n = (int64_t)*n_dev;
   for (int b = threadIdx.x; b < NB; b += kBlock) s_h[b] = 0u;
   __syncthreads();
   const uint32_t prefix = st->prefix;
@@ -180,6 +249,7 @@ __global__ __launch_bounds__(kBlock) void k_level_scan(SelState* __restrict__ st
   constexpr int BITS = LEVEL == 2 ? kL2Bits : 12;
   __shared__ uint32_t s_suf[kBlock + 1];
   const int t = threadIdx.x;
+  if (st->skip) return;
   // read the incoming rank before any barrier: the one thread that descends
   // overwrites st->krem after the barriers below
   const uint32_t krem = (LEVEL == 0) ? st->k : st->krem;
@@ -234,6 +304,9 @@ __global__ __launch_bounds__(kBlock) void k_level_scan(SelState* __restrict__ st
   }
 }
 
+// Zero the level histograms and reset a state for a new descent.  With
+// `from` given, the rank comes from the device (from->krem) and the descent
+// is skipped when from->skip == skip_when... see the callers.
 static __global__ void k_sel_begin(SelState* st, uint32_t* hist, int nhist, uint32_t k) {
   for (int i = threadIdx.x; i < nhist; i += blockDim.x) hist[i] = 0u;
   if (threadIdx.x == 0) {
@@ -241,6 +314,12 @@ static __global__ void k_sel_begin(SelState* st, uint32_t* hist, int nhist, uint
     z.k = k;
     *st = z;
   }
+}
+
+// Re-zero the level histograms ahead of the radix passes when they will run.
+static __global__ void k_hist_rezero(const SelState* st, uint32_t* hist, int nhist) {
+  if (st->skip) return;
+  for (int i = threadIdx.x; i < nhist; i += blockDim.x) hist[i] = 0u;
 }
 
 // Per-chunk (1024 elements, one wave) counts of keys above / equal to the
@@ -251,6 +330,7 @@ __global__ __launch_bounds__(kBlock) void k_tile_count(Src src, int64_t n,
                                                        const SelState* __restrict__ st,
                                                        uint32_t* __restrict__ tile_gt,
                                                        uint32_t* __restrict__ tile_eq) {
+  if (st->skip) return;
   const uint32_t T = st->thresh_bits;
   const int64_t n_chunks = cdiv64(n, kChunk);
   const int64_t wstride = (int64_t)gridDim.x * kChunksPerBlock;
@@ -482,18 +562,26 @@ static __global__ void k_sel_result(const SelState* st, sga_select_result* out) 
 
 // -------------------------------------------------------------- host drivers
 template <class Src>
+static inline void launch_level_hist_on(Src src, int64_t n, const uint32_t* n_dev, int level,
+                                        SelState* st, const SelWorkspace& w, hipStream_t s) {
+  dim3 grid(stream_grid(n, (int64_t)kBlock * kVec * 4, 256 * 8)), block(kBlock);
+  if (level == 0) hipLaunchKernelGGL((k_level_hist<Src, 0>), grid, block, 0, s, src, n, n_dev, st, w.hist);
+  else if (level == 1) hipLaunchKernelGGL((k_level_hist<Src, 1>), grid, block, 0, s, src, n, n_dev, st, w.hist + kBinsBig);
+  else hipLaunchKernelGGL((k_level_hist<Src, 2>), grid, block, 0, s, src, n, n_dev, st, w.hist + 2 * kBinsBig);
+}
+template <class Src>
 static inline void launch_level_hist(Src src, int64_t n, int level,
                                      const SelWorkspace& w, hipStream_t s) {
-  dim3 grid(stream_grid(n, (int64_t)kBlock * kVec * 4, 256 * 8)), block(kBlock);
-  if (level == 0) hipLaunchKernelGGL((k_level_hist<Src, 0>), grid, block, 0, s, src, n, w.st, w.hist);
-  else if (level == 1) hipLaunchKernelGGL((k_level_hist<Src, 1>), grid, block, 0, s, src, n, w.st, w.hist + kBinsBig);
-  else hipLaunchKernelGGL((k_level_hist<Src, 2>), grid, block, 0, s, src, n, w.st, w.hist + 2 * kBinsBig);
+  launch_level_hist_on(src, n, (const uint32_t*)nullptr, level, w.st, w, s);
 }
 
+static inline void launch_level_scan_on(int level, SelState* st, const SelWorkspace& w, hipStream_t s) {
+  if (level == 0) hipLaunchKernelGGL((k_level_scan<0>), dim3(1), dim3(kBlock), 0, s, st, w.hist);
+  else if (level == 1) hipLaunchKernelGGL((k_level_scan<1>), dim3(1), dim3(kBlock), 0, s, st, w.hist + kBinsBig);
+  else hipLaunchKernelGGL((k_level_scan<2>), dim3(1), dim3(kBlock), 0, s, st, w.hist + 2 * kBinsBig);
+}
 static inline void launch_level_scan(int level, const SelWorkspace& w, hipStream_t s) {
-  if (level == 0) hipLaunchKernelGGL((k_level_scan<0>), dim3(1), dim3(kBlock), 0, s, w.st, w.hist);
-  else if (level == 1) hipLaunchKernelGGL((k_level_scan<1>), dim3(1), dim3(kBlock), 0, s, w.st, w.hist + kBinsBig);
-  else hipLaunchKernelGGL((k_level_scan<2>), dim3(1), dim3(kBlock), 0, s, w.st, w.hist + 2 * kBinsBig);
+  launch_level_scan_on(level, w.st, w, s);
 }
 
 static inline void launch_begin(uint32_t k, const SelWorkspace& w, hipStream_t s) {
@@ -514,6 +602,250 @@ static inline void launch_tile_scan(int64_t n_tiles, int tie_all,
   const int nb = (int)cdiv64(n_tiles, kTileScanSpan);
   hipLaunchKernelGGL(k_tile_sums, dim3(nb), dim3(kBlock), 0, s, w.tile_gt, w.tile_eq, n_tiles, w.blk_gt, w.blk_eq);
   hipLaunchKernelGGL(k_tile_apply, dim3(nb), dim3(kBlock), 0, s, w.tile_gt, w.tile_eq, n_tiles, w.blk_gt, w.blk_eq, nb, tie_all, w.st);
+}
+
+// ===================================================== sampled-bracket path
+// The k-th largest key is bracketed from a small deterministic sample, so
+// the full data needs ONE sweep instead of four: that sweep counts, per
+// chunk, the keys above the bracket and collects the few keys inside it;
+// the exact threshold is then selected among those candidates only.  The
+// result is exact for any sample; if the bracket misses the k-th key (or the
+// candidate buffers overflow, e.g. on tie-heavy data) a flag routes the work
+// to the radix passes, all on the device.
+
+__device__ __forceinline__ uint32_t mix32(uint32_t x) {
+  x ^= x >> 16; x *= 0x7FEB352Du; x ^= x >> 15; x *= 0x846CA68Bu; x ^= x >> 16;
+  return x;
+}
+
+// One 4-element vector per window of `win` vectors, at a hashed offset.
+template <class Src>
+__global__ __launch_bounds__(kBlock) void k_sample(Src src, int64_t n, int64_t n_sv, int64_t win,
+                                                   uint32_t* __restrict__ keys) {
+  for (int64_t j = (int64_t)blockIdx.x * kBlock + threadIdx.x; j < n_sv;
+       j += (int64_t)gridDim.x * kBlock) {
+    const int64_t vec = j * win + (int64_t)(mix32((uint32_t)j) % (uint32_t)win);
+    uint32_t key[4];
+    src.load(vec * 4, n, key);
+    U4 o{key[0], key[1], key[2], key[3]};
+    *reinterpret_cast<U4*>(keys + j * 4) = o;
+  }
+}
+
+// Ranks of the bracket ends inside the sample: r = k*ns/n -/+ (5 sigma + 8).
+static __global__ void k_bracket_ranks(SelState* st, SelState* aux, uint32_t* hist, int nhist,
+                                       int which, uint32_t k, double n, double ns) {
+  for (int i = threadIdx.x; i < nhist; i += blockDim.x) hist[i] = 0u;
+  if (threadIdx.x != 0) return;
+  const double frac = (double)k / n;
+  const double r = frac * ns;
+  const double d = 5.0 * sqrt(r * (1.0 - frac) + 1.0) + 8.0;
+  SelState z = {};
+  if (which == 0) {            // upper end: a smaller rank = a larger key
+    const double rk = floor(r - d);
+    if (rk < 1.0) { z.skip = 1; st->t_hi = 0x80000000u; }
+    else z.k = (uint32_t)rk;
+  } else {                     // lower end
+    const double rk = ceil(r + d);
+    if (rk > ns) { z.skip = 1; st->t_lo = 0u; }
+    else z.k = (uint32_t)rk;
+  }
+  *aux = z;
+}
+
+static __global__ void k_bracket_set(SelState* st, const SelState* aux, int which) {
+  if (aux->skip) return;
+  if (which == 0) st->t_hi = aux->thresh_bits + 1u;   // keys equal to the sample key stay candidates
+  else st->t_lo = aux->thresh_bits;
+}
+
+// The one sweep over the data.  A persistent grid of kSegWaves waves; each
+// wave owns a private candidate segment, so no atomics are needed and the
+// candidates of a chunk stay in ascending index order.
+template <class Src>
+__global__ __launch_bounds__(kBlock) void k_bracket_sweep(
+    Src src, int64_t n, SelState* __restrict__ st, uint32_t* __restrict__ tile_gt,
+    uint32_t* __restrict__ tile_eq, uint32_t* __restrict__ seg_idx, uint32_t* __restrict__ seg_key,
+    uint32_t* __restrict__ seg_cnt, uint32_t seg_cap) {
+  __shared__ uint32_t s_hi[kChunksPerBlock], s_nf[kChunksPerBlock];
+  const uint32_t T_LO = st->t_lo, T_HI = st->t_hi;
+  const int64_t n_chunks = cdiv64(n, kChunk);
+  const int64_t gw = (int64_t)blockIdx.x * kChunksPerBlock + wave_id();
+  const int64_t W = (int64_t)gridDim.x * kChunksPerBlock;
+  uint32_t mycnt = 0, tot_hi = 0, tot_nf = 0;
+  uint32_t* my_idx = seg_idx + gw * seg_cap;
+  uint32_t* my_key = seg_key + gw * seg_cap;
+  for (int64_t c = gw; c < n_chunks; c += W) {
+    uint32_t chi = 0;
+#pragma unroll
+    for (int it = 0; it < kChunkIters; ++it) {
+      const int64_t i = c * kChunk + it * (kWave * kVec) + lane_id() * kVec;
+      uint32_t key[4] = {0, 0, 0, 0};
+      if (i < n) src.load(i, n, key);
+      bool cand[4];
+      uint32_t mine = 0;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const bool valid = i + e < n;
+        chi += (valid && key[e] >= T_HI);
+        tot_nf += (valid && key[e] >= 0x7F800000u);
+        cand[e] = valid && key[e] >= T_LO && key[e] < T_HI;
+        mine += cand[e];
+      }
+      if (ballot64(mine != 0)) {
+        const uint32_t incl = wave_incl_scan(mine);
+        uint32_t pos = mycnt + incl - mine;
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          if (cand[e]) {
+            if (pos < seg_cap) { my_idx[pos] = (uint32_t)(i + e); my_key[pos] = key[e]; }
+            ++pos;
+          }
+        mycnt += __shfl(incl, kWave - 1, kWave);
+      }
+    }
+    chi = wave_sum(chi);
+    tot_hi += chi;
+    if (lane_id() == 0) { tile_gt[c] = chi; tile_eq[c] = 0u; }
+  }
+  tot_nf = wave_sum(tot_nf);
+  if (lane_id() == 0) {
+    seg_cnt[gw] = mycnt < seg_cap ? mycnt : seg_cap;
+    s_hi[wave_id()] = tot_hi;
+    s_nf[wave_id()] = tot_nf;
+    if (mycnt > seg_cap) atomicOr(&st->overflow, 1u);
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    const uint32_t h = s_hi[0] + s_hi[1] + s_hi[2] + s_hi[3];
+    const uint32_t f = s_nf[0] + s_nf[1] + s_nf[2] + s_nf[3];
+    if (h) atomicAdd(&st->n_hi, h);
+    if (f) atomicAdd(&st->nonfinite, f);
+  }
+}
+
+// Single workgroup: segment counts -> offsets, validate the bracket, arm the
+// candidate descent (aux) or the radix passes (st->skip == 0).
+static __global__ __launch_bounds__(kBlock) void k_bracket_check(SelState* __restrict__ st,
+                                                                 SelState* __restrict__ aux,
+                                                                 uint32_t* __restrict__ seg_cnt,
+                                                                 uint32_t* __restrict__ hist, int nhist) {
+  __shared__ uint32_t s_w4[kChunksPerBlock];
+  constexpr int PER = kSegWaves / kBlock;   // 16
+  uint32_t v[PER], mine = 0;
+#pragma unroll
+  for (int j = 0; j < PER; ++j) { v[j] = seg_cnt[threadIdx.x * PER + j]; mine += v[j]; }
+  uint32_t total;
+  uint32_t run = block_excl_scan(mine, s_w4, total);
+#pragma unroll
+  for (int j = 0; j < PER; ++j) { seg_cnt[threadIdx.x * PER + j] = run; run += v[j]; }
+  for (int i = threadIdx.x; i < nhist; i += kBlock) hist[i] = 0u;
+  if (threadIdx.x == 0) {
+    seg_cnt[kSegWaves] = total;
+    const uint32_t k = st->k, n_hi = st->n_hi;
+    const bool ok = !st->overflow && n_hi < k && k <= n_hi + total;
+    st->cand_count = total;
+    st->bracket_ok = ok ? 1u : 0u;
+    st->skip = ok ? 1u : 0u;          // the radix passes run only when the bracket failed
+    st->path = ok ? 1u : 0u;
+    if (!ok) { st->nonfinite = 0u; st->status = 0u; }   // recounted by the radix passes
+    SelState z = {};
+    z.k = ok ? k - n_hi : 0u;
+    z.skip = ok ? 0u : 1u;
+    *aux = z;
+  }
+}
+
+// Dense candidate list from the per-wave segments (order: wave, then index).
+static __global__ __launch_bounds__(kBlock) void k_cand_compact(
+    const SelState* __restrict__ aux, const uint32_t* __restrict__ seg_off,
+    const uint32_t* __restrict__ seg_idx, const uint32_t* __restrict__ seg_key, uint32_t seg_cap,
+    uint32_t* __restrict__ cand_idx, uint32_t* __restrict__ cand_key) {
+  if (aux->skip) return;
+  for (int w = blockIdx.x * kChunksPerBlock + wave_id(); w < kSegWaves;
+       w += gridDim.x * kChunksPerBlock) {
+    const uint32_t off = seg_off[w], cnt = seg_off[w + 1] - off;
+    for (uint32_t j = lane_id(); j < cnt; j += kWave) {
+      cand_idx[off + j] = seg_idx[(int64_t)w * seg_cap + j];
+      cand_key[off + j] = seg_key[(int64_t)w * seg_cap + j];
+    }
+  }
+}
+
+// After the candidate descent: publish the exact threshold and fold each
+// candidate into its chunk's (above, equal) counts.
+static __global__ __launch_bounds__(kBlock) void k_cand_tiles(
+    SelState* __restrict__ st, const SelState* __restrict__ aux,
+    const uint32_t* __restrict__ cand_idx, const uint32_t* __restrict__ cand_key,
+    uint32_t* __restrict__ tile_gt, uint32_t* __restrict__ tile_eq) {
+  if (aux->skip) return;
+  const uint32_t T = aux->thresh_bits;
+  const uint32_t nc = st->cand_count;
+  if (blockIdx.x == 0 && threadIdx.x == 0) {
+    st->thresh_bits = T;
+    st->need = aux->need;
+    st->n_eq = aux->n_eq;
+    st->n_gt = st->k - aux->need;
+    st->status = aux->status;
+  }
+  for (uint32_t j = blockIdx.x * kBlock + threadIdx.x; j < nc; j += gridDim.x * kBlock) {
+    const uint32_t key = cand_key[j];
+    if (key > T) atomicAdd(&tile_gt[cand_idx[j] >> 10], 1u);
+    else if (key == T) atomicAdd(&tile_eq[cand_idx[j] >> 10], 1u);
+  }
+}
+static_assert(kChunk == 1024, "candidate -> chunk mapping uses idx >> 10");
+
+// Full select up to (and including) the tile scan: afterwards st holds the
+// threshold / need and tile_gt / tile_eq hold, per chunk, the number of
+// selected coordinates and of ties before it.
+template <class Src>
+static inline void run_select(Src src, int64_t n, int64_t k, int tie_all, bool fast,
+                              const SelWorkspace& w, hipStream_t s) {
+  const int nh = 2 * kBinsBig + kBinsSmall;
+  const int64_t n_tiles = cdiv64(n, kChunk);
+  launch_begin((uint32_t)k, w, s);
+  if (fast && n >= kFastMinN && w.sample && n < (1ll << 32)) {
+    int64_t n_sv = w.sample_cap / 4;
+    const int64_t n_vec = n / 4;
+    if (n_sv > n_vec) n_sv = n_vec;
+    const int64_t win = n_vec / n_sv;
+    const int64_t ns = n_sv * 4;
+    hipLaunchKernelGGL((k_sample<Src>), dim3(stream_grid(n_sv, kBlock)), dim3(kBlock), 0, s, src, n,
+                       n_sv, win, w.sample);
+    SrcU32 ssrc{w.sample};
+    for (int which = 0; which < 2; ++which) {
+      hipLaunchKernelGGL(k_bracket_ranks, dim3(1), dim3(kBlock), 0, s, w.st, w.aux, w.hist, nh, which,
+                         (uint32_t)k, (double)n, (double)ns);
+      for (int level = 0; level < 3; ++level) {
+        launch_level_hist_on(ssrc, ns, (const uint32_t*)nullptr, level, w.aux, w, s);
+        launch_level_scan_on(level, w.aux, w, s);
+      }
+      hipLaunchKernelGGL(k_bracket_set, dim3(1), dim3(1), 0, s, w.st, w.aux, which);
+    }
+    hipLaunchKernelGGL((k_bracket_sweep<Src>), dim3(kSegWaves / kChunksPerBlock), dim3(kBlock), 0, s,
+                       src, n, w.st, w.tile_gt, w.tile_eq, w.seg_idx, w.seg_key, w.seg_cnt,
+                       (uint32_t)w.seg_cap);
+    hipLaunchKernelGGL(k_bracket_check, dim3(1), dim3(kBlock), 0, s, w.st, w.aux, w.seg_cnt, w.hist, nh);
+    hipLaunchKernelGGL(k_cand_compact, dim3(256), dim3(kBlock), 0, s, w.aux, w.seg_cnt, w.seg_idx,
+                       w.seg_key, (uint32_t)w.seg_cap, w.cand_idx, w.cand_key);
+    SrcU32 csrc{w.cand_key};
+    const int64_t cmax = (int64_t)kSegWaves * w.seg_cap;
+    for (int level = 0; level < 3; ++level) {
+      launch_level_hist_on(csrc, cmax, &w.st->cand_count, level, w.aux, w, s);
+      launch_level_scan_on(level, w.aux, w, s);
+    }
+    hipLaunchKernelGGL(k_cand_tiles, dim3(256), dim3(kBlock), 0, s, w.st, w.aux, w.cand_idx,
+                       w.cand_key, w.tile_gt, w.tile_eq);
+    // radix passes: no-ops unless the bracket failed (st->skip == 0)
+    hipLaunchKernelGGL(k_hist_rezero, dim3(1), dim3(kBlock), 0, s, w.st, w.hist, nh);
+  }
+  for (int level = 0; level < 3; ++level) {
+    launch_level_hist(src, n, level, w, s);
+    launch_level_scan(level, w, s);
+  }
+  launch_tile_count(src, n, 0, w, s);
+  launch_tile_scan(n_tiles, tie_all, w, s);
 }
 
 #endif  // __HIPCC__

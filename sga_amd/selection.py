@@ -74,6 +74,14 @@ def select_exact_device(views, k, tie_mode, masks=None):
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
     res = torch.empty(8, dtype=torch.int32, device=dev)
     st = L.stream()
+    if masks is None:
+        masks = [torch.empty(g.numel(), dtype=torch.uint8, device=dev) for g in views]
+    if len(views) == 1:
+        # one contiguous array: the single-call entry point (sampled bracket
+        # with the radix passes as the on-device fallback)
+        L.call("sga_select_topk", L.ptr(views[0]), n_total, k, tie_mode, L.ptr(masks[0]),
+               L.ptr(res), L.ptr(ws), ws_bytes, st)
+        return res, masks
     L.call("sga_sel_begin", k, L.ptr(ws), ws_bytes, st)
     for level in range(3):
         for g in views:
@@ -82,8 +90,6 @@ def select_exact_device(views, k, tie_mode, masks=None):
     for g, b in zip(views, bases):
         L.call("sga_sel_count", L.ptr(g), g.numel(), b, L.ptr(ws), ws_bytes, st)
     L.call("sga_sel_tile_scan", max(nt, 1), tie_mode, L.ptr(ws), ws_bytes, st)
-    if masks is None:
-        masks = [torch.empty(g.numel(), dtype=torch.uint8, device=dev) for g in views]
     for g, b, m in zip(views, bases, masks):
         L.call("sga_sel_mask", L.ptr(g), g.numel(), b, tie_mode, L.ptr(m), L.ptr(ws),
                ws_bytes, st)

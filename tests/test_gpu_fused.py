@@ -113,3 +113,26 @@ def test_tie_heavy_gradients(dev):
         assert fs.read_result().thresh == th
         assert torch.equal(idx.cpu(), idx_ref) and torch.equal(vals.cpu(), val_ref)
         assert torch.equal(er.cpu(), rr) and torch.equal(em.cpu(), mm)
+
+
+def test_fast_and_radix_paths_agree(dev):
+    """Same inputs through the sampled-bracket path and the plain radix
+    passes: identical idx / values / state, and the fast path is really taken."""
+    from sga_amd.fused_step import FusedSparseStep
+    n = (1 << 21) + 4099
+    segs, _ = _segments([1 << 20, 4099, 1 << 20])
+    gen = torch.Generator().manual_seed(3)
+    base = [torch.randn(n, generator=gen) * 0.02, torch.zeros(n), torch.zeros(n),
+            student_t(n, 8) * 0.3]
+    g = student_t(n, 9).to(torch.bfloat16).to(dev)
+    outs = []
+    for fast in (True, False):
+        p, m, v, r = (t.to(dev).clone() for t in base)
+        fs = FusedSparseStep(n, segs, dev, values_dtype=torch.bfloat16, want_mask=True)
+        idx, vals = fs.step(g, r, p, m, v, 3, ratio_percent=1.0, fast=fast)
+        res = fs.read_result()
+        assert res.path == (1 if fast else 0) and res.status == 0
+        outs.append((idx.clone(), vals.clone(), p, m, v, r, fs.mask.clone(), res.thresh))
+    for a, b in zip(outs[0][:-1], outs[1][:-1]):
+        assert torch.equal(a, b)
+    assert outs[0][-1] == outs[1][-1]

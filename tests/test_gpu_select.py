@@ -148,3 +148,33 @@ def test_replay_select_building_blocks(dev):
     assert K.hist_top16(bad.to(dev))[1] == 2
     assert K.arm(True, torch.float32) and not K.arm(False, torch.float32)
     assert K.formula("update") is not None and K.formula("nope") is None
+
+
+def test_sampled_bracket_path_and_fallback(dev):
+    """n >= 2^20 arms the sampled-bracket path; heavy-tailed data must take
+    it (path == 1), tie-saturated data must fall back to the radix passes on
+    the device (path == 0); both bit-exact vs the oracle."""
+    from sga_amd import _lib as L
+    from sga_amd.selection import read_result, select_exact_device
+    n = (1 << 21) + 777
+    gen = torch.Generator().manual_seed(99)
+    fams = adversarial(n, gen)
+    fams["student-t"] = student_t(n, 5).abs()
+    fams["gauss"] = torch.randn(n, generator=gen).abs()
+    seen = set()
+    for name, sc in fams.items():
+        sd = sc.to(dev)
+        for k in sorted({1, n // 1000, n // 100, n // 10, n - 1}):
+            m_ref, t_ref = SEL.select_topk_flat(sc, k)
+            mask = torch.empty(n, dtype=torch.uint8, device=dev)
+            res, _ = select_exact_device([sd], k, L.TIE_LOWEST_INDEX, masks=[mask])
+            r = read_result(res)
+            assert r.status == 0 and r.n_selected == k, (name, k, vars(r))
+            assert r.thresh == t_ref, (name, k)
+            assert torch.equal(mask.cpu().bool(), m_ref), (name, k)
+            seen.add((name, r.path))
+            # ties-all mode through the same path
+            res2, (m2,) = select_exact_device([sd], k, L.TIE_ALL)
+            assert torch.equal(m2.cpu().bool(), sc >= t_ref), (name, k)
+    assert ("student-t", 1) in seen and ("gauss", 1) in seen
+    assert ("all-equal", 0) in seen
