@@ -28,7 +28,7 @@ def _hipcc():
     raise RuntimeError("hipcc not found")
 
 
-def build(verbose=True, jobs=8):
+def build(verbose=True, jobs=8, extra=()):
     hipcc = _hipcc()
     objdir = os.path.join(HERE, "build")
     os.makedirs(objdir, exist_ok=True)
@@ -36,7 +36,7 @@ def build(verbose=True, jobs=8):
 
     def one(src):
         obj = os.path.join(objdir, src.replace(".hip", ".o"))
-        cmd = [hipcc, *FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
+        cmd = [hipcc, *FLAGS, *extra, "-c", os.path.join(CSRC, src), "-o", obj]
         r = subprocess.run(cmd, capture_output=True, text=True)
         if r.returncode != 0:
             raise RuntimeError(f"hipcc failed on {src}:\n{r.stdout}\n{r.stderr}")
@@ -60,4 +60,4 @@ def build(verbose=True, jobs=8):
 
 
 if __name__ == "__main__":
-    build()
+    build(extra=tuple(a for a in sys.argv[1:] if a.startswith("-D")))

@@ -88,11 +88,26 @@ struct alignas(8) H4 { uint16_t x, y, z, w; };
 struct alignas(16) U4 { uint32_t x, y, z, w; };
 struct alignas(4) B4 { uint8_t x, y, z, w; };
 
+typedef float f4v __attribute__((ext_vector_type(4)));
 __device__ __forceinline__ F4 ld4(const float* p) {
   return *reinterpret_cast<const F4*>(p);
 }
 __device__ __forceinline__ void st4(float* p, const F4& v) {
   *reinterpret_cast<F4*>(p) = v;
+}
+// Streaming (non-temporal) 128-bit accesses for data touched once per sweep.
+__device__ __forceinline__ F4 ld4_nt(const float* p) {
+  const f4v t = __builtin_nontemporal_load(reinterpret_cast<const f4v*>(p));
+  return F4{t.x, t.y, t.z, t.w};
+}
+typedef unsigned short h4v __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ H4 ldh4_nt(const uint16_t* p) {
+  const h4v t = __builtin_nontemporal_load(reinterpret_cast<const h4v*>(p));
+  return H4{t.x, t.y, t.z, t.w};
+}
+__device__ __forceinline__ void st4_nt(float* p, const F4& v) {
+  f4v t = {v.x, v.y, v.z, v.w};
+  __builtin_nontemporal_store(t, reinterpret_cast<f4v*>(p));
 }
 
 // Load 4 consecutive elements starting at i (i % 4 == 0 relative to a
@@ -152,6 +167,57 @@ __device__ __forceinline__ void store4_u8(uint8_t* base, int64_t i, int64_t n,
 #pragma unroll
     for (int e = 0; e < 4; ++e)
       if (i + e < n) base[i + e] = (uint8_t)v[e];
+  }
+}
+
+// FULL variants: when the caller has established (wave-uniformly) that the
+// whole span is in range and vector-aligned, the access is a single
+// unconditional 64/128-bit instruction -- no per-lane branch, so the compiler
+// can keep many loads in flight before the first wait.
+template <bool FULL>
+__device__ __forceinline__ void ld_f32(const float* base, int64_t i, int64_t n, float out[4], bool vec) {
+  if (FULL) {
+    const F4 v = ld4_nt(base + i);
+    out[0] = v.x; out[1] = v.y; out[2] = v.z; out[3] = v.w;
+  } else {
+    load4_f32(base, i, n, out, vec);
+  }
+}
+template <bool FULL>
+__device__ __forceinline__ void ld_bf16(const uint16_t* base, int64_t i, int64_t n, float out[4], bool vec) {
+  if (FULL) {
+    const H4 v = ldh4_nt(base + i);
+    out[0] = bf16_to_f32(v.x); out[1] = bf16_to_f32(v.y);
+    out[2] = bf16_to_f32(v.z); out[3] = bf16_to_f32(v.w);
+  } else {
+    load4_bf16(base, i, n, out, vec);
+  }
+}
+template <bool FULL>
+__device__ __forceinline__ void ld_u8(const uint8_t* base, int64_t i, int64_t n, uint32_t out[4], bool vec) {
+  if (FULL) {
+    const B4 v = *reinterpret_cast<const B4*>(base + i);
+    out[0] = v.x; out[1] = v.y; out[2] = v.z; out[3] = v.w;
+  } else {
+    load4_u8(base, i, n, out, vec);
+  }
+}
+template <bool FULL>
+__device__ __forceinline__ void st_f32(float* base, int64_t i, int64_t n, const float v[4], bool vec) {
+  if (FULL) {
+    F4 t{v[0], v[1], v[2], v[3]};
+    st4_nt(base + i, t);
+  } else {
+    store4_f32(base, i, n, v, vec);
+  }
+}
+template <bool FULL>
+__device__ __forceinline__ void st_u8(uint8_t* base, int64_t i, int64_t n, const uint32_t v[4], bool vec) {
+  if (FULL) {
+    B4 t{(uint8_t)v[0], (uint8_t)v[1], (uint8_t)v[2], (uint8_t)v[3]};
+    *reinterpret_cast<B4*>(base + i) = t;
+  } else {
+    store4_u8(base, i, n, v, vec);
   }
 }
 

@@ -11,10 +11,10 @@
 
 namespace sga {
 
-template <bool BF16G>
+template <bool BF16G, bool FULL = false>
 __device__ __forceinline__ void load_g(const void* g, int64_t i, int64_t n, float out[4], bool vec) {
-  if (BF16G) load4_bf16(reinterpret_cast<const uint16_t*>(g), i, n, out, vec);
-  else load4_f32(reinterpret_cast<const float*>(g), i, n, out, vec);
+  if (BF16G) ld_bf16<FULL>(reinterpret_cast<const uint16_t*>(g), i, n, out, vec);
+  else ld_f32<FULL>(reinterpret_cast<const float*>(g), i, n, out, vec);
 }
 
 // Key source for the select sweeps.
@@ -28,26 +28,27 @@ struct SrcFused {
   const sga_segment* segs;
   int n_segs;
   bool vec;
+  template <bool FULL = false>
   __device__ __forceinline__ void load(int64_t i, int64_t n, uint32_t key[4]) const {
     float gg[4], rr[4];
-    load_g<BF16G>(g, i, n, gg, vec);
-    load4_f32(r, i, n, rr, vec);
+    load_g<BF16G, FULL>(g, i, n, gg, vec);
+    ld_f32<FULL>(r, i, n, rr, vec);
     if (SCORE == SGA_SCORE_ABS_G) {
 #pragma unroll
       for (int e = 0; e < 4; ++e) key[e] = abs_key(rr[e] + gg[e]);
       return;
     }
     float pp[4] = {0, 0, 0, 0}, mm[4], vv[4] = {0, 0, 0, 0};
-    load4_f32(m, i, n, mm, vec);
+    ld_f32<FULL>(m, i, n, mm, vec);
     if (SCORE != SGA_SCORE_ABS_M) {
-      load4_f32(p, i, n, pp, vec);
-      load4_f32(v, i, n, vv, vec);
+      ld_f32<FULL>(p, i, n, pp, vec);
+      ld_f32<FULL>(v, i, n, vv, vec);
     }
     SegCursor sc;
     sc.init(segs, n_segs);
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
-      if (i + e < n) {
+      if (FULL || i + e < n) {
         sc.seek(i + e);
         key[e] = score_key<SCORE>(rr[e] + gg[e], pp[e], mm[e], vv[e], sc.h);
       } else {
@@ -57,94 +58,195 @@ struct SrcFused {
   }
 };
 
-// Final sweep: select flags in index order, pack, residual, commit.
-template <bool BF16G, bool BF16V, int SCORE>
-__global__ __launch_bounds__(kBlock) void k_fused_final(
-    const void* __restrict__ g, float* __restrict__ r, float* __restrict__ p,
-    float* __restrict__ m, float* __restrict__ v, int64_t n, int64_t k,
-    const sga_segment* __restrict__ segs, int n_segs,
-    const SelState* __restrict__ st, const uint32_t* __restrict__ tile_sel,
-    const uint32_t* __restrict__ tile_eq, int32_t* __restrict__ idx_out,
-    void* __restrict__ values_out, uint8_t* __restrict__ mask_out, float factor,
-    float coeff, bool vec, bool mvec) {
-  const uint32_t T = st->thresh_bits;
-  const uint32_t need = st->need;
-  const bool scale = factor != 1.0f;
-  const bool apply_coeff = coeff != 1.0f;
-  const int64_t n_chunks = cdiv64(n, kChunk);
-  const int64_t wstride = (int64_t)gridDim.x * kChunksPerBlock;
-  SegCursor sc;
-  sc.init(segs, n_segs);
-  for (int64_t c = (int64_t)blockIdx.x * kChunksPerBlock + wave_id(); c < n_chunks;
-       c += wstride) {
-    ChunkCursor cur;
-    cur.sel_run = tile_sel[c];
-    cur.eq_run = tile_eq[c];
+// Commit used by the final sweep when the score does not depend on the
+// update itself (|g+r|, |m|): m' and v' are the exact separately-rounded
+// chain; the update direction uses reciprocal / hardware sqrt (about 1 ulp
+// each), which moves p by far less than 1e-6 of lr*|update|.
+struct FastHyper {
+  float inv_bc1, inv_bc2;
+};
+__device__ __forceinline__ void commit_fast(float& p, float g, float& m, float& v, const Hyper& h,
+                                            const FastHyper& f) {
+  const float sa = m * h.b1 + g * h.om1;
+  const float sb = v * h.b2 + (g * h.om2) * g;
+  const float den = __builtin_amdgcn_sqrtf(sb * f.inv_bc2) + h.eps;
+  const float u = (sa * f.inv_bc1) * __builtin_amdgcn_rcpf(den);
+  const float upd = h.wd * p + u;
+  p = p - h.lr * upd;
+  m = sa;
+  v = sb;
+}
+
+// Everything the final sweep needs besides the chunk index.
+struct FinalArgs {
+  const void* g;
+  float* r;
+  float* p;
+  float* m;
+  float* v;
+  int64_t n, k;
+  int32_t* idx_out;
+  void* values_out;
+  uint8_t* mask_out;
+  float factor, coeff;
+  uint32_t T, need;
+  bool vec, mvec, scale, apply_coeff;
+};
+
+// One 1024-element chunk of the final sweep, owned by one wave.  FULL: the
+// chunk is entirely in range and every array is vector-aligned, so all 20
+// loads are unconditional and issued before the first use.
+template <bool BF16G, bool BF16V, int SCORE, bool FULL>
+__device__ __forceinline__ void final_chunk(const FinalArgs& a, int64_t c, uint32_t sel_base,
+                                            uint32_t eq_base, SegCursor& sc, FastHyper& fh,
+                                            int64_t& fh_lo, int64_t& fh_hi) {
+  constexpr bool kFast = (SCORE == SGA_SCORE_ABS_G || SCORE == SGA_SCORE_ABS_M);
+  const int64_t n = a.n;
+  ChunkCursor cur;
+  cur.sel_run = sel_base;
+  cur.eq_run = eq_base;
+  float gg[kChunkIters][4], rr[kChunkIters][4], pp[kChunkIters][4], mm[kChunkIters][4],
+      vv[kChunkIters][4];
+  if (FULL) {
+    // raw loads first (bf16 kept packed), a scheduling fence, then unpacking:
+    // the wave has all 20 loads of its chunk in flight before the first wait
+    H4 graw_h[kChunkIters];
+    F4 graw_f[kChunkIters], rraw[kChunkIters], praw[kChunkIters], mraw[kChunkIters],
+        vraw[kChunkIters];
 #pragma unroll
     for (int it = 0; it < kChunkIters; ++it) {
       const int64_t i = c * kChunk + it * (kWave * kVec) + lane_id() * kVec;
-      float gg[4] = {0, 0, 0, 0}, rr[4] = {0, 0, 0, 0}, pp[4] = {0, 0, 0, 0},
-            mm[4] = {0, 0, 0, 0}, vv[4] = {0, 0, 0, 0};
-      if (i < n) {
-        load_g<BF16G>(g, i, n, gg, vec);
-        load4_f32(r, i, n, rr, vec);
-        load4_f32(p, i, n, pp, vec);
-        load4_f32(m, i, n, mm, vec);
-        load4_f32(v, i, n, vv, vec);
-      }
-      float q[4];
-      uint32_t key[4];
-      bool valid[4], sel[4];
+      if (BF16G) graw_h[it] = ldh4_nt(reinterpret_cast<const uint16_t*>(a.g) + i);
+      else graw_f[it] = ld4_nt(reinterpret_cast<const float*>(a.g) + i);
+      rraw[it] = ld4_nt(a.r + i);
+      praw[it] = ld4_nt(a.p + i);
+      mraw[it] = ld4_nt(a.m + i);
+      vraw[it] = ld4_nt(a.v + i);
+    }
+#ifndef SGA_NO_SCHED_BARRIER
+    __builtin_amdgcn_sched_barrier(0);
+#endif
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        valid[e] = i + e < n;
-        q[e] = rr[e] + gg[e];
-        if (valid[e]) sc.seek(i + e);
-        key[e] = valid[e] ? score_key<SCORE>(q[e], pp[e], mm[e], vv[e], sc.h) : 0u;
+    for (int it = 0; it < kChunkIters; ++it) {
+      if (BF16G) {
+        gg[it][0] = bf16_to_f32(graw_h[it].x); gg[it][1] = bf16_to_f32(graw_h[it].y);
+        gg[it][2] = bf16_to_f32(graw_h[it].z); gg[it][3] = bf16_to_f32(graw_h[it].w);
+      } else {
+        gg[it][0] = graw_f[it].x; gg[it][1] = graw_f[it].y; gg[it][2] = graw_f[it].z; gg[it][3] = graw_f[it].w;
       }
-      uint32_t pos;
-      slab_select(key, valid, T, need, cur, sel, pos);
-      if (i < n) {
-        uint32_t mk[4];
+      rr[it][0] = rraw[it].x; rr[it][1] = rraw[it].y; rr[it][2] = rraw[it].z; rr[it][3] = rraw[it].w;
+      pp[it][0] = praw[it].x; pp[it][1] = praw[it].y; pp[it][2] = praw[it].z; pp[it][3] = praw[it].w;
+      mm[it][0] = mraw[it].x; mm[it][1] = mraw[it].y; mm[it][2] = mraw[it].z; mm[it][3] = mraw[it].w;
+      vv[it][0] = vraw[it].x; vv[it][1] = vraw[it].y; vv[it][2] = vraw[it].z; vv[it][3] = vraw[it].w;
+    }
+  } else {
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          mk[e] = sel[e];
-          if (!valid[e]) continue;
-          sc.seek(i + e);
-          float ge = 0.0f;
-          if (sel[e]) {
-            float val = q[e];
-            if (scale) val = val * factor;
-            if (BF16V) {
-              const uint16_t hb = f32_to_bf16(val);
-              if ((int64_t)pos < k) {
-                idx_out[pos] = (int32_t)(i + e);
-                reinterpret_cast<uint16_t*>(values_out)[pos] = hb;
-              }
-              ge = bf16_to_f32(hb);
-            } else {
-              if ((int64_t)pos < k) {
-                idx_out[pos] = (int32_t)(i + e);
-                reinterpret_cast<float*>(values_out)[pos] = val;
-              }
-              ge = val;
-            }
-            ++pos;
-            if (apply_coeff) ge = ge * coeff;
-          }
-          const Commit cm = adamw_commit(pp[e], ge, mm[e], vv[e], sc.h);
-          pp[e] = pp[e] - sc.h.lr * cm.upd;
-          mm[e] = cm.m_new;
-          vv[e] = cm.v_new;
-          rr[e] = sel[e] ? 0.0f : q[e];
-        }
-        store4_f32(r, i, n, rr, vec);
-        store4_f32(m, i, n, mm, vec);
-        store4_f32(v, i, n, vv, vec);
-        store4_f32(p, i, n, pp, vec);
-        if (mask_out) store4_u8(mask_out, i, n, mk, mvec);
+    for (int it = 0; it < kChunkIters; ++it) {
+      const int64_t i = c * kChunk + it * (kWave * kVec) + lane_id() * kVec;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) gg[it][e] = rr[it][e] = pp[it][e] = mm[it][e] = vv[it][e] = 0.0f;
+      if (i < n) {
+        load_g<BF16G, false>(a.g, i, n, gg[it], a.vec);
+        load4_f32(a.r, i, n, rr[it], a.vec);
+        load4_f32(a.p, i, n, pp[it], a.vec);
+        load4_f32(a.m, i, n, mm[it], a.vec);
+        load4_f32(a.v, i, n, vv[it], a.vec);
       }
     }
+  }
+#pragma unroll
+  for (int it = 0; it < kChunkIters; ++it) {
+    const int64_t i = c * kChunk + it * (kWave * kVec) + lane_id() * kVec;
+    float q[4];
+    uint32_t key[4];
+    bool valid[4], sel[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      valid[e] = FULL || i + e < n;
+      q[e] = rr[it][e] + gg[it][e];
+      if (SCORE == SGA_SCORE_ABS_G) key[e] = abs_key(q[e]);
+      else if (SCORE == SGA_SCORE_ABS_M) key[e] = abs_key(mm[it][e]);
+      else {
+        if (valid[e]) sc.seek(i + e);
+        key[e] = valid[e] ? score_key<SCORE>(q[e], pp[it][e], mm[it][e], vv[it][e], sc.h) : 0u;
+      }
+    }
+    uint32_t pos;
+    slab_select(key, valid, a.T, a.need, cur, sel, pos);
+    if (FULL || i < n) {
+      uint32_t mk[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        mk[e] = sel[e];
+        if (!valid[e]) continue;
+        sc.seek(i + e);
+        float ge = 0.0f;
+        if (sel[e]) {
+          float val = q[e];
+          if (a.scale) val = val * a.factor;
+          if (BF16V) {
+            const uint16_t hb = f32_to_bf16(val);
+            if ((int64_t)pos < a.k) {
+              a.idx_out[pos] = (int32_t)(i + e);
+              reinterpret_cast<uint16_t*>(a.values_out)[pos] = hb;
+            }
+            ge = bf16_to_f32(hb);
+          } else {
+            if ((int64_t)pos < a.k) {
+              a.idx_out[pos] = (int32_t)(i + e);
+              reinterpret_cast<float*>(a.values_out)[pos] = val;
+            }
+            ge = val;
+          }
+          ++pos;
+          if (a.apply_coeff) ge = ge * a.coeff;
+        }
+        if (kFast) {
+          if (sc.lo != fh_lo || sc.hi != fh_hi) {
+            fh.inv_bc1 = __fdiv_rn(1.0f, sc.h.bc1);
+            fh.inv_bc2 = __fdiv_rn(1.0f, sc.h.bc2);
+            fh_lo = sc.lo; fh_hi = sc.hi;
+          }
+          commit_fast(pp[it][e], ge, mm[it][e], vv[it][e], sc.h, fh);
+        } else {
+          const Commit cm = adamw_commit(pp[it][e], ge, mm[it][e], vv[it][e], sc.h);
+          pp[it][e] = pp[it][e] - sc.h.lr * cm.upd;
+          mm[it][e] = cm.m_new;
+          vv[it][e] = cm.v_new;
+        }
+        rr[it][e] = sel[e] ? 0.0f : q[e];
+      }
+      st_f32<FULL>(a.r, i, n, rr[it], a.vec);
+      st_f32<FULL>(a.m, i, n, mm[it], a.vec);
+      st_f32<FULL>(a.v, i, n, vv[it], a.vec);
+      st_f32<FULL>(a.p, i, n, pp[it], a.vec);
+      if (a.mask_out) st_u8<FULL>(a.mask_out, i, n, mk, a.mvec);
+    }
+  }
+}
+
+// Final sweep: select flags in index order, pack, residual, commit.
+template <bool BF16G, bool BF16V, int SCORE>
+__global__ __launch_bounds__(kBlock) void k_fused_final(
+    FinalArgs a, const sga_segment* __restrict__ segs, int n_segs,
+    const SelState* __restrict__ st, const uint32_t* __restrict__ tile_sel,
+    const uint32_t* __restrict__ tile_eq) {
+  a.T = st->thresh_bits;
+  a.need = st->need;
+  const int64_t n_chunks = cdiv64(a.n, kChunk);
+  const int64_t wstride = (int64_t)gridDim.x * kChunksPerBlock;
+  SegCursor sc;
+  sc.init(segs, n_segs);
+  FastHyper fh{1.0f, 1.0f};
+  int64_t fh_lo = 1, fh_hi = 0;
+  const bool can_full = a.vec && (a.mask_out == nullptr || a.mvec);
+  for (int64_t c = (int64_t)blockIdx.x * kChunksPerBlock + wave_id(); c < n_chunks;
+       c += wstride) {
+    const uint32_t sb = tile_sel[c], eb = tile_eq[c];
+    if (can_full && (c + 1) * kChunk <= a.n)
+      final_chunk<BF16G, BF16V, SCORE, true>(a, c, sb, eb, sc, fh, fh_lo, fh_hi);
+    else
+      final_chunk<BF16G, BF16V, SCORE, false>(a, c, sb, eb, sc, fh, fh_lo, fh_hi);
   }
 }
 
@@ -177,10 +279,15 @@ static int run_fused(const void* g, float* resid, float* p, float* m, float* v, 
   const int64_t n_tiles = cdiv64(n, kChunk);
   ProfPair* pp = prof_next();
   if (pp) (void)hipEventRecord(pp->a, s);
+  FinalArgs fa;
+  fa.g = g; fa.r = resid; fa.p = p; fa.m = m; fa.v = v; fa.n = n; fa.k = k;
+  fa.idx_out = idx_out; fa.values_out = values_out; fa.mask_out = mask_out;
+  fa.factor = factor; fa.coeff = coeff; fa.T = 0; fa.need = 0;
+  fa.vec = vec; fa.mvec = aligned4(mask_out, 1);
+  fa.scale = factor != 1.0f; fa.apply_coeff = coeff != 1.0f;
   hipLaunchKernelGGL((k_fused_final<BF16G, BF16V, SCORE>),
-                     dim3(stream_grid(n_tiles, kChunksPerBlock, 1 << 20)), dim3(kBlock), 0, s, g,
-                     resid, p, m, v, n, k, segs, n_segs, w.st, w.tile_gt, w.tile_eq, idx_out,
-                     values_out, mask_out, factor, coeff, vec, aligned4(mask_out, 1));
+                     dim3(stream_grid(n_tiles, kChunksPerBlock, 1 << 20)), dim3(kBlock), 0, s, fa,
+                     segs, n_segs, w.st, w.tile_gt, w.tile_eq);
   if (pp) (void)hipEventRecord(pp->b, s);
   if (result) hipLaunchKernelGGL(k_sel_result, dim3(1), dim3(1), 0, s, w.st, result);
   return check_launch("sga_fused_sparse_step");

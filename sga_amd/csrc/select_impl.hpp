@@ -64,7 +64,7 @@ struct SelWorkspace {
   int64_t seg_cap;     // per-wave candidate capacity
 };
 
-constexpr int kSegWaves = 4096;            // persistent waves of the bracket sweep
+constexpr int kSegWaves = 8192;            // persistent waves of the bracket sweep
 constexpr int64_t kFastMinN = 1 << 20;     // below this the radix passes are cheap enough
 
 static inline int64_t fast_sample_vecs(int64_t n) {
@@ -154,12 +154,14 @@ static inline bool sel_ws_carve(void* ws, size_t bytes, int64_t n_tiles_needed,
 
 // ------------------------------------------------------------ key sources
 // A key source yields the 31-bit magnitude keys of 4 consecutive elements.
+// load<FULL>: FULL promises i + 4 <= n and vector alignment (see ld_f32).
 struct SrcF32 {                 // |x| of an fp32 score array
   const float* x;
   bool vec;
+  template <bool FULL = false>
   __device__ __forceinline__ void load(int64_t i, int64_t n, uint32_t key[4]) const {
     float v[4];
-    load4_f32(x, i, n, v, vec);
+    ld_f32<FULL>(x, i, n, v, vec);
 #pragma unroll
     for (int e = 0; e < 4; ++e) key[e] = abs_key(v[e]);
   }
@@ -167,8 +169,10 @@ struct SrcF32 {                 // |x| of an fp32 score array
 
 struct SrcU32 {                 // raw keys (sample / candidate buffers)
   const uint32_t* x;
+  static constexpr bool vec = true;
+  template <bool FULL = false>
   __device__ __forceinline__ void load(int64_t i, int64_t n, uint32_t key[4]) const {
-    if (i + 4 <= n) {
+    if (FULL || i + 4 <= n) {
       U4 v = *reinterpret_cast<const U4*>(x + i);
       key[0] = v.x; key[1] = v.y; key[2] = v.z; key[3] = v.w;
     } else {
@@ -224,12 +228,22 @@ __global__ __launch_bounds__(kBlock) void k_level_hist(Src src, int64_t n,
   for (int64_t base = first; base < n; base += stride) {
     const int64_t i = base + (int64_t)threadIdx.x * kVec;
     uint32_t key[4] = {0, 0, 0, 0};
-    if (i < n) src.load(i, n, key);
+    if (src.vec && base + kBlock * kVec <= n) {      // whole workgroup span in range
+      src.template load<true>(i, n, key);
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      uint32_t bin; bool part;
-      level_bin<LEVEL>(key[e], prefix, i + e < n, bin, part);
-      lds_hist_add(s_h, bin, part);
+      for (int e = 0; e < 4; ++e) {
+        uint32_t bin; bool part;
+        level_bin<LEVEL>(key[e], prefix, true, bin, part);
+        lds_hist_add(s_h, bin, part);
+      }
+    } else {
+      if (i < n) src.template load<false>(i, n, key);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        uint32_t bin; bool part;
+        level_bin<LEVEL>(key[e], prefix, i + e < n, bin, part);
+        lds_hist_add(s_h, bin, part);
+      }
     }
   }
   __syncthreads();
@@ -337,16 +351,27 @@ __global__ __launch_bounds__(kBlock) void k_tile_count(Src src, int64_t n,
   for (int64_t c = (int64_t)blockIdx.x * kChunksPerBlock + wave_id(); c < n_chunks;
        c += wstride) {
     uint32_t cg = 0, ce = 0;
+    if (src.vec && (c + 1) * kChunk <= n) {
+      uint32_t key[kChunkIters][4];
 #pragma unroll
-    for (int it = 0; it < kChunkIters; ++it) {
-      const int64_t i = c * kChunk + it * (kWave * kVec) + lane_id() * kVec;
-      uint32_t key[4] = {0, 0, 0, 0};
-      if (i < n) src.load(i, n, key);
+      for (int it = 0; it < kChunkIters; ++it)
+        src.template load<true>(c * kChunk + it * (kWave * kVec) + lane_id() * kVec, n, key[it]);
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const bool valid = i + e < n;
-        cg += (valid && key[e] > T);
-        ce += (valid && key[e] == T);
+      for (int it = 0; it < kChunkIters; ++it)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) { cg += key[it][e] > T; ce += key[it][e] == T; }
+    } else {
+#pragma unroll
+      for (int it = 0; it < kChunkIters; ++it) {
+        const int64_t i = c * kChunk + it * (kWave * kVec) + lane_id() * kVec;
+        uint32_t key[4] = {0, 0, 0, 0};
+        if (i < n) src.template load<false>(i, n, key);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const bool valid = i + e < n;
+          cg += (valid && key[e] > T);
+          ce += (valid && key[e] == T);
+        }
       }
     }
     cg = wave_sum(cg);
@@ -531,20 +556,27 @@ __global__ __launch_bounds__(kBlock) void k_write_mask(Src src, int64_t n, int64
     ChunkCursor cur;
     cur.sel_run = tile_sel[tile_base + c];
     cur.eq_run = tile_eq[tile_base + c];
+    const bool full = src.vec && mvec && (c + 1) * kChunk <= n;
+    uint32_t key[kChunkIters][4];
 #pragma unroll
     for (int it = 0; it < kChunkIters; ++it) {
       const int64_t i = c * kChunk + it * (kWave * kVec) + lane_id() * kVec;
-      uint32_t key[4] = {0, 0, 0, 0};
-      if (i < n) src.load(i, n, key);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) key[it][e] = 0u;
+      if (full) src.template load<true>(i, n, key[it]);
+      else if (i < n) src.template load<false>(i, n, key[it]);
+    }
+#pragma unroll
+    for (int it = 0; it < kChunkIters; ++it) {
+      const int64_t i = c * kChunk + it * (kWave * kVec) + lane_id() * kVec;
       bool valid[4], sel[4];
 #pragma unroll
-      for (int e = 0; e < 4; ++e) valid[e] = i + e < n;
+      for (int e = 0; e < 4; ++e) valid[e] = full || i + e < n;
       uint32_t pos;
-      slab_select(key, valid, T, need, cur, sel, pos);
-      if (i < n) {
-        uint32_t mk[4] = {sel[0], sel[1], sel[2], sel[3]};
-        store4_u8(mask, i, n, mk, mvec);
-      }
+      slab_select(key[it], valid, T, need, cur, sel, pos);
+      uint32_t mk[4] = {sel[0], sel[1], sel[2], sel[3]};
+      if (full) st_u8<true>(mask, i, n, mk, true);
+      else if (i < n) store4_u8(mask, i, n, mk, mvec);
     }
   }
 }
@@ -626,7 +658,7 @@ __global__ __launch_bounds__(kBlock) void k_sample(Src src, int64_t n, int64_t n
        j += (int64_t)gridDim.x * kBlock) {
     const int64_t vec = j * win + (int64_t)(mix32((uint32_t)j) % (uint32_t)win);
     uint32_t key[4];
-    src.load(vec * 4, n, key);
+    src.template load<false>(vec * 4, n, key);
     U4 o{key[0], key[1], key[2], key[3]};
     *reinterpret_cast<U4*>(keys + j * 4) = o;
   }
@@ -662,6 +694,50 @@ static __global__ void k_bracket_set(SelState* st, const SelState* aux, int whic
 // The one sweep over the data.  A persistent grid of kSegWaves waves; each
 // wave owns a private candidate segment, so no atomics are needed and the
 // candidates of a chunk stay in ascending index order.
+template <class Src, bool FULL>
+__device__ __forceinline__ void bracket_chunk(const Src& src, int64_t n, int64_t c, uint32_t T_LO,
+                                              uint32_t T_HI, uint32_t& chi, uint32_t& tot_nf,
+                                              uint32_t& mycnt, uint32_t seg_cap,
+                                              uint32_t* __restrict__ my_idx,
+                                              uint32_t* __restrict__ my_key) {
+  uint32_t keys[kChunkIters][4];
+#pragma unroll
+  for (int it = 0; it < kChunkIters; ++it) {
+    const int64_t i = c * kChunk + it * (kWave * kVec) + lane_id() * kVec;
+    if (!FULL) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) keys[it][e] = 0u;
+    }
+    if (FULL || i < n) src.template load<FULL>(i, n, keys[it]);
+  }
+#pragma unroll
+  for (int it = 0; it < kChunkIters; ++it) {
+    const int64_t i = c * kChunk + it * (kWave * kVec) + lane_id() * kVec;
+    const uint32_t* key = keys[it];
+    bool cand[4];
+    uint32_t mine = 0;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const bool valid = FULL || i + e < n;
+      chi += (valid && key[e] >= T_HI);
+      tot_nf += (valid && key[e] >= 0x7F800000u);
+      cand[e] = valid && key[e] >= T_LO && key[e] < T_HI;
+      mine += cand[e];
+    }
+    if (ballot64(mine != 0)) {
+      const uint32_t incl = wave_incl_scan(mine);
+      uint32_t pos = mycnt + incl - mine;
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        if (cand[e]) {
+          if (pos < seg_cap) { my_idx[pos] = (uint32_t)(i + e); my_key[pos] = key[e]; }
+          ++pos;
+        }
+      mycnt += __shfl(incl, kWave - 1, kWave);
+    }
+  }
+}
+
 template <class Src>
 __global__ __launch_bounds__(kBlock) void k_bracket_sweep(
     Src src, int64_t n, SelState* __restrict__ st, uint32_t* __restrict__ tile_gt,
@@ -677,33 +753,10 @@ __global__ __launch_bounds__(kBlock) void k_bracket_sweep(
   uint32_t* my_key = seg_key + gw * seg_cap;
   for (int64_t c = gw; c < n_chunks; c += W) {
     uint32_t chi = 0;
-#pragma unroll
-    for (int it = 0; it < kChunkIters; ++it) {
-      const int64_t i = c * kChunk + it * (kWave * kVec) + lane_id() * kVec;
-      uint32_t key[4] = {0, 0, 0, 0};
-      if (i < n) src.load(i, n, key);
-      bool cand[4];
-      uint32_t mine = 0;
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const bool valid = i + e < n;
-        chi += (valid && key[e] >= T_HI);
-        tot_nf += (valid && key[e] >= 0x7F800000u);
-        cand[e] = valid && key[e] >= T_LO && key[e] < T_HI;
-        mine += cand[e];
-      }
-      if (ballot64(mine != 0)) {
-        const uint32_t incl = wave_incl_scan(mine);
-        uint32_t pos = mycnt + incl - mine;
-#pragma unroll
-        for (int e = 0; e < 4; ++e)
-          if (cand[e]) {
-            if (pos < seg_cap) { my_idx[pos] = (uint32_t)(i + e); my_key[pos] = key[e]; }
-            ++pos;
-          }
-        mycnt += __shfl(incl, kWave - 1, kWave);
-      }
-    }
+    if (src.vec && (c + 1) * kChunk <= n)
+      bracket_chunk<Src, true>(src, n, c, T_LO, T_HI, chi, tot_nf, mycnt, seg_cap, my_idx, my_key);
+    else
+      bracket_chunk<Src, false>(src, n, c, T_LO, T_HI, chi, tot_nf, mycnt, seg_cap, my_idx, my_key);
     chi = wave_sum(chi);
     tot_hi += chi;
     if (lane_id() == 0) { tile_gt[c] = chi; tile_eq[c] = 0u; }
