@@ -79,7 +79,7 @@ def main():
     ap.add_argument("--ratio", type=float, default=1.0)
     ap.add_argument("--score", default="abs_g")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--cpu-sample", type=int, default=1 << 27)
+    ap.add_argument("--cpu-sample", type=int, default=1 << 29)
     ap.add_argument("--calib", action="store_true",
                     help="also launch one plain copy of 2^30 fp32 (k_calib_copy) so counter "
                          "runs can be scaled against a kernel of known traffic")
@@ -193,7 +193,7 @@ def main():
                        "ms_per_step": d * 1e3})
         out["sweep"] = sw
     if not args.no_cpu:
-        out["cpu_baseline"] = cpu_baseline(args.cpu_sample, 2, args.ratio)
+        out["cpu_baseline"] = cpu_baseline(args.cpu_sample, 3, args.ratio)
     else:
         out["cpu_baseline"] = None
     print(json.dumps(out))

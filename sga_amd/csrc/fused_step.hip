@@ -96,15 +96,14 @@ struct FinalArgs {
 // One 1024-element chunk of the final sweep, owned by one wave.  FULL: the
 // chunk is entirely in range and every array is vector-aligned, so all 20
 // loads are unconditional and issued before the first use.
-template <bool BF16G, bool BF16V, int SCORE, bool FULL>
-__device__ __forceinline__ void final_chunk(const FinalArgs& a, int64_t c, uint32_t sel_base,
-                                            uint32_t eq_base, SegCursor& sc, FastHyper& fh,
+// IT0 / NIT: the slabs [IT0, IT0+NIT) of the chunk are handled by this call;
+// `cur` carries the running selected / tie counts across calls.
+template <bool BF16G, bool BF16V, int SCORE, bool FULL, int IT0, int NIT>
+__device__ __forceinline__ void final_chunk(const FinalArgs& a, int64_t c, ChunkCursor& cur,
+                                            SegCursor& sc, FastHyper& fh,
                                             int64_t& fh_lo, int64_t& fh_hi) {
   constexpr bool kFast = (SCORE == SGA_SCORE_ABS_G || SCORE == SGA_SCORE_ABS_M);
   const int64_t n = a.n;
-  ChunkCursor cur;
-  cur.sel_run = sel_base;
-  cur.eq_run = eq_base;
   float gg[kChunkIters][4], rr[kChunkIters][4], pp[kChunkIters][4], mm[kChunkIters][4],
       vv[kChunkIters][4];
   if (FULL) {
@@ -114,7 +113,7 @@ __device__ __forceinline__ void final_chunk(const FinalArgs& a, int64_t c, uint3
     F4 graw_f[kChunkIters], rraw[kChunkIters], praw[kChunkIters], mraw[kChunkIters],
         vraw[kChunkIters];
 #pragma unroll
-    for (int it = 0; it < kChunkIters; ++it) {
+    for (int it = IT0; it < IT0 + NIT; ++it) {
       const int64_t i = c * kChunk + it * (kWave * kVec) + lane_id() * kVec;
       if (BF16G) graw_h[it] = ldh4_nt(reinterpret_cast<const uint16_t*>(a.g) + i);
       else graw_f[it] = ld4_nt(reinterpret_cast<const float*>(a.g) + i);
@@ -123,11 +122,9 @@ __device__ __forceinline__ void final_chunk(const FinalArgs& a, int64_t c, uint3
       mraw[it] = ld4_nt(a.m + i);
       vraw[it] = ld4_nt(a.v + i);
     }
-#ifndef SGA_NO_SCHED_BARRIER
     __builtin_amdgcn_sched_barrier(0);
-#endif
 #pragma unroll
-    for (int it = 0; it < kChunkIters; ++it) {
+    for (int it = IT0; it < IT0 + NIT; ++it) {
       if (BF16G) {
         gg[it][0] = bf16_to_f32(graw_h[it].x); gg[it][1] = bf16_to_f32(graw_h[it].y);
         gg[it][2] = bf16_to_f32(graw_h[it].z); gg[it][3] = bf16_to_f32(graw_h[it].w);
@@ -141,7 +138,7 @@ __device__ __forceinline__ void final_chunk(const FinalArgs& a, int64_t c, uint3
     }
   } else {
 #pragma unroll
-    for (int it = 0; it < kChunkIters; ++it) {
+    for (int it = IT0; it < IT0 + NIT; ++it) {
       const int64_t i = c * kChunk + it * (kWave * kVec) + lane_id() * kVec;
 #pragma unroll
       for (int e = 0; e < 4; ++e) gg[it][e] = rr[it][e] = pp[it][e] = mm[it][e] = vv[it][e] = 0.0f;
@@ -155,7 +152,7 @@ __device__ __forceinline__ void final_chunk(const FinalArgs& a, int64_t c, uint3
     }
   }
 #pragma unroll
-  for (int it = 0; it < kChunkIters; ++it) {
+  for (int it = IT0; it < IT0 + NIT; ++it) {
     const int64_t i = c * kChunk + it * (kWave * kVec) + lane_id() * kVec;
     float q[4];
     uint32_t key[4];
@@ -242,11 +239,19 @@ __global__ __launch_bounds__(kBlock) void k_fused_final(
   const bool can_full = a.vec && (a.mask_out == nullptr || a.mvec);
   for (int64_t c = (int64_t)blockIdx.x * kChunksPerBlock + wave_id(); c < n_chunks;
        c += wstride) {
-    const uint32_t sb = tile_sel[c], eb = tile_eq[c];
-    if (can_full && (c + 1) * kChunk <= a.n)
-      final_chunk<BF16G, BF16V, SCORE, true>(a, c, sb, eb, sc, fh, fh_lo, fh_hi);
-    else
-      final_chunk<BF16G, BF16V, SCORE, false>(a, c, sb, eb, sc, fh, fh_lo, fh_hi);
+    ChunkCursor cur;
+    cur.sel_run = tile_sel[c];
+    cur.eq_run = tile_eq[c];
+    if (can_full && (c + 1) * kChunk <= a.n) {
+      // one 256-element slab at a time (5 loads in flight per lane): measured
+      // as fast as batching all four slabs, at twice the occupancy
+      final_chunk<BF16G, BF16V, SCORE, true, 0, 1>(a, c, cur, sc, fh, fh_lo, fh_hi);
+      final_chunk<BF16G, BF16V, SCORE, true, 1, 1>(a, c, cur, sc, fh, fh_lo, fh_hi);
+      final_chunk<BF16G, BF16V, SCORE, true, 2, 1>(a, c, cur, sc, fh, fh_lo, fh_hi);
+      final_chunk<BF16G, BF16V, SCORE, true, 3, 1>(a, c, cur, sc, fh, fh_lo, fh_hi);
+    } else {
+      final_chunk<BF16G, BF16V, SCORE, false, 0, kChunkIters>(a, c, cur, sc, fh, fh_lo, fh_hi);
+    }
   }
 }
 

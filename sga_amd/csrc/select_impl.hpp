@@ -40,14 +40,15 @@ struct SelState {
   uint32_t sample_n;
   uint32_t overflow;    // a candidate segment ran out of room
   uint32_t skip;        // 1: kernels driven by this state do nothing
-  uint32_t pad_[11];
+  uint32_t done[3];     // per-level "workgroups finished" tickets (last one scans)
+  uint32_t pad_[8];
 };
 static_assert(sizeof(SelState) == 128, "SelState layout");
 
 struct SelWorkspace {
   SelState* st;        // main state (result, bracket)
-  SelState* aux;       // scratch state of the sample / candidate selects
-  uint32_t* hist;      // 3 levels: [0,4096) [4096,8192) [8192,8320)
+  SelState* aux;       // aux[0], aux[1]: states of the sample / candidate descents
+  uint32_t* hist;      // 2 sets of 3 levels: [0,4096) [4096,8192) [8192,8320)
   uint32_t* tile_gt;   // n_tiles -> selected-count prefix
   uint32_t* tile_eq;   // n_tiles -> tie-count prefix
   uint32_t* blk_gt;    // kMaxTileBlocks
@@ -70,7 +71,7 @@ constexpr int64_t kFastMinN = 1 << 20;     // below this the radix passes are ch
 static inline int64_t fast_sample_vecs(int64_t n) {
   int64_t v = n / 1024;
   if (v < 16384) v = 16384;
-  if (v > (1 << 20)) v = 1 << 20;
+  if (v > (1 << 18)) v = 1 << 18;
   return v;
 }
 static inline int64_t fast_seg_cap(int64_t n) {
@@ -84,8 +85,10 @@ static inline int64_t fast_seg_cap(int64_t n) {
 // [tile_gt[nt] | tile_eq[nt]] [fast-path buffers sized from nt].  nt is
 // derived from the byte size, so every entry point recovers the same carve
 // from (ws, ws_bytes) alone.
+constexpr int kHistEntries = 2 * kBinsBig + kBinsSmall;      // 8320
+constexpr int kHistStride = kHistEntries + 64;               // per-state stride
 constexpr size_t kSelFixedBytes =
-    256 + (size_t)(2 * kBinsBig + kBinsSmall + 64) * 4 + (size_t)kMaxTileBlocks * 4 * 2;
+    512 + (size_t)kHistStride * 2 * 4 + (size_t)kMaxTileBlocks * 4 * 2;
 
 static inline size_t fast_bytes_for_tiles(int64_t nt) {
   const int64_t n = nt * kChunk;
@@ -117,9 +120,9 @@ static inline bool sel_ws_carve(void* ws, size_t bytes, int64_t n_tiles_needed,
   char* p = reinterpret_cast<char*>(ws);
   out->st = reinterpret_cast<SelState*>(p);
   out->aux = reinterpret_cast<SelState*>(p + 128);
-  p += 256;
+  p += 512;
   out->hist = reinterpret_cast<uint32_t*>(p);
-  p += (size_t)(2 * kBinsBig + kBinsSmall + 64) * 4;
+  p += (size_t)kHistStride * 2 * 4;
   out->blk_gt = reinterpret_cast<uint32_t*>(p);
   p += (size_t)kMaxTileBlocks * 4;
   out->blk_eq = reinterpret_cast<uint32_t*>(p);
@@ -208,62 +211,16 @@ __device__ __forceinline__ void level_bin(uint32_t key, uint32_t prefix, bool va
   else { bin = key & (kBinsSmall - 1); part = valid && (key >> kL1Shift) == prefix; }
 }
 
-// n_dev (optional) caps n with a count produced on the device; a state whose
-// `skip` flag is set turns the kernel into a no-op.
-template <class Src, int LEVEL>
-__global__ __launch_bounds__(kBlock) void k_level_hist(Src src, int64_t n,
-                                                       const uint32_t* __restrict__ n_dev,
-                                                       const SelState* __restrict__ st,
-                                                       uint32_t* __restrict__ hist) {
-  constexpr int NB = LEVEL == 2 ? kBinsSmall : kBinsBig;
-  __shared__ uint32_t s_h[NB];
-  if (st->skip) return;
-  if (n_dev && (int64_t)*n_dev < n) n = (int64_t)*n_dev;
-  for (int b = threadIdx.x; b < NB; b += kBlock) s_h[b] = 0u;
-  __syncthreads();
-  const uint32_t prefix = st->prefix;
-  const int64_t stride = (int64_t)gridDim.x * kBlock * kVec;
-  // uniform trip count so the wave-level ballots inside lds_hist_add are safe
-  const int64_t first = ((int64_t)blockIdx.x * kBlock) * kVec;
-  for (int64_t base = first; base < n; base += stride) {
-    const int64_t i = base + (int64_t)threadIdx.x * kVec;
-    uint32_t key[4] = {0, 0, 0, 0};
-    if (src.vec && base + kBlock * kVec <= n) {      // whole workgroup span in range
-      src.template load<true>(i, n, key);
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        uint32_t bin; bool part;
-        level_bin<LEVEL>(key[e], prefix, true, bin, part);
-        lds_hist_add(s_h, bin, part);
-      }
-    } else {
-      if (i < n) src.template load<false>(i, n, key);
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        uint32_t bin; bool part;
-        level_bin<LEVEL>(key[e], prefix, i + e < n, bin, part);
-        lds_hist_add(s_h, bin, part);
-      }
-    }
-  }
-  __syncthreads();
-  for (int b = threadIdx.x; b < NB; b += kBlock) {
-    const uint32_t c = s_h[b];
-    if (c) atomicAdd(&hist[b], c);
-  }
-}
-
-// Single workgroup: find the bin where the descending cumulative count
-// crosses the remaining rank; descend one level.
+// One level of the descent for one state, run by a single workgroup: find
+// the bin where the descending cumulative count crosses the remaining rank.
 template <int LEVEL>
-__global__ __launch_bounds__(kBlock) void k_level_scan(SelState* __restrict__ st,
-                                                       const uint32_t* __restrict__ hist) {
+__device__ __forceinline__ void level_scan_body(SelState* __restrict__ st,
+                                                const uint32_t* __restrict__ hist,
+                                                uint32_t* s_suf /* kBlock + 1 */) {
   constexpr int NB = LEVEL == 2 ? kBinsSmall : kBinsBig;
   constexpr int PER = NB >= kBlock ? NB / kBlock : 1;
   constexpr int BITS = LEVEL == 2 ? kL2Bits : 12;
-  __shared__ uint32_t s_suf[kBlock + 1];
   const int t = threadIdx.x;
-  if (st->skip) return;
   // read the incoming rank before any barrier: the one thread that descends
   // overwrites st->krem after the barriers below
   const uint32_t krem = (LEVEL == 0) ? st->k : st->krem;
@@ -273,11 +230,11 @@ __global__ __launch_bounds__(kBlock) void k_level_scan(SelState* __restrict__ st
 #pragma unroll
   for (int j = 0; j < PER; ++j) {
     const int b = t * PER + j;
-    loc[j] = (b < NB) ? hist[b] : 0u;
+    loc[j] = (b < NB) ? __atomic_load_n(&hist[b], __ATOMIC_RELAXED) : 0u;
     mine += loc[j];
   }
-  // suffix sums over threads: s_suf[t] = sum of `mine` for threads >= t
-  s_suf[t] = mine;
+  __syncthreads();
+  s_suf[t] = mine;                       // suffix sums over threads
   if (t == 0) s_suf[kBlock] = 0u;
   __syncthreads();
   for (int o = 1; o < kBlock; o <<= 1) {
@@ -290,8 +247,8 @@ __global__ __launch_bounds__(kBlock) void k_level_scan(SelState* __restrict__ st
   if (LEVEL == 0 && t == 0) {
     st->total = total;
     uint32_t nf = 0;
-    for (int b = 0xFF0; b < kBinsBig; ++b) nf += hist[b];   // exponent 255
-    st->nonfinite = nf;
+    for (int b = 0xFF0; b < kBinsBig; ++b) nf += __atomic_load_n(&hist[b], __ATOMIC_RELAXED);
+    st->nonfinite = nf;                  // exponent 255: Inf / NaN
     if (krem < 1 || krem > total) st->status = 1;
   }
   const uint32_t above_me = s_suf[t + 1];
@@ -316,6 +273,96 @@ __global__ __launch_bounds__(kBlock) void k_level_scan(SelState* __restrict__ st
       }
     }
   }
+  __syncthreads();
+}
+
+template <int LEVEL>
+__device__ __forceinline__ uint32_t* level_hist_of(uint32_t* hist_set) {
+  return hist_set + (LEVEL == 0 ? 0 : LEVEL == 1 ? kBinsBig : 2 * kBinsBig);
+}
+
+// Histogram sweep of one radix level for NS states at once (NS = 2 lets the
+// two ends of the sample bracket descend together).  n_dev (optional) caps n
+// with a count produced on the device; a state whose `skip` flag is set does
+// not take part.  MERGE: the last workgroup to finish also runs the level's
+// scan, so hist + scan is one launch.
+template <class Src, int LEVEL, int NS, bool MERGE>
+__global__ __launch_bounds__(kBlock) void k_level_hist(Src src, int64_t n,
+                                                       const uint32_t* __restrict__ n_dev,
+                                                       SelState* __restrict__ st,
+                                                       uint32_t* __restrict__ hist) {
+  constexpr int NB = LEVEL == 2 ? kBinsSmall : kBinsBig;
+  __shared__ uint32_t s_h[NS][NB];
+  __shared__ uint32_t s_suf[kBlock + 1];
+  __shared__ uint32_t s_last;
+  bool on[NS];
+  uint32_t prefix[NS];
+  bool any = false;
+#pragma unroll
+  for (int q = 0; q < NS; ++q) {
+    on[q] = st[q].skip == 0;
+    prefix[q] = st[q].prefix;
+    any = any || on[q];
+  }
+  if (!any) return;
+  if (n_dev && (int64_t)*n_dev < n) n = (int64_t)*n_dev;
+#pragma unroll
+  for (int q = 0; q < NS; ++q)
+    for (int b = threadIdx.x; b < NB; b += kBlock) s_h[q][b] = 0u;
+  __syncthreads();
+  const int64_t stride = (int64_t)gridDim.x * kBlock * kVec;
+  // uniform trip count so the wave-level ballots inside lds_hist_add are safe
+  const int64_t first = ((int64_t)blockIdx.x * kBlock) * kVec;
+  for (int64_t base = first; base < n; base += stride) {
+    const int64_t i = base + (int64_t)threadIdx.x * kVec;
+    uint32_t key[4] = {0, 0, 0, 0};
+    const bool full = src.vec && base + kBlock * kVec <= n;   // whole workgroup span in range
+    if (full) src.template load<true>(i, n, key);
+    else if (i < n) src.template load<false>(i, n, key);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+#pragma unroll
+      for (int q = 0; q < NS; ++q) {
+        uint32_t bin; bool part;
+        level_bin<LEVEL>(key[e], prefix[q], full || i + e < n, bin, part);
+        lds_hist_add(s_h[q], bin, part && on[q]);
+      }
+    }
+  }
+  __syncthreads();
+#pragma unroll
+  for (int q = 0; q < NS; ++q) {
+    if (!on[q]) continue;
+    uint32_t* gh = level_hist_of<LEVEL>(hist + q * kHistStride);
+    for (int b = threadIdx.x; b < NB; b += kBlock) {
+      const uint32_t c = s_h[q][b];
+      if (c) atomicAdd(&gh[b], c);
+    }
+  }
+  if (!MERGE) return;
+  __threadfence();
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    const uint32_t ticket = atomicAdd(&st[0].done[LEVEL], 1u);
+    s_last = (ticket == gridDim.x - 1) ? 1u : 0u;
+  }
+  __syncthreads();
+  if (!s_last) return;
+  __threadfence();
+#pragma unroll
+  for (int q = 0; q < NS; ++q)
+    if (on[q]) level_scan_body<LEVEL>(&st[q], level_hist_of<LEVEL>(hist + q * kHistStride), s_suf);
+  if (threadIdx.x == 0) st[0].done[LEVEL] = 0u;
+}
+
+// Stand-alone scan (used when one level's histogram is built by several
+// launches, one per view).
+template <int LEVEL>
+__global__ __launch_bounds__(kBlock) void k_level_scan(SelState* __restrict__ st,
+                                                       uint32_t* __restrict__ hist) {
+  __shared__ uint32_t s_suf[kBlock + 1];
+  if (st->skip) return;
+  level_scan_body<LEVEL>(st, level_hist_of<LEVEL>(hist), s_suf);
 }
 
 // Zero the level histograms and reset a state for a new descent.  With
@@ -328,12 +375,6 @@ static __global__ void k_sel_begin(SelState* st, uint32_t* hist, int nhist, uint
     z.k = k;
     *st = z;
   }
-}
-
-// Re-zero the level histograms ahead of the radix passes when they will run.
-static __global__ void k_hist_rezero(const SelState* st, uint32_t* hist, int nhist) {
-  if (st->skip) return;
-  for (int i = threadIdx.x; i < nhist; i += blockDim.x) hist[i] = 0u;
 }
 
 // Per-chunk (1024 elements, one wave) counts of keys above / equal to the
@@ -593,32 +634,35 @@ static __global__ void k_sel_result(const SelState* st, sga_select_result* out) 
 }
 
 // -------------------------------------------------------------- host drivers
-template <class Src>
-static inline void launch_level_hist_on(Src src, int64_t n, const uint32_t* n_dev, int level,
-                                        SelState* st, const SelWorkspace& w, hipStream_t s) {
-  dim3 grid(stream_grid(n, (int64_t)kBlock * kVec * 4, 256 * 8)), block(kBlock);
-  if (level == 0) hipLaunchKernelGGL((k_level_hist<Src, 0>), grid, block, 0, s, src, n, n_dev, st, w.hist);
-  else if (level == 1) hipLaunchKernelGGL((k_level_hist<Src, 1>), grid, block, 0, s, src, n, n_dev, st, w.hist + kBinsBig);
-  else hipLaunchKernelGGL((k_level_hist<Src, 2>), grid, block, 0, s, src, n, n_dev, st, w.hist + 2 * kBinsBig);
+static inline dim3 hist_grid(int64_t n) {
+  return dim3(stream_grid(n, (int64_t)kBlock * kVec * 4, 256 * 8));
 }
+
+// hist (+ merged scan) of one level for NS states starting at `st`.
+template <class Src, int NS, bool MERGE>
+static inline void launch_level(Src src, int64_t n, const uint32_t* n_dev, int level,
+                                SelState* st, const SelWorkspace& w, hipStream_t s,
+                                unsigned max_blocks = 0) {
+  dim3 grid = hist_grid(n), block(kBlock);
+  if (max_blocks && grid.x > max_blocks) grid.x = max_blocks;
+  if (level == 0) hipLaunchKernelGGL((k_level_hist<Src, 0, NS, MERGE>), grid, block, 0, s, src, n, n_dev, st, w.hist);
+  else if (level == 1) hipLaunchKernelGGL((k_level_hist<Src, 1, NS, MERGE>), grid, block, 0, s, src, n, n_dev, st, w.hist);
+  else hipLaunchKernelGGL((k_level_hist<Src, 2, NS, MERGE>), grid, block, 0, s, src, n, n_dev, st, w.hist);
+}
+// piecewise API: histogram only (several views feed one level), then a scan
 template <class Src>
 static inline void launch_level_hist(Src src, int64_t n, int level,
                                      const SelWorkspace& w, hipStream_t s) {
-  launch_level_hist_on(src, n, (const uint32_t*)nullptr, level, w.st, w, s);
-}
-
-static inline void launch_level_scan_on(int level, SelState* st, const SelWorkspace& w, hipStream_t s) {
-  if (level == 0) hipLaunchKernelGGL((k_level_scan<0>), dim3(1), dim3(kBlock), 0, s, st, w.hist);
-  else if (level == 1) hipLaunchKernelGGL((k_level_scan<1>), dim3(1), dim3(kBlock), 0, s, st, w.hist + kBinsBig);
-  else hipLaunchKernelGGL((k_level_scan<2>), dim3(1), dim3(kBlock), 0, s, st, w.hist + 2 * kBinsBig);
+  launch_level<Src, 1, false>(src, n, (const uint32_t*)nullptr, level, w.st, w, s);
 }
 static inline void launch_level_scan(int level, const SelWorkspace& w, hipStream_t s) {
-  launch_level_scan_on(level, w.st, w, s);
+  if (level == 0) hipLaunchKernelGGL((k_level_scan<0>), dim3(1), dim3(kBlock), 0, s, w.st, w.hist);
+  else if (level == 1) hipLaunchKernelGGL((k_level_scan<1>), dim3(1), dim3(kBlock), 0, s, w.st, w.hist);
+  else hipLaunchKernelGGL((k_level_scan<2>), dim3(1), dim3(kBlock), 0, s, w.st, w.hist);
 }
 
 static inline void launch_begin(uint32_t k, const SelWorkspace& w, hipStream_t s) {
-  hipLaunchKernelGGL(k_sel_begin, dim3(1), dim3(kBlock), 0, s, w.st, w.hist,
-                     2 * kBinsBig + kBinsSmall, k);
+  hipLaunchKernelGGL(k_sel_begin, dim3(1), dim3(kBlock), 0, s, w.st, w.hist, kHistStride * 2, k);
 }
 
 template <class Src>
@@ -664,31 +708,22 @@ __global__ __launch_bounds__(kBlock) void k_sample(Src src, int64_t n, int64_t n
   }
 }
 
-// Ranks of the bracket ends inside the sample: r = k*ns/n -/+ (5 sigma + 8).
-static __global__ void k_bracket_ranks(SelState* st, SelState* aux, uint32_t* hist, int nhist,
-                                       int which, uint32_t k, double n, double ns) {
+// Ranks of the two bracket ends inside the sample, r = k*ns/n -/+ (5 sigma + 8):
+// aux[0] descends to the upper end (smaller rank = larger key), aux[1] to the
+// lower end.  Also zeroes both histogram sets.
+static __global__ void k_bracket_ranks(SelState* aux, uint32_t* hist, int nhist, uint32_t k,
+                                       double n, double ns) {
   for (int i = threadIdx.x; i < nhist; i += blockDim.x) hist[i] = 0u;
   if (threadIdx.x != 0) return;
   const double frac = (double)k / n;
   const double r = frac * ns;
   const double d = 5.0 * sqrt(r * (1.0 - frac) + 1.0) + 8.0;
-  SelState z = {};
-  if (which == 0) {            // upper end: a smaller rank = a larger key
-    const double rk = floor(r - d);
-    if (rk < 1.0) { z.skip = 1; st->t_hi = 0x80000000u; }
-    else z.k = (uint32_t)rk;
-  } else {                     // lower end
-    const double rk = ceil(r + d);
-    if (rk > ns) { z.skip = 1; st->t_lo = 0u; }
-    else z.k = (uint32_t)rk;
-  }
-  *aux = z;
-}
-
-static __global__ void k_bracket_set(SelState* st, const SelState* aux, int which) {
-  if (aux->skip) return;
-  if (which == 0) st->t_hi = aux->thresh_bits + 1u;   // keys equal to the sample key stay candidates
-  else st->t_lo = aux->thresh_bits;
+  SelState hi = {}, lo = {};
+  const double rh = floor(r - d), rl = ceil(r + d);
+  if (rh < 1.0) hi.skip = 1; else hi.k = (uint32_t)rh;
+  if (rl > ns) lo.skip = 1; else lo.k = (uint32_t)rl;
+  aux[0] = hi;
+  aux[1] = lo;
 }
 
 // The one sweep over the data.  A persistent grid of kSegWaves waves; each
@@ -740,11 +775,15 @@ __device__ __forceinline__ void bracket_chunk(const Src& src, int64_t n, int64_t
 
 template <class Src>
 __global__ __launch_bounds__(kBlock) void k_bracket_sweep(
-    Src src, int64_t n, SelState* __restrict__ st, uint32_t* __restrict__ tile_gt,
-    uint32_t* __restrict__ tile_eq, uint32_t* __restrict__ seg_idx, uint32_t* __restrict__ seg_key,
-    uint32_t* __restrict__ seg_cnt, uint32_t seg_cap) {
+    Src src, int64_t n, SelState* __restrict__ st, const SelState* __restrict__ aux,
+    uint32_t* __restrict__ tile_gt, uint32_t* __restrict__ tile_eq, uint32_t* __restrict__ seg_idx,
+    uint32_t* __restrict__ seg_key, uint32_t* __restrict__ seg_cnt, uint32_t seg_cap) {
   __shared__ uint32_t s_hi[kChunksPerBlock], s_nf[kChunksPerBlock];
-  const uint32_t T_LO = st->t_lo, T_HI = st->t_hi;
+  // keys equal to the upper sample key stay candidates; a skipped end means
+  // the bracket is open on that side
+  const uint32_t T_HI = aux[0].skip ? 0x80000000u : aux[0].thresh_bits + 1u;
+  const uint32_t T_LO = aux[1].skip ? 0u : aux[1].thresh_bits;
+  if (blockIdx.x == 0 && threadIdx.x == 0) { st->t_lo = T_LO; st->t_hi = T_HI; }
   const int64_t n_chunks = cdiv64(n, kChunk);
   const int64_t gw = (int64_t)blockIdx.x * kChunksPerBlock + wave_id();
   const int64_t W = (int64_t)gridDim.x * kChunksPerBlock;
@@ -805,7 +844,7 @@ static __global__ __launch_bounds__(kBlock) void k_bracket_check(SelState* __res
     SelState z = {};
     z.k = ok ? k - n_hi : 0u;
     z.skip = ok ? 0u : 1u;
-    *aux = z;
+    aux[0] = z;                       // the candidate descent runs on aux[0]
   }
 }
 
@@ -855,7 +894,6 @@ static_assert(kChunk == 1024, "candidate -> chunk mapping uses idx >> 10");
 template <class Src>
 static inline void run_select(Src src, int64_t n, int64_t k, int tie_all, bool fast,
                               const SelWorkspace& w, hipStream_t s) {
-  const int nh = 2 * kBinsBig + kBinsSmall;
   const int64_t n_tiles = cdiv64(n, kChunk);
   launch_begin((uint32_t)k, w, s);
   if (fast && n >= kFastMinN && w.sample && n < (1ll << 32)) {
@@ -866,37 +904,31 @@ static inline void run_select(Src src, int64_t n, int64_t k, int tie_all, bool f
     const int64_t ns = n_sv * 4;
     hipLaunchKernelGGL((k_sample<Src>), dim3(stream_grid(n_sv, kBlock)), dim3(kBlock), 0, s, src, n,
                        n_sv, win, w.sample);
+    hipLaunchKernelGGL(k_bracket_ranks, dim3(1), dim3(kBlock), 0, s, w.aux, w.hist, kHistStride * 2,
+                       (uint32_t)k, (double)n, (double)ns);
     SrcU32 ssrc{w.sample};
-    for (int which = 0; which < 2; ++which) {
-      hipLaunchKernelGGL(k_bracket_ranks, dim3(1), dim3(kBlock), 0, s, w.st, w.aux, w.hist, nh, which,
-                         (uint32_t)k, (double)n, (double)ns);
-      for (int level = 0; level < 3; ++level) {
-        launch_level_hist_on(ssrc, ns, (const uint32_t*)nullptr, level, w.aux, w, s);
-        launch_level_scan_on(level, w.aux, w, s);
-      }
-      hipLaunchKernelGGL(k_bracket_set, dim3(1), dim3(1), 0, s, w.st, w.aux, which);
-    }
+    for (int level = 0; level < 3; ++level)
+      launch_level<SrcU32, 2, true>(ssrc, ns, (const uint32_t*)nullptr, level, w.aux, w, s);
     hipLaunchKernelGGL((k_bracket_sweep<Src>), dim3(kSegWaves / kChunksPerBlock), dim3(kBlock), 0, s,
-                       src, n, w.st, w.tile_gt, w.tile_eq, w.seg_idx, w.seg_key, w.seg_cnt,
+                       src, n, w.st, w.aux, w.tile_gt, w.tile_eq, w.seg_idx, w.seg_key, w.seg_cnt,
                        (uint32_t)w.seg_cap);
-    hipLaunchKernelGGL(k_bracket_check, dim3(1), dim3(kBlock), 0, s, w.st, w.aux, w.seg_cnt, w.hist, nh);
+    hipLaunchKernelGGL(k_bracket_check, dim3(1), dim3(kBlock), 0, s, w.st, w.aux, w.seg_cnt, w.hist,
+                       kHistStride * 2);
     hipLaunchKernelGGL(k_cand_compact, dim3(256), dim3(kBlock), 0, s, w.aux, w.seg_cnt, w.seg_idx,
                        w.seg_key, (uint32_t)w.seg_cap, w.cand_idx, w.cand_key);
     SrcU32 csrc{w.cand_key};
     const int64_t cmax = (int64_t)kSegWaves * w.seg_cap;
-    for (int level = 0; level < 3; ++level) {
-      launch_level_hist_on(csrc, cmax, &w.st->cand_count, level, w.aux, w, s);
-      launch_level_scan_on(level, w.aux, w, s);
-    }
+    for (int level = 0; level < 3; ++level)
+      // the candidate count lives on the device (usually ~1e6): a small grid
+      // strides over it; a large grid would only add idle workgroups
+      launch_level<SrcU32, 1, true>(csrc, cmax, &w.st->cand_count, level, w.aux, w, s, 128);
     hipLaunchKernelGGL(k_cand_tiles, dim3(256), dim3(kBlock), 0, s, w.st, w.aux, w.cand_idx,
                        w.cand_key, w.tile_gt, w.tile_eq);
-    // radix passes: no-ops unless the bracket failed (st->skip == 0)
-    hipLaunchKernelGGL(k_hist_rezero, dim3(1), dim3(kBlock), 0, s, w.st, w.hist, nh);
+    // The radix passes below are no-ops unless the bracket failed
+    // (st->skip == 0); k_bracket_check left the histograms zeroed for them.
   }
-  for (int level = 0; level < 3; ++level) {
-    launch_level_hist(src, n, level, w, s);
-    launch_level_scan(level, w, s);
-  }
+  for (int level = 0; level < 3; ++level)
+    launch_level<Src, 1, true>(src, n, (const uint32_t*)nullptr, level, w.st, w, s);
   launch_tile_count(src, n, 0, w, s);
   launch_tile_scan(n_tiles, tie_all, w, s);
 }
