@@ -239,6 +239,72 @@ int sga_fused_sparse_step(const void* g, int g_dtype, float* resid, float* p,
                           int fast, sga_select_result* result, void* ws,
                           size_t ws_bytes, void* stream);
 
+/* ---- fused offline-replay group step (sga/replay_fused.py:1607-1914) ------ */
+
+/* One configuration's resident state for the current recorded step
+ * (states[c][param] = {ms, vs, ws, res, sel}, replay_fused.py:1548-1567),
+ * flattened over the shard.  sel / out_sel are byte masks (0/1). */
+typedef struct sga_replay_cfg {
+  float* w;
+  float* m;
+  float* v;
+  float* res;
+  const uint8_t* sel;
+  const uint8_t* out_sel; /* outgoing mask for the dual-lr split; NULL = sel */
+  double lr_scale;        /* dual-lr scale, lr_inactive = lr * lr_scale      */
+  int boundary;           /* si % T == 0                                     */
+  int adams;              /* optimizer == "adams"                            */
+  int split;              /* boundary dual-lr split active                   */
+  int pad_;
+} sga_replay_cfg;
+
+/* Per-tensor hyper-parameters of the replay commit (ShardParams entries +
+ * _lr_for_step + _bc_pair: replay_fused.py:251-271, replay.py:132-137).
+ * lr / wd are kept in double so 1-lr*wd, -lr and lr*lr_scale round like the
+ * reference's Python doubles; the rest are fp32 roundings. */
+typedef struct sga_replay_segment {
+  int64_t start, n;
+  double lr, wd;
+  float beta1, om1, beta2, om2, eps, bc1, bc2, wdf;
+} sga_replay_segment;
+
+/* pass 1 (replay_fused.py:1682-1743): qn2[c] = sum q_pre^2 over the shard
+ * (fp32 products, double accumulation, fixed order), coef[c] in double and
+ * fp32.  partials: sga_replay_partials() doubles.  cfgs is a HOST array. */
+int64_t sga_replay_partials(void);
+int sga_replay_pass1(const void* g, int g_dtype, int64_t n, float coef_dense,
+                     double clip, const sga_replay_cfg* cfgs, int G,
+                     double* partials, double* qn2, double* coef_d,
+                     float* coef_f, void* stream);
+
+/* pass 2 (replay_fused.py:1752-1825) for ONE boundary configuration:
+ * score = |formula(w,m,v,(g/coef_dense + res)*coef)|, exact top-k with
+ * lowest-index ties, written as a byte mask into sel_out.  The score is
+ * never materialised.  segs: sga_segment table (beta, eps, wd, bc of the
+ * upcoming commit); coef_f: device pointer to this configuration's coef. */
+int sga_replay_reselect(const void* g, int g_dtype, const float* res,
+                        const float* w, const float* m, const float* v,
+                        int64_t n, int64_t k, const sga_segment* segs,
+                        int n_segs, int score_id, const float* coef_f,
+                        float coef_dense, int adams, uint8_t* sel_out,
+                        sga_select_result* result, void* ws, size_t ws_bytes,
+                        void* stream);
+
+/* pass 3 (replay_fused.py:1836-1889): commit + residual for all G
+ * configurations in one sweep (the gradient is read once).  coef_f: device
+ * float[G] from pass 1.  segs: DEVICE array.  cfgs: HOST array. */
+int sga_replay_pass3(const void* g, int g_dtype, int64_t n, float coef_dense,
+                     const sga_replay_cfg* cfgs, int G, const float* coef_f,
+                     const sga_replay_segment* segs, int n_segs, void* stream);
+
+/* res /= T at fold boundaries (replay_fused.py:1632-1636), true division. */
+int sga_div_inplace(float* x, int64_t n, float d, void* stream);
+
+/* out[0] = sum (a-b)^2 in double (horizon numerators, :1890-1900).
+ * partials: 1024 doubles. */
+int sga_sq_dist(const float* a, const float* b, int64_t n, double* partials,
+                double* out, void* stream);
+
 /* Live timing of the fused step's final sweep with HIP events recorded on the
  * launch stream (no counterpart in the reference; used by the benchmark).
  * enable(1) resets and arms up to 512 launches; read() waits for the recorded

@@ -75,7 +75,8 @@ class Config:
 
 
 def group_replay(entries, w0, m0, v0, sel0, configs, g_steps, metas, t0,
-                 horizons=(), snapshots=None, norm_chunk=None):
+                 horizons=(), snapshots=None, norm_chunk=None, coef_hook=None,
+                 trace=None):
     """Fused-replay group loop on one shard (replay_fused.py:1536-1914).
 
     entries : list of dicts {"a": flat offset, "n": numel, "b1","b2","eps",
@@ -84,6 +85,9 @@ def group_replay(entries, w0, m0, v0, sel0, configs, g_steps, metas, t0,
     sel0    : list (per config) of flat bool masks (branch selection)
     g_steps : list of flat fp32 recorded gradients (post-clip, as logged)
     metas   : per step {"clip_grad", "grad_norm", "lr"}
+    coef_hook(si, ci, coef) -> coef lets a test substitute the clip
+    coefficient (e.g. the device's bits) so everything downstream is compared
+    on identical inputs; trace (a list) receives (si, ci, qn2, coef).
     Returns per-config dict with final w, m, v, res, sel and the per-horizon
     distances ``||w - snapshot||``.
     """
@@ -106,7 +110,7 @@ def group_replay(entries, w0, m0, v0, sel0, configs, g_steps, metas, t0,
             for ci, c in enumerate(configs):
                 if bnd[ci] and c.fold:
                     st[ci]["res"].div_(float(c.T))
-        gd = g_steps[si] / coef_dense                # (:1664)
+        gd = g_steps[si].float() / coef_dense        # (:1664)
         out_sel = {}
         # pass 1: fp32 chunk sums accumulated in a Python double (:1682-1720)
         coefs = []
@@ -122,6 +126,10 @@ def group_replay(entries, w0, m0, v0, sel0, configs, g_steps, metas, t0,
             coef = 1.0
             if clip > 0.0:
                 coef = min(1.0, clip / (math.sqrt(qn2) + 1.0e-6))
+            if trace is not None:
+                trace.append((si, ci, qn2, coef))
+            if coef_hook is not None:
+                coef = coef_hook(si, ci, coef)
             coefs.append(coef)
         # pass 2: boundary reselect (:1752-1825)
         for ci, c in enumerate(configs):

@@ -62,6 +62,13 @@ SIGNATURES = {
     "sga_gt_eq": (I32, [P, I64, F, P, P, P, P]),
     "sga_score_formula": (I32, [I32, P, P, P, P, P, I64] + [F] * 8 + [I32, I32, P]),
     "sga_opt_step_inplace": (I32, [P, P, P, P, P, P, I64] + [F] * 13 + [I32, P]),
+    "sga_replay_partials": (I64, []),
+    "sga_replay_pass1": (I32, [P, I32, I64, F, C.c_double, P, I32, P, P, P, P, P]),
+    "sga_replay_reselect": (I32, [P, I32, P, P, P, P, I64, I64, P, I32, I32, P, F, I32, P, P, P,
+                                  SZ, P]),
+    "sga_replay_pass3": (I32, [P, I32, I64, F, P, I32, P, P, I32, P]),
+    "sga_div_inplace": (I32, [P, I64, F, P]),
+    "sga_sq_dist": (I32, [P, P, I64, P, P, P]),
     "sga_calib_copy": (I32, [P, P, I64, P]),
     "sga_prof_enable": (I32, [I32]),
     "sga_prof_read": (I32, [P, P]),

@@ -1,0 +1,465 @@
+// Fused offline-replay group step: G configurations (score x ratio x cycle
+// length x optimizer x fold x dual-lr) advance over ONE recorded gradient;
+// the gradient is read once per pass and shared by all G state sets.
+//
+//   pass 1  qn2[c]  = sum q_pre^2,  q_pre = gd + res_c (boundary) | gd * sel_c
+//           coef[c] = min(1, clip / (sqrt(qn2[c]) + 1e-6))
+//   pass 2  (boundary re-selection) score = |formula(w,m,v,(gd+res)*coef)|,
+//           exact top-k -> new sel_c                       [select_impl.hpp]
+//   pass 3  boundary: q = (gd+res)*coef, res = 0
+//           else    : q = (gd*sel)*coef, res += gd*(1-sel)
+//           in-place AdamW / AdamS commit (optional dual-lr split)
+//
+// gd = fp32(g) / coef_dense.  Algorithmic HBM bytes per config-step at G
+// configs, bf16 g: non-boundary 34 + 4/G (sel 1 | sel 1 + res 8 + m,v,w 24),
+// boundary 36 + 4/G.
+#include "adam_math.hpp"
+#include "select_impl.hpp"
+
+namespace sga {
+
+constexpr int kMaxCfg = 16;
+
+struct RCfg {
+  float* w;
+  float* m;
+  float* v;
+  float* res;
+  const uint8_t* sel;       // current mask (bytes 0/1)
+  const uint8_t* out_sel;   // outgoing mask for the dual-lr split (may equal sel)
+  double lr_scale;          // dual-lr scale (lr_inactive = lr * lr_scale)
+  int boundary;
+  int adams;
+  int split;
+  int pad_;
+};
+
+struct RGroup {
+  RCfg c[kMaxCfg];
+  int G;
+};
+
+template <bool BF16G, bool FULL>
+__device__ __forceinline__ void load_gd(const void* g, int64_t i, int64_t n, float inv_is_one,
+                                        float coef_dense, float gd[4], bool vec) {
+  if (BF16G) ld_bf16<FULL>(reinterpret_cast<const uint16_t*>(g), i, n, gd, vec);
+  else ld_f32<FULL>(reinterpret_cast<const float*>(g), i, n, gd, vec);
+  if (inv_is_one == 0.0f) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) gd[e] = __fdiv_rn(gd[e], coef_dense);
+  }
+}
+
+// ------------------------------------------------------------------ pass 1
+template <bool BF16G>
+__global__ __launch_bounds__(kBlock) void k_replay_pass1(const void* __restrict__ g, int64_t n,
+                                                         float coef_dense, RGroup grp,
+                                                         double* __restrict__ partials, bool vec) {
+  __shared__ double s_w[kChunksPerBlock][kMaxCfg];
+  double acc[kMaxCfg];
+#pragma unroll
+  for (int c = 0; c < kMaxCfg; ++c) acc[c] = 0.0;
+  const float is_one = coef_dense == 1.0f ? 1.0f : 0.0f;
+  const int64_t stride = (int64_t)gridDim.x * kBlock * kVec;
+  for (int64_t base = (int64_t)blockIdx.x * kBlock * kVec; base < n; base += stride) {
+    const int64_t i = base + (int64_t)threadIdx.x * kVec;
+    const bool full = vec && base + kBlock * kVec <= n;
+    if (!full && i >= n) continue;
+    float gd[4];
+    if (full) load_gd<BF16G, true>(g, i, n, is_one, coef_dense, gd, true);
+    else load_gd<BF16G, false>(g, i, n, is_one, coef_dense, gd, vec);
+#pragma unroll
+    for (int c = 0; c < kMaxCfg; ++c) {
+      if (c >= grp.G) break;
+      float q[4];
+      if (grp.c[c].boundary) {
+        float rr[4];
+        if (full) ld_f32<true>(grp.c[c].res, i, n, rr, true);
+        else load4_f32(grp.c[c].res, i, n, rr, vec);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) q[e] = gd[e] + rr[e];
+      } else {
+        uint32_t sl[4];
+        if (full) ld_u8<true>(grp.c[c].sel, i, n, sl, true);
+        else load4_u8(grp.c[c].sel, i, n, sl, vec);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) q[e] = gd[e] * (sl[e] ? 1.0f : 0.0f);
+      }
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        if (full || i + e < n) acc[c] += (double)(q[e] * q[e]);
+    }
+  }
+#pragma unroll
+  for (int c = 0; c < kMaxCfg; ++c) {
+    if (c >= grp.G) break;
+    const double t = wave_sum(acc[c]);
+    if (lane_id() == 0) s_w[wave_id()][c] = t;
+  }
+  __syncthreads();
+  if (threadIdx.x < grp.G) {
+    const int c = threadIdx.x;
+    partials[(int64_t)blockIdx.x * kMaxCfg + c] = s_w[0][c] + s_w[1][c] + s_w[2][c] + s_w[3][c];
+  }
+}
+
+// One wave per config folds the workgroup partials in a fixed order and
+// forms the clip coefficient in double (the host formula of the reference).
+__global__ __launch_bounds__(kBlock) void k_replay_coef(const double* __restrict__ partials,
+                                                        int n_blocks, int G, double clip,
+                                                        double* __restrict__ qn2,
+                                                        double* __restrict__ coef_d,
+                                                        float* __restrict__ coef_f) {
+  for (int c = wave_id(); c < G; c += kChunksPerBlock) {
+    double a = 0.0;
+    for (int b = lane_id(); b < n_blocks; b += kWave) a += partials[(int64_t)b * kMaxCfg + c];
+    a = wave_sum(a);
+    if (lane_id() == 0) {
+      double coef = 1.0;
+      if (clip > 0.0) {
+        coef = clip / (sqrt(a) + 1.0e-6);
+        if (coef > 1.0) coef = 1.0;
+      }
+      qn2[c] = a;
+      coef_d[c] = coef;
+      coef_f[c] = (float)coef;
+    }
+  }
+}
+
+// ------------------------------------------------------------------ pass 3
+struct RSeg {          // sga_replay_segment, see the header
+  int64_t start, n;
+  double lr, wd;
+  float b1, om1, b2, om2, eps, bc1, bc2, wdf;
+};
+
+struct RSegCursor {
+  const RSeg* segs;
+  int n_segs;
+  int64_t lo, hi;
+  RSeg s;
+  float omlwd, neglr, lrf;
+  __device__ __forceinline__ void init(const RSeg* p, int ns) { segs = p; n_segs = ns; lo = 1; hi = 0; }
+  __device__ __forceinline__ void seek(int64_t i) {
+    if (i >= lo && i < hi) return;
+    int a = 0, b = n_segs - 1;
+    while (a < b) {
+      const int mid = (a + b + 1) >> 1;
+      if (segs[mid].start <= i) a = mid; else b = mid - 1;
+    }
+    s = segs[a];
+    lo = s.start;
+    hi = lo + s.n;
+    omlwd = (float)(1.0 - s.lr * s.wd);
+    neglr = (float)(-s.lr);
+    lrf = (float)s.lr;
+  }
+};
+
+template <bool BF16G, bool FULL>
+__device__ __forceinline__ void pass3_vec(const void* g, int64_t i, int64_t n, float is_one,
+                                          float coef_dense, const RGroup& grp,
+                                          const float* __restrict__ coef_f, RSegCursor& sc,
+                                          bool vec) {
+  float gd[4];
+  load_gd<BF16G, FULL>(g, i, n, is_one, coef_dense, gd, vec);
+#pragma unroll 1
+  for (int c = 0; c < grp.G; ++c) {
+    const RCfg& cf = grp.c[c];
+    const float coef = coef_f[c];
+    float rr[4], mm[4], vv[4] = {0, 0, 0, 0}, ww[4];
+    uint32_t sl[4] = {1, 1, 1, 1}, so[4] = {1, 1, 1, 1};
+    ld_f32<FULL>(cf.res, i, n, rr, vec);
+    ld_f32<FULL>(cf.m, i, n, mm, vec);
+    if (!cf.adams) ld_f32<FULL>(cf.v, i, n, vv, vec);
+    ld_f32<FULL>(cf.w, i, n, ww, vec);
+    if (!cf.boundary) ld_u8<FULL>(cf.sel, i, n, sl, vec);
+    if (cf.split) ld_u8<FULL>(cf.out_sel, i, n, so, vec);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      if (!FULL && i + e >= n) continue;
+      sc.seek(i + e);
+      float q;
+      if (cf.boundary) {
+        q = (gd[e] + rr[e]) * coef;
+        rr[e] = 0.0f;
+      } else {
+        const float on = sl[e] ? 1.0f : 0.0f;
+        q = (gd[e] * on) * coef;
+        rr[e] = rr[e] + gd[e] * (1.0f - on);
+      }
+      const float bc1 = cf.adams ? 1.0f : sc.s.bc1, bc2 = cf.adams ? 1.0f : sc.s.bc2;
+      const float vb = cf.adams ? (mm[e] * mm[e]) * sc.s.b2 : vv[e] * sc.s.b2;
+      const float vn = __fmaf_rn(q * sc.s.om2, q, vb);
+      const float mn = __fmaf_rn(q, sc.s.om1, mm[e] * sc.s.b1);
+      const float mh = __fdiv_rn(mn, bc1);
+      const float vh = __fsqrt_rn(__fdiv_rn(vn, bc2));
+      const float upd = __fdiv_rn(mh, vh + sc.s.eps);
+      if (cf.split) {
+        const float lri = (float)(sc.s.lr * cf.lr_scale);
+        const float step = so[e] ? sc.lrf : lri;          // inactive = NOT in the outgoing mask
+        const float full_u = ww[e] * sc.s.wdf + upd;
+        ww[e] = __fmaf_rn(-full_u, step, ww[e]);
+      } else {
+        ww[e] = __fmaf_rn(upd, sc.neglr, ww[e] * sc.omlwd);
+      }
+      mm[e] = mn;
+      vv[e] = vn;
+    }
+    st_f32<FULL>(cf.res, i, n, rr, vec);
+    st_f32<FULL>(cf.m, i, n, mm, vec);
+    st_f32<FULL>(cf.v, i, n, vv, vec);
+    st_f32<FULL>(cf.w, i, n, ww, vec);
+  }
+}
+
+template <bool BF16G>
+__global__ __launch_bounds__(kBlock) void k_replay_pass3(const void* __restrict__ g, int64_t n,
+                                                         float coef_dense, RGroup grp,
+                                                         const float* __restrict__ coef_f,
+                                                         const RSeg* __restrict__ segs, int n_segs,
+                                                         bool vec) {
+  const float is_one = coef_dense == 1.0f ? 1.0f : 0.0f;
+  RSegCursor sc;
+  sc.init(segs, n_segs);
+  const int64_t stride = (int64_t)gridDim.x * kBlock * kVec;
+  for (int64_t base = (int64_t)blockIdx.x * kBlock * kVec; base < n; base += stride) {
+    const int64_t i = base + (int64_t)threadIdx.x * kVec;
+    if (vec && base + kBlock * kVec <= n)
+      pass3_vec<BF16G, true>(g, i, n, is_one, coef_dense, grp, coef_f, sc, true);
+    else if (i < n)
+      pass3_vec<BF16G, false>(g, i, n, is_one, coef_dense, grp, coef_f, sc, vec);
+  }
+}
+
+// --------------------------------------------------- pass 2 score source
+// key = |registry score| of q = (gd + res) * coef against one config's state.
+template <bool BF16G, int SCORE>
+struct SrcReplay {
+  const void* g;
+  const float* res;
+  const float* w;
+  const float* m;
+  const float* v;
+  const sga_segment* segs;   // b1, b2, eps, wd, bc1, bc2 per tensor
+  int n_segs;
+  const float* coef_f;       // device scalar of this config
+  float coef_dense;
+  int adams;
+  bool vec;
+  template <bool FULL = false>
+  __device__ __forceinline__ void load(int64_t i, int64_t n, uint32_t key[4]) const {
+    float gd[4], rr[4];
+    load_gd<BF16G, FULL>(g, i, n, coef_dense == 1.0f ? 1.0f : 0.0f, coef_dense, gd, vec);
+    ld_f32<FULL>(res, i, n, rr, vec);
+    const float coef = coef_f[0];
+    float q[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) q[e] = (gd[e] + rr[e]) * coef;
+    if (SCORE == SGA_SCORE_ABS_G) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) key[e] = abs_key(q[e]);
+      return;
+    }
+    float ww[4] = {0, 0, 0, 0}, mm[4], vv[4] = {0, 0, 0, 0};
+    ld_f32<FULL>(m, i, n, mm, vec);
+    if (SCORE != SGA_SCORE_ABS_M) {
+      ld_f32<FULL>(w, i, n, ww, vec);
+      if (!adams) ld_f32<FULL>(v, i, n, vv, vec);
+    }
+    SegCursor sc;
+    sc.init(segs, n_segs);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      if (FULL || i + e < n) {
+        sc.seek(i + e);
+        Hyper h = sc.h;
+        float ve = vv[e];
+        if (adams) { ve = mm[e] * mm[e]; h.bc1 = 1.0f; h.bc2 = 1.0f; }
+        key[e] = score_key<SCORE>(q[e], ww[e], mm[e], ve, h);
+      } else {
+        key[e] = 0u;
+      }
+    }
+  }
+};
+
+__global__ __launch_bounds__(kBlock) void k_div_inplace(float* __restrict__ x, int64_t n, float d,
+                                                        bool vec) {
+  const int64_t stride = (int64_t)gridDim.x * kBlock * kVec;
+  for (int64_t i = ((int64_t)blockIdx.x * kBlock + threadIdx.x) * kVec; i < n; i += stride) {
+    float v[4];
+    load4_f32(x, i, n, v, vec);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) v[e] = __fdiv_rn(v[e], d);
+    store4_f32(x, i, n, v, vec);
+  }
+}
+
+// sum (a - b)^2 in double, two-stage
+__global__ __launch_bounds__(kBlock) void k_sqdist_stage1(const float* __restrict__ a,
+                                                          const float* __restrict__ b, int64_t n,
+                                                          double* __restrict__ partials, bool vec) {
+  __shared__ double s_w[kChunksPerBlock];
+  double acc = 0.0;
+  const int64_t stride = (int64_t)gridDim.x * kBlock * kVec;
+  for (int64_t i = ((int64_t)blockIdx.x * kBlock + threadIdx.x) * kVec; i < n; i += stride) {
+    float x[4], y[4];
+    load4_f32(a, i, n, x, vec);
+    load4_f32(b, i, n, y, vec);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const double d = (double)(x[e] - y[e]);
+      acc += d * d;
+    }
+  }
+  acc = wave_sum(acc);
+  if (lane_id() == 0) s_w[wave_id()] = acc;
+  __syncthreads();
+  if (threadIdx.x == 0) partials[blockIdx.x] = s_w[0] + s_w[1] + s_w[2] + s_w[3];
+}
+__global__ __launch_bounds__(kWave) void k_sqdist_stage2(const double* __restrict__ partials, int nb,
+                                                         double* __restrict__ out) {
+  double a = 0.0;
+  for (int b = lane_id(); b < nb; b += kWave) a += partials[b];
+  a = wave_sum(a);
+  if (lane_id() == 0) out[0] = a;
+}
+
+static bool fill_group(RGroup* grp, const sga_replay_cfg* cfgs, int G) {
+  if (G < 1 || G > kMaxCfg || !cfgs) return false;
+  grp->G = G;
+  for (int c = 0; c < G; ++c) {
+    const sga_replay_cfg& s = cfgs[c];
+    if (!s.w || !s.m || !s.v || !s.res || !s.sel) return false;
+    RCfg& d = grp->c[c];
+    d.w = s.w; d.m = s.m; d.v = s.v; d.res = s.res; d.sel = s.sel;
+    d.out_sel = s.out_sel ? s.out_sel : s.sel;
+    d.lr_scale = s.lr_scale; d.boundary = s.boundary; d.adams = s.adams; d.split = s.split;
+    d.pad_ = 0;
+  }
+  for (int c = G; c < kMaxCfg; ++c) grp->c[c] = grp->c[0];
+  return true;
+}
+
+static bool group_aligned(const RGroup& grp) {
+  for (int c = 0; c < grp.G; ++c) {
+    const RCfg& d = grp.c[c];
+    if (!aligned4(d.w, 4) || !aligned4(d.m, 4) || !aligned4(d.v, 4) || !aligned4(d.res, 4) ||
+        !aligned4(d.sel, 1) || !aligned4(d.out_sel, 1))
+      return false;
+  }
+  return true;
+}
+
+constexpr int kReplayBlocks = 2048;
+
+}  // namespace sga
+
+using namespace sga;
+
+static_assert(sizeof(RSeg) == sizeof(sga_replay_segment), "replay segment layout");
+
+extern "C" int64_t sga_replay_partials(void) { return (int64_t)kReplayBlocks * kMaxCfg; }
+
+extern "C" int sga_replay_pass1(const void* g, int g_dtype, int64_t n, float coef_dense, double clip,
+                                const sga_replay_cfg* cfgs, int G, double* partials, double* qn2,
+                                double* coef_d, float* coef_f, void* stream) {
+  RGroup grp;
+  if (!g || n < 1 || !partials || !qn2 || !coef_d || !coef_f || !fill_group(&grp, cfgs, G) ||
+      (g_dtype != SGA_F32 && g_dtype != SGA_BF16)) {
+    set_error("sga_replay_pass1: bad argument (1 <= G <= %d, all state pointers set)", kMaxCfg);
+    return SGA_ERR_ARG;
+  }
+  const bool bg = g_dtype == SGA_BF16;
+  const bool vec = aligned4(g, bg ? 2 : 4) && group_aligned(grp);
+  const unsigned nb = stream_grid(n, (int64_t)kBlock * kVec, kReplayBlocks);
+  hipStream_t s = (hipStream_t)stream;
+  if (bg) hipLaunchKernelGGL((k_replay_pass1<true>), dim3(nb), dim3(kBlock), 0, s, g, n, coef_dense, grp, partials, vec);
+  else hipLaunchKernelGGL((k_replay_pass1<false>), dim3(nb), dim3(kBlock), 0, s, g, n, coef_dense, grp, partials, vec);
+  hipLaunchKernelGGL(k_replay_coef, dim3(1), dim3(kBlock), 0, s, partials, (int)nb, G, clip, qn2, coef_d, coef_f);
+  return check_launch("sga_replay_pass1");
+}
+
+extern "C" int sga_replay_pass3(const void* g, int g_dtype, int64_t n, float coef_dense,
+                                const sga_replay_cfg* cfgs, int G, const float* coef_f,
+                                const sga_replay_segment* segs, int n_segs, void* stream) {
+  RGroup grp;
+  if (!g || n < 1 || !coef_f || !segs || n_segs < 1 || !fill_group(&grp, cfgs, G) ||
+      (g_dtype != SGA_F32 && g_dtype != SGA_BF16)) {
+    set_error("sga_replay_pass3: bad argument");
+    return SGA_ERR_ARG;
+  }
+  const bool bg = g_dtype == SGA_BF16;
+  const bool vec = aligned4(g, bg ? 2 : 4) && group_aligned(grp);
+  const unsigned nb = stream_grid(n, (int64_t)kBlock * kVec, kReplayBlocks * 4);
+  hipStream_t s = (hipStream_t)stream;
+  const RSeg* rs = reinterpret_cast<const RSeg*>(segs);
+  if (bg) hipLaunchKernelGGL((k_replay_pass3<true>), dim3(nb), dim3(kBlock), 0, s, g, n, coef_dense, grp, coef_f, rs, n_segs, vec);
+  else hipLaunchKernelGGL((k_replay_pass3<false>), dim3(nb), dim3(kBlock), 0, s, g, n, coef_dense, grp, coef_f, rs, n_segs, vec);
+  return check_launch("sga_replay_pass3");
+}
+
+template <bool BF16G, int SCORE>
+static int run_reselect(const void* g, const float* res, const float* w, const float* m,
+                        const float* v, int64_t n, int64_t k, const sga_segment* segs, int n_segs,
+                        const float* coef_f, float coef_dense, int adams, uint8_t* sel_out,
+                        sga_select_result* result, const SelWorkspace& ws, hipStream_t s) {
+  const bool vec = aligned4(g, BF16G ? 2 : 4) && aligned4(res, 4) && aligned4(w, 4) &&
+                   aligned4(m, 4) && aligned4(v, 4);
+  SrcReplay<BF16G, SCORE> src{g, res, w, m, v, segs, n_segs, coef_f, coef_dense, adams, vec};
+  run_select(src, n, k, 0, true, ws, s);
+  const int64_t nc = cdiv64(n, kChunk);
+  hipLaunchKernelGGL((k_write_mask<SrcReplay<BF16G, SCORE>>), dim3(stream_grid(nc, kChunksPerBlock, 1 << 20)),
+                     dim3(kBlock), 0, s, src, n, (int64_t)0, 0, ws.st, ws.tile_gt, ws.tile_eq, sel_out,
+                     aligned4(sel_out, 1));
+  if (result) hipLaunchKernelGGL(k_sel_result, dim3(1), dim3(1), 0, s, ws.st, result);
+  return check_launch("sga_replay_reselect");
+}
+
+extern "C" int sga_replay_reselect(const void* g, int g_dtype, const float* res, const float* w,
+                                   const float* m, const float* v, int64_t n, int64_t k,
+                                   const sga_segment* segs, int n_segs, int score_id,
+                                   const float* coef_f, float coef_dense, int adams,
+                                   uint8_t* sel_out, sga_select_result* result, void* ws,
+                                   size_t ws_bytes, void* stream) {
+  if (!g || !res || !w || !m || !v || !segs || !coef_f || !sel_out || n < 1 || n >= (1ll << 31) ||
+      k < 1 || k > n || n_segs < 1 || score_id < 0 || score_id > 3 ||
+      (g_dtype != SGA_F32 && g_dtype != SGA_BF16)) {
+    set_error("sga_replay_reselect: bad argument (n=%lld k=%lld)", (long long)n, (long long)k);
+    return SGA_ERR_ARG;
+  }
+  SelWorkspace sw;
+  if (!sel_ws_carve(ws, ws_bytes, cdiv64(n, kChunk), &sw)) {
+    set_error("sga_replay_reselect: workspace too small (sga_select_workspace_bytes(n))");
+    return SGA_ERR_WORKSPACE;
+  }
+  hipStream_t s = (hipStream_t)stream;
+#define SGA_RS(BG, SC) return run_reselect<BG, SC>(g, res, w, m, v, n, k, segs, n_segs, coef_f, coef_dense, adams, sel_out, result, sw, s)
+  if (g_dtype == SGA_BF16) {
+    switch (score_id) { case 0: SGA_RS(true, 0); case 1: SGA_RS(true, 1); case 2: SGA_RS(true, 2); default: SGA_RS(true, 3); }
+  } else {
+    switch (score_id) { case 0: SGA_RS(false, 0); case 1: SGA_RS(false, 1); case 2: SGA_RS(false, 2); default: SGA_RS(false, 3); }
+  }
+#undef SGA_RS
+}
+
+extern "C" int sga_div_inplace(float* x, int64_t n, float d, void* stream) {
+  if (n == 0) return SGA_OK;
+  if (!x || n < 0) { set_error("sga_div_inplace: bad argument"); return SGA_ERR_ARG; }
+  hipLaunchKernelGGL(k_div_inplace, dim3(stream_grid(n, (int64_t)kBlock * kVec)), dim3(kBlock), 0,
+                     (hipStream_t)stream, x, n, d, aligned4(x, 4));
+  return check_launch("sga_div_inplace");
+}
+
+extern "C" int sga_sq_dist(const float* a, const float* b, int64_t n, double* partials, double* out,
+                           void* stream) {
+  if (!a || !b || !partials || !out || n < 1) { set_error("sga_sq_dist: bad argument"); return SGA_ERR_ARG; }
+  const unsigned nb = stream_grid(n, (int64_t)kBlock * kVec, 1024);
+  hipStream_t s = (hipStream_t)stream;
+  hipLaunchKernelGGL(k_sqdist_stage1, dim3(nb), dim3(kBlock), 0, s, a, b, n, partials,
+                     aligned4(a, 4) && aligned4(b, 4));
+  hipLaunchKernelGGL(k_sqdist_stage2, dim3(1), dim3(kWave), 0, s, partials, (int)nb, out);
+  return check_launch("sga_sq_dist");
+}

@@ -1,0 +1,188 @@
+"""Fused offline-replay group step on MI355X: the per-recorded-step loop of
+``sga/replay_fused.py:1607-1914`` at world == 1.  G configurations
+(score x ratio x cycle length x optimizer x fold x dual-lr) share one read of
+the recorded gradient per pass; state stays resident on the device."""
+import ctypes as C
+import math
+
+import torch
+
+from . import _lib as L
+from .scores import SCORE_MAP
+from .selection import read_result
+
+MAX_CONFIGS = 16
+
+
+class ReplayCfg(C.Structure):
+    """struct sga_replay_cfg"""
+    _fields_ = [("w", C.c_void_p), ("m", C.c_void_p), ("v", C.c_void_p), ("res", C.c_void_p),
+                ("sel", C.c_void_p), ("out_sel", C.c_void_p), ("lr_scale", C.c_double),
+                ("boundary", C.c_int), ("adams", C.c_int), ("split", C.c_int), ("pad_", C.c_int)]
+
+
+class ReplaySegment(C.Structure):
+    """struct sga_replay_segment"""
+    _fields_ = [("start", C.c_int64), ("n", C.c_int64), ("lr", C.c_double), ("wd", C.c_double),
+                ("beta1", C.c_float), ("om1", C.c_float), ("beta2", C.c_float),
+                ("om2", C.c_float), ("eps", C.c_float), ("bc1", C.c_float), ("bc2", C.c_float),
+                ("wdf", C.c_float)]
+
+
+class Config:
+    """One replay arm (``replay_fused.py:1501-1505``)."""
+
+    def __init__(self, score, ratio, T, optimizer="adamw", fold=False, dual_lr=1.0):
+        if score not in SCORE_MAP:
+            raise ValueError(f"Unknown SGA score '{score}'. Registered: {sorted(SCORE_MAP)}")
+        if optimizer not in ("adamw", "adams"):
+            raise ValueError(f"unknown optimizer {optimizer!r}")
+        self.score, self.ratio, self.T = score, float(ratio), int(T)
+        self.optimizer, self.fold, self.dual_lr = optimizer, bool(fold), float(dual_lr)
+
+
+def coef_dense_for(clip_grad, grad_norm):
+    """``sga/replay.py:628-645``"""
+    if clip_grad <= 0.0 or not math.isfinite(grad_norm) or grad_norm <= 0.0:
+        return 1.0
+    return min(clip_grad / (grad_norm + 1.0e-6), 1.0)
+
+
+def _upload(struct_array, dev_buf):
+    host = torch.frombuffer(bytearray(bytes(struct_array)), dtype=torch.uint8)
+    dev_buf.copy_(host)
+
+
+class ReplayGroup:
+    """Resident state of one config group over a flat shard of N elements.
+
+    entries : list of dicts {"a", "n", "b1", "b2", "eps", "wd"} tiling [0, N)
+              (ShardParams entries, ``replay_fused.py:251-271``)
+    w0/m0/v0: flat fp32 device tensors, the branch-point state (copied per config)
+    sel0    : per-config flat bool/uint8 device masks (branch selection)
+    """
+
+    def __init__(self, entries, w0, m0, v0, sel0, configs, t0, window):
+        if not (1 <= len(configs) <= MAX_CONFIGS):
+            raise ValueError(f"1..{MAX_CONFIGS} configs per group")
+        L.require_dev(w0, m0, v0, *sel0)
+        self.N = w0.numel()
+        off = 0
+        for e in entries:
+            if e["a"] != off:
+                raise ValueError("entries must tile [0, N) in order")
+            off += e["n"]
+        if off != self.N:
+            raise ValueError("entries do not cover the shard")
+        self.entries, self.configs, self.t0, self.W = entries, configs, t0, window
+        dev = w0.device
+        self.dev = dev
+        self.state = []
+        for ci, _ in enumerate(configs):
+            self.state.append({
+                "w": w0.clone(), "m": m0.clone(), "v": v0.clone(),
+                "res": torch.zeros(self.N, dtype=torch.float32, device=dev),
+                "sel": sel0[ci].reshape(-1).to(torch.uint8).clone(),
+                "spare": torch.empty(self.N, dtype=torch.uint8, device=dev)})
+        G = len(configs)
+        self.ks = {c.ratio: max(1, int(round(c.ratio / 100.0 * self.N))) for c in configs}
+        self.partials = torch.empty(int(L.raw("sga_replay_partials")), dtype=torch.float64,
+                                    device=dev)
+        self.qn2 = torch.zeros(G, dtype=torch.float64, device=dev)
+        self.coef_d = torch.ones(G, dtype=torch.float64, device=dev)
+        self.coef_f = torch.ones(G, dtype=torch.float32, device=dev)
+        self.ws_bytes = int(L.raw("sga_select_workspace_bytes", self.N))
+        self.ws = torch.empty(self.ws_bytes, dtype=torch.uint8, device=dev)
+        self.sel_result = torch.zeros(8, dtype=torch.int32, device=dev)
+        self._cfg_host = (ReplayCfg * G)()
+        self._rseg_host = (ReplaySegment * len(entries))()
+        self._rseg_dev = torch.empty(C.sizeof(self._rseg_host), dtype=torch.uint8, device=dev)
+        self._seg_host = (L.Segment * len(entries))()
+        self._seg_dev = {o: torch.empty(C.sizeof(self._seg_host), dtype=torch.uint8, device=dev)
+                         for o in ("adamw", "adams")}
+        self.dist_at = [dict() for _ in configs]
+        self.si = 0
+
+    # -- per-step tables ----------------------------------------------------
+    def _fill_segments(self, count, lr_of):
+        for i, e in enumerate(self.entries):
+            r = self._rseg_host[i]
+            r.start, r.n = e["a"], e["n"]
+            r.lr, r.wd = float(lr_of(e)), float(e["wd"])
+            r.beta1, r.om1 = L.f32(e["b1"]), L.f32(1.0 - e["b1"])
+            r.beta2, r.om2 = L.f32(e["b2"]), L.f32(1.0 - e["b2"])
+            r.eps, r.wdf = L.f32(e["eps"]), L.f32(e["wd"])
+            r.bc1 = L.f32(1.0 - e["b1"] ** count)
+            r.bc2 = L.f32(1.0 - e["b2"] ** count)
+            s = self._seg_host[i]
+            s.start, s.n, s.lr = e["a"], e["n"], L.f32(lr_of(e))
+            s.beta1, s.om1, s.beta2, s.om2 = r.beta1, r.om1, r.beta2, r.om2
+            s.eps, s.wd, s.bc1, s.bc2 = r.eps, r.wdf, r.bc1, r.bc2
+        _upload(self._rseg_host, self._rseg_dev)
+        _upload(self._seg_host, self._seg_dev["adamw"])
+
+    def _fill_cfgs(self, bnd, out_sel):
+        for ci, c in enumerate(self.configs):
+            s, h = self.state[ci], self._cfg_host[ci]
+            h.w, h.m, h.v, h.res = (s[k].data_ptr() for k in ("w", "m", "v", "res"))
+            h.sel = s["sel"].data_ptr()
+            split = bool(bnd[ci] and c.dual_lr != 1.0)
+            h.out_sel = (out_sel.get(ci, s["sel"])).data_ptr() if split else None
+            h.lr_scale = c.dual_lr
+            h.boundary, h.adams, h.split = int(bnd[ci]), int(c.optimizer == "adams"), int(split)
+
+    # -- one recorded step ----------------------------------------------------
+    def step(self, g, meta, snapshots=None, horizons=()):
+        """Advance every config over the recorded (post-clip) gradient ``g``
+        (flat bf16/fp32 device tensor).  ``meta``: {"clip_grad", "grad_norm",
+        "lr"} (``lr`` a float, or a callable entry -> float)."""
+        si, N, G = self.si, self.N, len(self.configs)
+        L.require_dev(g)
+        L.require_contig(g=g)
+        assert g.numel() == N
+        clip = float(meta.get("clip_grad", 0.0))
+        coef_dense = coef_dense_for(clip, float(meta.get("grad_norm", float("nan"))))
+        lr = meta["lr"]
+        lr_of = lr if callable(lr) else (lambda e: lr)
+        count = self.t0 + si + 1
+        bnd = [si % c.T == 0 for c in self.configs]
+        st = L.stream()
+        if si > 0:                                   # residual fold
+            for ci, c in enumerate(self.configs):
+                if bnd[ci] and c.fold:
+                    L.call("sga_div_inplace", L.ptr(self.state[ci]["res"]), N,
+                           L.f32(float(c.T)), st)
+        self._fill_segments(count, lr_of)
+        self._fill_cfgs(bnd, {})
+        gd = L.dtype_code(g)
+        L.call("sga_replay_pass1", L.ptr(g), gd, N, L.f32(coef_dense), clip, self._cfg_host, G,
+               L.ptr(self.partials), L.ptr(self.qn2), L.ptr(self.coef_d), L.ptr(self.coef_f), st)
+        out_sel = {}
+        for ci, c in enumerate(self.configs):        # boundary re-selection
+            if not (bnd[ci] and si > 0 and si + 1 < self.W):
+                continue
+            s = self.state[ci]
+            L.call("sga_replay_reselect", L.ptr(g), gd, L.ptr(s["res"]), L.ptr(s["w"]),
+                   L.ptr(s["m"]), L.ptr(s["v"]), N, self.ks[c.ratio],
+                   L.ptr(self._seg_dev["adamw"]), len(self.entries), SCORE_MAP[c.score],
+                   C.c_void_p(self.coef_f.data_ptr() + 4 * ci), L.f32(coef_dense),
+                   int(c.optimizer == "adams"), L.ptr(s["spare"]), L.ptr(self.sel_result),
+                   L.ptr(self.ws), self.ws_bytes, st)
+            if c.dual_lr != 1.0:
+                out_sel[ci] = s["sel"]
+            s["sel"], s["spare"] = s["spare"], s["sel"]
+        self._fill_cfgs(bnd, out_sel)
+        L.call("sga_replay_pass3", L.ptr(g), gd, N, L.f32(coef_dense), self._cfg_host, G,
+               L.ptr(self.coef_f), L.ptr(self._rseg_dev), len(self.entries), st)
+        hz = si + 1
+        if hz in horizons and snapshots is not None:
+            out = torch.zeros(1, dtype=torch.float64, device=self.dev)
+            part = torch.empty(1024, dtype=torch.float64, device=self.dev)
+            for ci in range(G):
+                L.call("sga_sq_dist", L.ptr(self.state[ci]["w"]), L.ptr(snapshots[hz]), N,
+                       L.ptr(part), L.ptr(out), st)
+                self.dist_at[ci][hz] = math.sqrt(float(out.item()))
+        self.si += 1
+
+    def last_select(self):
+        return read_result(self.sel_result)

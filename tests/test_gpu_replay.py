@@ -1,0 +1,196 @@
+"""GPU parity of the replay kernels: score formulas, in-place AdamW/AdamS
+commit (dual-lr, label accumulation) and the fused group step vs the CPU
+oracle.  Masks and thresholds bit-exact; m/v bit-exact (same FMA recipe);
+w within 1e-6 relative of the commit's operands; clip norms within the
+reference's 1e-6 reordering band."""
+import pytest
+import torch
+
+from oracle import replay as OR
+from oracle import scores as OS
+from oracle import select as SEL
+from tests.util import adv, rel_close, student_t
+
+pytestmark = pytest.mark.gpu
+
+
+def _state(n, seed):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(n, generator=g) * 0.02, torch.randn(n, generator=g) * 1e-3,
+            torch.rand(n, generator=g) * 1e-6 + 1e-12, torch.randn(n, generator=g) * 1e-3)
+
+
+@pytest.mark.parametrize("opt", ["adamw", "adams"])
+@pytest.mark.parametrize("name", ["update", "abs_g", "abs_m", "coi"])
+def test_score_formulas(dev, name, opt):
+    from sga_amd import replay_kernels as K
+    from sga_amd.replay import score_formula
+    from sga_amd.scores import get_score_spec
+    b1, b2, eps, wd, step = 0.9, 0.95, 1e-8, 1e-2, 7
+    bc1, bc2 = 1 - b1 ** step, 1 - b2 ** step
+    w, m, v, g = _state(100_003, 3)
+    ref = OS.score_formula(name, w, m, v, g, b1, b2, eps, wd, bc1, bc2, opt,
+                           update_includes_wd=True)
+    got = score_formula(name, *(t.to(dev) for t in (w, m, v, g)), b1, b2, eps, wd, bc1, bc2,
+                        opt, update_includes_wd=True).cpu()
+    if name in ("abs_g", "abs_m"):
+        assert torch.equal(got, ref)
+    else:
+        atol = 2e-6 * float(ref.abs().max()) if name == "coi" else 0.0
+        bad, worst = rel_close(got, ref, 2e-6, atol)
+        assert bad == 0, worst
+    if opt == "adamw":
+        spec = get_score_spec(name).formula(*(t.to(dev) for t in (w, m, v, g)), b1, b2, eps, wd,
+                                            bc1, bc2)
+        assert torch.equal(spec.cpu(), got)
+        assert torch.equal(K.formula(name)(*(t.to(dev) for t in (w, m, v, g)), b1, b2, eps, wd,
+                                           bc1, bc2).cpu(), got)
+
+
+@pytest.mark.parametrize("opt", ["adamw", "adams"])
+@pytest.mark.parametrize("lr,wd,count", [(1e-3, .01, 7), (3e-4, .01, 1), (1e-3, 0.0, 100)])
+def test_opt_step_inplace(dev, opt, lr, wd, count):
+    from sga_amd import replay_kernels as K
+    from sga_amd.replay import _opt_step_inplace
+    b1, b2, eps = 0.9, 0.999, 1e-8
+    n = 70_001
+    for adversarial in (False, True):
+        if adversarial:
+            q, m, w = (adv(n, s).clamp(-1e15, 1e15) for s in (1, 2, 3))
+            v = adv(n, 4, nonneg=True).clamp(0, 1e30)
+        else:
+            w, m, v, q = _state(n, count)
+        bc1, bc2 = OR.bc_pair(opt, count, b1, b2)
+        inactive = torch.rand(n, generator=torch.Generator().manual_seed(3)) < 0.5
+        for ina, lri, with_lab in ((None, None, True), (inactive, lr * 0.3, False)):
+            rm, rv, rw = m.clone(), v.clone(), w.clone()
+            rlab = torch.zeros(n) if with_lab else None
+            OR.opt_step_inplace(q, rm, rv, rw, rlab, lr, wd, b1, b2, bc1, bc2, eps,
+                                optimizer=opt, inactive=ina, lr_inactive=lri)
+            dm, dv, dw = (t.to(dev) for t in (m, v, w))
+            dlab = torch.zeros(n, device=dev) if with_lab else None
+            _opt_step_inplace(q.to(dev), dm, dv, dw, dlab, lr, wd, b1, b2, bc1, bc2, eps,
+                              optimizer=opt, inactive=None if ina is None else ina.to(dev),
+                              lr_inactive=lri)
+            assert torch.equal(dm.cpu().view(torch.int32), rm.view(torch.int32))
+            assert torch.equal(dv.cpu().view(torch.int32), rv.view(torch.int32))
+            ok = torch.isfinite(rw)
+            scale = torch.maximum(w.abs(), (rw - w).abs())
+            bad, worst = rel_close(dw.cpu()[ok], rw[ok], 1e-6, 1e-38, scale=scale[ok])
+            assert bad == 0, (adversarial, worst)
+            if with_lab and not adversarial:
+                bad, worst = rel_close(dlab.cpu(), rlab, 4e-6)
+                assert bad == 0, worst
+    with pytest.raises(ValueError, match="come as a pair"):
+        K.opt_step_inplace(q.to(dev), dm, dv, dw, None, lr, wd, b1, b2, bc1, bc2, eps,
+                           inactive=inactive.to(dev))
+
+
+def _fixture(n_sizes, W, seed=2026, bf16=False):
+    n = sum(n_sizes)
+    gen = torch.Generator().manual_seed(seed)
+    w0 = torch.randn(n, generator=gen) * 0.02
+    m0 = torch.randn(n, generator=gen) * 1e-3
+    v0 = torch.rand(n, generator=gen) * 1e-6
+    grads = []
+    for s in range(W):
+        g = student_t(n, seed + s, scale=1e-2 * (1 + 0.05 * s))
+        if s in (2, 3):
+            g[n_sizes[0]:n_sizes[0] + n_sizes[1]] = 0.0      # a param absent from the payload
+        grads.append(g.to(torch.bfloat16) if bf16 else g)
+    entries, off = [], 0
+    for i, s in enumerate(n_sizes):
+        entries.append({"a": off, "n": s, "b1": 0.9, "b2": 0.95, "eps": 1e-8,
+                        "wd": 0.1 if i % 2 == 0 else 0.0})
+        off += s
+    return n, w0, m0, v0, grads, entries
+
+
+def _run_group(dev, cfg_specs, clip, W=9, bf16=False, t0=10, sizes=(400_000, 300_000, 170_000)):
+    from sga_amd.replay_group import Config, ReplayGroup
+    n, w0, m0, v0, grads, entries = _fixture(list(sizes), W, bf16=bf16)
+    lr = 5e-5
+    norms = [float(g.float().norm()) * 1.3 for g in grads]
+    metas = [{"clip_grad": clip, "grad_norm": norms[i], "lr": lr} for i in range(W)]
+    ocfg = [OR.Config(*c) for c in cfg_specs]
+    dcfg = [Config(*c) for c in cfg_specs]
+    sel0 = []
+    for c in ocfg:
+        sc = OS.score_formula(c.score, w0, m0, v0, grads[0].float(), 0.9, 0.95, 1e-8, 0.1,
+                              *OR.bc_pair(c.optimizer, t0 + 1, 0.9, 0.95), c.optimizer,
+                              update_includes_wd=True).abs()
+        sel0.append(SEL.select_topk_flat(sc, SEL.replay_k(n, c.ratio))[0])
+    grp = ReplayGroup(entries, w0.to(dev), m0.to(dev), v0.to(dev), [s.to(dev) for s in sel0],
+                      dcfg, t0, W)
+    dev_coefs, dev_qn2 = {}, {}
+    for si in range(W):
+        grp.step(grads[si].to(dev), metas[si])
+        cf, q2 = grp.coef_d.cpu().tolist(), grp.qn2.cpu().tolist()
+        for ci in range(len(dcfg)):
+            dev_coefs[(si, ci)], dev_qn2[(si, ci)] = cf[ci], q2[ci]
+    trace = []
+    out = OR.group_replay(entries, w0, m0, v0, sel0, ocfg, grads, metas, t0,
+                          coef_hook=lambda si, ci, c: dev_coefs[(si, ci)], trace=trace)
+    for si, ci, qn2, coef in trace:             # clip norms: 1e-6 reordering band
+        assert abs(dev_qn2[(si, ci)] - qn2) <= 1e-6 * max(qn2, 1e-30), (si, ci)
+        assert abs(dev_coefs[(si, ci)] - coef) <= 1e-6 * coef, (si, ci)
+    return grp, out, w0
+
+
+def test_group_step_no_clip_bitwise(dev):
+    specs = [("abs_g", 1.0, 1), ("abs_g", 10.0, 4), ("abs_m", 1.0, 4), ("abs_g", 0.1, 3, "adams"),
+             ("abs_g", 1.0, 4, "adamw", True), ("abs_g", 1.0, 4, "adamw", False, 0.25),
+             ("abs_g", 1.0, 16)]
+    grp, out, w0 = _run_group(dev, specs, clip=0.0, bf16=True)
+    for ci, o in enumerate(out):
+        s = grp.state[ci]
+        assert torch.equal(s["sel"].cpu().bool(), o["sel"]), ci
+        assert torch.equal(s["res"].cpu().view(torch.int32), o["res"].view(torch.int32)), ci
+        assert torch.equal(s["m"].cpu(), o["m"]) and torch.equal(s["v"].cpu(), o["v"]), ci
+        # 1e-6 of |w| or of the total displacement the W commits can apply (W * lr * |upd|, |upd| <= ~3)
+        bad, worst = rel_close(s["w"], o["w"], 1e-6, atol=1e-6 * 9 * 5e-5 * 3)
+        assert bad == 0, (ci, worst)
+    assert float(grp.state[0]["res"].abs().max()) == 0.0       # T = 1: no residual survives
+
+
+def test_group_step_with_clip(dev):
+    specs = [("abs_g", 1.0, 1), ("abs_g", 10.0, 4), ("abs_g", 1.0, 4, "adams", True),
+             ("abs_m", 0.1, 3, "adamw", False, 2.0)]
+    grp, out, w0 = _run_group(dev, specs, clip=0.3, bf16=False)
+    for ci, o in enumerate(out):
+        s = grp.state[ci]
+        assert torch.equal(s["sel"].cpu().bool(), o["sel"]), ci
+        assert torch.equal(s["res"].cpu().view(torch.int32), o["res"].view(torch.int32)), ci
+        assert torch.equal(s["m"].cpu(), o["m"]) and torch.equal(s["v"].cpu(), o["v"]), ci
+        # 1e-6 of |w| or of the total displacement the W commits can apply (W * lr * |upd|, |upd| <= ~3)
+        bad, worst = rel_close(s["w"], o["w"], 1e-6, atol=1e-6 * 9 * 5e-5 * 3)
+        assert bad == 0, (ci, worst)
+
+
+@pytest.mark.parametrize("score", ["update", "coi"])
+def test_reselect_on_identical_score_bits(dev, score):
+    """Adam-normalised scores: the boundary re-selection is compared with the
+    oracle selector fed the device's own score bits."""
+    from sga_amd.replay_group import Config, ReplayGroup
+    from sga_amd.scores import SCORE_MAP, device_formula
+    n, w0, m0, v0, grads, entries = _fixture([300_000, 1024, 200_000], 3)
+    t0, lr = 5, 1e-4
+    cfg = Config(score, 1.0, 1)
+    k = SEL.replay_k(n, 1.0)
+    sel0 = torch.zeros(n, dtype=torch.bool)
+    grp = ReplayGroup(entries, w0.to(dev), m0.to(dev), v0.to(dev), [sel0.to(dev)], [cfg], t0, 3)
+    grp.step(grads[0].to(dev), {"clip_grad": 0.0, "lr": lr})
+    s = grp.state[0]
+    w1, m1, v1 = (s[x].clone() for x in ("w", "m", "v"))
+    grp.step(grads[1].to(dev), {"clip_grad": 0.0, "lr": lr})     # si = 1: reselects
+    count = t0 + 2
+    sc = torch.empty(n)
+    q = grads[1].to(dev)                                           # res == 0 at T = 1, coef == 1
+    for e in entries:
+        a, b = e["a"], e["a"] + e["n"]
+        sc[a:b] = device_formula(SCORE_MAP[score], w1[a:b], m1[a:b], v1[a:b], q[a:b], e["b1"],
+                                 e["b2"], e["eps"], e["wd"], 1 - e["b1"] ** count,
+                                 1 - e["b2"] ** count, absolute=True).cpu()
+    ref, th = SEL.select_topk_flat(sc, k)
+    assert torch.equal(s["sel"].cpu().bool(), ref)
+    assert grp.last_select().thresh == th
