@@ -71,6 +71,69 @@ def cpu_baseline(sample_n, steps, ratio):
                       f"{dt:.1f} s; host cpu_count={os.cpu_count()}"}
 
 
+def replay_bench(G=8, W=32, seed=4):
+    """Fused offline replay on the Qwen3-0.6B shapes: a window of W recorded
+    bf16 gradient steps resident in HBM, G configs drawn with a fixed seed from
+    score x ratio x cycle length; per-config fp32 w/m/v/residual + byte mask."""
+    import random
+    import torch
+    from sga_amd import _lib as L
+    from sga_amd.replay import select_topk_flat
+    from sga_amd.replay_group import Config, ReplayGroup
+    from sga_amd.shapes import qwen3_06b, segments_for
+    dev = torch.device("cuda:0")
+    segs, n = segments_for(qwen3_06b())
+    entries = [{"a": s["start"], "n": s["n"], "b1": s["b1"], "b2": s["b2"], "eps": s["eps"],
+                "wd": s["wd"]} for s in segs]
+    rnd = random.Random(seed)
+    axes = [(sc, r, t) for sc in ("abs_g", "update", "coi") for r in (0.1, 1.0, 10.0)
+            for t in (1, 4, 16)]
+    picks = rnd.sample(axes, G)
+    cfgs = [Config(*p) for p in picks]
+    gen = torch.Generator(device=dev).manual_seed(1)
+    w0 = torch.randn(n, generator=gen, device=dev) * 0.02
+    m0 = torch.randn(n, generator=gen, device=dev) * 1e-4
+    v0 = torch.rand(n, generator=gen, device=dev) * 1e-8
+    # slowly drifting per-tensor scale: one scale vector per step applied on the fly
+    window = []
+    for s in range(W):
+        g = student_t_dev(n, 500 + s, dev, scale=1e-3 * (1.0 + 0.02 * s))
+        window.append(g)
+    sel0 = []
+    base = window[0].float().abs()
+    for c in cfgs:                       # branch selection on |g0| (cheap stand-in for the front block)
+        sel0.append(select_topk_flat(base, max(1, int(round(c.ratio / 100.0 * n))))[0])
+    del base
+    grp = ReplayGroup(entries, w0, m0, v0, sel0, cfgs, t0=100, window=W)
+    del sel0
+    meta = {"clip_grad": 1.0, "grad_norm": float("nan"), "lr": 1e-4}
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for s in range(W):
+        grp.step(window[s], meta)
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    # algorithmic bytes of this calendar (bf16 g read once per pass for the group)
+    alg = 0.0
+    n_resel = 0
+    for s in range(W):
+        alg += 2 * 2.0 * n                                   # g in pass 1 and pass 3
+        for c in cfgs:
+            bnd = s % c.T == 0
+            alg += (4.0 if bnd else 1.0) * n                 # pass 1: res | sel
+            alg += (32.0 if bnd else 33.0) * n               # pass 3: res, m, v, w r/w (+ sel)
+            if bnd and s > 0 and s + 1 < W:
+                per = 6.0 if c.score == "abs_g" else 18.0    # g, res (+ w, m, v)
+                alg += (2 * per + 1.0) * n                   # bracket sweep + mask sweep + mask
+                n_resel += 1
+    return {"metric": "replay config-steps/s", "value": G * W / dt, "unit": "config-steps/s",
+            "ms_per_window": dt * 1e3, "G": G, "W": W, "n": n, "reselects": n_resel,
+            "configs": [list(p) for p in picks],
+            "alg_bytes": alg, "achieved_GBps": alg / dt / 1e9, "frac": alg / dt / HBM_PEAK,
+            "workload": "Qwen3-0.6B shapes (596,049,920 elems, 310 tensors), bf16 Student-t(3) "
+                        "window, per-config fp32 w/m/v/res + u8 mask resident, clip 1.0"}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -83,6 +146,9 @@ def main():
     ap.add_argument("--calib", action="store_true",
                     help="also launch one plain copy of 2^30 fp32 (k_calib_copy) so counter "
                          "runs can be scaled against a kernel of known traffic")
+    ap.add_argument("--no-replay", action="store_true", help="skip the fused replay leg")
+    ap.add_argument("--only-replay", action="store_true",
+                    help="run just the fused replay leg (for profiling) and print its JSON")
     ap.add_argument("--sweep", action="store_true",
                     help="also time ratios 0.1/1/10 % and the update score")
     args = ap.parse_args()
@@ -97,6 +163,10 @@ def main():
     from sga_amd.shapes import llama32_1b, segments_for
 
     L.load()
+    if args.only_replay:
+        torch.cuda.set_device(0)
+        print(json.dumps(replay_bench()))
+        return
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     segs, n = segments_for(llama32_1b())
@@ -192,6 +262,10 @@ def main():
             sw.append({"score": score, "ratio_percent": ratio, "elem_per_s": n / d,
                        "ms_per_step": d * 1e3})
         out["sweep"] = sw
+    if not args.no_replay:
+        del p, m, v, r, grads, fs
+        torch.cuda.empty_cache()
+        out["replay"] = replay_bench()
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(args.cpu_sample, 3, args.ratio)
     else:

@@ -68,7 +68,7 @@ struct SegCursor {
   int n_segs;
   int64_t lo, hi;
   Hyper h;
-  __device__ __forceinline__ void init(const sga_segment* s, int ns) {
+  __host__ __device__ __forceinline__ void init(const sga_segment* s, int ns) {
     segs = s; n_segs = ns; lo = 1; hi = 0;
   }
   __device__ __forceinline__ void seek(int64_t i) {

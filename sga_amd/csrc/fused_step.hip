@@ -25,11 +25,10 @@ struct SrcFused {
   const float* p;
   const float* m;
   const float* v;
-  const sga_segment* segs;
-  int n_segs;
   bool vec;
+  SegCursor sc;        // per-thread cache of the current segment's hyper-parameters
   template <bool FULL = false>
-  __device__ __forceinline__ void load(int64_t i, int64_t n, uint32_t key[4]) const {
+  __device__ __forceinline__ void load(int64_t i, int64_t n, uint32_t key[4]) {
     float gg[4], rr[4];
     load_g<BF16G, FULL>(g, i, n, gg, vec);
     ld_f32<FULL>(r, i, n, rr, vec);
@@ -44,8 +43,6 @@ struct SrcFused {
       ld_f32<FULL>(p, i, n, pp, vec);
       ld_f32<FULL>(v, i, n, vv, vec);
     }
-    SegCursor sc;
-    sc.init(segs, n_segs);
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
       if (FULL || i + e < n) {
@@ -279,7 +276,8 @@ static int run_fused(const void* g, float* resid, float* p, float* m, float* v, 
                      sga_select_result* result, const SelWorkspace& w, hipStream_t s) {
   const bool vec = aligned4(g, BF16G ? 2 : 4) && aligned4(resid, 4) && aligned4(p, 4) &&
                    aligned4(m, 4) && aligned4(v, 4);
-  SrcFused<BF16G, SCORE> src{g, resid, p, m, v, segs, n_segs, vec};
+  SrcFused<BF16G, SCORE> src{g, resid, p, m, v, vec, {}};
+  src.sc.init(segs, n_segs);
   run_select(src, n, k, 0, fast != 0, w, s);
   const int64_t n_tiles = cdiv64(n, kChunk);
   ProfPair* pp = prof_next();

@@ -242,14 +242,13 @@ struct SrcReplay {
   const float* w;
   const float* m;
   const float* v;
-  const sga_segment* segs;   // b1, b2, eps, wd, bc1, bc2 per tensor
-  int n_segs;
   const float* coef_f;       // device scalar of this config
   float coef_dense;
   int adams;
   bool vec;
+  SegCursor sc;              // b1, b2, eps, wd, bc1, bc2 per tensor (cached per thread)
   template <bool FULL = false>
-  __device__ __forceinline__ void load(int64_t i, int64_t n, uint32_t key[4]) const {
+  __device__ __forceinline__ void load(int64_t i, int64_t n, uint32_t key[4]) {
     float gd[4], rr[4];
     load_gd<BF16G, FULL>(g, i, n, coef_dense == 1.0f ? 1.0f : 0.0f, coef_dense, gd, vec);
     ld_f32<FULL>(res, i, n, rr, vec);
@@ -268,8 +267,6 @@ struct SrcReplay {
       ld_f32<FULL>(w, i, n, ww, vec);
       if (!adams) ld_f32<FULL>(v, i, n, vv, vec);
     }
-    SegCursor sc;
-    sc.init(segs, n_segs);
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
       if (FULL || i + e < n) {
@@ -408,7 +405,8 @@ static int run_reselect(const void* g, const float* res, const float* w, const f
                         sga_select_result* result, const SelWorkspace& ws, hipStream_t s) {
   const bool vec = aligned4(g, BF16G ? 2 : 4) && aligned4(res, 4) && aligned4(w, 4) &&
                    aligned4(m, 4) && aligned4(v, 4);
-  SrcReplay<BF16G, SCORE> src{g, res, w, m, v, segs, n_segs, coef_f, coef_dense, adams, vec};
+  SrcReplay<BF16G, SCORE> src{g, res, w, m, v, coef_f, coef_dense, adams, vec, {}};
+  src.sc.init(segs, n_segs);
   run_select(src, n, k, 0, true, ws, s);
   const int64_t nc = cdiv64(n, kChunk);
   hipLaunchKernelGGL((k_write_mask<SrcReplay<BF16G, SCORE>>), dim3(stream_grid(nc, kChunksPerBlock, 1 << 20)),

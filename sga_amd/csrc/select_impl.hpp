@@ -162,7 +162,7 @@ struct SrcF32 {                 // |x| of an fp32 score array
   const float* x;
   bool vec;
   template <bool FULL = false>
-  __device__ __forceinline__ void load(int64_t i, int64_t n, uint32_t key[4]) const {
+  __device__ __forceinline__ void load(int64_t i, int64_t n, uint32_t key[4]) {
     float v[4];
     ld_f32<FULL>(x, i, n, v, vec);
 #pragma unroll
@@ -174,7 +174,7 @@ struct SrcU32 {                 // raw keys (sample / candidate buffers)
   const uint32_t* x;
   static constexpr bool vec = true;
   template <bool FULL = false>
-  __device__ __forceinline__ void load(int64_t i, int64_t n, uint32_t key[4]) const {
+  __device__ __forceinline__ void load(int64_t i, int64_t n, uint32_t key[4]) {
     if (FULL || i + 4 <= n) {
       U4 v = *reinterpret_cast<const U4*>(x + i);
       key[0] = v.x; key[1] = v.y; key[2] = v.z; key[3] = v.w;
@@ -730,25 +730,19 @@ static __global__ void k_bracket_ranks(SelState* aux, uint32_t* hist, int nhist,
 // wave owns a private candidate segment, so no atomics are needed and the
 // candidates of a chunk stay in ascending index order.
 template <class Src, bool FULL>
-__device__ __forceinline__ void bracket_chunk(const Src& src, int64_t n, int64_t c, uint32_t T_LO,
+__device__ __forceinline__ void bracket_chunk(Src& src, int64_t n, int64_t c, uint32_t T_LO,
                                               uint32_t T_HI, uint32_t& chi, uint32_t& tot_nf,
                                               uint32_t& mycnt, uint32_t seg_cap,
                                               uint32_t* __restrict__ my_idx,
                                               uint32_t* __restrict__ my_key) {
-  uint32_t keys[kChunkIters][4];
+  // one 256-element slab at a time: keeps the register footprint of
+  // expensive key sources (Adam-normalised scores) small enough for full
+  // occupancy; slabs of different waves overlap their loads
 #pragma unroll
   for (int it = 0; it < kChunkIters; ++it) {
     const int64_t i = c * kChunk + it * (kWave * kVec) + lane_id() * kVec;
-    if (!FULL) {
-#pragma unroll
-      for (int e = 0; e < 4; ++e) keys[it][e] = 0u;
-    }
-    if (FULL || i < n) src.template load<FULL>(i, n, keys[it]);
-  }
-#pragma unroll
-  for (int it = 0; it < kChunkIters; ++it) {
-    const int64_t i = c * kChunk + it * (kWave * kVec) + lane_id() * kVec;
-    const uint32_t* key = keys[it];
+    uint32_t key[4] = {0u, 0u, 0u, 0u};
+    if (FULL || i < n) src.template load<FULL>(i, n, key);
     bool cand[4];
     uint32_t mine = 0;
 #pragma unroll
