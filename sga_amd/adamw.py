@@ -3,6 +3,7 @@
 ``adamw_grad_correct_compact``, ``build_dir_table`` and ``SgaAdamW`` with the
 reference's signatures, refusals and step order."""
 import math
+from dataclasses import dataclass, field
 from types import SimpleNamespace
 from typing import Optional
 
@@ -145,6 +146,56 @@ def adamw_grad_correct_compact(param_buffer, grad_buffer, exp_avg_buffer,
            L.f32(1.0 - beta1), L.f32(beta2), L.f32(1.0 - beta2), L.f32(eps),
            L.f32(weight_decay), L.f32(bias_correction1), L.f32(bias_correction2),
            L.f32(coeff), L.f32(interval), flags, L.ptr(dir_table), n_table, L.stream())
+
+
+@dataclass
+class ParamRecord:
+    """One (model param, fp32 main param) pair and its hyper-parameters
+    (``sga/plugins/optimizer/__init__.py:20-60``)."""
+    model_param: object
+    main_param: object
+    bucket_state: object
+    start: int
+    end: int
+    lr: float
+    beta1: float
+    beta2: float
+    eps: float
+    weight_decay: float
+    step: int
+    _state: dict = field(default=None, repr=False)
+
+    @property
+    def grad(self):
+        return self.main_param.grad
+
+    @property
+    def m(self):
+        return self._state["exp_avg"]
+
+    @property
+    def v(self):
+        return self._state["exp_avg_sq"]
+
+    def mask_u8(self):
+        bs = self.bucket_state
+        if bs is None or bs.active_mask_u8 is None:
+            return None
+        return bs.active_mask_u8[self.start:self.end]
+
+
+@dataclass
+class OptContext:
+    """What the optimizer sees for one step
+    (``sga/plugins/optimizer/__init__.py:63-87``)."""
+    records: list
+    phase: str
+    support: object = None
+    bucket_states: list = None
+    fold_window: int = 1
+    next_step_is_full: bool = False
+    apply_coeff: float = 1.0
+    compact_values: dict = None
 
 
 class SgaAdamW:

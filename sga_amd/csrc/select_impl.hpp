@@ -902,7 +902,9 @@ static inline void run_select(Src src, int64_t n, int64_t k, int tie_all, bool f
                        (uint32_t)k, (double)n, (double)ns);
     SrcU32 ssrc{w.sample};
     for (int level = 0; level < 3; ++level)
-      launch_level<SrcU32, 2, true>(ssrc, ns, (const uint32_t*)nullptr, level, w.aux, w, s);
+      // <= 1M keys: 64 fat workgroups keep the histogram flush (one atomic per
+      // non-empty bin per workgroup) far below one atomic per key
+      launch_level<SrcU32, 2, true>(ssrc, ns, (const uint32_t*)nullptr, level, w.aux, w, s, 64);
     hipLaunchKernelGGL((k_bracket_sweep<Src>), dim3(kSegWaves / kChunksPerBlock), dim3(kBlock), 0, s,
                        src, n, w.st, w.aux, w.tile_gt, w.tile_eq, w.seg_idx, w.seg_key, w.seg_cnt,
                        (uint32_t)w.seg_cap);
@@ -915,7 +917,7 @@ static inline void run_select(Src src, int64_t n, int64_t k, int tie_all, bool f
     for (int level = 0; level < 3; ++level)
       // the candidate count lives on the device (usually ~1e6): a small grid
       // strides over it; a large grid would only add idle workgroups
-      launch_level<SrcU32, 1, true>(csrc, cmax, &w.st->cand_count, level, w.aux, w, s, 128);
+      launch_level<SrcU32, 1, true>(csrc, cmax, &w.st->cand_count, level, w.aux, w, s, 64);
     hipLaunchKernelGGL(k_cand_tiles, dim3(256), dim3(kBlock), 0, s, w.st, w.aux, w.cand_idx,
                        w.cand_key, w.tile_gt, w.tile_eq);
     // The radix passes below are no-ops unless the bracket failed
