@@ -125,7 +125,9 @@ int sga_mask_fill(const uint8_t* mask, int64_t n, const uint32_t* chunk_offsets,
 
 /* adamw_grad_correct / _grad_correct_kernel, adamw.py:88-213, 502-634.
  * emit_mode -1 = sparse step, 0..3 = full step writing that score into g.
- * flags: SGA_GC_*.  interval is the fold divisor (fp32 division). */
+ * flags: SGA_GC_*.  interval is the fold divisor (fp32 division).
+ * SGA_GC_ADAMS selects the AdamS tail of adams.py:87-213, 392-504 (v rebuilt
+ * from the pre-commit m, no bias corrections: bc1/bc2 are ignored). */
 int sga_adamw_grad_correct(float* p, float* g, float* m, float* v,
                            const uint8_t* mask, int64_t n, float lr,
                            float beta1, float om1, float beta2, float om2,
@@ -135,7 +137,8 @@ int sga_adamw_grad_correct(float* p, float* g, float* m, float* v,
 
 /* adamw_grad_correct_compact, adamw.py:217-322, 637-792: the commit reads its
  * gradient from the bucket-level sorted (idx, values) by merge-join.
- * flags: SGA_GC_APPLY_COEFF | SGA_GC_FOLD.  dir_table may be NULL. */
+ * flags: SGA_GC_APPLY_COEFF | SGA_GC_FOLD | SGA_GC_ADAMS (adams.py:507-654).
+ * dir_table may be NULL. */
 int sga_adamw_grad_correct_compact(float* p, float* g, float* m, float* v,
                                    const int32_t* idx, const void* values,
                                    int values_dtype, int64_t rec_start,

@@ -123,3 +123,43 @@ def build_dir_table(idx, total_n):
     n_table = (total_n >> 10) + 2
     keys = torch.arange(n_table, dtype=torch.int64) * 1024
     return torch.searchsorted(idx.long(), keys).to(torch.int32)
+
+
+def adams_grad_correct(param, grad, m, v, lr, b1, b2, eps, wd, mask=None,
+                       emit_score=None, coeff=1.0, clear=False, fold=False,
+                       interval=1.0, inactive_lr_scale=1.0):
+    """AdamS twin (``sga/plugins/optimizer/adams_torch.py:34-85``): v is
+    rebuilt from the pre-commit m, no bias corrections."""
+    check_knobs(mask, emit_score, coeff, clear, fold, inactive_lr_scale)
+    if param.numel() == 0:
+        return
+    if inactive_lr_scale != 1.0:
+        g = grad
+        lr_apply = torch.where(mask > 0, lr, lr * inactive_lr_scale)
+    elif mask is not None:
+        g = torch.where(mask > 0, grad, torch.zeros_like(grad))
+        lr_apply = lr
+    else:
+        g = grad
+        lr_apply = lr
+    if coeff != 1.0:
+        g = torch.where(mask > 0, g * coeff, g)
+    upd = S.update(param, m, v, g, b1, b2, eps, wd, 1.0, 1.0, optimizer="adams")
+    score = None
+    if emit_score == "update":
+        score = upd
+    elif emit_score is not None:
+        score = S.get_formula(emit_score)(param, m, v, g, b1, b2, eps, wd, 1.0, 1.0,
+                                          optimizer="adams")
+    m_new = b1 * m + (1.0 - b1) * g
+    v_new = b2 * (m * m) + (1.0 - b2) * g * g
+    m.copy_(m_new)
+    v.copy_(v_new)
+    if emit_score is not None:
+        grad.copy_(score)
+    else:
+        if clear and mask is not None:
+            grad.masked_fill_(mask > 0, 0.0)
+        if fold:
+            grad.div_(interval)
+    param.sub_(lr_apply * upd)

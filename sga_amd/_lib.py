@@ -14,7 +14,7 @@ LIB_PATH = os.path.join(_HERE, "libsga_hip.so")
 
 SGA_F32, SGA_BF16 = 0, 1
 TIE_ALL, TIE_LOWEST_INDEX = 0, 1
-GC_HAS_MASK, GC_APPLY_COEFF, GC_CLEAR, GC_FOLD, GC_LR_SPLIT = 1, 2, 4, 8, 16
+GC_HAS_MASK, GC_APPLY_COEFF, GC_CLEAR, GC_FOLD, GC_LR_SPLIT, GC_ADAMS = 1, 2, 4, 8, 16, 32
 RP_HAS_LAB, RP_ADAMS, RP_SPLIT = 1, 2, 4
 
 P, I64, I32, F, SZ = C.c_void_p, C.c_int64, C.c_int, C.c_float, C.c_size_t

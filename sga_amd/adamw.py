@@ -27,7 +27,7 @@ def _flat32(**named):
 def adamw_grad_correct(param_buffer, grad_buffer, exp_avg_buffer, exp_avg_sq_buffer,
                        lr, beta1, beta2, eps, weight_decay, step, mask=None,
                        emit_score: Optional[str] = None, coeff=1.0, clear=False,
-                       fold=False, interval=1.0, inactive_lr_scale=1.0):
+                       fold=False, interval=1.0, inactive_lr_scale=1.0, _adams=False):
     """One fused commit on contiguous same-size 1-D fp32 buffers
     (``adamw.py:502-634``).  ``emit_score=None`` is the sparse step; a score
     name is the full step that also writes that score into ``grad_buffer``."""
@@ -78,6 +78,8 @@ def adamw_grad_correct(param_buffer, grad_buffer, exp_avg_buffer, exp_avg_sq_buf
         flags |= L.GC_FOLD
     if inactive_lr_scale != 1.0:
         flags |= L.GC_LR_SPLIT
+    if _adams:
+        flags |= L.GC_ADAMS
     L.call("sga_adamw_grad_correct", L.ptr(param_buffer), L.ptr(grad_buffer),
            L.ptr(exp_avg_buffer), L.ptr(exp_avg_sq_buffer), L.ptr(mk), n, L.f32(lr),
            L.f32(beta1), L.f32(1.0 - beta1), L.f32(beta2), L.f32(1.0 - beta2),
@@ -107,7 +109,7 @@ def build_dir_table(idx, total_n):
 def adamw_grad_correct_compact(param_buffer, grad_buffer, exp_avg_buffer,
                                exp_avg_sq_buffer, idx, values, rec_start, lr, beta1,
                                beta2, eps, weight_decay, step, coeff=1.0, fold=False,
-                               interval=1.0, dir_table=None):
+                               interval=1.0, dir_table=None, _adams=False):
     """Compact-emission commit: the gradient comes from the bucket-level sorted
     ``(idx, values)`` by merge-join (``adamw.py:637-792``).  ``values`` may be
     fp32 or bf16."""
@@ -139,7 +141,8 @@ def adamw_grad_correct_compact(param_buffer, grad_buffer, exp_avg_buffer,
             f"adamw_grad_correct_compact: dir_table has {dir_table.numel()} entries "
             f"but the record's last block needs >= {((rec_start + n - 1) >> 10) + 2}")
         n_table = dir_table.numel()
-    flags = (L.GC_APPLY_COEFF if coeff != 1.0 else 0) | (L.GC_FOLD if fold else 0)
+    flags = ((L.GC_APPLY_COEFF if coeff != 1.0 else 0) | (L.GC_FOLD if fold else 0)
+             | (L.GC_ADAMS if _adams else 0))
     L.call("sga_adamw_grad_correct_compact", L.ptr(param_buffer), L.ptr(grad_buffer),
            L.ptr(exp_avg_buffer), L.ptr(exp_avg_sq_buffer), L.ptr(idx), L.ptr(values),
            L.dtype_code(values), rec_start, n, k_total, L.f32(lr), L.f32(beta1),
@@ -222,6 +225,10 @@ class SgaAdamW:
     def ensure_state(self, bucket_states):
         pass
 
+    # the two commit entry points (SgaAdamS swaps in the AdamS recursion)
+    _commit = staticmethod(adamw_grad_correct)
+    _commit_compact = staticmethod(adamw_grad_correct_compact)
+
     @staticmethod
     def _state(rec):
         st = rec._state
@@ -235,7 +242,7 @@ class SgaAdamW:
         for rec in ctx.records:
             st = self._state(rec)
             m = rec.mask_u8() if use_mask else None
-            adamw_grad_correct(
+            self._commit(
                 rec.main_param.data.view(-1), rec.grad.data.view(-1),
                 st["exp_avg"].view(-1), st["exp_avg_sq"].view(-1), rec.lr, rec.beta1,
                 rec.beta2, rec.eps, rec.weight_decay, rec.step, mask=m,
@@ -250,14 +257,14 @@ class SgaAdamW:
             bs = rec.bucket_state
             values = ctx.compact_values.get(id(bs))
             if values is None:
-                adamw_grad_correct(
+                self._commit(
                     rec.main_param.data.view(-1), rec.grad.data.view(-1),
                     st["exp_avg"].view(-1), st["exp_avg_sq"].view(-1), rec.lr,
                     rec.beta1, rec.beta2, rec.eps, rec.weight_decay, rec.step)
                 continue
             bucket = ctx.support.buckets[bs.support_index]
             table = bucket.dir_table if self.compact_search == "table" else None
-            adamw_grad_correct_compact(
+            self._commit_compact(
                 rec.main_param.data.view(-1), rec.grad.data.view(-1),
                 st["exp_avg"].view(-1), st["exp_avg_sq"].view(-1), bucket.idx, values,
                 rec.start, rec.lr, rec.beta1, rec.beta2, rec.eps, rec.weight_decay,

@@ -24,6 +24,7 @@ __global__ __launch_bounds__(kBlock) void k_grad_correct(
   const bool clear = flags & SGA_GC_CLEAR;
   const bool fold = flags & SGA_GC_FOLD;
   const bool split = flags & SGA_GC_LR_SPLIT;
+  const bool adams = flags & SGA_GC_ADAMS;   // v basis = pre-commit m*m, h.bc1 = h.bc2 = 1
   const int64_t stride = (int64_t)gridDim.x * kBlock * kVec;
   for (int64_t i = ((int64_t)blockIdx.x * kBlock + threadIdx.x) * kVec; i < n;
        i += stride) {
@@ -32,7 +33,12 @@ __global__ __launch_bounds__(kBlock) void k_grad_correct(
     load4_f32(p, i, n, pp, vec);
     load4_f32(g, i, n, gg, vec);
     load4_f32(m, i, n, mm, vec);
-    load4_f32(v, i, n, vv, vec);
+    if (adams) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) vv[e] = mm[e] * mm[e];
+    } else {
+      load4_f32(v, i, n, vv, vec);
+    }
     if (has_mask) load4_u8(mask, i, n, mk, vec);
     float gout[4];
 #pragma unroll
@@ -106,6 +112,7 @@ __global__ __launch_bounds__(kBlock) void k_grad_correct_compact(
   __shared__ int64_t s_bounds[2];
   const bool apply_coeff = flags & SGA_GC_APPLY_COEFF;
   const bool fold = flags & SGA_GC_FOLD;
+  const bool adams = flags & SGA_GC_ADAMS;
   const int64_t n_spans = cdiv64(n, kBlockSpan);
   for (int64_t span = blockIdx.x; span < n_spans; span += gridDim.x) {
     const int64_t off0 = span * kBlockSpan;
@@ -149,7 +156,12 @@ __global__ __launch_bounds__(kBlock) void k_grad_correct_compact(
         float pp[4], mm[4], vv[4], raw[4] = {0, 0, 0, 0};
         load4_f32(p, i, n, pp, vec);
         load4_f32(m, i, n, mm, vec);
-        load4_f32(v, i, n, vv, vec);
+        if (adams) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) vv[e] = mm[e] * mm[e];
+        } else {
+          load4_f32(v, i, n, vv, vec);
+        }
         if (fold) load4_f32(g, i, n, raw, vec);
         const uint32_t fw = s_found[t0 >> 5] >> (t0 & 31);
 #pragma unroll
@@ -218,10 +230,7 @@ extern "C" int sga_adamw_grad_correct(float* p, float* g, float* m, float* v,
     set_error("sga_adamw_grad_correct: LR_SPLIT needs a full step with a mask");
     return SGA_ERR_ARG;
   }
-  if (flags & SGA_GC_ADAMS) {
-    set_error("sga_adamw_grad_correct: the AdamS recursion is not built");
-    return SGA_ERR_ARG;
-  }
+  if (flags & SGA_GC_ADAMS) { bc1 = 1.0f; bc2 = 1.0f; }
   const Hyper h = mk_hyper(lr, beta1, om1, beta2, om2, eps, wd, bc1, bc2);
   const bool vec = aligned4(p, 4) && aligned4(g, 4) && aligned4(m, 4) &&
                    aligned4(v, 4) && aligned4(mask, 1);
@@ -265,6 +274,7 @@ extern "C" int sga_adamw_grad_correct_compact(
               (long long)n_table, (long long)(((rec_start + n - 1) >> 10) + 2));
     return SGA_ERR_ARG;
   }
+  if (flags & SGA_GC_ADAMS) { bc1 = 1.0f; bc2 = 1.0f; }
   const Hyper h = mk_hyper(lr, beta1, om1, beta2, om2, eps, wd, bc1, bc2);
   const bool vec = aligned4(p, 4) && aligned4(g, 4) && aligned4(m, 4) && aligned4(v, 4);
   dim3 grid(stream_grid(n, kBlockSpan)), block(kBlock);

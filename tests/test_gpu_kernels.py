@@ -236,3 +236,48 @@ def test_dir_table_geometries(dev):
         t = A.build_dir_table(idx.to(dev), n)
         assert t.dtype == torch.int32 and t.numel() == (n >> 10) + 2
         assert torch.equal(t.cpu(), OA.build_dir_table(idx, n))
+
+
+@pytest.mark.parametrize("kw", [dict(), dict(mask=True), dict(mask=True, coeff=0.5, clear=True, fold=True, interval=4.0),
+                                dict(emit_score="update"), dict(emit_score="coi"), dict(emit_score="abs_m"),
+                                dict(mask=True, emit_score="abs_g", inactive_lr_scale=0.5)])
+def test_adams_grad_correct(dev, kw):
+    from sga_amd import adams as AS
+    n = 90_001
+    p, m, v, g = _state(n, 31)
+    kw = dict(kw)
+    mask = None
+    if kw.pop("mask", False):
+        mask = (torch.rand(n, generator=torch.Generator().manual_seed(2)) < 0.3).to(torch.uint8)
+    ref = [t.clone() for t in (p, g, m, v)]
+    OA.adams_grad_correct(*ref, 1e-3, 0.9, 0.95, 1e-8, 0.1, mask=mask, **kw)
+    devt = [t.to(dev) for t in (p, g, m, v)]
+    AS.adams_grad_correct(*devt, 1e-3, 0.9, 0.95, 1e-8, 0.1,
+                          mask=None if mask is None else mask.to(dev), **kw)
+    assert torch.equal(devt[2].cpu(), ref[2]) and torch.equal(devt[3].cpu(), ref[3])
+    if kw.get("emit_score") in (None, "abs_g", "abs_m"):
+        assert torch.equal(devt[1].cpu(), ref[1])
+    else:
+        atol = 2e-6 * float(ref[1].abs().max()) if kw["emit_score"] == "coi" else 0.0
+        assert rel_close(devt[1], ref[1], 2e-6, atol)[0] == 0
+    assert rel_close(devt[0], ref[0], 1e-6, scale=sub_scale(p, ref[0]))[0] == 0
+
+
+def test_adams_compact_equals_masked(dev):
+    from sga_amd import adams as AS
+    from sga_amd.adamw import build_dir_table
+    from sga_amd.kernels import pack_selected
+    from sga_amd.support import compact_mask_u8
+    n = 70_001
+    p, m, v, g = _state(n, 41)
+    mask = (torch.rand(n, generator=torch.Generator().manual_seed(4)) < 0.2).to(torch.uint8)
+    a = [t.to(dev) for t in (p, g, m, v)]
+    AS.adams_grad_correct(*a, 1e-3, 0.9, 0.95, 1e-8, 0.1, mask=mask.to(dev), coeff=0.5, clear=True)
+    b = [t.to(dev) for t in (p, g, m, v)]
+    idx = compact_mask_u8(mask.to(dev))
+    vals = torch.empty(idx.numel(), device=dev)
+    pack_selected(b[1], idx, vals, 1.0)
+    AS.adams_grad_correct_compact(b[0], b[1], b[2], b[3], idx, vals, 0, 1e-3, 0.9, 0.95, 1e-8, 0.1,
+                                  coeff=0.5, dir_table=build_dir_table(idx, n))
+    for x, y in zip(a, b):
+        assert torch.equal(x, y)

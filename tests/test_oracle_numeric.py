@@ -318,3 +318,26 @@ def test_fused_step_end_state_invariant():
                                    1e-4, 0.9, 0.95, 1e-8, 0.1, step)
         torch.testing.assert_close(p[:10000].double(), rp, rtol=1e-5, atol=1e-7)
         torch.testing.assert_close(m[:10000].double(), rm, rtol=1e-5, atol=1e-9)
+
+
+def test_adams_grad_correct_vs_f64():
+    n = 2000
+    lr, b1, b2, eps, wd = 1e-3, 0.9, 0.95, 1e-8, 0.1
+    p, m, v, g = _state(n, 21)
+    mask = (torch.rand(n, generator=torch.Generator().manual_seed(1)) < 0.3).to(torch.uint8)
+    pp, gg, mm, vv = p.clone(), g.clone(), m.clone(), v.clone()
+    A.adams_grad_correct(pp, gg, mm, vv, lr, b1, b2, eps, wd, mask=mask, clear=True)
+    ge = torch.where(mask > 0, g, torch.zeros(())).double()
+    m2 = b1 * m.double() + (1 - b1) * ge
+    v2 = b2 * m.double() ** 2 + (1 - b2) * ge * ge
+    p2 = p.double() - lr * (wd * p.double() + m2 / (v2.sqrt() + eps))
+    torch.testing.assert_close(mm.double(), m2, rtol=1e-5, atol=1e-7)
+    torch.testing.assert_close(vv.double(), v2, rtol=1e-4, atol=1e-7)
+    torch.testing.assert_close(pp.double(), p2, rtol=1e-5, atol=1e-7)
+    assert bool((gg[mask > 0] == 0).all()) and torch.equal(gg[mask == 0], g[mask == 0])
+    for name in S.FORMULAS:
+        p3, g3 = p.clone(), g.clone()
+        A.adams_grad_correct(p3, g3, m.clone(), v.clone(), lr, b1, b2, eps, wd, emit_score=name)
+        ref = _f64_scores(p, m, v, g, b1, b2, eps, wd, 1.0, 1.0, adams=True)
+        torch.testing.assert_close(g3.double(), ref[name], rtol=1e-5,
+                                   atol=2e-6 if name == "coi" else 1e-7)
