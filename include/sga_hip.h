@@ -109,6 +109,21 @@ int sga_scatter_selected_blocks(float* dst, const uint8_t* mask,
                                 const int32_t* block_idx, const float* src,
                                 int64_t kb, int x, int64_t n_dst, void* stream);
 
+/* Block-granular selection helpers (x a power of two in [1, 1024]).
+ * sga_block_reduce: out[b] = mean (mode 0) or max (mode 1) of |g| over the
+ *   b-th x-element block of one view, tail block over its real length
+ *   (_block_reduce_views, selection/_histogram.py:219-251).
+ * sga_block_any: any_out[b] = block b of the span has a set mask byte
+ *   (block_idx_from_mask, support.py:102-142).
+ * sga_expand_blocks: out[i] = bmask[i / x], i < n
+ *   (bm.repeat_interleave(x)[:n], _histogram.py:303-306). */
+int sga_block_reduce(const float* g, int64_t n, int x, int mode, float* out,
+                     void* stream);
+int sga_block_any(const uint8_t* mask, int64_t n, int x, uint8_t* any_out,
+                  void* stream);
+int sga_expand_blocks(const uint8_t* bmask, int x, int64_t n, uint8_t* out,
+                      void* stream);
+
 /* ---- support: mask -> sorted int32 idx (sga/support.py:57-99) ----------- */
 
 /* Phase 1: per-chunk set-byte counts + total.  chunk_counts has

@@ -189,3 +189,43 @@ def shard_select_balanced(score, k, entries):
     hist = build_histogram(views, shift, nbins, stride, phases)
     b = balanced_crossing_bin(hist, n_total, n_sampled, k)
     return abs_bit_top(score, shift) >= b, bin_edge_float(b, shift)
+
+
+def block_reduce_views(views, x, reduce):
+    """|g| reduced over x-element blocks, tail over its real length
+    (``_histogram.py:219-251``)."""
+    out = []
+    for g in views:
+        c = g.reshape(-1).abs()
+        if c.numel() == 0:
+            out.append(torch.empty(0))
+            continue
+        nb, rem = divmod(c.numel(), x)
+        parts = []
+        if nb:
+            b = c[:nb * x].view(nb, x)
+            parts.append(b.mean(dim=1) if reduce == "mean" else b.amax(dim=1))
+        if rem:
+            t = c[nb * x:]
+            parts.append((t.mean() if reduce == "mean" else t.amax()).reshape(1))
+        out.append(torch.cat(parts))
+    return out
+
+
+def select_masks_blocks(views, k, x, reduce="mean", mode="exact"):
+    """Block-granular histogram select (``_histogram.py:291-307``)."""
+    k_blocks = max(1, int(round(k / x)))
+    bviews = block_reduce_views(views, x, reduce)
+    thresh, bmasks = select_masks_histogram(bviews, k_blocks, mode=mode)
+    return thresh, [bm.repeat_interleave(x)[:g.numel()] for bm, g in zip(bmasks, views)]
+
+
+def block_idx_from_mask(mask_u8, spans, x):
+    """Block starts with ANY set byte, per span (``support.py:102-142``)."""
+    out = []
+    m = mask_u8.tolist()
+    for start, end in spans:
+        for lo in range(start, end, x):
+            if any(m[lo:min(lo + x, end)]):
+                out.append(lo)
+    return torch.tensor(out, dtype=torch.int32)

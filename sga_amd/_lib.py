@@ -39,6 +39,9 @@ SIGNATURES = {
     "sga_masked_norm_sq": (I32, [P, P, I64, P, P, P]),
     "sga_gather_selected_blocks": (I32, [P, P, P, P, I64, I32, F, I64, P]),
     "sga_scatter_selected_blocks": (I32, [P, P, P, P, I64, I32, I64, P]),
+    "sga_block_reduce": (I32, [P, I64, I32, I32, P, P]),
+    "sga_block_any": (I32, [P, I64, I32, P, P]),
+    "sga_expand_blocks": (I32, [P, I32, I64, P, P]),
     "sga_mask_chunks": (I64, [I64]),
     "sga_mask_count": (I32, [P, I64, P, P, P]),
     "sga_mask_fill": (I32, [P, I64, P, P, I64, P]),

@@ -128,6 +128,67 @@ __global__ __launch_bounds__(kBlock) void k_scatter_blocks(
   }
 }
 
+// ------------------------------------------------ block-granular helpers
+// A group of L = min(x, 64) lanes cooperates on one x-element block of a
+// view (the tail block of a view is short and reduces over its real length).
+// MODE 0: mean of |g|, 1: max of |g|  -> float out[block]
+template <int MODE>
+__global__ __launch_bounds__(kBlock) void k_block_reduce(const float* __restrict__ g, int64_t n,
+                                                         int x, int lanes, float* __restrict__ out,
+                                                         int64_t n_blocks) {
+  const int per_wave = kWave / lanes;
+  const int sub = lane_id() / lanes, l = lane_id() % lanes;
+  const int64_t wstride = (int64_t)gridDim.x * kChunksPerBlock * per_wave;
+  for (int64_t b0 = ((int64_t)blockIdx.x * kChunksPerBlock + wave_id()) * per_wave; b0 < n_blocks;
+       b0 += wstride) {
+    const int64_t b = b0 + sub;
+    float acc = 0.0f;
+    int64_t len = 0;
+    if (b < n_blocks) {
+      const int64_t lo = b * x;
+      len = n - lo < x ? n - lo : x;
+      for (int64_t j = l; j < len; j += lanes) {
+        const float a = fabsf(g[lo + j]);
+        acc = MODE == 0 ? acc + a : fmaxf(acc, a);
+      }
+    }
+    for (int o = lanes / 2; o > 0; o >>= 1) {
+      const float t = __shfl_xor(acc, o, kWave);
+      acc = MODE == 0 ? acc + t : fmaxf(acc, t);
+    }
+    if (b < n_blocks && l == 0) out[b] = MODE == 0 ? __fdiv_rn(acc, (float)len) : acc;
+  }
+}
+
+// any_out[b] = 1 when block b of the span has a set byte
+__global__ __launch_bounds__(kBlock) void k_block_any(const uint8_t* __restrict__ mask, int64_t n,
+                                                      int x, int lanes, uint8_t* __restrict__ any_out,
+                                                      int64_t n_blocks) {
+  const int per_wave = kWave / lanes;
+  const int sub = lane_id() / lanes, l = lane_id() % lanes;
+  const int64_t wstride = (int64_t)gridDim.x * kChunksPerBlock * per_wave;
+  for (int64_t b0 = ((int64_t)blockIdx.x * kChunksPerBlock + wave_id()) * per_wave; b0 < n_blocks;
+       b0 += wstride) {
+    const int64_t b = b0 + sub;
+    uint32_t acc = 0;
+    if (b < n_blocks) {
+      const int64_t lo = b * x;
+      const int64_t len = n - lo < x ? n - lo : x;
+      for (int64_t j = l; j < len; j += lanes) acc |= mask[lo + j];
+    }
+    for (int o = lanes / 2; o > 0; o >>= 1) acc |= __shfl_xor(acc, o, kWave);
+    if (b < n_blocks && l == 0) any_out[b] = acc ? 1 : 0;
+  }
+}
+
+// out[i] = bmask[i / x]  (repeat_interleave(x)[:n])
+__global__ __launch_bounds__(kBlock) void k_expand_blocks(const uint8_t* __restrict__ bmask, int xlog,
+                                                          int64_t n, uint8_t* __restrict__ out) {
+  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n;
+       i += (int64_t)gridDim.x * kBlock)
+    out[i] = bmask[i >> xlog];
+}
+
 // ------------------------------------------------------- mask compaction
 // Chunk = 1024 consecutive bytes owned by one wave (4 x 4 bytes per lane).
 // Phase 1 counts the non-zero bytes of each chunk; a two-level exclusive scan
@@ -245,6 +306,48 @@ extern "C" int sga_pack_selected(float* grad, const int32_t* idx, void* values,
 }
 
 static const int64_t kNormMaxBlocks = 2048;
+
+static int xlog_of(int x);
+
+extern "C" int sga_block_reduce(const float* g, int64_t n, int x, int mode, float* out,
+                                void* stream) {
+  if (n == 0) return SGA_OK;
+  if (!g || !out || n < 0 || xlog_of(x) < 0 || (mode != 0 && mode != 1)) {
+    set_error("sga_block_reduce: bad argument (x=%d mode=%d)", x, mode);
+    return SGA_ERR_ARG;
+  }
+  const int64_t nb = cdiv64(n, x);
+  const int lanes = x < kWave ? x : kWave;
+  dim3 grid(stream_grid(nb, kChunksPerBlock * (kWave / lanes))), block(kBlock);
+  if (mode == 0) hipLaunchKernelGGL((k_block_reduce<0>), grid, block, 0, (hipStream_t)stream, g, n, x, lanes, out, nb);
+  else hipLaunchKernelGGL((k_block_reduce<1>), grid, block, 0, (hipStream_t)stream, g, n, x, lanes, out, nb);
+  return check_launch("sga_block_reduce");
+}
+
+extern "C" int sga_block_any(const uint8_t* mask, int64_t n, int x, uint8_t* any_out, void* stream) {
+  if (n == 0) return SGA_OK;
+  if (!mask || !any_out || n < 0 || xlog_of(x) < 0) {
+    set_error("sga_block_any: bad argument (x=%d)", x);
+    return SGA_ERR_ARG;
+  }
+  const int64_t nb = cdiv64(n, x);
+  const int lanes = x < kWave ? x : kWave;
+  hipLaunchKernelGGL(k_block_any, dim3(stream_grid(nb, kChunksPerBlock * (kWave / lanes))),
+                     dim3(kBlock), 0, (hipStream_t)stream, mask, n, x, lanes, any_out, nb);
+  return check_launch("sga_block_any");
+}
+
+extern "C" int sga_expand_blocks(const uint8_t* bmask, int x, int64_t n, uint8_t* out, void* stream) {
+  if (n == 0) return SGA_OK;
+  const int xl = xlog_of(x);
+  if (!bmask || !out || n < 0 || xl < 0) {
+    set_error("sga_expand_blocks: bad argument (x=%d)", x);
+    return SGA_ERR_ARG;
+  }
+  hipLaunchKernelGGL(k_expand_blocks, dim3(stream_grid(n, kBlock)), dim3(kBlock), 0,
+                     (hipStream_t)stream, bmask, xl, n, out);
+  return check_launch("sga_expand_blocks");
+}
 
 extern "C" int64_t sga_norm_partials(int64_t n) {
   return stream_grid(n, (int64_t)kBlock * kVec, kNormMaxBlocks);

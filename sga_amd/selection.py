@@ -149,14 +149,42 @@ class HistogramSelect:
                 f"block_size must be a power of two in [1, 1024], got {block_size!r}")
         if block_reduce not in ("mean", "max"):
             raise ValueError(f"block_reduce must be 'mean' or 'max', got {block_reduce!r}")
-        if block_size != 1:
-            raise NotImplementedError("block-granular selection is not built")
         self.mode, self.block_size = mode, block_size
         self.block_reduce, self.global_allreduce = block_reduce, global_allreduce
 
     def select(self, grads, k, comm_group, warmup_target=None):
-        return select_masks_histogram(grads, k, comm_group, mode=self.mode,
-                                      global_allreduce=self.global_allreduce)
+        if self.block_size == 1:
+            return select_masks_histogram(grads, k, comm_group, mode=self.mode,
+                                          global_allreduce=self.global_allreduce)
+        # block mode (_histogram.py:291-307): select over per-block scores,
+        # then expand the block masks back to element masks
+        x = self.block_size
+        k_blocks = max(1, int(round(k / x)))
+        bviews = block_reduce_views(grads, x, self.block_reduce)
+        thresh, bmasks = select_masks_histogram(bviews, k_blocks, comm_group, mode=self.mode,
+                                                global_allreduce=self.global_allreduce)
+        masks = []
+        st = L.stream()
+        for bm, g in zip(bmasks, grads):
+            m = torch.empty(g.numel(), dtype=torch.uint8, device=g.device)
+            L.call("sga_expand_blocks", L.ptr(bm), x, g.numel(), L.ptr(m), st)
+            masks.append(m)
+        return thresh, masks
+
+
+def block_reduce_views(grads, x, reduce):
+    """Per-view block scores: |g| reduced (mean | max) over contiguous
+    x-element blocks, the tail block over its real length
+    (``_histogram.py:219-251``)."""
+    out = []
+    st = L.stream()
+    for g in _flat_views(grads):
+        nb = -(-g.numel() // x)
+        o = torch.empty(nb, dtype=torch.float32, device=g.device)
+        L.call("sga_block_reduce", L.ptr(g), g.numel(), x, 0 if reduce == "mean" else 1,
+               L.ptr(o), st)
+        out.append(o)
+    return out
 
 
 class ExactKthvalue:

@@ -49,3 +49,41 @@ def compact_mask_u8(mask_u8, pool: Optional[IndexPool] = None):
         L.call("sga_mask_fill", L.ptr(mk), n, L.ptr(counts), L.ptr(buf), buf.numel(),
                L.stream())
     return buf[:k]
+
+
+def block_idx_from_mask(mask_u8, spans, x):
+    """int32 block-start index per x-element block that has ANY set byte, per
+    span; blocks tile each span from its start, the tail block may be short
+    (``sga/support.py:102-142``).  With x == 1 equals ``compact_mask_u8``."""
+    assert mask_u8.numel() < 2 ** 31, (
+        f"int32 block-start indices assume < 2^31 elements, got {mask_u8.numel()}")
+    L.require_dev(mask_u8)
+    mk = mask_u8.reshape(-1)
+    if mk.dtype == torch.bool:
+        mk = mk.view(torch.uint8)
+    dev = mk.device
+    prev_end, counts = 0, []
+    for start, end in spans:
+        assert start >= prev_end, (
+            f"spans must be ascending and non-overlapping, got span starting at {start} "
+            f"after one ending at {prev_end}")
+        prev_end = end
+        counts.append(-(-(end - start) // x))
+    total = sum(counts)
+    if total == 0:
+        return torch.empty(0, dtype=torch.int32, device=dev)
+    any_b = torch.empty(total, dtype=torch.uint8, device=dev)
+    st = L.stream()
+    off = 0
+    for (start, end), nb in zip(spans, counts):
+        if nb:
+            L.call("sga_block_any", L.ptr(mk[start:end]), end - start, x,
+                   L.ptr(any_b[off:off + nb]), st)
+        off += nb
+    ordinal = compact_mask_u8(any_b).long()        # selected block ordinals, ascending
+    if ordinal.numel() == 0:
+        return torch.empty(0, dtype=torch.int32, device=dev)
+    first = torch.tensor([0] + list(torch.tensor(counts).cumsum(0)[:-1]), device=dev)
+    starts = torch.tensor([s for s, _ in spans], device=dev)
+    owner = torch.searchsorted(first, ordinal, right=True) - 1
+    return ((ordinal - first[owner]) * x + starts[owner]).to(torch.int32)

@@ -178,3 +178,47 @@ def test_sampled_bracket_path_and_fallback(dev):
             assert torch.equal(m2.cpu().bool(), sc >= t_ref), (name, k)
     assert ("student-t", 1) in seen and ("gauss", 1) in seen
     assert ("all-equal", 0) in seen
+
+
+@pytest.mark.parametrize("x,reduce", [(4, "max"), (64, "max"), (1024, "max"), (8, "mean")])
+def test_block_granular_selection(dev, x, reduce):
+    from sga_amd.selection import HistogramSelect, block_reduce_views
+    from sga_amd.support import block_idx_from_mask
+    g = torch.Generator().manual_seed(x)
+    views = [torch.randn(40001, generator=g), torch.randn(7, generator=g),
+             torch.randn(65536, generator=g) * 3, torch.randn(100009, generator=g)]
+    dviews = [v.to(dev) for v in views]
+    n_total = sum(v.numel() for v in views)
+    k = SEL.k_for(n_total, 5.0)
+    bv_ref = SEL.block_reduce_views(views, x, reduce)
+    bv_dev = block_reduce_views(dviews, x, reduce)
+    for a, b in zip(bv_dev, bv_ref):
+        if reduce == "max":
+            assert torch.equal(a.cpu(), b)
+        else:                      # fp32 summation order differs: tolerance class
+            torch.testing.assert_close(a.cpu(), b, rtol=1e-6, atol=0)
+    if reduce == "max":
+        th_ref, m_ref = SEL.select_masks_blocks(views, k, x, reduce)
+        th_dev, m_dev = HistogramSelect("exact", block_size=x, block_reduce=reduce).select(
+            dviews, k, None)
+        assert th_dev == th_ref
+        for a, b in zip(m_dev, m_ref):
+            assert torch.equal(a.cpu(), b)
+        mask = torch.cat(m_ref)
+    else:
+        mask = (torch.rand(n_total, generator=g) < 0.01).to(torch.uint8)
+    spans, off = [], 0
+    for v in views:
+        spans.append((off, off + v.numel()))
+        off += v.numel()
+    got = block_idx_from_mask(mask.to(dev), spans, x)
+    assert got.dtype == torch.int32
+    assert torch.equal(got.cpu(), SEL.block_idx_from_mask(mask, spans, x))
+    # the block gather moves exactly the set bytes of every listed block
+    from sga_amd.kernels import gather_selected_blocks, scatter_selected_blocks
+    flat = torch.cat(views)
+    vals = torch.empty(got.numel() * x, device=dev)
+    gather_selected_blocks(flat.to(dev), mask.to(dev), got, vals, x, 1.0)
+    dst = torch.zeros(n_total, device=dev)
+    scatter_selected_blocks(dst, mask.to(dev), got, vals, x)
+    assert torch.equal(dst.cpu(), torch.where(mask.bool(), flat, torch.zeros(())))

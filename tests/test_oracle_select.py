@@ -163,3 +163,15 @@ def test_compact_mask_kats():
     g = torch.Generator().manual_seed(4)
     m = (torch.rand(300000, generator=g) < 0.4).to(torch.uint8)
     assert OK.compact_mask_u8(m).tolist() == [i for i, b in enumerate(m.tolist()) if b]
+
+
+def test_block_helpers_kats():
+    """Literal block KATs: ANY rule, short tail blocks, x == 1 == compaction."""
+    m = torch.tensor([0, 1, 0, 0, 0, 0, 1, 1, 0, 0, 1], dtype=torch.uint8)
+    assert SEL.block_idx_from_mask(m, [(0, 6), (6, 11)], 4).tolist() == [0, 6, 10]
+    assert SEL.block_idx_from_mask(m, [(0, 11)], 1).tolist() == OK.compact_mask_u8(m).tolist()
+    g = torch.tensor([1.0, -3.0, 2.0, 0.0, 5.0])
+    assert SEL.block_reduce_views([g], 2, "max")[0].tolist() == [3.0, 2.0, 5.0]
+    assert SEL.block_reduce_views([g], 2, "mean")[0].tolist() == [2.0, 1.0, 5.0]
+    th, masks = SEL.select_masks_blocks([g], 2, 2, "max")
+    assert masks[0].tolist() == [0, 0, 0, 0, 1] and th == 5.0
