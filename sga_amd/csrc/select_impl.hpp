@@ -815,12 +815,17 @@ __global__ __launch_bounds__(kBlock) void k_bracket_sweep(
 static __global__ __launch_bounds__(kBlock) void k_bracket_check(SelState* __restrict__ st,
                                                                  SelState* __restrict__ aux,
                                                                  uint32_t* __restrict__ seg_cnt,
-                                                                 uint32_t* __restrict__ hist, int nhist) {
+                                                                 uint32_t* __restrict__ hist, int nhist,
+                                                                 int n_waves) {
   __shared__ uint32_t s_w4[kChunksPerBlock];
   constexpr int PER = kSegWaves / kBlock;   // 16
   uint32_t v[PER], mine = 0;
 #pragma unroll
-  for (int j = 0; j < PER; ++j) { v[j] = seg_cnt[threadIdx.x * PER + j]; mine += v[j]; }
+  for (int j = 0; j < PER; ++j) {
+    const int wv = threadIdx.x * PER + j;
+    v[j] = wv < n_waves ? seg_cnt[wv] : 0u;   // waves the sweep did not launch own nothing
+    mine += v[j];
+  }
   uint32_t total;
   uint32_t run = block_excl_scan(mine, s_w4, total);
 #pragma unroll
@@ -905,11 +910,26 @@ static inline void run_select(Src src, int64_t n, int64_t k, int tie_all, bool f
       // <= 1M keys: 64 fat workgroups keep the histogram flush (one atomic per
       // non-empty bin per workgroup) far below one atomic per key
       launch_level<SrcU32, 2, true>(ssrc, ns, (const uint32_t*)nullptr, level, w.aux, w, s, 64);
-    hipLaunchKernelGGL((k_bracket_sweep<Src>), dim3(kSegWaves / kChunksPerBlock), dim3(kBlock), 0, s,
+    // persistent grid = exactly what the device holds at once for THIS
+    // instantiation (a partial second round would idle most of the chip)
+    static int sweep_blocks = 0;
+    if (sweep_blocks == 0) {
+      int per_cu = 0, dev = 0;
+      hipDeviceProp_t prop;
+      if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess &&
+          hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, k_bracket_sweep<Src>, kBlock, 0) ==
+              hipSuccess && per_cu > 0) {
+        sweep_blocks = per_cu * prop.multiProcessorCount;
+      } else {
+        sweep_blocks = 1024;
+      }
+      if (sweep_blocks > kSegWaves / kChunksPerBlock) sweep_blocks = kSegWaves / kChunksPerBlock;
+    }
+    hipLaunchKernelGGL((k_bracket_sweep<Src>), dim3(sweep_blocks), dim3(kBlock), 0, s,
                        src, n, w.st, w.aux, w.tile_gt, w.tile_eq, w.seg_idx, w.seg_key, w.seg_cnt,
                        (uint32_t)w.seg_cap);
     hipLaunchKernelGGL(k_bracket_check, dim3(1), dim3(kBlock), 0, s, w.st, w.aux, w.seg_cnt, w.hist,
-                       kHistStride * 2);
+                       kHistStride * 2, sweep_blocks * kChunksPerBlock);
     hipLaunchKernelGGL(k_cand_compact, dim3(256), dim3(kBlock), 0, s, w.aux, w.seg_cnt, w.seg_idx,
                        w.seg_key, (uint32_t)w.seg_cap, w.cand_idx, w.cand_key);
     SrcU32 csrc{w.cand_key};
