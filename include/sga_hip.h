@@ -210,6 +210,11 @@ int sga_hist_topbits(const float* score, int64_t n, int shift, int stride,
 int sga_mask_topbits_ge(const float* score, int64_t n, int shift, int32_t bin,
                         uint8_t* mask_out, void* stream);
 
+/* Adaptive-tau threshold mask (_adaptive.py:44-66): mask = |score| >= tau,
+ * count[0] (device int64, may be NULL) += number of set bytes. */
+int sga_mask_abs_ge(const float* score, int64_t n, float tau, uint8_t* mask_out,
+                    int64_t* count, void* stream);
+
 /* replay_kernels.py:372-414 building blocks with the same outputs. */
 int sga_cand_extract_count(const float* score, int64_t n, int32_t bin,
                            uint32_t* chunk_counts, int64_t* total,

@@ -229,3 +229,57 @@ def block_idx_from_mask(mask_u8, spans, x):
             if any(m[lo:min(lo + x, end)]):
                 out.append(lo)
     return torch.tensor(out, dtype=torch.int32)
+
+
+ADAPT_BAND = 0.01          # _adaptive.py:21
+ADAPT_LOG_GAIN = 0.5       # _adaptive.py:22
+ADAPT_MAX_UP = 1.15        # _adaptive.py:23
+ADAPT_MAX_DOWN = 0.9       # _adaptive.py:24
+
+
+def adapt_threshold(thresh, measured, target):
+    """Dead-band multiplicative tau update (``_adaptive.py:27-41``)."""
+    if abs(measured - target) <= ADAPT_BAND:
+        return thresh
+    f = (measured / target) ** ADAPT_LOG_GAIN
+    return thresh * min(max(f, ADAPT_MAX_DOWN), ADAPT_MAX_UP)
+
+
+class AdaptiveTau:
+    """Persistent-threshold selector state machine (``_adaptive.py:79-187``,
+    world 1)."""
+
+    def __init__(self, ratio_percent, warmup_syncs, warmup_mode):
+        self.target = ratio_percent / 100.0
+        self.warmup_syncs = warmup_syncs
+        self.mode = warmup_mode
+        self.tau = None
+        self.warmup_passed = 0
+
+    def warmup_sync_target(self, start_iter, period):
+        if self.warmup_syncs is None:
+            return None
+        return max(0, (self.warmup_syncs * period - 1 - start_iter) // period)
+
+    def _boot(self, views, k):
+        thresh, masks = select_masks_histogram(views, k, self.mode)
+        self.tau = thresh if thresh > 0.0 else bin_edge_float(1, HIST_MODES[self.mode][0])
+        return masks
+
+    def select(self, views, k, warmup_target=None):
+        n = sum(g.numel() for g in views)
+        required = max(warmup_target if warmup_target is not None else
+                       (self.warmup_syncs if self.warmup_syncs is not None else 1), 1)
+        if self.tau is None or self.warmup_passed < required:
+            masks = self._boot(views, k)
+            r = sum(int(m.sum()) for m in masks) / n
+            self.warmup_passed = self.warmup_passed + 1 if abs(r - self.target) <= ADAPT_BAND else 0
+            return self.tau, masks
+        masks = [(g.reshape(-1).abs() >= self.tau).to(torch.uint8) for g in views]
+        r = sum(int(m.sum()) for m in masks) / n
+        if r == 0.0 or self.tau <= 0.0:
+            masks = self._boot(views, k)
+            return self.tau, masks
+        used = self.tau
+        self.tau = adapt_threshold(used, r, self.target)
+        return used, masks

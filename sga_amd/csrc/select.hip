@@ -129,6 +129,35 @@ __global__ __launch_bounds__(kBlock) void k_gt_eq(
   }
 }
 
+// mask = |x| >= tau (float compare, NaN -> 0), count accumulated (u64 atomic
+// per workgroup: order-free)
+__global__ __launch_bounds__(kBlock) void k_mask_abs_ge(const float* __restrict__ x, int64_t n,
+                                                        float tau, uint8_t* __restrict__ mask,
+                                                        unsigned long long* __restrict__ count,
+                                                        bool vec) {
+  __shared__ uint32_t s_w[kChunksPerBlock];
+  uint32_t c = 0;
+  const int64_t stride = (int64_t)gridDim.x * kBlock * kVec;
+  for (int64_t i = ((int64_t)blockIdx.x * kBlock + threadIdx.x) * kVec; i < n; i += stride) {
+    float v[4];
+    load4_f32(x, i, n, v, vec);
+    uint32_t mk[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      mk[e] = (i + e < n) && fabsf(v[e]) >= tau;
+      c += mk[e];
+    }
+    store4_u8(mask, i, n, mk, vec);
+  }
+  c = wave_sum(c);
+  if (lane_id() == 0) s_w[wave_id()] = c;
+  __syncthreads();
+  if (threadIdx.x == 0 && count) {
+    const uint32_t t = s_w[0] + s_w[1] + s_w[2] + s_w[3];
+    if (t) atomicAdd(count, (unsigned long long)t);
+  }
+}
+
 __global__ void k_zero_i32(int32_t* p, int n) {
   for (int i = threadIdx.x; i < n; i += blockDim.x) p[i] = 0;
 }
@@ -276,6 +305,17 @@ extern "C" int sga_mask_topbits_ge(const float* score, int64_t n, int shift, int
                      0, (hipStream_t)stream, score, n, shift, (uint32_t)bin, mask_out,
                      aligned4(score, 4) && aligned4(mask_out, 1));
   return check_launch("sga_mask_topbits_ge");
+}
+
+extern "C" int sga_mask_abs_ge(const float* score, int64_t n, float tau, uint8_t* mask_out,
+                               int64_t* count, void* stream) {
+  if (n == 0) return SGA_OK;
+  if (!score || !mask_out || n < 0) { set_error("sga_mask_abs_ge: bad argument"); return SGA_ERR_ARG; }
+  hipLaunchKernelGGL(k_mask_abs_ge, dim3(stream_grid(n, (int64_t)kBlock * kVec * 4, 256 * 8)),
+                     dim3(kBlock), 0, (hipStream_t)stream, score, n, tau, mask_out,
+                     reinterpret_cast<unsigned long long*>(count),
+                     aligned4(score, 4) && aligned4(mask_out, 1));
+  return check_launch("sga_mask_abs_ge");
 }
 
 extern "C" int sga_cand_extract_count(const float* score, int64_t n, int32_t bin,

@@ -187,6 +187,108 @@ def block_reduce_views(grads, x, reduce):
     return out
 
 
+def count_on(mask_u8):
+    """Number of set bytes of a device uint8 mask (``_adaptive.py:44-51``)."""
+    n = mask_u8.numel()
+    if n == 0:
+        return 0
+    L.require_dev(mask_u8)
+    dev = mask_u8.device
+    counts = torch.empty(int(L.raw("sga_mask_chunks", n)), dtype=torch.int32, device=dev)
+    total = torch.empty(1, dtype=torch.int64, device=dev)
+    L.call("sga_mask_count", L.ptr(mask_u8), n, L.ptr(counts), L.ptr(total), L.stream())
+    return int(total.item())
+
+
+def threshold_masks(grads, tau):
+    """``|g| >= tau`` uint8 masks per view and their total set count in one
+    sweep each (``_adaptive.py:44-66``: ``_threshold_masks`` + ``_count_on``)."""
+    views = _flat_views(grads)
+    dev = views[0].device
+    count = torch.zeros(1, dtype=torch.int64, device=dev)
+    masks = []
+    st = L.stream()
+    for g in views:
+        m = torch.empty(g.numel(), dtype=torch.uint8, device=dev)
+        L.call("sga_mask_abs_ge", L.ptr(g), g.numel(), L.f32(tau), L.ptr(m), L.ptr(count), st)
+        masks.append(m)
+    return masks, int(count.item())
+
+
+def adapt_threshold(thresh, measured_ratio, target_ratio, gain=0.5, max_up=1.15,
+                    max_down=0.9, band=0.01):
+    """One multiplicative dead-band update of tau (``_adaptive.py:28-41``)."""
+    if abs(measured_ratio - target_ratio) <= band:
+        return thresh
+    factor = (measured_ratio / target_ratio) ** gain
+    return thresh * min(max(factor, max_down), max_up)
+
+
+_ADAPT_BAND = 0.01            # _adaptive.py:21-24
+
+
+class AdaptiveTau:
+    """Persistent-threshold selector (``_adaptive.py:79-187``).
+
+    While warming up (and whenever the threshold has collapsed) the mask
+    comes from the histogram select in ``warmup_mode``; afterwards one
+    ``|g| >= tau`` sweep produces masks and their count, and tau follows the
+    measured ratio by the dead-band multiplicative rule.
+    """
+
+    def __init__(self, ratio_percent, warmup_syncs, warmup_mode, global_allreduce=True):
+        if warmup_mode not in _HIST_MODES:
+            raise ValueError(f"unknown adaptive_warmup_mode: {warmup_mode!r} "
+                             f"(expected one of {sorted(_HIST_MODES)})")
+        if not isinstance(global_allreduce, bool):
+            raise ValueError(f"global_allreduce must be a bool, got {global_allreduce!r}")
+        self.target_ratio = ratio_percent / 100.0
+        self.warmup_syncs = warmup_syncs
+        self.warmup_mode = warmup_mode
+        self.global_allreduce = global_allreduce
+        self.tau = None
+        self.warmup_passed = 0
+
+    def warmup_sync_target(self, start_iter, period):
+        """Gated warmup selects left for a selection that starts at
+        ``start_iter`` (``_adaptive.py:104-122``); a boundary exactly on the
+        window edge is post-warmup."""
+        if self.warmup_syncs is None:
+            return None
+        return max(0, (self.warmup_syncs * period - 1 - start_iter) // period)
+
+    def _bootstrap(self, grads, k, comm_group):
+        thresh, masks = select_masks_histogram(grads, k, comm_group, mode=self.warmup_mode,
+                                               global_allreduce=self.global_allreduce)
+        # bin 0's edge is 0.0, which the multiplicative rule can never leave
+        self.tau = thresh if thresh > 0.0 else _bin_edge_float(
+            1, _HIST_MODES[self.warmup_mode][0])
+        return masks
+
+    @staticmethod
+    def _measured(masks, grads):
+        return sum(count_on(m) for m in masks) / sum(g.numel() for g in grads)
+
+    def select(self, grads, k, comm_group, warmup_target):
+        if warmup_target is not None:
+            required = max(warmup_target, 1)
+        else:
+            required = max(self.warmup_syncs if self.warmup_syncs is not None else 1, 1)
+        if self.tau is None or self.warmup_passed < required:
+            masks = self._bootstrap(grads, k, comm_group)
+            hit = abs(self._measured(masks, grads) - self.target_ratio) <= _ADAPT_BAND
+            self.warmup_passed = self.warmup_passed + 1 if hit else 0
+            return self.tau, masks
+        masks, on = threshold_masks(grads, self.tau)
+        measured = on / sum(g.numel() for g in grads)
+        if measured == 0.0 or self.tau <= 0.0:
+            masks = self._bootstrap(grads, k, comm_group)
+            return self.tau, masks
+        used = self.tau
+        self.tau = adapt_threshold(used, measured, self.target_ratio)
+        return used, masks
+
+
 class ExactKthvalue:
     def select(self, grads, k, comm_group, warmup_target=None):
         return select_masks_exact_kthvalue(grads, k, comm_group)
@@ -211,8 +313,12 @@ class TopkSelection:
         elif self.method == "exact":
             self._impl = ExactKthvalue()
         elif self.method == "adaptive":
-            raise NotImplementedError("the adaptive-tau controller is host control "
-                                      "logic outside this build")
+            ws = getattr(args, "sga_selection_adaptive_warmup_syncs", None)
+            self._impl = AdaptiveTau(
+                self.ratio_percent, int(ws) if ws is not None else None,
+                getattr(args, "sga_selection_adaptive_warmup_mode", "fast"),
+                global_allreduce=bool(getattr(
+                    args, "sga_selection_topk_histogram_add_global_allreduce", False)))
         else:
             raise ValueError("sga_selection_method must be adaptive|exact|histogram "
                              f"(got {self.method!r})")
@@ -222,8 +328,20 @@ class TopkSelection:
     def block_size(self):
         return getattr(self._impl, "block_size", 1)
 
+    @property
+    def tau(self):
+        return getattr(self._impl, "tau", None)
+
+    @property
+    def warmup_passed(self):
+        return getattr(self._impl, "warmup_passed", None)
+
     def k_for(self, n_total):
         return max(1, int(round(n_total * self.ratio_percent / 100.0)))
+
+    def warmup_sync_target(self, start_iter, period):
+        hook = getattr(self._impl, "warmup_sync_target", None)
+        return hook(start_iter, period) if callable(hook) else None
 
     def select(self, ctx):
         k = self.k_for(sum(g.numel() for g in ctx.grad_views))

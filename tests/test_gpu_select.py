@@ -222,3 +222,55 @@ def test_block_granular_selection(dev, x, reduce):
     dst = torch.zeros(n_total, device=dev)
     scatter_selected_blocks(dst, mask.to(dev), got, vals, x)
     assert torch.equal(dst.cpu(), torch.where(mask.bool(), flat, torch.zeros(())))
+
+
+def test_adaptive_threshold_masks(dev):
+    from sga_amd.selection import adapt_threshold, threshold_masks
+    g = torch.Generator().manual_seed(11)
+    views = [torch.randn(100_003, generator=g), torch.randn(5, generator=g),
+             torch.randn(65_536, generator=g) * 2]
+    views[0][7] = float("nan")
+    tau = 1.25
+    masks, cnt = threshold_masks([v.to(dev) for v in views], tau)
+    ref = [(v.abs() >= tau).to(torch.uint8) for v in views]
+    for a, b in zip(masks, ref):
+        assert torch.equal(a.cpu(), b)
+    assert cnt == sum(int(m.sum()) for m in ref)
+    assert adapt_threshold(2.0, 0.105, 0.10) == 2.0
+    assert adapt_threshold(2.0, 0.4, 0.10) == 2.0 * 1.15
+    assert abs(adapt_threshold(2.0, 0.12, 0.10, band=0.0) - 2.0 * 1.2 ** 0.5) < 1e-12
+
+
+def test_adaptive_tau_trajectory_matches_oracle(dev):
+    """Bootstrap, gated warmup, tau feedback and collapse re-bootstrap over a
+    drifting gradient scale: thresholds, masks and controller state track
+    the oracle's state machine cycle by cycle."""
+    from types import SimpleNamespace
+
+    from oracle import select as OS
+    from sga_amd.selection import TopkSelection
+    args = SimpleNamespace(sga_selection_method="adaptive", sga_selection_ratio_percent=10.0,
+                           sga_selection_adaptive_warmup_syncs=2,
+                           sga_selection_adaptive_warmup_mode="fast")
+    sel = TopkSelection(args)
+    ref = OS.AdaptiveTau(10.0, 2, "fast")
+    assert sel.warmup_sync_target(0, 4) == ref.warmup_sync_target(0, 4) == 1
+    gen = torch.Generator().manual_seed(5)
+    scales = [1.0, 1.0, 1.0, 1.3, 1.3, 0.7, 0.7, 1e-6, 1.0, 1.0]
+    for cyc, sc in enumerate(scales):
+        grads = [torch.randn(50_000, generator=gen) * sc, torch.randn(1_237, generator=gen) * sc]
+        k = OS.k_for(51_237, 10.0)
+        thr_r, m_r = ref.select(grads, k, 2)
+        ctx = SimpleNamespace(grad_views=[g.to(dev) for g in grads], comm_group=None,
+                              warmup_target=2)
+        m_d = sel.select(ctx)
+        assert sel.last_threshold == thr_r, (cyc, sel.last_threshold, thr_r)
+        assert sel.tau == ref.tau and sel.warmup_passed == ref.warmup_passed, cyc
+        for a, b in zip(m_d, m_r):
+            assert torch.equal(a.cpu(), b), cyc
+    # zero-tau latch re-bootstraps to the smallest positive bin edge
+    sel._impl.tau = 0.0
+    sel._impl.warmup_passed = 5
+    sel.select(SimpleNamespace(grad_views=[torch.zeros(64, device=dev)], comm_group=None,
+                               warmup_target=0))
+    assert sel.tau == OS.bin_edge_float(1, 19)

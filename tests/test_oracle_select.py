@@ -175,3 +175,52 @@ def test_block_helpers_kats():
     assert SEL.block_reduce_views([g], 2, "mean")[0].tolist() == [2.0, 1.0, 5.0]
     th, masks = SEL.select_masks_blocks([g], 2, 2, "max")
     assert masks[0].tolist() == [0, 0, 0, 0, 1] and th == 5.0
+
+
+def test_adaptive_threshold_reference_vectors():
+    # known answers held by the reference's own unit test
+    # (tests/test_plugins_unit.py:603-616)
+    f = SEL.adapt_threshold
+    assert f(1.0, 0.105, 0.10) == 1.0 and f(1.0, 0.095, 0.10) == 1.0
+    assert f(1.0, 0.13, 0.10) == 1.3 ** 0.5
+    assert f(1.0, 0.085, 0.10) == 0.85 ** 0.5
+    assert f(1.0, 0.20, 0.10) == 1.15
+    assert f(1.0, 0.0001, 0.10) == 0.9
+
+
+def test_adaptive_warmup_anchor_reference_vectors():
+    # tests/test_plugins_unit.py:346-362
+    a = SEL.AdaptiveTau(40.0, 5, "fast")
+    assert a.warmup_sync_target(0, 4) == 4
+    assert a.warmup_sync_target(6, 4) == (20 - 1 - 6) // 4
+    assert a.warmup_sync_target(25, 4) == 0
+    assert SEL.AdaptiveTau(40.0, None, "fast").warmup_sync_target(0, 4) is None
+
+
+def test_adaptive_lifecycle_oracle():
+    # the phases the reference's lifecycle test walks
+    # (tests/test_plugins_unit.py:619-677)
+    torch.manual_seed(12)
+    grads = [torch.randn(4096), torch.randn(1000)]
+    k = SEL.k_for(5096, 10.0)
+    a = SEL.AdaptiveTau(10.0, None, "fast")
+    thr, _ = a.select(grads, k, 3)
+    bits = torch.tensor(thr, dtype=torch.float32).view(torch.int32).item()
+    assert bits & ((1 << 19) - 1) == 0 and a.tau == thr and a.warmup_passed in (0, 1)
+    a.warmup_passed = 0
+    thr, _ = a.select(grads, k, 3)
+    assert a.tau == thr
+    a.warmup_passed = 3
+    tau = a.tau
+    thr, masks = a.select(grads, k, 3)
+    assert thr == tau
+    for g, m in zip(grads, masks):
+        assert torch.equal(m, (g.abs() >= tau).to(torch.uint8))
+    a.tau = 1e30
+    _, masks = a.select(grads, k, 3)
+    assert a.tau < 1e30 and any(int(m.sum()) for m in masks)
+    # zero-tau latch: an all-zero input bootstraps to bin 0 -> floor edge
+    a.warmup_passed = 5
+    a.tau = 0.0
+    a.select([torch.zeros(64)], 6, 0)
+    assert a.tau == SEL.bin_edge_float(1, 19) and a.tau > 0.0
