@@ -99,6 +99,12 @@ int sga_compact_norm_sq(const float* values, int64_t k, float* partials,
 int sga_masked_norm_sq(const float* grad, const uint8_t* mask, int64_t n,
                        float* partials, float* total, void* stream);
 
+/* grad[i] *= coeff where mask[i] != 0 (mask NULL: everywhere) -- the explicit
+ * clip scale of the masked clip service, engine.py:1172-1216
+ * (`grad.mul_(coeff)`, `grad.view(-1)[m > 0] *= coeff`). */
+int sga_scale_masked(float* grad, const uint8_t* mask, int64_t n, float coeff,
+                     void* stream);
+
 /* block gather / scatter  -- gather_selected_blocks / scatter_selected_blocks,
  * kernels.py:190-249 */
 int sga_gather_selected_blocks(const float* grad, const uint8_t* mask,

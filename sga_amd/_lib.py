@@ -60,6 +60,7 @@ SIGNATURES = {
     "sga_sel_result": (I32, [P, P, SZ, P]),
     "sga_hist_topbits": (I32, [P, I64, I32, I32, I32, P, I32, P, P]),
     "sga_mask_topbits_ge": (I32, [P, I64, I32, I32, P, P]),
+    "sga_scale_masked": (I32, [P, P, I64, F, P]),
     "sga_mask_abs_ge": (I32, [P, I64, F, P, P, P]),
     "sga_cand_extract_count": (I32, [P, I64, I32, P, P, P]),
     "sga_cand_extract_fill": (I32, [P, I64, I32, P, P, I64, P]),

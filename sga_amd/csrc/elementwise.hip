@@ -387,6 +387,37 @@ extern "C" int sga_masked_norm_sq(const float* grad, const uint8_t* mask,
   return check_launch("sga_masked_norm_sq");
 }
 
+// g[i] *= coeff where mask[i] (every i when mask is null): the explicit clip
+// scale, one fp32 multiply per touched coordinate.
+template <bool MASKED>
+__global__ __launch_bounds__(kBlock) void k_scale_masked(float* __restrict__ g,
+                                                         const uint8_t* __restrict__ mask,
+                                                         int64_t n, float coeff, bool vec) {
+  const int64_t stride = (int64_t)gridDim.x * kBlock * kVec;
+  for (int64_t i = ((int64_t)blockIdx.x * kBlock + threadIdx.x) * kVec; i < n; i += stride) {
+    float v[4];
+    load4_f32(g, i, n, v, vec);
+    uint32_t mk[4] = {1u, 1u, 1u, 1u};
+    if (MASKED) load4_u8(mask, i, n, mk, vec);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) v[e] = mk[e] ? v[e] * coeff : v[e];
+    store4_f32(g, i, n, v, vec);
+  }
+}
+
+extern "C" int sga_scale_masked(float* grad, const uint8_t* mask, int64_t n, float coeff,
+                                void* stream) {
+  if (n == 0) return SGA_OK;
+  if (!grad || n < 0) { set_error("sga_scale_masked: bad argument"); return SGA_ERR_ARG; }
+  dim3 grid(stream_grid(n, (int64_t)kBlock * kVec * 4, 256 * 8)), block(kBlock);
+  const bool vec = aligned4(grad, 4) && aligned4(mask, 1);
+  if (mask)
+    hipLaunchKernelGGL((k_scale_masked<true>), grid, block, 0, (hipStream_t)stream, grad, mask, n, coeff, vec);
+  else
+    hipLaunchKernelGGL((k_scale_masked<false>), grid, block, 0, (hipStream_t)stream, grad, mask, n, coeff, vec);
+  return check_launch("sga_scale_masked");
+}
+
 static int xlog_of(int x) {
   if (x < 1 || x > 1024 || (x & (x - 1))) return -1;
   int l = 0;
