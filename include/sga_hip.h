@@ -242,6 +242,16 @@ int sga_score_formula(int score_id, const float* w, const float* m,
                       float bc1, float bc2, float eps, int absolute, int adams,
                       void* stream);
 
+/* Branch-point score of the replay front select (replay_fused.py:1236-1265):
+ * the same registry formula evaluated in double on fp32 inputs with double
+ * scalars, out = fp32(|score|).  adams != 0: v := m*m, bc := 1.  include_wd
+ * adds wd*w to the update score (the online cycle semantics). */
+int sga_branch_score_f64(int score_id, const float* w, const float* m,
+                         const float* v, const float* g, float* out, int64_t n,
+                         double beta1, double beta2, double eps, double wd,
+                         double bc1, double bc2, int adams, int include_wd,
+                         void* stream);
+
 /* opt_step_inplace / _k_adam, replay_kernels.py:163-216, 330-369 and
  * replay.py:674-744.  flags: SGA_RP_*. */
 int sga_opt_step_inplace(const float* q, float* m, float* v, float* w,
@@ -325,6 +335,16 @@ int sga_replay_reselect(const void* g, int g_dtype, const float* res,
 int sga_replay_pass3(const void* g, int g_dtype, int64_t n, float coef_dense,
                      const sga_replay_cfg* cfgs, int G, const float* coef_f,
                      const sga_replay_segment* segs, int n_segs, void* stream);
+
+/* Dense reference step of the replay (dense_replay_dev, replay.py:848-926):
+ * in-place AdamW/AdamS commit of the recorded gradient g over the whole flat
+ * shard with per-tensor hyper-parameters from segs, lab += (lr*upd)^2 when lab
+ * is not NULL, and recon2[0] = sum((g / coef_dense)^2) in double.  partials:
+ * sga_replay_partials() doubles of workspace. */
+int sga_dense_replay_step(const void* g, int g_dtype, float* w, float* m, float* v,
+                          float* lab, int64_t n, const sga_replay_segment* segs,
+                          int n_segs, int adams, double coef_dense, double* partials,
+                          double* recon2, void* stream);
 
 /* res /= T at fold boundaries (replay_fused.py:1632-1636), true division. */
 int sga_div_inplace(float* x, int64_t n, float d, void* stream);

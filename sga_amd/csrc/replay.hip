@@ -37,6 +37,54 @@ __global__ __launch_bounds__(kBlock) void k_score_formula(
   }
 }
 
+// Branch-point score: the registry formula evaluated in double on fp32
+// inputs, |.| rounded once to fp32 (the replay's front select ranks these).
+struct BranchK {
+  double b1, om1, b2, om2, eps, wd, bc1, bc2;
+};
+
+template <int SCORE>
+__global__ __launch_bounds__(kBlock) void k_branch_score(
+    const float* __restrict__ w, const float* __restrict__ m, const float* __restrict__ v,
+    const float* __restrict__ g, float* __restrict__ out, int64_t n, BranchK c, bool adams,
+    bool include_wd, bool vec) {
+  const int64_t stride = (int64_t)gridDim.x * kBlock * kVec;
+  for (int64_t i = ((int64_t)blockIdx.x * kBlock + threadIdx.x) * kVec; i < n; i += stride) {
+    float ww[4] = {0, 0, 0, 0}, mm[4] = {0, 0, 0, 0}, vv[4] = {0, 0, 0, 0}, gg[4] = {0, 0, 0, 0};
+    if (SCORE != SGA_SCORE_ABS_M) load4_f32(g, i, n, gg, vec);
+    if (SCORE != SGA_SCORE_ABS_G) load4_f32(m, i, n, mm, vec);
+    if (SCORE == SGA_SCORE_UPDATE || SCORE == SGA_SCORE_COI) {
+      load4_f32(w, i, n, ww, vec);
+      if (!adams) load4_f32(v, i, n, vv, vec);
+    }
+    float o[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const double gd = gg[e], md = mm[e], wd_ = ww[e];
+      const double vd = adams ? md * md : (double)vv[e];
+      double r;
+      if (SCORE == SGA_SCORE_ABS_G) {
+        r = gd;
+      } else if (SCORE == SGA_SCORE_ABS_M) {
+        r = md;
+      } else {
+        const double sa = __ddiv_rn(md * c.b1 + gd * c.om1, c.bc1);
+        const double sb = __ddiv_rn(vd * c.b2 + (gd * c.om2) * gd, c.bc2);
+        const double ug = __ddiv_rn(sa, __dsqrt_rn(sb) + c.eps);
+        if (SCORE == SGA_SCORE_UPDATE) {
+          r = include_wd ? c.wd * wd_ + ug : ug;
+        } else {
+          const double u0 = __ddiv_rn(__ddiv_rn(md * c.b1, c.bc1),
+                                      __dsqrt_rn(__ddiv_rn(vd * c.b2, c.bc2)) + c.eps);
+          r = ug - u0;
+        }
+      }
+      o[e] = (float)fabs(r);
+    }
+    store4_f32(out, i, n, o, vec);
+  }
+}
+
 struct StepK {
   float b1, om1, b2, om2, bc1, bc2, eps, omlwd, neglr, lr2, lr, lri, wd;
 };
@@ -116,6 +164,38 @@ extern "C" int sga_score_formula(int score_id, const float* w, const float* m, c
   }
 #undef SGA_SF
   return check_launch("sga_score_formula");
+}
+
+extern "C" int sga_branch_score_f64(int score_id, const float* w, const float* m, const float* v,
+                                    const float* g, float* out, int64_t n, double beta1,
+                                    double beta2, double eps, double wd, double bc1, double bc2,
+                                    int adams, int include_wd, void* stream) {
+  if (n == 0) return SGA_OK;
+  if (!out || n < 0 || score_id < 0 || score_id > 3) {
+    set_error("sga_branch_score_f64: bad argument (score_id=%d)", score_id);
+    return SGA_ERR_ARG;
+  }
+  const bool need_g = score_id != SGA_SCORE_ABS_M, need_m = score_id != SGA_SCORE_ABS_G;
+  const bool need_wv = score_id == SGA_SCORE_UPDATE || score_id == SGA_SCORE_COI;
+  if ((need_g && !g) || (need_m && !m) || (need_wv && (!w || (!adams && !v)))) {
+    set_error("sga_branch_score_f64: missing input tensor for score %d", score_id);
+    return SGA_ERR_ARG;
+  }
+  if (adams) { bc1 = 1.0; bc2 = 1.0; }
+  const BranchK c{beta1, 1.0 - beta1, beta2, 1.0 - beta2, eps, wd, bc1, bc2};
+  const bool vec = aligned4(w, 4) && aligned4(m, 4) && aligned4(v, 4) && aligned4(g, 4) &&
+                   aligned4(out, 4);
+  dim3 grid(stream_grid(n, (int64_t)kBlock * kVec)), block(kBlock);
+  hipStream_t st = (hipStream_t)stream;
+#define SGA_BS(S) hipLaunchKernelGGL((k_branch_score<S>), grid, block, 0, st, w, m, v, g, out, n, c, adams != 0, include_wd != 0, vec)
+  switch (score_id) {
+    case 0: SGA_BS(0); break;
+    case 1: SGA_BS(1); break;
+    case 2: SGA_BS(2); break;
+    default: SGA_BS(3); break;
+  }
+#undef SGA_BS
+  return check_launch("sga_branch_score_f64");
 }
 
 extern "C" int sga_opt_step_inplace(const float* q, float* m, float* v, float* w, float* lab,

@@ -233,6 +233,71 @@ __global__ __launch_bounds__(kBlock) void k_replay_pass3(const void* __restrict_
   }
 }
 
+// ------------------------------------------------------- dense reference step
+// One commit of the recorded (post-clip) gradient on the dense trajectory,
+// with the per-coordinate label lab += (lr*upd)^2 and the pre-clip
+// reconstruction sum((q / coef_dense)^2) in double.
+template <bool BF16G, bool FULL>
+__device__ __forceinline__ double dense_vec(const void* g, int64_t i, int64_t n, float* w,
+                                            float* m, float* v, float* lab, int adams,
+                                            double coef_dense, RSegCursor& sc, bool vec) {
+  float q[4], mm[4], vv[4] = {0, 0, 0, 0}, ww[4], ll[4] = {0, 0, 0, 0};
+  if (BF16G) ld_bf16<FULL>(reinterpret_cast<const uint16_t*>(g), i, n, q, vec);
+  else ld_f32<FULL>(reinterpret_cast<const float*>(g), i, n, q, vec);
+  ld_f32<FULL>(m, i, n, mm, vec);
+  if (!adams) ld_f32<FULL>(v, i, n, vv, vec);
+  ld_f32<FULL>(w, i, n, ww, vec);
+  if (lab) ld_f32<FULL>(lab, i, n, ll, vec);
+  double acc = 0.0;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    if (!FULL && i + e >= n) continue;
+    sc.seek(i + e);
+    const float bc1 = adams ? 1.0f : sc.s.bc1, bc2 = adams ? 1.0f : sc.s.bc2;
+    const float vb = adams ? (mm[e] * mm[e]) * sc.s.b2 : vv[e] * sc.s.b2;
+    const float vn = __fmaf_rn(q[e] * sc.s.om2, q[e], vb);
+    const float mn = __fmaf_rn(q[e], sc.s.om1, mm[e] * sc.s.b1);
+    const float mh = __fdiv_rn(mn, bc1);
+    const float vh = __fsqrt_rn(__fdiv_rn(vn, bc2));
+    const float upd = __fdiv_rn(mh, vh + sc.s.eps);
+    ww[e] = __fmaf_rn(upd, sc.neglr, ww[e] * sc.omlwd);
+    ll[e] = __fmaf_rn(upd * (float)(sc.s.lr * sc.s.lr), upd, ll[e]);
+    mm[e] = mn;
+    vv[e] = vn;
+    const double qd = (double)q[e] / coef_dense;
+    acc += qd * qd;
+  }
+  st_f32<FULL>(m, i, n, mm, vec);
+  st_f32<FULL>(v, i, n, vv, vec);
+  st_f32<FULL>(w, i, n, ww, vec);
+  if (lab) st_f32<FULL>(lab, i, n, ll, vec);
+  return acc;
+}
+
+template <bool BF16G>
+__global__ __launch_bounds__(kBlock) void k_dense_step(const void* __restrict__ g, int64_t n,
+                                                       float* w, float* m, float* v, float* lab,
+                                                       int adams, double coef_dense,
+                                                       const RSeg* __restrict__ segs, int n_segs,
+                                                       double* __restrict__ partials, bool vec) {
+  __shared__ double s_w[kChunksPerBlock];
+  RSegCursor sc;
+  sc.init(segs, n_segs);
+  double acc = 0.0;
+  const int64_t stride = (int64_t)gridDim.x * kBlock * kVec;
+  for (int64_t base = (int64_t)blockIdx.x * kBlock * kVec; base < n; base += stride) {
+    const int64_t i = base + (int64_t)threadIdx.x * kVec;
+    if (vec && base + kBlock * kVec <= n)
+      acc += dense_vec<BF16G, true>(g, i, n, w, m, v, lab, adams, coef_dense, sc, true);
+    else if (i < n)
+      acc += dense_vec<BF16G, false>(g, i, n, w, m, v, lab, adams, coef_dense, sc, vec);
+  }
+  acc = wave_sum(acc);
+  if (lane_id() == 0) s_w[wave_id()] = acc;
+  __syncthreads();
+  if (threadIdx.x == 0) partials[blockIdx.x] = s_w[0] + s_w[1] + s_w[2] + s_w[3];
+}
+
 // --------------------------------------------------- pass 2 score source
 // key = |registry score| of q = (gd + res) * coef against one config's state.
 template <bool BF16G, int SCORE>
@@ -441,6 +506,27 @@ extern "C" int sga_replay_reselect(const void* g, int g_dtype, const float* res,
     switch (score_id) { case 0: SGA_RS(false, 0); case 1: SGA_RS(false, 1); case 2: SGA_RS(false, 2); default: SGA_RS(false, 3); }
   }
 #undef SGA_RS
+}
+
+extern "C" int sga_dense_replay_step(const void* g, int g_dtype, float* w, float* m, float* v,
+                                     float* lab, int64_t n, const sga_replay_segment* segs,
+                                     int n_segs, int adams, double coef_dense, double* partials,
+                                     double* recon2, void* stream) {
+  if (!g || !w || !m || !v || !segs || !partials || !recon2 || n < 1 || n_segs < 1 ||
+      !(coef_dense > 0.0) || (g_dtype != SGA_F32 && g_dtype != SGA_BF16)) {
+    set_error("sga_dense_replay_step: bad argument");
+    return SGA_ERR_ARG;
+  }
+  const bool bg = g_dtype == SGA_BF16;
+  const bool vec = aligned4(g, bg ? 2 : 4) && aligned4(w, 4) && aligned4(m, 4) && aligned4(v, 4) &&
+                   aligned4(lab, 4);
+  const unsigned nb = stream_grid(n, (int64_t)kBlock * kVec, kReplayBlocks);
+  hipStream_t s = (hipStream_t)stream;
+  const RSeg* rs = reinterpret_cast<const RSeg*>(segs);
+  if (bg) hipLaunchKernelGGL((k_dense_step<true>), dim3(nb), dim3(kBlock), 0, s, g, n, w, m, v, lab, adams, coef_dense, rs, n_segs, partials, vec);
+  else hipLaunchKernelGGL((k_dense_step<false>), dim3(nb), dim3(kBlock), 0, s, g, n, w, m, v, lab, adams, coef_dense, rs, n_segs, partials, vec);
+  hipLaunchKernelGGL(k_sqdist_stage2, dim3(1), dim3(kWave), 0, s, partials, (int)nb, recon2);
+  return check_launch("sga_dense_replay_step");
 }
 
 extern "C" int sga_div_inplace(float* x, int64_t n, float d, void* stream) {
