@@ -200,6 +200,20 @@ def main():
         calib = {"kernel": "k_calib_copy", "bytes": cn * 8, "avg_ms": ms,
                  "GBps": cn * 8 / ms / 1e6}
         del src, dst
+        # the final sweep's own mix of streams without its math, on scratch arrays
+        sg = torch.zeros(n, dtype=torch.bfloat16, device=dev)
+        sc = [torch.zeros(n, device=dev) for _ in range(4)]
+        sargs = [L.ptr(sg)] + [L.ptr(t) for t in sc] + [n, L.stream()]
+        L.call("sga_calib_streams", *sargs)
+        ev[0].record()
+        for _ in range(5):
+            L.call("sga_calib_streams", *sargs)
+        ev[1].record()
+        torch.cuda.synchronize()
+        ms = ev[0].elapsed_time(ev[1]) / 5
+        calib["streams"] = {"kernel": "k_calib_streams", "bytes": n * 34, "avg_ms": ms,
+                            "GBps": n * 34 / ms / 1e6}
+        del sg, sc
     run(args.warmup, 0, args.ratio, args.score)
     torch.cuda.synchronize()
     L.raw("sga_prof_enable", 1)

@@ -362,6 +362,13 @@ int sga_prof_enable(int on);
 /* dst[0..n) = src[0..n), fp32, n % 4 == 0: plain copy of known size used to
  * calibrate the HBM traffic counters (no counterpart in the reference). */
 int sga_calib_copy(float* dst, const float* src, int64_t n, void* stream);
+
+/* Math-free kernel with the fused final sweep's stream structure (reads bf16
+ * g and fp32 r/p/m/v, rewrites r/p/m/v: 34 B per element), to measure what that
+ * mix of streams reaches on the device (no counterpart in the reference).
+ * Overwrites r/p/m/v with meaningless values: use scratch buffers. */
+int sga_calib_streams(const void* g_bf16, float* r, float* p, float* m, float* v,
+                      int64_t n, void* stream);
 int sga_prof_read(double* total_ms, int* launches);
 
 #ifdef __cplusplus

@@ -77,6 +77,7 @@ SIGNATURES = {
     "sga_div_inplace": (I32, [P, I64, F, P]),
     "sga_sq_dist": (I32, [P, P, I64, P, P, P]),
     "sga_calib_copy": (I32, [P, P, I64, P]),
+    "sga_calib_streams": (I32, [P, P, P, P, P, I64, P]),
     "sga_prof_enable": (I32, [I32]),
     "sga_prof_read": (I32, [P, P]),
     "sga_fused_workspace_bytes": (SZ, [I64]),

@@ -472,11 +472,8 @@ static int run_reselect(const void* g, const float* res, const float* w, const f
                    aligned4(m, 4) && aligned4(v, 4);
   SrcReplay<BF16G, SCORE> src{g, res, w, m, v, coef_f, coef_dense, adams, vec, {}};
   src.sc.init(segs, n_segs);
-  run_select(src, n, k, 0, true, ws, s);
-  const int64_t nc = cdiv64(n, kChunk);
-  hipLaunchKernelGGL((k_write_mask<SrcReplay<BF16G, SCORE>>), dim3(stream_grid(nc, kChunksPerBlock, 1 << 20)),
-                     dim3(kBlock), 0, s, src, n, (int64_t)0, 0, ws.st, ws.tile_gt, ws.tile_eq, sel_out,
-                     aligned4(sel_out, 1));
+  run_select(src, n, k, 0, true, ws, s, true);
+  finish_mask(src, n, 0, ws, sel_out, s);
   if (result) hipLaunchKernelGGL(k_sel_result, dim3(1), dim3(1), 0, s, ws.st, result);
   return check_launch("sga_replay_reselect");
 }

@@ -268,11 +268,8 @@ extern "C" int sga_select_topk(const float* score, int64_t n, int64_t k, int tie
   hipStream_t s = (hipStream_t)stream;
   SrcF32 src{score, aligned4(score, 4)};
   const int tie_all = tie_mode == SGA_TIE_ALL;
-  run_select(src, n, k, tie_all, true, w, s);
-  const int64_t nc = cdiv64(n, kChunk);
-  hipLaunchKernelGGL((k_write_mask<SrcF32>), dim3(stream_grid(nc, kChunksPerBlock)), dim3(kBlock), 0,
-                     s, src, n, (int64_t)0, tie_all, w.st, w.tile_gt, w.tile_eq, mask_out,
-                     aligned4(mask_out, 1));
+  run_select(src, n, k, tie_all, true, w, s, true);
+  finish_mask(src, n, tie_all, w, mask_out, s);
   if (result) hipLaunchKernelGGL(k_sel_result, dim3(1), dim3(1), 0, s, w.st, result);
   return check_launch("sga_select_topk");
 }

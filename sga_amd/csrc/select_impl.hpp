@@ -61,6 +61,7 @@ struct SelWorkspace {
   uint32_t* seg_key;
   uint32_t* cand_idx;  // dense candidates
   uint32_t* cand_key;
+  uint32_t* pbits;     // 32 words per chunk: bit planes of "key above the bracket"
   int64_t sample_cap;
   int64_t seg_cap;     // per-wave candidate capacity
 };
@@ -95,7 +96,7 @@ static inline size_t fast_bytes_for_tiles(int64_t nt) {
   if (n < kFastMinN) return 0;
   const int64_t sc = fast_seg_cap(n);
   return (size_t)fast_sample_vecs(n) * 16 + (size_t)(kSegWaves + 64) * 4 +
-         (size_t)kSegWaves * sc * 4 * 4 + 256;
+         (size_t)kSegWaves * sc * 4 * 4 + (size_t)nt * 128 + 256;
 }
 
 static inline size_t sel_ws_bytes(int64_t n) {
@@ -133,6 +134,8 @@ static inline bool sel_ws_carve(void* ws, size_t bytes, int64_t n_tiles_needed,
   p += (size_t)nt * 4;
   out->n_tiles_cap = nt;
   out->sample = nullptr;
+  out->seg_cnt = out->seg_idx = out->seg_key = out->cand_idx = out->cand_key = nullptr;
+  out->pbits = nullptr;
   out->sample_cap = 0;
   out->seg_cap = 0;
   if (fast_bytes_for_tiles(nt) > 0) {
@@ -148,7 +151,8 @@ static inline bool sel_ws_carve(void* ws, size_t bytes, int64_t n_tiles_needed,
     out->seg_idx = reinterpret_cast<uint32_t*>(p); p += seg_bytes;
     out->seg_key = reinterpret_cast<uint32_t*>(p); p += seg_bytes;
     out->cand_idx = reinterpret_cast<uint32_t*>(p); p += seg_bytes;
-    out->cand_key = reinterpret_cast<uint32_t*>(p);
+    out->cand_key = reinterpret_cast<uint32_t*>(p); p += seg_bytes;
+    out->pbits = reinterpret_cast<uint32_t*>(p);
   }
   return true;
 }
@@ -587,7 +591,9 @@ __global__ __launch_bounds__(kBlock) void k_write_mask(Src src, int64_t n, int64
                                                        const SelState* __restrict__ st,
                                                        const uint32_t* __restrict__ tile_sel,
                                                        const uint32_t* __restrict__ tile_eq,
-                                                       uint8_t* __restrict__ mask, bool mvec) {
+                                                       uint8_t* __restrict__ mask, bool mvec,
+                                                       int unless_settled = 0) {
+  if (unless_settled && st->bracket_ok) return;
   const uint32_t T = st->thresh_bits;
   const uint32_t need = tie_all ? 0xFFFFFFFFu : st->need;
   const int64_t n_chunks = cdiv64(n, kChunk);
@@ -729,29 +735,45 @@ static __global__ void k_bracket_ranks(SelState* aux, uint32_t* hist, int nhist,
 // The one sweep over the data.  A persistent grid of kSegWaves waves; each
 // wave owns a private candidate segment, so no atomics are needed and the
 // candidates of a chunk stay in ascending index order.
-template <class Src, bool FULL>
+template <class Src, bool FULL, bool PM>
 __device__ __forceinline__ void bracket_chunk(Src& src, int64_t n, int64_t c, uint32_t T_LO,
                                               uint32_t T_HI, uint32_t& chi, uint32_t& tot_nf,
                                               uint32_t& mycnt, uint32_t seg_cap,
                                               uint32_t* __restrict__ my_idx,
-                                              uint32_t* __restrict__ my_key) {
+                                              uint32_t* __restrict__ my_key,
+                                              uint32_t* __restrict__ pbits) {
   // one 256-element slab at a time: keeps the register footprint of
   // expensive key sources (Adam-normalised scores) small enough for full
   // occupancy; slabs of different waves overlap their loads
+  uint32_t pword = 0u;
 #pragma unroll
   for (int it = 0; it < kChunkIters; ++it) {
     const int64_t i = c * kChunk + it * (kWave * kVec) + lane_id() * kVec;
     uint32_t key[4] = {0u, 0u, 0u, 0u};
     if (FULL || i < n) src.template load<FULL>(i, n, key);
     bool cand[4];
-    uint32_t mine = 0;
+    uint32_t mine = 0, above[4];
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
       const bool valid = FULL || i + e < n;
-      chi += (valid && key[e] >= T_HI);
+      above[e] = (valid && key[e] >= T_HI);
+      chi += above[e];
       tot_nf += (valid && key[e] >= 0x7F800000u);
       cand[e] = valid && key[e] >= T_LO && key[e] < T_HI;
       mine += cand[e];
+    }
+    if (PM) {
+      // provisional mask as bit planes: everything above the bracket is
+      // certainly selected; the few keys inside it are settled after the
+      // candidate descent.  Lane 8*it + 2e + h keeps the word with lanes
+      // [32h, 32h+32) of element e of slab `it`; one 128-byte store per chunk.
+      const uint64_t b0 = ballot64(above[0]), b1 = ballot64(above[1]);
+      const uint64_t b2 = ballot64(above[2]), b3 = ballot64(above[3]);
+      const int l = lane_id();
+      if ((l >> 3) == it) {
+        const uint64_t bb = (l & 4) ? ((l & 2) ? b3 : b2) : ((l & 2) ? b1 : b0);
+        pword = (l & 1) ? (uint32_t)(bb >> 32) : (uint32_t)bb;
+      }
     }
     if (ballot64(mine != 0)) {
       const uint32_t incl = wave_incl_scan(mine);
@@ -765,13 +787,15 @@ __device__ __forceinline__ void bracket_chunk(Src& src, int64_t n, int64_t c, ui
       mycnt += __shfl(incl, kWave - 1, kWave);
     }
   }
+  if (PM && lane_id() < 32) pbits[c * 32 + lane_id()] = pword;
 }
 
-template <class Src>
+template <class Src, bool PM>
 __global__ __launch_bounds__(kBlock) void k_bracket_sweep(
     Src src, int64_t n, SelState* __restrict__ st, const SelState* __restrict__ aux,
     uint32_t* __restrict__ tile_gt, uint32_t* __restrict__ tile_eq, uint32_t* __restrict__ seg_idx,
-    uint32_t* __restrict__ seg_key, uint32_t* __restrict__ seg_cnt, uint32_t seg_cap) {
+    uint32_t* __restrict__ seg_key, uint32_t* __restrict__ seg_cnt, uint32_t seg_cap,
+    uint32_t* __restrict__ pbits) {
   __shared__ uint32_t s_hi[kChunksPerBlock], s_nf[kChunksPerBlock];
   // keys equal to the upper sample key stay candidates; a skipped end means
   // the bracket is open on that side
@@ -787,9 +811,9 @@ __global__ __launch_bounds__(kBlock) void k_bracket_sweep(
   for (int64_t c = gw; c < n_chunks; c += W) {
     uint32_t chi = 0;
     if (src.vec && (c + 1) * kChunk <= n)
-      bracket_chunk<Src, true>(src, n, c, T_LO, T_HI, chi, tot_nf, mycnt, seg_cap, my_idx, my_key);
+      bracket_chunk<Src, true, PM>(src, n, c, T_LO, T_HI, chi, tot_nf, mycnt, seg_cap, my_idx, my_key, pbits);
     else
-      bracket_chunk<Src, false>(src, n, c, T_LO, T_HI, chi, tot_nf, mycnt, seg_cap, my_idx, my_key);
+      bracket_chunk<Src, false, PM>(src, n, c, T_LO, T_HI, chi, tot_nf, mycnt, seg_cap, my_idx, my_key, pbits);
     chi = wave_sum(chi);
     tot_hi += chi;
     if (lane_id() == 0) { tile_gt[c] = chi; tile_eq[c] = 0u; }
@@ -887,12 +911,101 @@ static __global__ __launch_bounds__(kBlock) void k_cand_tiles(
 }
 static_assert(kChunk == 1024, "candidate -> chunk mapping uses idx >> 10");
 
-// Full select up to (and including) the tile scan: afterwards st holds the
-// threshold / need and tile_gt / tile_eq hold, per chunk, the number of
-// selected coordinates and of ties before it.
+// Bit planes of the bracket sweep -> mask bytes (keys above the bracket).
+// Each lane expands 16 consecutive bytes: 4 lanes x 4 elements of one slab.
+static __global__ __launch_bounds__(kBlock) void k_expand_mask(
+    const SelState* __restrict__ st, const uint32_t* __restrict__ pbits, int64_t n,
+    uint8_t* __restrict__ mask, bool mvec) {
+  if (!st->bracket_ok) return;
+  const int64_t n_chunks = cdiv64(n, kChunk);
+  const int64_t wstride = (int64_t)gridDim.x * kChunksPerBlock;
+  const int l = lane_id();
+  const int it = l >> 4, sl0 = (l & 15) * 4;        // slab, first slab-lane
+  for (int64_t c = (int64_t)blockIdx.x * kChunksPerBlock + wave_id(); c < n_chunks; c += wstride) {
+    const U4* pw = reinterpret_cast<const U4*>(pbits + c * 32 + it * 8);
+    const U4 lo = pw[0], hi = pw[1];
+    const uint32_t w[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+    uint32_t out[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {                   // slab-lane sl0 + j -> 4 bytes
+      const int sl = sl0 + j;
+      uint32_t v = 0;
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        v |= (((sl < 32 ? w[2 * e] : w[2 * e + 1]) >> (sl & 31)) & 1u) << (8 * e);
+      out[j] = v;
+    }
+    const int64_t i = c * kChunk + (int64_t)l * 16;
+    if (mvec && i + 16 <= n) {
+      *reinterpret_cast<U4*>(mask + i) = U4{out[0], out[1], out[2], out[3]};
+    } else {
+      for (int b = 0; b < 16; ++b)
+        if (i + b < n) mask[i + b] = (uint8_t)((out[b >> 2] >> (8 * (b & 3))) & 1u);
+    }
+  }
+}
+
+// Settles the bracket's candidates in the expanded mask: keys above the
+// threshold are selected; of the ties, the first `need` by index.  After the
+// tile scan tile_eq[c] counts the ties before chunk c, so only the one chunk
+// where the quota runs out has to rank its ties (a chunk's candidates are
+// contiguous and index-ordered in the list).
+static __global__ __launch_bounds__(kBlock) void k_cand_mask(
+    const SelState* __restrict__ st, const uint32_t* __restrict__ cand_idx,
+    const uint32_t* __restrict__ cand_key, const uint32_t* __restrict__ tile_eq,
+    int64_t n_tiles, int tie_all, uint8_t* __restrict__ mask) {
+  if (!st->bracket_ok) return;
+  const uint32_t T = st->thresh_bits, nc = st->cand_count, n_eq = st->n_eq;
+  const uint32_t need = tie_all ? 0xFFFFFFFFu : st->need;
+  for (uint32_t j = blockIdx.x * kBlock + threadIdx.x; j < nc; j += gridDim.x * kBlock) {
+    const uint32_t key = cand_key[j];
+    if (key < T) continue;
+    const uint32_t idx = cand_idx[j];
+    bool on = true;
+    if (key == T && need < n_eq) {
+      const uint32_t c = idx >> 10;
+      const uint32_t before = tile_eq[c];
+      const uint32_t upto = (int64_t)c + 1 < n_tiles ? tile_eq[c + 1] : n_eq;
+      if (before >= need) {
+        on = false;
+      } else if (upto > need) {            // the quota ends inside this chunk
+        uint32_t rank = before;
+        for (uint32_t q = j; q > 0 && (cand_idx[q - 1] >> 10) == c; --q)
+          rank += cand_key[q - 1] == T;
+        on = rank < need;
+      }
+    }
+    if (on) mask[idx] = 1;
+  }
+}
+
+// Persistent grid of the bracket sweep = exactly what the device holds at
+// once for THIS instantiation (a partial second round would idle most of the
+// chip).
+template <class Src, bool PM>
+static inline int sweep_grid() {
+  static int blocks = 0;
+  if (blocks == 0) {
+    int per_cu = 0, dev = 0;
+    hipDeviceProp_t prop;
+    if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess &&
+        hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, k_bracket_sweep<Src, PM>, kBlock, 0) ==
+            hipSuccess && per_cu > 0) {
+      blocks = per_cu * prop.multiProcessorCount;
+    } else {
+      blocks = 1024;
+    }
+    if (blocks > kSegWaves / kChunksPerBlock) blocks = kSegWaves / kChunksPerBlock;
+  }
+  return blocks;
+}
+
+// want_mask: the sweep also records, as bit planes, which keys lie above the
+// bracket, so a caller that only wants the mask can finish from those bits
+// and the candidates (finish_mask) instead of re-reading the data.
 template <class Src>
 static inline void run_select(Src src, int64_t n, int64_t k, int tie_all, bool fast,
-                              const SelWorkspace& w, hipStream_t s) {
+                              const SelWorkspace& w, hipStream_t s, bool want_mask = false) {
   const int64_t n_tiles = cdiv64(n, kChunk);
   launch_begin((uint32_t)k, w, s);
   if (fast && n >= kFastMinN && w.sample && n < (1ll << 32)) {
@@ -910,24 +1023,15 @@ static inline void run_select(Src src, int64_t n, int64_t k, int tie_all, bool f
       // <= 1M keys: 64 fat workgroups keep the histogram flush (one atomic per
       // non-empty bin per workgroup) far below one atomic per key
       launch_level<SrcU32, 2, true>(ssrc, ns, (const uint32_t*)nullptr, level, w.aux, w, s, 64);
-    // persistent grid = exactly what the device holds at once for THIS
-    // instantiation (a partial second round would idle most of the chip)
-    static int sweep_blocks = 0;
-    if (sweep_blocks == 0) {
-      int per_cu = 0, dev = 0;
-      hipDeviceProp_t prop;
-      if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess &&
-          hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, k_bracket_sweep<Src>, kBlock, 0) ==
-              hipSuccess && per_cu > 0) {
-        sweep_blocks = per_cu * prop.multiProcessorCount;
-      } else {
-        sweep_blocks = 1024;
-      }
-      if (sweep_blocks > kSegWaves / kChunksPerBlock) sweep_blocks = kSegWaves / kChunksPerBlock;
-    }
-    hipLaunchKernelGGL((k_bracket_sweep<Src>), dim3(sweep_blocks), dim3(kBlock), 0, s,
-                       src, n, w.st, w.aux, w.tile_gt, w.tile_eq, w.seg_idx, w.seg_key, w.seg_cnt,
-                       (uint32_t)w.seg_cap);
+    const int sweep_blocks = want_mask ? sweep_grid<Src, true>() : sweep_grid<Src, false>();
+    if (want_mask)
+      hipLaunchKernelGGL((k_bracket_sweep<Src, true>), dim3(sweep_blocks), dim3(kBlock), 0, s,
+                         src, n, w.st, w.aux, w.tile_gt, w.tile_eq, w.seg_idx, w.seg_key, w.seg_cnt,
+                         (uint32_t)w.seg_cap, w.pbits);
+    else
+      hipLaunchKernelGGL((k_bracket_sweep<Src, false>), dim3(sweep_blocks), dim3(kBlock), 0, s,
+                         src, n, w.st, w.aux, w.tile_gt, w.tile_eq, w.seg_idx, w.seg_key, w.seg_cnt,
+                         (uint32_t)w.seg_cap, (uint32_t*)nullptr);
     hipLaunchKernelGGL(k_bracket_check, dim3(1), dim3(kBlock), 0, s, w.st, w.aux, w.seg_cnt, w.hist,
                        kHistStride * 2, sweep_blocks * kChunksPerBlock);
     hipLaunchKernelGGL(k_cand_compact, dim3(256), dim3(kBlock), 0, s, w.aux, w.seg_cnt, w.seg_idx,
@@ -947,6 +1051,24 @@ static inline void run_select(Src src, int64_t n, int64_t k, int tie_all, bool f
     launch_level<Src, 1, true>(src, n, (const uint32_t*)nullptr, level, w.st, w, s);
   launch_tile_count(src, n, 0, w, s);
   launch_tile_scan(n_tiles, tie_all, w, s);
+}
+
+// Mask of the selection after run_select(..., want_mask = true): the bit
+// planes and the candidates settle it when the bracket held, else the
+// ordered full pass writes it.
+template <class Src>
+static inline void finish_mask(Src src, int64_t n, int tie_all, const SelWorkspace& w,
+                               uint8_t* mask, hipStream_t s) {
+  const int64_t nc = cdiv64(n, kChunk);
+  if (w.pbits && n >= kFastMinN && n < (1ll << 32)) {
+    hipLaunchKernelGGL(k_expand_mask, dim3(stream_grid(nc, kChunksPerBlock, 1 << 14)), dim3(kBlock),
+                       0, s, w.st, w.pbits, n, mask, (reinterpret_cast<uintptr_t>(mask) & 15) == 0);
+    hipLaunchKernelGGL(k_cand_mask, dim3(256), dim3(kBlock), 0, s, w.st, w.cand_idx, w.cand_key,
+                       w.tile_eq, nc, tie_all, mask);
+  }
+  hipLaunchKernelGGL((k_write_mask<Src>), dim3(stream_grid(nc, kChunksPerBlock, 1 << 14)),
+                     dim3(kBlock), 0, s, src, n, (int64_t)0, tie_all, w.st, w.tile_gt, w.tile_eq,
+                     mask, aligned4(mask, 1), 1);
 }
 
 #endif  // __HIPCC__

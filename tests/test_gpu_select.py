@@ -180,6 +180,30 @@ def test_sampled_bracket_path_and_fallback(dev):
     assert ("all-equal", 0) in seen
 
 
+def test_bracket_path_partial_ties(dev):
+    """bf16-quantised magnitudes: the k-th value sits on a plateau of ties of
+    which only the first few (by index) are selected, while the sampled
+    bracket still holds -- the mask is settled from the sweep's bit planes
+    and the candidate list."""
+    from sga_amd import _lib as L
+    from sga_amd.selection import read_result, select_exact_device
+    n = (1 << 22) + 4321
+    sc = student_t(n, 3).abs().to(torch.bfloat16).float()
+    sd = sc.to(dev)
+    partial = 0
+    for k in (n // 1000, n // 100, n // 100 + 17, n // 10, n // 10 + 5, n // 3):
+        m_ref, t_ref = SEL.select_topk_flat(sc, k)
+        mask = torch.full((n,), 7, dtype=torch.uint8, device=dev)
+        res, _ = select_exact_device([sd], k, L.TIE_LOWEST_INDEX, masks=[mask])
+        r = read_result(res)
+        assert r.status == 0 and r.n_selected == k and r.thresh == t_ref, (k, vars(r))
+        assert torch.equal(mask.cpu().bool(), m_ref) and int(mask.max()) == 1, k
+        partial += int(r.path == 1 and r.need < r.n_eq)
+        res2, (m2,) = select_exact_device([sd], k, L.TIE_ALL)
+        assert torch.equal(m2.cpu().bool(), sc >= t_ref), k
+    assert partial >= 3
+
+
 @pytest.mark.parametrize("x,reduce", [(4, "max"), (64, "max"), (1024, "max"), (8, "mean")])
 def test_block_granular_selection(dev, x, reduce):
     from sga_amd.selection import HistogramSelect, block_reduce_views
