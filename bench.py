@@ -124,7 +124,7 @@ def replay_bench(G=8, W=32, seed=4):
             alg += (32.0 if bnd else 33.0) * n               # pass 3: res, m, v, w r/w (+ sel)
             if bnd and s > 0 and s + 1 < W:
                 per = 6.0 if c.score == "abs_g" else 18.0    # g, res (+ w, m, v)
-                alg += (2 * per + 1.0) * n                   # bracket sweep + mask sweep + mask
+                alg += (per + 1.0) * n                       # one score sweep + the new mask
                 n_resel += 1
     return {"metric": "replay config-steps/s", "value": G * W / dt, "unit": "config-steps/s",
             "ms_per_window": dt * 1e3, "G": G, "W": W, "n": n, "reselects": n_resel,

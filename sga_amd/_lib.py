@@ -152,3 +152,35 @@ def dtype_code(t):
     if t.dtype == torch.bfloat16:
         return SGA_BF16
     raise TypeError(f"unsupported dtype {t.dtype} (fp32 or bf16)")
+
+
+class TableUploader:
+    """Ships small per-step parameter tables (ctypes struct arrays) to one
+    device buffer without stalling the host: the bytes go through a ring of
+    pinned staging buffers and an asynchronous copy on the current stream, so
+    the copy is ordered after the kernels that still read the previous table
+    and before the ones launched next."""
+
+    def __init__(self, nbytes, device, slots=4):
+        import torch
+        self.nbytes = int(nbytes)
+        self.dev = torch.empty(self.nbytes, dtype=torch.uint8, device=device)
+        self._host = [torch.empty(self.nbytes, dtype=torch.uint8, pin_memory=True)
+                      for _ in range(slots)]
+        self._done = [None] * slots
+        self._i = 0
+
+    def upload(self, struct_array):
+        import torch
+        if C.sizeof(struct_array) != self.nbytes:
+            raise ValueError("table size changed")
+        slot = self._i % len(self._host)
+        self._i += 1
+        if self._done[slot] is not None:
+            self._done[slot].synchronize()
+        C.memmove(self._host[slot].data_ptr(), C.addressof(struct_array), self.nbytes)
+        self.dev.copy_(self._host[slot], non_blocking=True)
+        ev = torch.cuda.Event()
+        ev.record()
+        self._done[slot] = ev
+        return self.dev

@@ -51,14 +51,23 @@ __device__ __forceinline__ void load_gd(const void* g, int64_t i, int64_t n, flo
 }
 
 // ------------------------------------------------------------------ pass 1
-template <bool BF16G>
+// Two launches per step, each with its config count as a template argument
+// so the per-config loads are unrolled and all in flight together: one over
+// the configs at a cycle boundary (q = gd + res), one over the others
+// (q = gd * sel).  Both write their configs' slots of the same partials table.
+struct P1List {
+  const void* ptr[kMaxCfg];   // res (boundary list) or sel (masked list)
+  int slot[kMaxCfg];          // config index of each entry
+};
+
+template <bool BF16G, bool BOUNDARY, int NC>
 __global__ __launch_bounds__(kBlock) void k_replay_pass1(const void* __restrict__ g, int64_t n,
-                                                         float coef_dense, RGroup grp,
+                                                         float coef_dense, P1List lst,
                                                          double* __restrict__ partials, bool vec) {
-  __shared__ double s_w[kChunksPerBlock][kMaxCfg];
-  double acc[kMaxCfg];
+  __shared__ double s_w[kChunksPerBlock][NC];
+  double acc[NC];
 #pragma unroll
-  for (int c = 0; c < kMaxCfg; ++c) acc[c] = 0.0;
+  for (int c = 0; c < NC; ++c) acc[c] = 0.0;
   const float is_one = coef_dense == 1.0f ? 1.0f : 0.0f;
   const int64_t stride = (int64_t)gridDim.x * kBlock * kVec;
   for (int64_t base = (int64_t)blockIdx.x * kBlock * kVec; base < n; base += stride) {
@@ -68,38 +77,49 @@ __global__ __launch_bounds__(kBlock) void k_replay_pass1(const void* __restrict_
     float gd[4];
     if (full) load_gd<BF16G, true>(g, i, n, is_one, coef_dense, gd, true);
     else load_gd<BF16G, false>(g, i, n, is_one, coef_dense, gd, vec);
+    if (BOUNDARY) {
+      float rr[NC][4];
 #pragma unroll
-    for (int c = 0; c < kMaxCfg; ++c) {
-      if (c >= grp.G) break;
-      float q[4];
-      if (grp.c[c].boundary) {
-        float rr[4];
-        if (full) ld_f32<true>(grp.c[c].res, i, n, rr, true);
-        else load4_f32(grp.c[c].res, i, n, rr, vec);
-#pragma unroll
-        for (int e = 0; e < 4; ++e) q[e] = gd[e] + rr[e];
-      } else {
-        uint32_t sl[4];
-        if (full) ld_u8<true>(grp.c[c].sel, i, n, sl, true);
-        else load4_u8(grp.c[c].sel, i, n, sl, vec);
-#pragma unroll
-        for (int e = 0; e < 4; ++e) q[e] = gd[e] * (sl[e] ? 1.0f : 0.0f);
+      for (int c = 0; c < NC; ++c) {
+        const float* rp = reinterpret_cast<const float*>(lst.ptr[c]);
+        if (full) ld_f32<true>(rp, i, n, rr[c], true);
+        else load4_f32(rp, i, n, rr[c], vec);
       }
 #pragma unroll
-      for (int e = 0; e < 4; ++e)
-        if (full || i + e < n) acc[c] += (double)(q[e] * q[e]);
+      for (int c = 0; c < NC; ++c)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const float q = gd[e] + rr[c][e];
+          if (full || i + e < n) acc[c] += (double)(q * q);
+        }
+    } else {
+      // q = gd * {0, 1}: q*q is gd*gd or 0, squared once for all configs
+      float gd2[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) gd2[e] = (full || i + e < n) ? gd[e] * gd[e] : 0.0f;
+      uint32_t sl[NC][4];
+#pragma unroll
+      for (int c = 0; c < NC; ++c) {
+        const uint8_t* sp = reinterpret_cast<const uint8_t*>(lst.ptr[c]);
+        if (full) ld_u8<true>(sp, i, n, sl[c], true);
+        else load4_u8(sp, i, n, sl[c], vec);
+      }
+#pragma unroll
+      for (int c = 0; c < NC; ++c)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc[c] += (double)(sl[c][e] ? gd2[e] : 0.0f);
     }
   }
 #pragma unroll
-  for (int c = 0; c < kMaxCfg; ++c) {
-    if (c >= grp.G) break;
+  for (int c = 0; c < NC; ++c) {
     const double t = wave_sum(acc[c]);
     if (lane_id() == 0) s_w[wave_id()][c] = t;
   }
   __syncthreads();
-  if (threadIdx.x < grp.G) {
+  if (threadIdx.x < NC) {
     const int c = threadIdx.x;
-    partials[(int64_t)blockIdx.x * kMaxCfg + c] = s_w[0][c] + s_w[1][c] + s_w[2][c] + s_w[3][c];
+    partials[(int64_t)blockIdx.x * kMaxCfg + lst.slot[c]] =
+        s_w[0][c] + s_w[1][c] + s_w[2][c] + s_w[3][c];
   }
 }
 
@@ -423,6 +443,29 @@ using namespace sga;
 
 static_assert(sizeof(RSeg) == sizeof(sga_replay_segment), "replay segment layout");
 
+template <bool BOUNDARY, bool BF16G, int NC>
+static void launch_pass1_n(unsigned nb, hipStream_t s, const void* g, int64_t n, float coef_dense,
+                           const P1List& lst, double* partials, bool vec) {
+  hipLaunchKernelGGL((k_replay_pass1<BF16G, BOUNDARY, NC>), dim3(nb), dim3(kBlock), 0, s, g, n,
+                     coef_dense, lst, partials, vec);
+}
+
+template <bool BOUNDARY>
+static void launch_pass1(bool bg, int count, unsigned nb, hipStream_t s, const void* g, int64_t n,
+                         float coef_dense, const P1List& lst, double* partials, bool vec) {
+#define SGA_P1(NC)                                                                             \
+  case NC:                                                                                     \
+    if (bg) launch_pass1_n<BOUNDARY, true, NC>(nb, s, g, n, coef_dense, lst, partials, vec);   \
+    else launch_pass1_n<BOUNDARY, false, NC>(nb, s, g, n, coef_dense, lst, partials, vec);     \
+    break;
+  switch (count) {
+    SGA_P1(1) SGA_P1(2) SGA_P1(3) SGA_P1(4) SGA_P1(5) SGA_P1(6) SGA_P1(7) SGA_P1(8)
+    SGA_P1(9) SGA_P1(10) SGA_P1(11) SGA_P1(12) SGA_P1(13) SGA_P1(14) SGA_P1(15) SGA_P1(16)
+    default: break;                       // no config of this kind at this step
+  }
+#undef SGA_P1
+}
+
 extern "C" int64_t sga_replay_partials(void) { return (int64_t)kReplayBlocks * kMaxCfg; }
 
 extern "C" int sga_replay_pass1(const void* g, int g_dtype, int64_t n, float coef_dense, double clip,
@@ -438,8 +481,14 @@ extern "C" int sga_replay_pass1(const void* g, int g_dtype, int64_t n, float coe
   const bool vec = aligned4(g, bg ? 2 : 4) && group_aligned(grp);
   const unsigned nb = stream_grid(n, (int64_t)kBlock * kVec, kReplayBlocks);
   hipStream_t s = (hipStream_t)stream;
-  if (bg) hipLaunchKernelGGL((k_replay_pass1<true>), dim3(nb), dim3(kBlock), 0, s, g, n, coef_dense, grp, partials, vec);
-  else hipLaunchKernelGGL((k_replay_pass1<false>), dim3(nb), dim3(kBlock), 0, s, g, n, coef_dense, grp, partials, vec);
+  P1List lb = {}, lm = {};
+  int n_b = 0, n_m = 0;
+  for (int c = 0; c < G; ++c) {
+    if (grp.c[c].boundary) { lb.ptr[n_b] = grp.c[c].res; lb.slot[n_b++] = c; }
+    else { lm.ptr[n_m] = grp.c[c].sel; lm.slot[n_m++] = c; }
+  }
+  launch_pass1<true>(bg, n_b, nb, s, g, n, coef_dense, lb, partials, vec);
+  launch_pass1<false>(bg, n_m, nb, s, g, n, coef_dense, lm, partials, vec);
   hipLaunchKernelGGL(k_replay_coef, dim3(1), dim3(kBlock), 0, s, partials, (int)nb, G, clip, qn2, coef_d, coef_f);
   return check_launch("sga_replay_pass1");
 }

@@ -44,24 +44,27 @@ class FusedSparseStep:
         self.mask = (torch.empty(n, dtype=torch.uint8, device=device)
                      if want_mask else None)
         self._seg_host = (L.Segment * len(segments))()
-        self._seg_dev = torch.empty(C.sizeof(self._seg_host), dtype=torch.uint8,
-                                    device=device)
-        self._seg_step = None
-
-    def _upload_segments(self, step):
-        if self._seg_step == step:
-            return
-        for i, s in enumerate(self.segments):
-            e = self._seg_host[i]
+        for e, s in zip(self._seg_host, segments):
             e.start, e.n = s["start"], s["n"]
             e.lr = L.f32(s["lr"])
             e.beta1, e.om1 = L.f32(s["b1"]), L.f32(1.0 - s["b1"])
             e.beta2, e.om2 = L.f32(s["b2"]), L.f32(1.0 - s["b2"])
             e.eps, e.wd = L.f32(s["eps"]), L.f32(s["wd"])
-            e.bc1 = L.f32(1.0 - s["b1"] ** step)
-            e.bc2 = L.f32(1.0 - s["b2"] ** step)
-        host = torch.frombuffer(bytearray(bytes(self._seg_host)), dtype=torch.uint8)
-        self._seg_dev.copy_(host)
+        self._seg_up = L.TableUploader(C.sizeof(self._seg_host), device)
+        self._seg_dev = self._seg_up.dev
+        self._seg_step = None
+
+    def _upload_segments(self, step):
+        if self._seg_step == step:
+            return
+        bc = {}
+        for e, s in zip(self._seg_host, self.segments):
+            key = (s["b1"], s["b2"])
+            if key not in bc:
+                bc[key] = (L.f32(1.0 - s["b1"] ** step), L.f32(1.0 - s["b2"] ** step))
+            e.lr = L.f32(s["lr"])                      # callers may retune lr between steps
+            e.bc1, e.bc2 = bc[key]
+        self._seg_up.upload(self._seg_host)
         self._seg_step = step
 
     def step(self, g, resid, p, m, v, step, k=None, ratio_percent=None,

@@ -47,7 +47,8 @@ class DenseReplay:
         self._recon2 = torch.zeros(1, dtype=torch.float64, device=dev)
         self._dist = torch.zeros(1, dtype=torch.float64, device=dev)
         self._seg_host = (ReplaySegment * len(entries))()
-        self._seg_dev = torch.empty(C.sizeof(self._seg_host), dtype=torch.uint8, device=dev)
+        self._seg_up = L.TableUploader(C.sizeof(self._seg_host), dev)
+        self._seg_dev = self._seg_up.dev
         self.si = 0
         self.den_at, self.snapshots, self.recon_steps = {}, {}, []
 
@@ -68,7 +69,7 @@ class DenseReplay:
             r.beta1, r.om1 = L.f32(e["b1"]), L.f32(1.0 - e["b1"])
             r.beta2, r.om2 = L.f32(e["b2"]), L.f32(1.0 - e["b2"])
             r.eps, r.wdf, r.bc1, r.bc2 = L.f32(e["eps"]), L.f32(e["wd"]), L.f32(bc1), L.f32(bc2)
-        _upload(self._seg_host, self._seg_dev)
+        _upload(self._seg_host, self._seg_up)
         st = L.stream()
         L.call("sga_dense_replay_step", L.ptr(g), L.dtype_code(g), L.ptr(self.w), L.ptr(self.m),
                L.ptr(self.v), L.ptr(self.label), self.N, L.ptr(self._seg_dev),

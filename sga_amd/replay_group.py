@@ -48,9 +48,8 @@ def coef_dense_for(clip_grad, grad_norm):
     return min(clip_grad / (grad_norm + 1.0e-6), 1.0)
 
 
-def _upload(struct_array, dev_buf):
-    host = torch.frombuffer(bytearray(bytes(struct_array)), dtype=torch.uint8)
-    dev_buf.copy_(host)
+def _upload(struct_array, uploader):
+    uploader.upload(struct_array)
 
 
 class ReplayGroup:
@@ -96,10 +95,11 @@ class ReplayGroup:
         self.sel_result = torch.zeros(8, dtype=torch.int32, device=dev)
         self._cfg_host = (ReplayCfg * G)()
         self._rseg_host = (ReplaySegment * len(entries))()
-        self._rseg_dev = torch.empty(C.sizeof(self._rseg_host), dtype=torch.uint8, device=dev)
+        self._rseg_up = L.TableUploader(C.sizeof(self._rseg_host), dev)
+        self._rseg_dev = self._rseg_up.dev
         self._seg_host = (L.Segment * len(entries))()
-        self._seg_dev = {o: torch.empty(C.sizeof(self._seg_host), dtype=torch.uint8, device=dev)
-                         for o in ("adamw", "adams")}
+        self._seg_up = L.TableUploader(C.sizeof(self._seg_host), dev)
+        self._seg_dev = {"adamw": self._seg_up.dev}
         self.dist_at = [dict() for _ in configs]
         self.si = 0
 
@@ -118,8 +118,8 @@ class ReplayGroup:
             s.start, s.n, s.lr = e["a"], e["n"], L.f32(lr_of(e))
             s.beta1, s.om1, s.beta2, s.om2 = r.beta1, r.om1, r.beta2, r.om2
             s.eps, s.wd, s.bc1, s.bc2 = r.eps, r.wdf, r.bc1, r.bc2
-        _upload(self._rseg_host, self._rseg_dev)
-        _upload(self._seg_host, self._seg_dev["adamw"])
+        _upload(self._rseg_host, self._rseg_up)
+        _upload(self._seg_host, self._seg_up)
 
     def _fill_cfgs(self, bnd, out_sel):
         for ci, c in enumerate(self.configs):
