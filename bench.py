@@ -147,6 +147,8 @@ def main():
                     help="also launch one plain copy of 2^30 fp32 (k_calib_copy) so counter "
                          "runs can be scaled against a kernel of known traffic")
     ap.add_argument("--no-replay", action="store_true", help="skip the fused replay leg")
+    ap.add_argument("--no-packed", action="store_true",
+                    help="skip the packed-state variant of the fused step")
     ap.add_argument("--only-replay", action="store_true",
                     help="run just the fused replay leg (for profiling) and print its JSON")
     ap.add_argument("--sweep", action="store_true",
@@ -259,6 +261,33 @@ def main():
                           "frac": value * ALG_BYTES_STEP / HBM_PEAK},
         "select": {"thresh": res.thresh, "n_gt": res.n_gt, "n_eq": res.n_eq, "path": res.path},
     }
+    if not args.no_packed:
+        # same workload with resid/p/m/v interleaved in 64 KiB records (the
+        # library-owned state layout); identical arithmetic and outputs
+        from sga_amd.fused_step import PackedState
+        st = PackedState(n, dev).pack(r, p, m, v)
+
+        def run_packed(steps, step0):
+            for s in range(steps):
+                fs.step_packed(grads[(step0 + s) % 2], st, step0 + s + 1, k=k, score=args.score)
+        step0 = args.warmup + args.steps
+        run_packed(args.warmup, step0)
+        torch.cuda.synchronize()
+        L.raw("sga_prof_enable", 1)
+        t1 = time.perf_counter()
+        run_packed(args.steps, step0 + args.warmup)
+        torch.cuda.synchronize()
+        dtp = time.perf_counter() - t1
+        L.call("sga_prof_read", ctypes.byref(tot_ms), ctypes.byref(cnt))
+        L.raw("sga_prof_enable", 0)
+        st.unpack(r, p, m, v)
+        del st
+        pms = tot_ms.value / max(cnt.value, 1)
+        out["packed_state"] = {
+            "layout": "resid/p/m/v interleaved, 64 KiB records (sga_fused_sparse_step_packed)",
+            "value": n * args.steps / dtp, "ms_per_step": dtp / args.steps * 1e3,
+            "step_frac": n * args.steps / dtp * ALG_BYTES_STEP / HBM_PEAK,
+            "final_avg_ms": pms, "final_frac": final_bytes / (pms * 1e-3) / HBM_PEAK}
     if calib:
         out["copy_calibration"] = calib
     if args.sweep:

@@ -278,6 +278,28 @@ int sga_fused_sparse_step(const void* g, int g_dtype, float* resid, float* p,
                           int fast, sga_select_result* result, void* ws,
                           size_t ws_bytes, void* stream);
 
+/* Packed-state variant of the fused step for callers that let the library
+ * lay out the optimizer-side state (no counterpart in the reference, whose
+ * buffers are separate tensors): resid, p, m, v are interleaved in 64 KiB
+ * records [resid[4096] | p[4096] | m[4096] | v[4096]], i.e. element i of
+ * array a (0 resid, 1 p, 2 m, 3 v) is state[(i >> 12) * 16384 + a * 4096 +
+ * (i & 4095)].  state holds sga_packed_state_elems(n) floats, 16-byte
+ * aligned.  Same arithmetic, same outputs as sga_fused_sparse_step; the four
+ * streams of a workgroup then always fall into different DRAM banks of one
+ * physical page, which the device rewards with higher streaming efficiency.
+ * sga_state_repack converts between the two layouts (unpack = 0: arrays ->
+ * state, 1: state -> arrays; a NULL array is skipped). */
+int64_t sga_packed_state_elems(int64_t n);
+int sga_fused_sparse_step_packed(const void* g, int g_dtype, float* state,
+                                 int64_t n, int64_t k, const sga_segment* segs,
+                                 int n_segs, int score_id, int32_t* idx_out,
+                                 void* values_out, int values_dtype,
+                                 uint8_t* mask_out, float factor, float coeff,
+                                 int fast, sga_select_result* result, void* ws,
+                                 size_t ws_bytes, void* stream);
+int sga_state_repack(float* resid, float* p, float* m, float* v, float* state,
+                     int64_t n, int unpack, void* stream);
+
 /* ---- fused offline-replay group step (sga/replay_fused.py:1607-1914) ------ */
 
 /* One configuration's resident state for the current recorded step

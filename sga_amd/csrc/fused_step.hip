@@ -17,6 +17,16 @@ __device__ __forceinline__ void load_g(const void* g, int64_t i, int64_t n, floa
   else ld_f32<FULL>(reinterpret_cast<const float*>(g), i, n, out, vec);
 }
 
+// Packed state: resid, p, m, v interleaved in records of 4 x kPackRun floats
+// ([resid run | p run | m run | v run], 64 KiB), so the four streams of a
+// workgroup always sit in different DRAM banks of one physical page.  Element
+// i of array a lives at state[(i >> 12) * 16384 + a * 4096 + (i & 4095)]; with
+// the array bases set to state + a * 4096 that is base[i + (i >> 12) * 12288].
+constexpr int kPackRunLog = 12;
+constexpr int64_t kPackRun = 1ll << kPackRunLog;
+constexpr int64_t kPackExtra = 3 * kPackRun;
+static_assert(kPackRun % kChunk == 0 && kChunk == 1024, "a chunk never straddles two runs");
+
 // Key source for the select sweeps.
 template <bool BF16G, int SCORE>
 struct SrcFused {
@@ -27,8 +37,14 @@ struct SrcFused {
   const float* v;
   bool vec;
   SegCursor sc;        // per-thread cache of the current segment's hyper-parameters
+  int64_t pack_extra;  // 0: separate arrays; else extra floats per kPackRun elements (packed state)
   template <bool FULL = false>
   __device__ __forceinline__ void load(int64_t i, int64_t n, uint32_t key[4]) {
+    const int64_t sh = (i >> kPackRunLog) * pack_extra;
+    const float* r = this->r + sh;
+    const float* p = this->p + sh;
+    const float* m = this->m + sh;
+    const float* v = this->v + sh;
     float gg[4], rr[4];
     load_g<BF16G, FULL>(g, i, n, gg, vec);
     ld_f32<FULL>(r, i, n, rr, vec);
@@ -88,6 +104,7 @@ struct FinalArgs {
   float factor, coeff;
   uint32_t T, need;
   bool vec, mvec, scale, apply_coeff;
+  int64_t pack_extra;
 };
 
 // One 1024-element chunk of the final sweep, owned by one wave.  FULL: the
@@ -101,6 +118,11 @@ __device__ __forceinline__ void final_chunk(const FinalArgs& a, int64_t c, Chunk
                                             int64_t& fh_lo, int64_t& fh_hi) {
   constexpr bool kFast = (SCORE == SGA_SCORE_ABS_G || SCORE == SGA_SCORE_ABS_M);
   const int64_t n = a.n;
+  const int64_t sh = (c >> (kPackRunLog - 10)) * a.pack_extra;
+  float* const R = a.r + sh;
+  float* const P = a.p + sh;
+  float* const M = a.m + sh;
+  float* const V = a.v + sh;
   float gg[kChunkIters][4], rr[kChunkIters][4], pp[kChunkIters][4], mm[kChunkIters][4],
       vv[kChunkIters][4];
   if (FULL) {
@@ -114,10 +136,10 @@ __device__ __forceinline__ void final_chunk(const FinalArgs& a, int64_t c, Chunk
       const int64_t i = c * kChunk + it * (kWave * kVec) + lane_id() * kVec;
       if (BF16G) graw_h[it] = ldh4_nt(reinterpret_cast<const uint16_t*>(a.g) + i);
       else graw_f[it] = ld4_nt(reinterpret_cast<const float*>(a.g) + i);
-      rraw[it] = ld4_nt(a.r + i);
-      praw[it] = ld4_nt(a.p + i);
-      mraw[it] = ld4_nt(a.m + i);
-      vraw[it] = ld4_nt(a.v + i);
+      rraw[it] = ld4_nt(R + i);
+      praw[it] = ld4_nt(P + i);
+      mraw[it] = ld4_nt(M + i);
+      vraw[it] = ld4_nt(V + i);
     }
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -141,10 +163,10 @@ __device__ __forceinline__ void final_chunk(const FinalArgs& a, int64_t c, Chunk
       for (int e = 0; e < 4; ++e) gg[it][e] = rr[it][e] = pp[it][e] = mm[it][e] = vv[it][e] = 0.0f;
       if (i < n) {
         load_g<BF16G, false>(a.g, i, n, gg[it], a.vec);
-        load4_f32(a.r, i, n, rr[it], a.vec);
-        load4_f32(a.p, i, n, pp[it], a.vec);
-        load4_f32(a.m, i, n, mm[it], a.vec);
-        load4_f32(a.v, i, n, vv[it], a.vec);
+        load4_f32(R, i, n, rr[it], a.vec);
+        load4_f32(P, i, n, pp[it], a.vec);
+        load4_f32(M, i, n, mm[it], a.vec);
+        load4_f32(V, i, n, vv[it], a.vec);
       }
     }
   }
@@ -210,10 +232,10 @@ __device__ __forceinline__ void final_chunk(const FinalArgs& a, int64_t c, Chunk
         }
         rr[it][e] = sel[e] ? 0.0f : q[e];
       }
-      st_f32<FULL>(a.r, i, n, rr[it], a.vec);
-      st_f32<FULL>(a.m, i, n, mm[it], a.vec);
-      st_f32<FULL>(a.v, i, n, vv[it], a.vec);
-      st_f32<FULL>(a.p, i, n, pp[it], a.vec);
+      st_f32<FULL>(R, i, n, rr[it], a.vec);
+      st_f32<FULL>(M, i, n, mm[it], a.vec);
+      st_f32<FULL>(V, i, n, vv[it], a.vec);
+      st_f32<FULL>(P, i, n, pp[it], a.vec);
       if (a.mask_out) st_u8<FULL>(a.mask_out, i, n, mk, a.mvec);
     }
   }
@@ -273,10 +295,11 @@ template <bool BF16G, bool BF16V, int SCORE>
 static int run_fused(const void* g, float* resid, float* p, float* m, float* v, int64_t n,
                      int64_t k, const sga_segment* segs, int n_segs, int32_t* idx_out,
                      void* values_out, uint8_t* mask_out, float factor, float coeff, int fast,
-                     sga_select_result* result, const SelWorkspace& w, hipStream_t s) {
+                     sga_select_result* result, const SelWorkspace& w, hipStream_t s,
+                     int64_t pack_extra) {
   const bool vec = aligned4(g, BF16G ? 2 : 4) && aligned4(resid, 4) && aligned4(p, 4) &&
                    aligned4(m, 4) && aligned4(v, 4);
-  SrcFused<BF16G, SCORE> src{g, resid, p, m, v, vec, {}};
+  SrcFused<BF16G, SCORE> src{g, resid, p, m, v, vec, {}, pack_extra};
   src.sc.init(segs, n_segs);
   run_select(src, n, k, 0, fast != 0, w, s);
   const int64_t n_tiles = cdiv64(n, kChunk);
@@ -288,6 +311,7 @@ static int run_fused(const void* g, float* resid, float* p, float* m, float* v, 
   fa.factor = factor; fa.coeff = coeff; fa.T = 0; fa.need = 0;
   fa.vec = vec; fa.mvec = aligned4(mask_out, 1);
   fa.scale = factor != 1.0f; fa.apply_coeff = coeff != 1.0f;
+  fa.pack_extra = pack_extra;
   hipLaunchKernelGGL((k_fused_final<BF16G, BF16V, SCORE>),
                      dim3(stream_grid(n_tiles, kChunksPerBlock, 1 << 20)), dim3(kBlock), 0, s, fa,
                      segs, n_segs, w.st, w.tile_gt, w.tile_eq);
@@ -327,31 +351,31 @@ extern "C" int sga_prof_read(double* total_ms, int* launches) {
 
 extern "C" size_t sga_fused_workspace_bytes(int64_t n) { return sel_ws_bytes(n < 0 ? 0 : n); }
 
-extern "C" int sga_fused_sparse_step(const void* g, int g_dtype, float* resid, float* p, float* m,
-                                     float* v, int64_t n, int64_t k, const sga_segment* segs,
-                                     int n_segs, int score_id, int32_t* idx_out, void* values_out,
-                                     int values_dtype, uint8_t* mask_out, float factor,
-                                     float coeff, int fast, sga_select_result* result, void* ws,
-                                     size_t ws_bytes, void* stream) {
+static int fused_entry(const char* who, const void* g, int g_dtype, float* resid, float* p,
+                       float* m, float* v, int64_t pack_extra, int64_t n, int64_t k,
+                       const sga_segment* segs, int n_segs, int score_id, int32_t* idx_out,
+                       void* values_out, int values_dtype, uint8_t* mask_out, float factor,
+                       float coeff, int fast, sga_select_result* result, void* ws, size_t ws_bytes,
+                       void* stream) {
   if (!g || !resid || !p || !m || !v || !segs || !idx_out || !values_out || n < 1 ||
       n >= (1ll << 31) || k < 1 || k > n || n_segs < 1 ||
       (g_dtype != SGA_F32 && g_dtype != SGA_BF16) ||
       (values_dtype != SGA_F32 && values_dtype != SGA_BF16) || score_id < 0 || score_id > 3) {
-    set_error("sga_fused_sparse_step: bad argument (n=%lld k=%lld n_segs=%d score=%d; need "
-              "1 <= k <= n < 2^31)", (long long)n, (long long)k, n_segs, score_id);
+    set_error("%s: bad argument (n=%lld k=%lld n_segs=%d score=%d; need 1 <= k <= n < 2^31)", who,
+              (long long)n, (long long)k, n_segs, score_id);
     return SGA_ERR_ARG;
   }
   SelWorkspace w;
   if (!sel_ws_carve(ws, ws_bytes, cdiv64(n, kChunk), &w)) {
-    set_error("sga_fused_sparse_step: workspace missing, misaligned or smaller than "
-              "sga_fused_workspace_bytes(n)=%zu", sel_ws_bytes(n));
+    set_error("%s: workspace missing, misaligned or smaller than "
+              "sga_fused_workspace_bytes(n)=%zu", who, sel_ws_bytes(n));
     return SGA_ERR_WORKSPACE;
   }
   hipStream_t s = (hipStream_t)stream;
   const bool bg = g_dtype == SGA_BF16, bv = values_dtype == SGA_BF16;
 #define SGA_RUN(BG, BV, SC)                                                                   \
   return run_fused<BG, BV, SC>(g, resid, p, m, v, n, k, segs, n_segs, idx_out, values_out,   \
-                               mask_out, factor, coeff, fast, result, w, s)
+                               mask_out, factor, coeff, fast, result, w, s, pack_extra)
 #define SGA_RUN_SC(BG, BV)                    \
   switch (score_id) {                         \
     case 0: SGA_RUN(BG, BV, 0);               \
@@ -365,4 +389,65 @@ extern "C" int sga_fused_sparse_step(const void* g, int g_dtype, float* resid, f
   else { SGA_RUN_SC(false, false) }
 #undef SGA_RUN_SC
 #undef SGA_RUN
+}
+
+extern "C" int sga_fused_sparse_step(const void* g, int g_dtype, float* resid, float* p, float* m,
+                                     float* v, int64_t n, int64_t k, const sga_segment* segs,
+                                     int n_segs, int score_id, int32_t* idx_out, void* values_out,
+                                     int values_dtype, uint8_t* mask_out, float factor,
+                                     float coeff, int fast, sga_select_result* result, void* ws,
+                                     size_t ws_bytes, void* stream) {
+  return fused_entry("sga_fused_sparse_step", g, g_dtype, resid, p, m, v, 0, n, k, segs, n_segs,
+                     score_id, idx_out, values_out, values_dtype, mask_out, factor, coeff, fast,
+                     result, ws, ws_bytes, stream);
+}
+
+extern "C" int64_t sga_packed_state_elems(int64_t n) {
+  return n <= 0 ? 0 : cdiv64(n, kPackRun) * 4 * kPackRun;
+}
+
+extern "C" int sga_fused_sparse_step_packed(const void* g, int g_dtype, float* state, int64_t n,
+                                            int64_t k, const sga_segment* segs, int n_segs,
+                                            int score_id, int32_t* idx_out, void* values_out,
+                                            int values_dtype, uint8_t* mask_out, float factor,
+                                            float coeff, int fast, sga_select_result* result,
+                                            void* ws, size_t ws_bytes, void* stream) {
+  if (state && (reinterpret_cast<uintptr_t>(state) & 15)) {
+    set_error("sga_fused_sparse_step_packed: state must be 16-byte aligned");
+    return SGA_ERR_ARG;
+  }
+  return fused_entry("sga_fused_sparse_step_packed", g, g_dtype, state,
+                     state ? state + kPackRun : nullptr, state ? state + 2 * kPackRun : nullptr,
+                     state ? state + 3 * kPackRun : nullptr, kPackExtra, n, k, segs, n_segs,
+                     score_id, idx_out, values_out, values_dtype, mask_out, factor, coeff, fast,
+                     result, ws, ws_bytes, stream);
+}
+
+// resid/p/m/v <-> packed state (dir 0: pack, 1: unpack); a null array is skipped.
+static __global__ __launch_bounds__(kBlock) void k_state_repack(float* __restrict__ r,
+                                                                float* __restrict__ p,
+                                                                float* __restrict__ m,
+                                                                float* __restrict__ v,
+                                                                float* __restrict__ state,
+                                                                int64_t n, int dir) {
+  float* arr[4] = {r, p, m, v};
+  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n;
+       i += (int64_t)gridDim.x * kBlock) {
+    const int64_t j = i + (i >> kPackRunLog) * kPackExtra;
+#pragma unroll
+    for (int a = 0; a < 4; ++a) {
+      if (!arr[a]) continue;
+      if (dir == 0) state[j + a * kPackRun] = arr[a][i];
+      else arr[a][i] = state[j + a * kPackRun];
+    }
+  }
+}
+
+extern "C" int sga_state_repack(float* resid, float* p, float* m, float* v, float* state,
+                                int64_t n, int unpack, void* stream) {
+  if (n == 0) return SGA_OK;
+  if (!state || n < 0) { set_error("sga_state_repack: bad argument"); return SGA_ERR_ARG; }
+  hipLaunchKernelGGL(k_state_repack, dim3(stream_grid(n, kBlock, 1 << 16)), dim3(kBlock), 0,
+                     (hipStream_t)stream, resid, p, m, v, state, n, unpack ? 1 : 0);
+  return check_launch("sga_state_repack");
 }

@@ -136,3 +136,42 @@ def test_fast_and_radix_paths_agree(dev):
     for a, b in zip(outs[0][:-1], outs[1][:-1]):
         assert torch.equal(a, b)
     assert outs[0][-1] == outs[1][-1]
+
+
+@pytest.mark.parametrize("score,gdtype", [("abs_g", torch.bfloat16), ("update", torch.float32),
+                                          ("abs_m", torch.bfloat16)])
+def test_packed_state_is_bitwise_the_separate_layout(dev, score, gdtype):
+    """The packed-state entry point runs the same arithmetic on interleaved
+    64 KiB records: after unpacking, every output equals the separate-array
+    entry point's bit for bit, over several steps, ragged sizes, both select
+    paths (n below and above the sampled-bracket cut-in)."""
+    from sga_amd.fused_step import FusedSparseStep, PackedState
+    for sizes in ([4097, 3, 12_289, 1000], [1 << 20, 4099, (1 << 20) + 5]):
+        segs, n = _segments(sizes)
+        gen = torch.Generator().manual_seed(5)
+        p0 = (torch.randn(n, generator=gen) * 0.02).to(dev)
+        m0 = (torch.randn(n, generator=gen) * 1e-3).to(dev)
+        v0 = (torch.rand(n, generator=gen) * 1e-5).to(dev)
+        r0 = (student_t(n, 77) * 0.1).to(dev)
+        p, m, v, r = (t.clone() for t in (p0, m0, v0, r0))
+        st = PackedState(n, dev).pack(r0, p0, m0, v0)
+        back = [torch.empty(n, device=dev) for _ in range(4)]
+        st.unpack(*back)
+        for a, b in zip(back, (r0, p0, m0, v0)):
+            assert torch.equal(a, b)
+        fa = FusedSparseStep(n, segs, dev, values_dtype=torch.bfloat16, want_mask=True)
+        fb = FusedSparseStep(n, segs, dev, values_dtype=torch.bfloat16, want_mask=True)
+        for step in range(1, 4):
+            g = student_t(n, 100 + step).to(gdtype).to(dev)
+            ia, va = fa.step(g, r, p, m, v, step, ratio_percent=1.0, score=score)
+            ib, vb = fb.step_packed(g, st, step, ratio_percent=1.0, score=score)
+            ra, rb = fa.read_result(), fb.read_result()
+            assert (ra.thresh_bits, ra.need, ra.n_selected, ra.path) == \
+                (rb.thresh_bits, rb.need, rb.n_selected, rb.path)
+            assert torch.equal(ia, ib) and torch.equal(va.view(torch.int16), vb.view(torch.int16))
+            assert torch.equal(fa.mask, fb.mask)
+            st.unpack(*back)
+            for a, b in zip(back, (r, p, m, v)):
+                assert torch.equal(a.view(torch.int32), b.view(torch.int32)), (sizes, step)
+    with pytest.raises(ValueError):
+        fb.step_packed(g, PackedState(n + 1, dev), 1, ratio_percent=1.0)
