@@ -316,7 +316,10 @@ typedef struct sga_replay_cfg {
   int boundary;           /* si % T == 0                                     */
   int adams;              /* optimizer == "adams"                            */
   int split;              /* boundary dual-lr split active                   */
-  int pad_;
+  int packed;             /* 1: res/w/m/v are the run bases state, state+4096,
+                             state+8192, state+12288 of ONE packed state (the
+                             layout of sga_fused_sparse_step_packed, array
+                             order res, w, m, v); the same for every config  */
 } sga_replay_cfg;
 
 /* Per-tensor hyper-parameters of the replay commit (ShardParams entries +
@@ -347,7 +350,7 @@ int sga_replay_reselect(const void* g, int g_dtype, const float* res,
                         const float* w, const float* m, const float* v,
                         int64_t n, int64_t k, const sga_segment* segs,
                         int n_segs, int score_id, const float* coef_f,
-                        float coef_dense, int adams, uint8_t* sel_out,
+                        float coef_dense, int adams, int packed, uint8_t* sel_out,
                         sga_select_result* result, void* ws, size_t ws_bytes,
                         void* stream);
 
@@ -368,13 +371,15 @@ int sga_dense_replay_step(const void* g, int g_dtype, float* w, float* m, float*
                           int n_segs, int adams, double coef_dense, double* partials,
                           double* recon2, void* stream);
 
-/* res /= T at fold boundaries (replay_fused.py:1632-1636), true division. */
-int sga_div_inplace(float* x, int64_t n, float d, void* stream);
+/* res /= T at fold boundaries (replay_fused.py:1632-1636), true division.
+ * packed != 0: x is the run base of one array inside a packed state. */
+int sga_div_inplace(float* x, int64_t n, float d, int packed, void* stream);
 
 /* out[0] = sum (a-b)^2 in double (horizon numerators, :1890-1900).
- * partials: 1024 doubles. */
-int sga_sq_dist(const float* a, const float* b, int64_t n, double* partials,
-                double* out, void* stream);
+ * partials: 1024 doubles.  a_packed != 0: a is the run base of one array
+ * inside a packed state; b is always flat. */
+int sga_sq_dist(const float* a, int a_packed, const float* b, int64_t n,
+                double* partials, double* out, void* stream);
 
 /* Live timing of the fused step's final sweep with HIP events recorded on the
  * launch stream (no counterpart in the reference; used by the benchmark).

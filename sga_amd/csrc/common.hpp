@@ -15,6 +15,17 @@ constexpr int kChunk = kWave * kVec * kChunkIters;   // 1024 elements / wave
 constexpr int kChunksPerBlock = kBlock / kWave;      // 4
 constexpr int kBlockSpan = kChunk * kChunksPerBlock; // 4096 elements / block
 
+// Packed state: four fp32 arrays of one bucket interleaved in records of
+// 4 x kPackRun floats ([a0 run | a1 run | a2 run | a3 run], 64 KiB), so the
+// four streams of a workgroup always sit in different DRAM banks of one
+// physical page.  Element i of array a lives at
+// state[(i >> 12) * 16384 + a * 4096 + (i & 4095)]; with the array bases set
+// to state + a * 4096 that is base[i + (i >> 12) * 12288].
+constexpr int kPackRunLog = 12;
+constexpr int64_t kPackRun = 1ll << kPackRunLog;
+constexpr int64_t kPackExtra = 3 * kPackRun;
+static_assert(kPackRun % kChunk == 0 && kChunk == 1024, "a chunk never straddles two runs");
+
 void set_error(const char* fmt, ...);
 int check_launch(const char* what);
 
@@ -55,6 +66,19 @@ __device__ __forceinline__ uint16_t f32_to_bf16(float f) {
 }
 
 __device__ __forceinline__ int lane_id() { return threadIdx.x & (kWave - 1); }
+
+// Offset (in floats) that moves an array's run base to the record holding
+// element i of a packed state.  UNIFORM promises that every lane of the wave
+// addresses the same run (chunk-structured sweeps), so the offset is formed
+// once on the scalar unit.
+template <bool UNIFORM>
+__device__ __forceinline__ int64_t pack_shift(int64_t i, int64_t pack_extra) {
+  if (UNIFORM) {
+    const int run = __builtin_amdgcn_readfirstlane((int)(i >> kPackRunLog));
+    return (int64_t)run * pack_extra;
+  }
+  return (i >> kPackRunLog) * pack_extra;
+}
 __device__ __forceinline__ int wave_id() { return threadIdx.x >> 6; }
 
 // Number of set bits of `mask` strictly below the calling lane.

@@ -17,16 +17,6 @@ __device__ __forceinline__ void load_g(const void* g, int64_t i, int64_t n, floa
   else ld_f32<FULL>(reinterpret_cast<const float*>(g), i, n, out, vec);
 }
 
-// Packed state: resid, p, m, v interleaved in records of 4 x kPackRun floats
-// ([resid run | p run | m run | v run], 64 KiB), so the four streams of a
-// workgroup always sit in different DRAM banks of one physical page.  Element
-// i of array a lives at state[(i >> 12) * 16384 + a * 4096 + (i & 4095)]; with
-// the array bases set to state + a * 4096 that is base[i + (i >> 12) * 12288].
-constexpr int kPackRunLog = 12;
-constexpr int64_t kPackRun = 1ll << kPackRunLog;
-constexpr int64_t kPackExtra = 3 * kPackRun;
-static_assert(kPackRun % kChunk == 0 && kChunk == 1024, "a chunk never straddles two runs");
-
 // Key source for the select sweeps.
 template <bool BF16G, int SCORE>
 struct SrcFused {
@@ -40,7 +30,7 @@ struct SrcFused {
   int64_t pack_extra;  // 0: separate arrays; else extra floats per kPackRun elements (packed state)
   template <bool FULL = false>
   __device__ __forceinline__ void load(int64_t i, int64_t n, uint32_t key[4]) {
-    const int64_t sh = (i >> kPackRunLog) * pack_extra;
+    const int64_t sh = pack_shift<FULL>(i, pack_extra);
     const float* r = this->r + sh;
     const float* p = this->p + sh;
     const float* m = this->m + sh;
@@ -118,7 +108,7 @@ __device__ __forceinline__ void final_chunk(const FinalArgs& a, int64_t c, Chunk
                                             int64_t& fh_lo, int64_t& fh_hi) {
   constexpr bool kFast = (SCORE == SGA_SCORE_ABS_G || SCORE == SGA_SCORE_ABS_M);
   const int64_t n = a.n;
-  const int64_t sh = (c >> (kPackRunLog - 10)) * a.pack_extra;
+  const int64_t sh = pack_shift<true>(c << 10, a.pack_extra);     // c is wave-uniform
   float* const R = a.r + sh;
   float* const P = a.p + sh;
   float* const M = a.m + sh;

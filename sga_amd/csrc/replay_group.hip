@@ -31,12 +31,13 @@ struct RCfg {
   int boundary;
   int adams;
   int split;
-  int pad_;
+  int packed;
 };
 
 struct RGroup {
   RCfg c[kMaxCfg];
   int G;
+  int64_t pack_extra;       // 0, or kPackExtra when every config's w/m/v/res is one packed state
 };
 
 template <bool BF16G, bool FULL>
@@ -63,7 +64,8 @@ struct P1List {
 template <bool BF16G, bool BOUNDARY, int NC>
 __global__ __launch_bounds__(kBlock) void k_replay_pass1(const void* __restrict__ g, int64_t n,
                                                          float coef_dense, P1List lst,
-                                                         double* __restrict__ partials, bool vec) {
+                                                         double* __restrict__ partials, bool vec,
+                                                         int64_t pack_extra) {
   __shared__ double s_w[kChunksPerBlock][NC];
   double acc[NC];
 #pragma unroll
@@ -81,7 +83,8 @@ __global__ __launch_bounds__(kBlock) void k_replay_pass1(const void* __restrict_
       float rr[NC][4];
 #pragma unroll
       for (int c = 0; c < NC; ++c) {
-        const float* rp = reinterpret_cast<const float*>(lst.ptr[c]);
+        const float* rp = reinterpret_cast<const float*>(lst.ptr[c]) +
+                          (full ? pack_shift<true>(i, pack_extra) : pack_shift<false>(i, pack_extra));
         if (full) ld_f32<true>(rp, i, n, rr[c], true);
         else load4_f32(rp, i, n, rr[c], vec);
       }
@@ -184,16 +187,21 @@ __device__ __forceinline__ void pass3_vec(const void* g, int64_t i, int64_t n, f
                                           bool vec) {
   float gd[4];
   load_gd<BF16G, FULL>(g, i, n, is_one, coef_dense, gd, vec);
+  const int64_t sh = pack_shift<FULL>(i, grp.pack_extra);
 #pragma unroll 1
   for (int c = 0; c < grp.G; ++c) {
     const RCfg& cf = grp.c[c];
     const float coef = coef_f[c];
+    float* const RES = cf.res + sh;
+    float* const MM = cf.m + sh;
+    float* const VV = cf.v + sh;
+    float* const WW = cf.w + sh;
     float rr[4], mm[4], vv[4] = {0, 0, 0, 0}, ww[4];
     uint32_t sl[4] = {1, 1, 1, 1}, so[4] = {1, 1, 1, 1};
-    ld_f32<FULL>(cf.res, i, n, rr, vec);
-    ld_f32<FULL>(cf.m, i, n, mm, vec);
-    if (!cf.adams) ld_f32<FULL>(cf.v, i, n, vv, vec);
-    ld_f32<FULL>(cf.w, i, n, ww, vec);
+    ld_f32<FULL>(RES, i, n, rr, vec);
+    ld_f32<FULL>(MM, i, n, mm, vec);
+    if (!cf.adams) ld_f32<FULL>(VV, i, n, vv, vec);
+    ld_f32<FULL>(WW, i, n, ww, vec);
     if (!cf.boundary) ld_u8<FULL>(cf.sel, i, n, sl, vec);
     if (cf.split) ld_u8<FULL>(cf.out_sel, i, n, so, vec);
 #pragma unroll
@@ -227,10 +235,10 @@ __device__ __forceinline__ void pass3_vec(const void* g, int64_t i, int64_t n, f
       mm[e] = mn;
       vv[e] = vn;
     }
-    st_f32<FULL>(cf.res, i, n, rr, vec);
-    st_f32<FULL>(cf.m, i, n, mm, vec);
-    st_f32<FULL>(cf.v, i, n, vv, vec);
-    st_f32<FULL>(cf.w, i, n, ww, vec);
+    st_f32<FULL>(RES, i, n, rr, vec);
+    st_f32<FULL>(MM, i, n, mm, vec);
+    st_f32<FULL>(VV, i, n, vv, vec);
+    st_f32<FULL>(WW, i, n, ww, vec);
   }
 }
 
@@ -332,8 +340,14 @@ struct SrcReplay {
   int adams;
   bool vec;
   SegCursor sc;              // b1, b2, eps, wd, bc1, bc2 per tensor (cached per thread)
+  int64_t pack_extra;        // 0 or kPackExtra (res/w/m/v of one packed state)
   template <bool FULL = false>
   __device__ __forceinline__ void load(int64_t i, int64_t n, uint32_t key[4]) {
+    const int64_t sh = pack_shift<FULL>(i, pack_extra);
+    const float* res = this->res + sh;
+    const float* w = this->w + sh;
+    const float* m = this->m + sh;
+    const float* v = this->v + sh;
     float gd[4], rr[4];
     load_gd<BF16G, FULL>(g, i, n, coef_dense == 1.0f ? 1.0f : 0.0f, coef_dense, gd, vec);
     ld_f32<FULL>(res, i, n, rr, vec);
@@ -368,27 +382,29 @@ struct SrcReplay {
 };
 
 __global__ __launch_bounds__(kBlock) void k_div_inplace(float* __restrict__ x, int64_t n, float d,
-                                                        bool vec) {
+                                                        bool vec, int64_t pack_extra) {
   const int64_t stride = (int64_t)gridDim.x * kBlock * kVec;
   for (int64_t i = ((int64_t)blockIdx.x * kBlock + threadIdx.x) * kVec; i < n; i += stride) {
+    float* xs = x + (i >> kPackRunLog) * pack_extra;
     float v[4];
-    load4_f32(x, i, n, v, vec);
+    load4_f32(xs, i, n, v, vec);
 #pragma unroll
     for (int e = 0; e < 4; ++e) v[e] = __fdiv_rn(v[e], d);
-    store4_f32(x, i, n, v, vec);
+    store4_f32(xs, i, n, v, vec);
   }
 }
 
 // sum (a - b)^2 in double, two-stage
 __global__ __launch_bounds__(kBlock) void k_sqdist_stage1(const float* __restrict__ a,
                                                           const float* __restrict__ b, int64_t n,
-                                                          double* __restrict__ partials, bool vec) {
+                                                          double* __restrict__ partials, bool vec,
+                                                          int64_t a_pack_extra) {
   __shared__ double s_w[kChunksPerBlock];
   double acc = 0.0;
   const int64_t stride = (int64_t)gridDim.x * kBlock * kVec;
   for (int64_t i = ((int64_t)blockIdx.x * kBlock + threadIdx.x) * kVec; i < n; i += stride) {
     float x[4], y[4];
-    load4_f32(a, i, n, x, vec);
+    load4_f32(a + (i >> kPackRunLog) * a_pack_extra, i, n, x, vec);
     load4_f32(b, i, n, y, vec);
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
@@ -419,8 +435,10 @@ static bool fill_group(RGroup* grp, const sga_replay_cfg* cfgs, int G) {
     d.w = s.w; d.m = s.m; d.v = s.v; d.res = s.res; d.sel = s.sel;
     d.out_sel = s.out_sel ? s.out_sel : s.sel;
     d.lr_scale = s.lr_scale; d.boundary = s.boundary; d.adams = s.adams; d.split = s.split;
-    d.pad_ = 0;
+    d.packed = s.packed != 0;
+    if (d.packed != (cfgs[0].packed != 0)) return false;     // one layout per group
   }
+  grp->pack_extra = cfgs[0].packed ? kPackExtra : 0;
   for (int c = G; c < kMaxCfg; ++c) grp->c[c] = grp->c[0];
   return true;
 }
@@ -445,18 +463,19 @@ static_assert(sizeof(RSeg) == sizeof(sga_replay_segment), "replay segment layout
 
 template <bool BOUNDARY, bool BF16G, int NC>
 static void launch_pass1_n(unsigned nb, hipStream_t s, const void* g, int64_t n, float coef_dense,
-                           const P1List& lst, double* partials, bool vec) {
+                           const P1List& lst, double* partials, bool vec, int64_t pack_extra) {
   hipLaunchKernelGGL((k_replay_pass1<BF16G, BOUNDARY, NC>), dim3(nb), dim3(kBlock), 0, s, g, n,
-                     coef_dense, lst, partials, vec);
+                     coef_dense, lst, partials, vec, pack_extra);
 }
 
 template <bool BOUNDARY>
 static void launch_pass1(bool bg, int count, unsigned nb, hipStream_t s, const void* g, int64_t n,
-                         float coef_dense, const P1List& lst, double* partials, bool vec) {
+                         float coef_dense, const P1List& lst, double* partials, bool vec,
+                         int64_t pack_extra) {
 #define SGA_P1(NC)                                                                             \
   case NC:                                                                                     \
-    if (bg) launch_pass1_n<BOUNDARY, true, NC>(nb, s, g, n, coef_dense, lst, partials, vec);   \
-    else launch_pass1_n<BOUNDARY, false, NC>(nb, s, g, n, coef_dense, lst, partials, vec);     \
+    if (bg) launch_pass1_n<BOUNDARY, true, NC>(nb, s, g, n, coef_dense, lst, partials, vec, pack_extra); \
+    else launch_pass1_n<BOUNDARY, false, NC>(nb, s, g, n, coef_dense, lst, partials, vec, pack_extra);   \
     break;
   switch (count) {
     SGA_P1(1) SGA_P1(2) SGA_P1(3) SGA_P1(4) SGA_P1(5) SGA_P1(6) SGA_P1(7) SGA_P1(8)
@@ -487,8 +506,8 @@ extern "C" int sga_replay_pass1(const void* g, int g_dtype, int64_t n, float coe
     if (grp.c[c].boundary) { lb.ptr[n_b] = grp.c[c].res; lb.slot[n_b++] = c; }
     else { lm.ptr[n_m] = grp.c[c].sel; lm.slot[n_m++] = c; }
   }
-  launch_pass1<true>(bg, n_b, nb, s, g, n, coef_dense, lb, partials, vec);
-  launch_pass1<false>(bg, n_m, nb, s, g, n, coef_dense, lm, partials, vec);
+  launch_pass1<true>(bg, n_b, nb, s, g, n, coef_dense, lb, partials, vec, grp.pack_extra);
+  launch_pass1<false>(bg, n_m, nb, s, g, n, coef_dense, lm, partials, vec, 0);
   hipLaunchKernelGGL(k_replay_coef, dim3(1), dim3(kBlock), 0, s, partials, (int)nb, G, clip, qn2, coef_d, coef_f);
   return check_launch("sga_replay_pass1");
 }
@@ -515,11 +534,13 @@ extern "C" int sga_replay_pass3(const void* g, int g_dtype, int64_t n, float coe
 template <bool BF16G, int SCORE>
 static int run_reselect(const void* g, const float* res, const float* w, const float* m,
                         const float* v, int64_t n, int64_t k, const sga_segment* segs, int n_segs,
-                        const float* coef_f, float coef_dense, int adams, uint8_t* sel_out,
-                        sga_select_result* result, const SelWorkspace& ws, hipStream_t s) {
+                        const float* coef_f, float coef_dense, int adams, int packed,
+                        uint8_t* sel_out, sga_select_result* result, const SelWorkspace& ws,
+                        hipStream_t s) {
   const bool vec = aligned4(g, BF16G ? 2 : 4) && aligned4(res, 4) && aligned4(w, 4) &&
                    aligned4(m, 4) && aligned4(v, 4);
-  SrcReplay<BF16G, SCORE> src{g, res, w, m, v, coef_f, coef_dense, adams, vec, {}};
+  SrcReplay<BF16G, SCORE> src{g, res, w, m, v, coef_f, coef_dense, adams, vec, {},
+                              packed ? kPackExtra : 0};
   src.sc.init(segs, n_segs);
   run_select(src, n, k, 0, true, ws, s, true);
   finish_mask(src, n, 0, ws, sel_out, s);
@@ -530,7 +551,7 @@ static int run_reselect(const void* g, const float* res, const float* w, const f
 extern "C" int sga_replay_reselect(const void* g, int g_dtype, const float* res, const float* w,
                                    const float* m, const float* v, int64_t n, int64_t k,
                                    const sga_segment* segs, int n_segs, int score_id,
-                                   const float* coef_f, float coef_dense, int adams,
+                                   const float* coef_f, float coef_dense, int adams, int packed,
                                    uint8_t* sel_out, sga_select_result* result, void* ws,
                                    size_t ws_bytes, void* stream) {
   if (!g || !res || !w || !m || !v || !segs || !coef_f || !sel_out || n < 1 || n >= (1ll << 31) ||
@@ -545,7 +566,7 @@ extern "C" int sga_replay_reselect(const void* g, int g_dtype, const float* res,
     return SGA_ERR_WORKSPACE;
   }
   hipStream_t s = (hipStream_t)stream;
-#define SGA_RS(BG, SC) return run_reselect<BG, SC>(g, res, w, m, v, n, k, segs, n_segs, coef_f, coef_dense, adams, sel_out, result, sw, s)
+#define SGA_RS(BG, SC) return run_reselect<BG, SC>(g, res, w, m, v, n, k, segs, n_segs, coef_f, coef_dense, adams, packed, sel_out, result, sw, s)
   if (g_dtype == SGA_BF16) {
     switch (score_id) { case 0: SGA_RS(true, 0); case 1: SGA_RS(true, 1); case 2: SGA_RS(true, 2); default: SGA_RS(true, 3); }
   } else {
@@ -575,21 +596,21 @@ extern "C" int sga_dense_replay_step(const void* g, int g_dtype, float* w, float
   return check_launch("sga_dense_replay_step");
 }
 
-extern "C" int sga_div_inplace(float* x, int64_t n, float d, void* stream) {
+extern "C" int sga_div_inplace(float* x, int64_t n, float d, int packed, void* stream) {
   if (n == 0) return SGA_OK;
   if (!x || n < 0) { set_error("sga_div_inplace: bad argument"); return SGA_ERR_ARG; }
   hipLaunchKernelGGL(k_div_inplace, dim3(stream_grid(n, (int64_t)kBlock * kVec)), dim3(kBlock), 0,
-                     (hipStream_t)stream, x, n, d, aligned4(x, 4));
+                     (hipStream_t)stream, x, n, d, aligned4(x, 4), packed ? kPackExtra : 0);
   return check_launch("sga_div_inplace");
 }
 
-extern "C" int sga_sq_dist(const float* a, const float* b, int64_t n, double* partials, double* out,
-                           void* stream) {
+extern "C" int sga_sq_dist(const float* a, int a_packed, const float* b, int64_t n, double* partials,
+                           double* out, void* stream) {
   if (!a || !b || !partials || !out || n < 1) { set_error("sga_sq_dist: bad argument"); return SGA_ERR_ARG; }
   const unsigned nb = stream_grid(n, (int64_t)kBlock * kVec, 1024);
   hipStream_t s = (hipStream_t)stream;
   hipLaunchKernelGGL(k_sqdist_stage1, dim3(nb), dim3(kBlock), 0, s, a, b, n, partials,
-                     aligned4(a, 4) && aligned4(b, 4));
+                     aligned4(a, 4) && aligned4(b, 4), a_packed ? kPackExtra : 0);
   hipLaunchKernelGGL(k_sqdist_stage2, dim3(1), dim3(kWave), 0, s, partials, (int)nb, out);
   return check_launch("sga_sq_dist");
 }

@@ -85,7 +85,7 @@ class DenseReplay:
                               if math.isfinite(norm) and norm > 0.0 else None)})
         self.si += 1
         if self.si in horizons:
-            L.call("sga_sq_dist", L.ptr(self.w), L.ptr(self.w0), self.N, L.ptr(self._partials),
+            L.call("sga_sq_dist", L.ptr(self.w), 0, L.ptr(self.w0), self.N, L.ptr(self._partials),
                    L.ptr(self._dist), st)
             self.den_at[self.si] = math.sqrt(float(self._dist.item()))
             self.snapshots[self.si] = self.w.clone()

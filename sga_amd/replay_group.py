@@ -18,7 +18,7 @@ class ReplayCfg(C.Structure):
     """struct sga_replay_cfg"""
     _fields_ = [("w", C.c_void_p), ("m", C.c_void_p), ("v", C.c_void_p), ("res", C.c_void_p),
                 ("sel", C.c_void_p), ("out_sel", C.c_void_p), ("lr_scale", C.c_double),
-                ("boundary", C.c_int), ("adams", C.c_int), ("split", C.c_int), ("pad_", C.c_int)]
+                ("boundary", C.c_int), ("adams", C.c_int), ("split", C.c_int), ("packed", C.c_int)]
 
 
 class ReplaySegment(C.Structure):
@@ -52,6 +52,39 @@ def _upload(struct_array, uploader):
     uploader.upload(struct_array)
 
 
+_RUN = 4096                       # floats per array per packed record
+_ARRAY_SLOT = {"res": 0, "w": 1, "m": 2, "v": 3}
+
+
+class ConfigState:
+    """One config's resident state: res / w / m / v interleaved in one packed
+    buffer (64 KiB records, array order res, w, m, v) plus the byte masks.
+    ``state["w"]`` etc. return flat unpacked copies for inspection."""
+
+    def __init__(self, n, w0, m0, v0, sel):
+        dev = w0.device
+        self.n = n
+        self.data = torch.zeros(int(L.raw("sga_packed_state_elems", n)), dtype=torch.float32,
+                                device=dev)
+        L.call("sga_state_repack", None, L.ptr(w0), L.ptr(m0), L.ptr(v0), L.ptr(self.data), n, 0,
+               L.stream())
+        self.sel = sel.reshape(-1).to(torch.uint8).clone()
+        self.spare = torch.empty(n, dtype=torch.uint8, device=dev)
+
+    def base(self, name):
+        """Device address of an array's first run inside the packed buffer."""
+        return self.data.data_ptr() + 4 * _RUN * _ARRAY_SLOT[name]
+
+    def __getitem__(self, name):
+        if name in ("sel", "spare"):
+            return getattr(self, name)
+        out = torch.empty(self.n, dtype=torch.float32, device=self.data.device)
+        args = [None] * 4
+        args[_ARRAY_SLOT[name]] = L.ptr(out)
+        L.call("sga_state_repack", *args, L.ptr(self.data), self.n, 1, L.stream())
+        return out
+
+
 class ReplayGroup:
     """Resident state of one config group over a flat shard of N elements.
 
@@ -76,13 +109,7 @@ class ReplayGroup:
         self.entries, self.configs, self.t0, self.W = entries, configs, t0, window
         dev = w0.device
         self.dev = dev
-        self.state = []
-        for ci, _ in enumerate(configs):
-            self.state.append({
-                "w": w0.clone(), "m": m0.clone(), "v": v0.clone(),
-                "res": torch.zeros(self.N, dtype=torch.float32, device=dev),
-                "sel": sel0[ci].reshape(-1).to(torch.uint8).clone(),
-                "spare": torch.empty(self.N, dtype=torch.uint8, device=dev)})
+        self.state = [ConfigState(self.N, w0, m0, v0, sel0[ci]) for ci in range(len(configs))]
         G = len(configs)
         self.ks = {c.ratio: max(1, int(round(c.ratio / 100.0 * self.N))) for c in configs}
         self.partials = torch.empty(int(L.raw("sga_replay_partials")), dtype=torch.float64,
@@ -124,11 +151,11 @@ class ReplayGroup:
     def _fill_cfgs(self, bnd, out_sel):
         for ci, c in enumerate(self.configs):
             s, h = self.state[ci], self._cfg_host[ci]
-            h.w, h.m, h.v, h.res = (s[k].data_ptr() for k in ("w", "m", "v", "res"))
-            h.sel = s["sel"].data_ptr()
+            h.w, h.m, h.v, h.res = (s.base(k) for k in ("w", "m", "v", "res"))
+            h.sel = s.sel.data_ptr()
             split = bool(bnd[ci] and c.dual_lr != 1.0)
-            h.out_sel = (out_sel.get(ci, s["sel"])).data_ptr() if split else None
-            h.lr_scale = c.dual_lr
+            h.out_sel = (out_sel.get(ci, s.sel)).data_ptr() if split else None
+            h.lr_scale, h.packed = c.dual_lr, 1
             h.boundary, h.adams, h.split = int(bnd[ci]), int(c.optimizer == "adams"), int(split)
 
     # -- one recorded step ----------------------------------------------------
@@ -150,8 +177,8 @@ class ReplayGroup:
         if si > 0:                                   # residual fold
             for ci, c in enumerate(self.configs):
                 if bnd[ci] and c.fold:
-                    L.call("sga_div_inplace", L.ptr(self.state[ci]["res"]), N,
-                           L.f32(float(c.T)), st)
+                    L.call("sga_div_inplace", C.c_void_p(self.state[ci].base("res")), N,
+                           L.f32(float(c.T)), 1, st)
         self._fill_segments(count, lr_of)
         self._fill_cfgs(bnd, {})
         gd = L.dtype_code(g)
@@ -162,15 +189,16 @@ class ReplayGroup:
             if not (bnd[ci] and si > 0 and si + 1 < self.W):
                 continue
             s = self.state[ci]
-            L.call("sga_replay_reselect", L.ptr(g), gd, L.ptr(s["res"]), L.ptr(s["w"]),
-                   L.ptr(s["m"]), L.ptr(s["v"]), N, self.ks[c.ratio],
+            L.call("sga_replay_reselect", L.ptr(g), gd, C.c_void_p(s.base("res")),
+                   C.c_void_p(s.base("w")), C.c_void_p(s.base("m")), C.c_void_p(s.base("v")), N,
+                   self.ks[c.ratio],
                    L.ptr(self._seg_dev["adamw"]), len(self.entries), SCORE_MAP[c.score],
                    C.c_void_p(self.coef_f.data_ptr() + 4 * ci), L.f32(coef_dense),
-                   int(c.optimizer == "adams"), L.ptr(s["spare"]), L.ptr(self.sel_result),
+                   int(c.optimizer == "adams"), 1, L.ptr(s.spare), L.ptr(self.sel_result),
                    L.ptr(self.ws), self.ws_bytes, st)
             if c.dual_lr != 1.0:
-                out_sel[ci] = s["sel"]
-            s["sel"], s["spare"] = s["spare"], s["sel"]
+                out_sel[ci] = s.sel
+            s.sel, s.spare = s.spare, s.sel
         self._fill_cfgs(bnd, out_sel)
         L.call("sga_replay_pass3", L.ptr(g), gd, N, L.f32(coef_dense), self._cfg_host, G,
                L.ptr(self.coef_f), L.ptr(self._rseg_dev), len(self.entries), st)
@@ -179,7 +207,7 @@ class ReplayGroup:
             out = torch.zeros(1, dtype=torch.float64, device=self.dev)
             part = torch.empty(1024, dtype=torch.float64, device=self.dev)
             for ci in range(G):
-                L.call("sga_sq_dist", L.ptr(self.state[ci]["w"]), L.ptr(snapshots[hz]), N,
+                L.call("sga_sq_dist", C.c_void_p(self.state[ci].base("w")), 1, L.ptr(snapshots[hz]), N,
                        L.ptr(part), L.ptr(out), st)
                 self.dist_at[ci][hz] = math.sqrt(float(out.item()))
         self.si += 1
