@@ -6,9 +6,15 @@ One "step" = score |g+r| -> exact top-k (1 %, lowest-index ties) -> index pack
 Llama-3.2-1B-shaped gradient set (1,235,814,400 elements, 146 tensors, bf16
 Student-t(3) gradients, fp32 p/m/v/residual) with every input resident in HBM.
 
+The step is timed on both state layouts: the library-owned packed layout
+(resid/p/m/v interleaved in 64 KiB records -- the headline) and the drop-in
+one (four flat tensors, as the reference's buffers are); both run the same
+arithmetic and produce the same bits.
+
 Prints ONE JSON line: whole-job elements/s, the roofline of the dominant
-kernel (the final sweep, timed live with HIP events on its launch stream) and
-the CPU oracle timed on a bounded sample of the same workload.
+kernel (the final sweep, timed live with HIP events on its launch stream),
+both layouts under "layouts", the fused replay leg and the CPU oracle timed on
+a bounded sample of the same workload.
 """
 import argparse
 import ctypes
@@ -147,8 +153,9 @@ def main():
                     help="also launch one plain copy of 2^30 fp32 (k_calib_copy) so counter "
                          "runs can be scaled against a kernel of known traffic")
     ap.add_argument("--no-replay", action="store_true", help="skip the fused replay leg")
-    ap.add_argument("--no-packed", action="store_true",
-                    help="skip the packed-state variant of the fused step")
+    ap.add_argument("--layout", choices=("both", "packed", "separate"), default="both",
+                    help="state layout(s) to time; the headline is the packed layout unless "
+                         "only the separate one runs")
     ap.add_argument("--only-replay", action="store_true",
                     help="run just the fused replay leg (for profiling) and print its JSON")
     ap.add_argument("--sweep", action="store_true",
@@ -181,11 +188,6 @@ def main():
     fs = FusedSparseStep(n, segs, dev, values_dtype=torch.bfloat16,
                          max_k=k_for(n, 10.0) + 16)
 
-    def run(steps, step0, ratio, score):
-        k = k_for(n, ratio)
-        for s in range(steps):
-            fs.step(grads[(step0 + s) % 2], r, p, m, v, step0 + s + 1, k=k, score=score)
-
     calib = None
     if args.calib:
         cn = 1 << 30
@@ -216,22 +218,51 @@ def main():
         calib["streams"] = {"kernel": "k_calib_streams", "bytes": n * 34, "avg_ms": ms,
                             "GBps": n * 34 / ms / 1e6}
         del sg, sc
-    run(args.warmup, 0, args.ratio, args.score)
-    torch.cuda.synchronize()
-    L.raw("sga_prof_enable", 1)
-    t0 = time.perf_counter()
-    run(args.steps, args.warmup, args.ratio, args.score)
-    torch.cuda.synchronize()
-    dt = time.perf_counter() - t0
-    tot_ms, cnt = ctypes.c_double(0), ctypes.c_int(0)
-    L.call("sga_prof_read", ctypes.byref(tot_ms), ctypes.byref(cnt))
-    L.raw("sga_prof_enable", 0)
-    res = fs.read_result()
-    assert res.status == 0 and res.n_selected == k_for(n, args.ratio), vars(res)
-
     k = k_for(n, args.ratio)
-    final_ms = tot_ms.value / max(cnt.value, 1)
     final_bytes = n * ALG_BYTES_FINAL + k * 6.0
+
+    def time_leg(step_fn, step0):
+        """W warm-up + K timed steps of one layout; returns (seconds, final-sweep ms)."""
+        for s in range(args.warmup):
+            step_fn(step0 + s)
+        torch.cuda.synchronize()
+        L.raw("sga_prof_enable", 1)
+        t0 = time.perf_counter()
+        for s in range(args.steps):
+            step_fn(step0 + args.warmup + s)
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        tot_ms, cnt = ctypes.c_double(0), ctypes.c_int(0)
+        L.call("sga_prof_read", ctypes.byref(tot_ms), ctypes.byref(cnt))
+        L.raw("sga_prof_enable", 0)
+        res = fs.read_result()
+        assert res.status == 0 and res.n_selected == k, vars(res)
+        return dt, tot_ms.value / max(cnt.value, 1), res
+
+    def leg_summary(dt, final_ms):
+        return {"value": n * args.steps / dt, "ms_per_step": dt / args.steps * 1e3,
+                "step_frac": n * args.steps / dt * ALG_BYTES_STEP / HBM_PEAK,
+                "final_avg_ms": final_ms,
+                "final_frac": final_bytes / (final_ms * 1e-3) / HBM_PEAK}
+
+    legs, step0 = {}, 0
+    if args.layout in ("separate", "both"):
+        # the drop-in entry point: resid / p / m / v are the caller's four flat tensors
+        dt_s, ms_s, res = time_leg(
+            lambda t: fs.step(grads[t % 2], r, p, m, v, t + 1, k=k, score=args.score), step0)
+        legs["separate"] = (dt_s, ms_s)
+        step0 += args.warmup + args.steps
+    if args.layout in ("packed", "both"):
+        # the library-owned state layout: the same four arrays interleaved in 64 KiB
+        # records; identical arithmetic and outputs (asserted bitwise by the tests)
+        from sga_amd.fused_step import PackedState
+        st = PackedState(n, dev).pack(r, p, m, v)
+        dt_p, ms_p, res = time_leg(
+            lambda t: fs.step_packed(grads[t % 2], st, t + 1, k=k, score=args.score), step0)
+        legs["packed"] = (dt_p, ms_p)
+        step0 += args.warmup + args.steps
+    head = "packed" if "packed" in legs else "separate"
+    dt, final_ms = legs[head]
     achieved = final_bytes / (final_ms * 1e-3) if final_ms > 0 else 0.0
     traffic = None
     tpath = os.path.join(ROOT, "profiles", "fused_final_llama1b_traffic.json")
@@ -241,6 +272,9 @@ def main():
         except Exception:
             traffic = None
     value = n * args.steps / dt
+    layout_txt = ("resid/p/m/v interleaved in 64 KiB records (sga_fused_sparse_step_packed)"
+                  if head == "packed" else
+                  "resid/p/m/v as four flat tensors (sga_fused_sparse_step)")
     out = {
         "metric": "grad elems/s (score+top-k+resid AdamW)",
         "value": value, "unit": "elem/s", "n_gpus": 1, "steps": args.steps,
@@ -250,8 +284,9 @@ def main():
         "config": {"workload": "Llama-3.2-1B-shaped set, 1,235,814,400 elems / 146 tensors, "
                                "bf16 Student-t(3) grads, fp32 p/m/v/residual, score "
                                f"{args.score}, exact top-k {args.ratio}% (k={k}), index pack "
-                               "int32+bf16, residual-aware AdamW",
-                   "ratio_percent": args.ratio, "score": args.score, "k": k},
+                               "int32+bf16, residual-aware AdamW; state layout: " + layout_txt,
+                   "ratio_percent": args.ratio, "score": args.score, "k": k,
+                   "state_layout": head},
         "roofline": {"bound": "hbm", "achieved": achieved / 1e9, "peak": HBM_PEAK / 1e9,
                      "unit": "GB/s", "frac": achieved / HBM_PEAK, "traffic": traffic,
                      "kernel": "k_fused_final", "avg_ms": final_ms,
@@ -260,39 +295,19 @@ def main():
                           "achieved_GBps": value * ALG_BYTES_STEP / 1e9,
                           "frac": value * ALG_BYTES_STEP / HBM_PEAK},
         "select": {"thresh": res.thresh, "n_gt": res.n_gt, "n_eq": res.n_eq, "path": res.path},
+        "layouts": {name: leg_summary(*v) for name, v in legs.items()},
     }
-    if not args.no_packed:
-        # same workload with resid/p/m/v interleaved in 64 KiB records (the
-        # library-owned state layout); identical arithmetic and outputs
-        from sga_amd.fused_step import PackedState
-        st = PackedState(n, dev).pack(r, p, m, v)
-
-        def run_packed(steps, step0):
-            for s in range(steps):
-                fs.step_packed(grads[(step0 + s) % 2], st, step0 + s + 1, k=k, score=args.score)
-        step0 = args.warmup + args.steps
-        run_packed(args.warmup, step0)
-        torch.cuda.synchronize()
-        L.raw("sga_prof_enable", 1)
-        t1 = time.perf_counter()
-        run_packed(args.steps, step0 + args.warmup)
-        torch.cuda.synchronize()
-        dtp = time.perf_counter() - t1
-        L.call("sga_prof_read", ctypes.byref(tot_ms), ctypes.byref(cnt))
-        L.raw("sga_prof_enable", 0)
-        st.unpack(r, p, m, v)
-        del st
-        pms = tot_ms.value / max(cnt.value, 1)
-        out["packed_state"] = {
-            "layout": "resid/p/m/v interleaved, 64 KiB records (sga_fused_sparse_step_packed)",
-            "value": n * args.steps / dtp, "ms_per_step": dtp / args.steps * 1e3,
-            "step_frac": n * args.steps / dtp * ALG_BYTES_STEP / HBM_PEAK,
-            "final_avg_ms": pms, "final_frac": final_bytes / (pms * 1e-3) / HBM_PEAK}
     if calib:
         out["copy_calibration"] = calib
     if args.sweep:
         sw = []
-        step0 = args.warmup + args.steps
+        def run(steps, t0_, ratio, score):          # on the headline layout
+            kk = k_for(n, ratio)
+            for t in range(t0_, t0_ + steps):
+                if head == "packed":
+                    fs.step_packed(grads[t % 2], st, t + 1, k=kk, score=score)
+                else:
+                    fs.step(grads[t % 2], r, p, m, v, t + 1, k=kk, score=score)
         for score, ratio in (("abs_g", 0.1), ("abs_g", 10.0), ("update", 0.1),
                              ("update", 1.0), ("update", 10.0)):
             run(1, step0, ratio, score)
@@ -305,6 +320,9 @@ def main():
             sw.append({"score": score, "ratio_percent": ratio, "elem_per_s": n / d,
                        "ms_per_step": d * 1e3})
         out["sweep"] = sw
+    if head == "packed":
+        st.unpack(r, p, m, v)
+        del st
     if not args.no_replay:
         del p, m, v, r, grads, fs
         torch.cuda.empty_cache()
