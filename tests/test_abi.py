@@ -79,3 +79,24 @@ def test_oracle_is_not_imported_by_the_product():
             if f.endswith((".py", ".hip", ".hpp")):
                 src = open(os.path.join(dp, f)).read()
                 assert "oracle" not in src.replace("# oracle", ""), f
+
+
+def test_header_is_plain_c_and_struct_sizes_agree(tmp_path):
+    """include/sga_hip.h compiles as C99 on its own, and the struct sizes a C
+    caller sees are the ones the ctypes mirrors use."""
+    import subprocess
+    from sga_amd import _lib as L
+    from sga_amd.replay_group import ReplayCfg, ReplaySegment
+    from sga_amd.selection import SelectResult
+    src = tmp_path / "sizes.c"
+    src.write_text('#include <stdio.h>\n#include "sga_hip.h"\n'
+                   'int main(void) { printf("%zu %zu %zu %zu\\n", sizeof(sga_segment), '
+                   'sizeof(sga_select_result), sizeof(sga_replay_cfg), '
+                   'sizeof(sga_replay_segment)); return 0; }\n')
+    exe = tmp_path / "sizes"
+    subprocess.run(["gcc", "-std=c99", "-Wall", "-Werror", "-pedantic",
+                    "-I", os.path.join(ROOT, "include"), str(src), "-o", str(exe)], check=True)
+    got = [int(x) for x in subprocess.run([str(exe)], check=True, capture_output=True,
+                                          text=True).stdout.split()]
+    assert got == [ctypes.sizeof(L.Segment), ctypes.sizeof(SelectResult),
+                   ctypes.sizeof(ReplayCfg), ctypes.sizeof(ReplaySegment)]
