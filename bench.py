@@ -140,6 +140,63 @@ def replay_bench(G=8, W=32, seed=4):
                         "window, per-config fp32 w/m/v/res + u8 mask resident, clip 1.0"}
 
 
+def trace_io_bench(W=4, tmp=None):
+    """Recorded-trace leg: writes a W-step bf16 trace of the Qwen3-0.6B shapes in
+    the reference writer's layout under a temp dir, then streams it back through
+    the pread reader (page cache warm) -- once on its own and once feeding the
+    dense reference pass -- to measure the PCIe-inclusive rates."""
+    import shutil
+    import tempfile
+    import torch
+    from sga_amd import trace_io as T
+    from sga_amd.replay_dense import DenseReplay
+    from sga_amd.shapes import qwen3_06b
+    dev = torch.device("cuda:0")
+    shapes = qwen3_06b()
+    d = tempfile.mkdtemp(prefix="sga_trace_", dir=tmp)
+    try:
+        cat = {name: {"shape": [n], "dtype": "torch.float32"} for name, n in shapes}
+        meta = {"step": 100, "phase": "shadow", "lr": [1e-4], "grad_norm": float("nan"),
+                "clip_grad": 0.0, "weight_decay": 0.1, "adam_beta1": 0.9, "adam_beta2": 0.95,
+                "adam_eps": 1e-8}
+        T.write_catalog(d, cat, meta, "bf16")
+        gen = torch.Generator().manual_seed(0)
+        zeros = {name: torch.zeros(n) for name, n in shapes}
+        w = {name: torch.randn(n, generator=gen) * 0.02 for name, n in shapes}
+        T.write_state(d, 100, meta, w, zeros, zeros)
+        del zeros
+        for s in range(W):
+            T.write_grad(d, 100 + s, dict(meta, step=100 + s),
+                         {name: (torch.randn(n, generator=gen) * 1e-3) for name, n in shapes},
+                         torch.bfloat16)
+        catalog, names, _o, N, s_files, g_files = T.discover_trace(d)
+        sp = T.ShardParams(names, catalog, meta, 0, N)
+        steps = T.window_steps_for(g_files, 100, W)
+        cache = {}
+        for _gs, _m, g in T.WindowReader(g_files, steps, sp, dev, index_cache=cache):
+            pass                                           # warm: page cache, index, buffers
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _gs, _m, g in T.WindowReader(g_files, steps, sp, dev, index_cache=cache):
+            pass
+        torch.cuda.synchronize()
+        dt_read = time.perf_counter() - t0
+        w0, m0, v0, _ = T.load_branch_state(s_files[100], sp, dev)
+        dense = DenseReplay(sp.entries, w0, m0, v0, 100)
+        t0 = time.perf_counter()
+        for gs, gm, g in T.WindowReader(g_files, steps, sp, dev, index_cache=cache):
+            dense.step(gs, g, gm)
+        torch.cuda.synchronize()
+        dt_dense = time.perf_counter() - t0
+        return {"workload": f"Qwen3-0.6B shapes, {W} recorded bf16 steps ({N} elems each), "
+                            "files in the page cache",
+                "reader_GBps": W * N * 2 / dt_read / 1e9, "reader_ms_per_step": dt_read / W * 1e3,
+                "dense_pass_ms_per_step": dt_dense / W * 1e3,
+                "dense_pass_elem_per_s": W * N / dt_dense}
+    finally:
+        shutil.rmtree(d, ignore_errors=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -156,6 +213,9 @@ def main():
     ap.add_argument("--layout", choices=("both", "packed", "separate"), default="both",
                     help="state layout(s) to time; the headline is the packed layout unless "
                          "only the separate one runs")
+    ap.add_argument("--trace-io", action="store_true",
+                    help="run just the recorded-trace leg (writes a temporary trace, streams it "
+                         "back through the pread reader and the dense pass) and print its JSON")
     ap.add_argument("--only-replay", action="store_true",
                     help="run just the fused replay leg (for profiling) and print its JSON")
     ap.add_argument("--sweep", action="store_true",
@@ -175,6 +235,10 @@ def main():
     if args.only_replay:
         torch.cuda.set_device(0)
         print(json.dumps(replay_bench()))
+        return
+    if args.trace_io:
+        torch.cuda.set_device(0)
+        print(json.dumps(trace_io_bench()))
         return
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)

@@ -313,12 +313,15 @@ class WindowReader:
     iteration step re-uses its slot, so consume it before advancing.
 
     ``depth`` host staging buffers (pinned on a GPU) bound the read-ahead;
-    the upload runs on its own stream and the consumer's current stream is
-    made to wait on it.
+    ``read_threads`` threads copy disjoint pieces of a step out of the page
+    cache side by side (positional reads release the GIL); the upload runs on
+    its own stream and the consumer's current stream is made to wait on it.
     """
 
-    def __init__(self, g_files, window_steps, sp, device, depth=2, index_cache=None):
+    def __init__(self, g_files, window_steps, sp, device, depth=2, index_cache=None,
+                 read_threads=8):
         self.g_files, self.steps, self.sp = g_files, list(window_steps), sp
+        self.read_threads = max(1, int(read_threads))
         self.device = torch.device(device)
         self.index_cache = {} if index_cache is None else index_cache
         self.depth = max(1, int(depth))
@@ -341,6 +344,9 @@ class WindowReader:
         return self._host[key]
 
     def _read_loop(self):
+        from concurrent.futures import ThreadPoolExecutor
+        piece = 32 << 20                       # elements per read task
+        pool = ThreadPoolExecutor(self.read_threads) if self.read_threads > 1 else None
         try:
             for gstep in self.steps:
                 path = self.g_files[gstep]
@@ -361,12 +367,23 @@ class WindowReader:
                 hb, size = _bytes_of(host), _ITEMSIZE[dtype]
                 fd = os.open(path, os.O_RDONLY)
                 try:
+                    # positional reads release the GIL and are independent, so a few
+                    # threads copy disjoint pieces out of the page cache side by side
+                    jobs = []
                     for e, card in cards:
-                        dst = hb[size * e["a"]:size * (e["a"] + e["n"])]
                         if card is None:
-                            dst[:] = 0
-                        else:
-                            tf.read_into(fd, card, e["p_off"], e["n"], dst)
+                            hb[size * e["a"]:size * (e["a"] + e["n"])] = 0
+                            continue
+                        for lo in range(0, e["n"], piece):
+                            cnt = min(piece, e["n"] - lo)
+                            dst = hb[size * (e["a"] + lo):size * (e["a"] + lo + cnt)]
+                            jobs.append((card, e["p_off"] + lo, cnt, dst))
+                    if pool is None:
+                        for card, first, cnt, dst in jobs:
+                            tf.read_into(fd, card, first, cnt, dst)
+                    else:
+                        for fut in [pool.submit(tf.read_into, fd, *j) for j in jobs]:
+                            fut.result()
                 finally:
                     os.close(fd)
                 self._ready.put((gstep, tf.meta, slot, dtype))
@@ -374,6 +391,9 @@ class WindowReader:
         except BaseException as exc:          # surface in the consumer
             self._exc = exc
             self._ready.put(None)
+        finally:
+            if pool is not None:
+                pool.shutdown(wait=False)
 
     def __iter__(self):
         cur = torch.cuda.current_stream(self.device) if self._pin else None
