@@ -188,11 +188,17 @@ def trace_io_bench(W=4, tmp=None):
             dense.step(gs, g, gm)
         torch.cuda.synchronize()
         dt_dense = time.perf_counter() - t0
+        t0 = time.perf_counter()
+        for _ in range(W):                                 # same step, gradient resident
+            dense.step(gs, g, gm)
+        torch.cuda.synchronize()
+        dt_res = time.perf_counter() - t0
         return {"workload": f"Qwen3-0.6B shapes, {W} recorded bf16 steps ({N} elems each), "
                             "files in the page cache",
                 "reader_GBps": W * N * 2 / dt_read / 1e9, "reader_ms_per_step": dt_read / W * 1e3,
                 "dense_pass_ms_per_step": dt_dense / W * 1e3,
-                "dense_pass_elem_per_s": W * N / dt_dense}
+                "dense_pass_elem_per_s": W * N / dt_dense,
+                "dense_step_resident_ms": dt_res / W * 1e3}
     finally:
         shutil.rmtree(d, ignore_errors=True)
 
