@@ -126,10 +126,13 @@ def replay_bench(G=8, W=32, seed=4):
         alg += 2 * 2.0 * n                                   # g in pass 1 and pass 3
         for c in cfgs:
             bnd = s % c.T == 0
-            alg += (4.0 if bnd else 1.0) * n                 # pass 1: res | sel
-            alg += (32.0 if bnd else 33.0) * n               # pass 3: res, m, v, w r/w (+ sel)
+            rz = s == 0 or (s - 1) % c.T == 0                # res is all zeros: no traffic for it
+            alg += ((0.0 if rz else 4.0) if bnd else 1.0) * n  # pass 1: res | sel
+            # pass 3: m, v, w read+write; res read unless zero, written unless it stays zero
+            alg += (24.0 + (0.0 if rz else 4.0) + (0.0 if (bnd and rz) else 4.0)
+                    + (0.0 if bnd else 1.0)) * n
             if bnd and s > 0 and s + 1 < W:
-                per = 6.0 if c.score == "abs_g" else 18.0    # g, res (+ w, m, v)
+                per = (6.0 if c.score == "abs_g" else 18.0) - (4.0 if rz else 0.0)
                 alg += (per + 1.0) * n                       # one score sweep + the new mask
                 n_resel += 1
     return {"metric": "replay config-steps/s", "value": G * W / dt, "unit": "config-steps/s",

@@ -320,6 +320,11 @@ typedef struct sga_replay_cfg {
                              state+8192, state+12288 of ONE packed state (the
                              layout of sga_fused_sparse_step_packed, array
                              order res, w, m, v); the same for every config  */
+  int res_zero;           /* 1: the caller knows res is all zeros when this
+                             step starts (first step, or the step after a
+                             boundary): it is then neither read nor, at a
+                             boundary, rewritten                              */
+  int pad_;
 } sga_replay_cfg;
 
 /* Per-tensor hyper-parameters of the replay commit (ShardParams entries +
@@ -350,7 +355,8 @@ int sga_replay_reselect(const void* g, int g_dtype, const float* res,
                         const float* w, const float* m, const float* v,
                         int64_t n, int64_t k, const sga_segment* segs,
                         int n_segs, int score_id, const float* coef_f,
-                        float coef_dense, int adams, int packed, uint8_t* sel_out,
+                        float coef_dense, int adams, int packed, int res_zero,
+                        uint8_t* sel_out,
                         sga_select_result* result, void* ws, size_t ws_bytes,
                         void* stream);
 

@@ -32,6 +32,8 @@ struct RCfg {
   int adams;
   int split;
   int packed;
+  int res_zero;             // res is known to be all zeros when the step starts
+  int pad_;
 };
 
 struct RGroup {
@@ -56,6 +58,10 @@ __device__ __forceinline__ void load_gd(const void* g, int64_t i, int64_t n, flo
 // so the per-config loads are unrolled and all in flight together: one over
 // the configs at a cycle boundary (q = gd + res), one over the others
 // (q = gd * sel).  Both write their configs' slots of the same partials table.
+struct P1Alias {
+  int src[kMaxCfg];           // partials slot that holds config c's sums
+};
+
 struct P1List {
   const void* ptr[kMaxCfg];   // res (boundary list) or sel (masked list)
   int slot[kMaxCfg];          // config index of each entry
@@ -104,8 +110,13 @@ __global__ __launch_bounds__(kBlock) void k_replay_pass1(const void* __restrict_
 #pragma unroll
       for (int c = 0; c < NC; ++c) {
         const uint8_t* sp = reinterpret_cast<const uint8_t*>(lst.ptr[c]);
-        if (full) ld_u8<true>(sp, i, n, sl[c], true);
-        else load4_u8(sp, i, n, sl[c], vec);
+        if (!sp) {                       // no mask: every coordinate counts (q = gd)
+          sl[c][0] = sl[c][1] = sl[c][2] = sl[c][3] = 1u;
+        } else if (full) {
+          ld_u8<true>(sp, i, n, sl[c], true);
+        } else {
+          load4_u8(sp, i, n, sl[c], vec);
+        }
       }
 #pragma unroll
       for (int c = 0; c < NC; ++c)
@@ -132,10 +143,11 @@ __global__ __launch_bounds__(kBlock) void k_replay_coef(const double* __restrict
                                                         int n_blocks, int G, double clip,
                                                         double* __restrict__ qn2,
                                                         double* __restrict__ coef_d,
-                                                        float* __restrict__ coef_f) {
+                                                        float* __restrict__ coef_f, P1Alias al) {
   for (int c = wave_id(); c < G; c += kChunksPerBlock) {
     double a = 0.0;
-    for (int b = lane_id(); b < n_blocks; b += kWave) a += partials[(int64_t)b * kMaxCfg + c];
+    const int src = al.src[c];
+    for (int b = lane_id(); b < n_blocks; b += kWave) a += partials[(int64_t)b * kMaxCfg + src];
     a = wave_sum(a);
     if (lane_id() == 0) {
       double coef = 1.0;
@@ -198,7 +210,8 @@ __device__ __forceinline__ void pass3_vec(const void* g, int64_t i, int64_t n, f
     float* const WW = cf.w + sh;
     float rr[4], mm[4], vv[4] = {0, 0, 0, 0}, ww[4];
     uint32_t sl[4] = {1, 1, 1, 1}, so[4] = {1, 1, 1, 1};
-    ld_f32<FULL>(RES, i, n, rr, vec);
+    if (cf.res_zero) rr[0] = rr[1] = rr[2] = rr[3] = 0.0f;
+    else ld_f32<FULL>(RES, i, n, rr, vec);
     ld_f32<FULL>(MM, i, n, mm, vec);
     if (!cf.adams) ld_f32<FULL>(VV, i, n, vv, vec);
     ld_f32<FULL>(WW, i, n, ww, vec);
@@ -235,7 +248,7 @@ __device__ __forceinline__ void pass3_vec(const void* g, int64_t i, int64_t n, f
       mm[e] = mn;
       vv[e] = vn;
     }
-    st_f32<FULL>(RES, i, n, rr, vec);
+    if (!(cf.boundary && cf.res_zero)) st_f32<FULL>(RES, i, n, rr, vec);   // zero stays zero
     st_f32<FULL>(MM, i, n, mm, vec);
     st_f32<FULL>(VV, i, n, vv, vec);
     st_f32<FULL>(WW, i, n, ww, vec);
@@ -341,6 +354,7 @@ struct SrcReplay {
   bool vec;
   SegCursor sc;              // b1, b2, eps, wd, bc1, bc2 per tensor (cached per thread)
   int64_t pack_extra;        // 0 or kPackExtra (res/w/m/v of one packed state)
+  int res_zero;              // res is known to be all zeros: not read
   template <bool FULL = false>
   __device__ __forceinline__ void load(int64_t i, int64_t n, uint32_t key[4]) {
     const int64_t sh = pack_shift<FULL>(i, pack_extra);
@@ -350,7 +364,8 @@ struct SrcReplay {
     const float* v = this->v + sh;
     float gd[4], rr[4];
     load_gd<BF16G, FULL>(g, i, n, coef_dense == 1.0f ? 1.0f : 0.0f, coef_dense, gd, vec);
-    ld_f32<FULL>(res, i, n, rr, vec);
+    if (res_zero) rr[0] = rr[1] = rr[2] = rr[3] = 0.0f;
+    else ld_f32<FULL>(res, i, n, rr, vec);
     const float coef = coef_f[0];
     float q[4];
 #pragma unroll
@@ -436,6 +451,8 @@ static bool fill_group(RGroup* grp, const sga_replay_cfg* cfgs, int G) {
     d.out_sel = s.out_sel ? s.out_sel : s.sel;
     d.lr_scale = s.lr_scale; d.boundary = s.boundary; d.adams = s.adams; d.split = s.split;
     d.packed = s.packed != 0;
+    d.res_zero = s.res_zero != 0;
+    d.pad_ = 0;
     if (d.packed != (cfgs[0].packed != 0)) return false;     // one layout per group
   }
   grp->pack_extra = cfgs[0].packed ? kPackExtra : 0;
@@ -501,14 +518,24 @@ extern "C" int sga_replay_pass1(const void* g, int g_dtype, int64_t n, float coe
   const unsigned nb = stream_grid(n, (int64_t)kBlock * kVec, kReplayBlocks);
   hipStream_t s = (hipStream_t)stream;
   P1List lb = {}, lm = {};
-  int n_b = 0, n_m = 0;
+  P1Alias al;
+  int n_b = 0, n_m = 0, plain = -1;
   for (int c = 0; c < G; ++c) {
-    if (grp.c[c].boundary) { lb.ptr[n_b] = grp.c[c].res; lb.slot[n_b++] = c; }
-    else { lm.ptr[n_m] = grp.c[c].sel; lm.slot[n_m++] = c; }
+    al.src[c] = c;
+    if (grp.c[c].boundary && grp.c[c].res_zero) {
+      // q = gd + 0: one unmasked sum of squares serves every such config
+      if (plain < 0) { plain = c; lm.ptr[n_m] = nullptr; lm.slot[n_m++] = c; }
+      al.src[c] = plain;
+    } else if (grp.c[c].boundary) {
+      lb.ptr[n_b] = grp.c[c].res; lb.slot[n_b++] = c;
+    } else {
+      lm.ptr[n_m] = grp.c[c].sel; lm.slot[n_m++] = c;
+    }
   }
+  for (int c = G; c < kMaxCfg; ++c) al.src[c] = 0;
   launch_pass1<true>(bg, n_b, nb, s, g, n, coef_dense, lb, partials, vec, grp.pack_extra);
   launch_pass1<false>(bg, n_m, nb, s, g, n, coef_dense, lm, partials, vec, 0);
-  hipLaunchKernelGGL(k_replay_coef, dim3(1), dim3(kBlock), 0, s, partials, (int)nb, G, clip, qn2, coef_d, coef_f);
+  hipLaunchKernelGGL(k_replay_coef, dim3(1), dim3(kBlock), 0, s, partials, (int)nb, G, clip, qn2, coef_d, coef_f, al);
   return check_launch("sga_replay_pass1");
 }
 
@@ -534,13 +561,13 @@ extern "C" int sga_replay_pass3(const void* g, int g_dtype, int64_t n, float coe
 template <bool BF16G, int SCORE>
 static int run_reselect(const void* g, const float* res, const float* w, const float* m,
                         const float* v, int64_t n, int64_t k, const sga_segment* segs, int n_segs,
-                        const float* coef_f, float coef_dense, int adams, int packed,
+                        const float* coef_f, float coef_dense, int adams, int packed, int res_zero,
                         uint8_t* sel_out, sga_select_result* result, const SelWorkspace& ws,
                         hipStream_t s) {
   const bool vec = aligned4(g, BF16G ? 2 : 4) && aligned4(res, 4) && aligned4(w, 4) &&
                    aligned4(m, 4) && aligned4(v, 4);
   SrcReplay<BF16G, SCORE> src{g, res, w, m, v, coef_f, coef_dense, adams, vec, {},
-                              packed ? kPackExtra : 0};
+                              packed ? kPackExtra : 0, res_zero};
   src.sc.init(segs, n_segs);
   run_select(src, n, k, 0, true, ws, s, true);
   finish_mask(src, n, 0, ws, sel_out, s);
@@ -552,7 +579,7 @@ extern "C" int sga_replay_reselect(const void* g, int g_dtype, const float* res,
                                    const float* m, const float* v, int64_t n, int64_t k,
                                    const sga_segment* segs, int n_segs, int score_id,
                                    const float* coef_f, float coef_dense, int adams, int packed,
-                                   uint8_t* sel_out, sga_select_result* result, void* ws,
+                                   int res_zero, uint8_t* sel_out, sga_select_result* result, void* ws,
                                    size_t ws_bytes, void* stream) {
   if (!g || !res || !w || !m || !v || !segs || !coef_f || !sel_out || n < 1 || n >= (1ll << 31) ||
       k < 1 || k > n || n_segs < 1 || score_id < 0 || score_id > 3 ||
@@ -566,7 +593,7 @@ extern "C" int sga_replay_reselect(const void* g, int g_dtype, const float* res,
     return SGA_ERR_WORKSPACE;
   }
   hipStream_t s = (hipStream_t)stream;
-#define SGA_RS(BG, SC) return run_reselect<BG, SC>(g, res, w, m, v, n, k, segs, n_segs, coef_f, coef_dense, adams, packed, sel_out, result, sw, s)
+#define SGA_RS(BG, SC) return run_reselect<BG, SC>(g, res, w, m, v, n, k, segs, n_segs, coef_f, coef_dense, adams, packed, res_zero, sel_out, result, sw, s)
   if (g_dtype == SGA_BF16) {
     switch (score_id) { case 0: SGA_RS(true, 0); case 1: SGA_RS(true, 1); case 2: SGA_RS(true, 2); default: SGA_RS(true, 3); }
   } else {

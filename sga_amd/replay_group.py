@@ -18,7 +18,8 @@ class ReplayCfg(C.Structure):
     """struct sga_replay_cfg"""
     _fields_ = [("w", C.c_void_p), ("m", C.c_void_p), ("v", C.c_void_p), ("res", C.c_void_p),
                 ("sel", C.c_void_p), ("out_sel", C.c_void_p), ("lr_scale", C.c_double),
-                ("boundary", C.c_int), ("adams", C.c_int), ("split", C.c_int), ("packed", C.c_int)]
+                ("boundary", C.c_int), ("adams", C.c_int), ("split", C.c_int), ("packed", C.c_int),
+                ("res_zero", C.c_int), ("pad_", C.c_int)]
 
 
 class ReplaySegment(C.Structure):
@@ -128,6 +129,9 @@ class ReplayGroup:
         self._seg_up = L.TableUploader(C.sizeof(self._seg_host), dev)
         self._seg_dev = {"adamw": self._seg_up.dev}
         self.dist_at = [dict() for _ in configs]
+        # res is all zeros at the start and again after every boundary commit;
+        # the kernels then skip its traffic (same values either way)
+        self.res_zero = [True] * len(configs)
         self.si = 0
 
     # -- per-step tables ----------------------------------------------------
@@ -155,7 +159,7 @@ class ReplayGroup:
             h.sel = s.sel.data_ptr()
             split = bool(bnd[ci] and c.dual_lr != 1.0)
             h.out_sel = (out_sel.get(ci, s.sel)).data_ptr() if split else None
-            h.lr_scale, h.packed = c.dual_lr, 1
+            h.lr_scale, h.packed, h.res_zero = c.dual_lr, 1, int(self.res_zero[ci])
             h.boundary, h.adams, h.split = int(bnd[ci]), int(c.optimizer == "adams"), int(split)
 
     # -- one recorded step ----------------------------------------------------
@@ -176,7 +180,7 @@ class ReplayGroup:
         st = L.stream()
         if si > 0:                                   # residual fold
             for ci, c in enumerate(self.configs):
-                if bnd[ci] and c.fold:
+                if bnd[ci] and c.fold and not self.res_zero[ci]:
                     L.call("sga_div_inplace", C.c_void_p(self.state[ci].base("res")), N,
                            L.f32(float(c.T)), 1, st)
         self._fill_segments(count, lr_of)
@@ -194,7 +198,8 @@ class ReplayGroup:
                    self.ks[c.ratio],
                    L.ptr(self._seg_dev["adamw"]), len(self.entries), SCORE_MAP[c.score],
                    C.c_void_p(self.coef_f.data_ptr() + 4 * ci), L.f32(coef_dense),
-                   int(c.optimizer == "adams"), 1, L.ptr(s.spare), L.ptr(self.sel_result),
+                   int(c.optimizer == "adams"), 1, int(self.res_zero[ci]), L.ptr(s.spare),
+                   L.ptr(self.sel_result),
                    L.ptr(self.ws), self.ws_bytes, st)
             if c.dual_lr != 1.0:
                 out_sel[ci] = s.sel
@@ -202,6 +207,7 @@ class ReplayGroup:
         self._fill_cfgs(bnd, out_sel)
         L.call("sga_replay_pass3", L.ptr(g), gd, N, L.f32(coef_dense), self._cfg_host, G,
                L.ptr(self.coef_f), L.ptr(self._rseg_dev), len(self.entries), st)
+        self.res_zero = list(bnd)
         hz = si + 1
         if hz in horizons and snapshots is not None:
             out = torch.zeros(1, dtype=torch.float64, device=self.dev)
