@@ -791,7 +791,7 @@ __device__ __forceinline__ void bracket_chunk(Src& src, int64_t n, int64_t c, ui
 }
 
 template <class Src, bool PM>
-__global__ __launch_bounds__(kBlock) void k_bracket_sweep(
+__global__ __launch_bounds__(kBlock, 4) void k_bracket_sweep(
     Src src, int64_t n, SelState* __restrict__ st, const SelState* __restrict__ aux,
     uint32_t* __restrict__ tile_gt, uint32_t* __restrict__ tile_eq, uint32_t* __restrict__ seg_idx,
     uint32_t* __restrict__ seg_key, uint32_t* __restrict__ seg_cnt, uint32_t seg_cap,
