@@ -83,9 +83,10 @@ static inline int64_t fast_seg_cap(int64_t n) {
 }
 
 // Workspace layout: [fixed: states | level histograms | tile-scan block sums]
-// [tile_gt[nt] | tile_eq[nt]] [fast-path buffers sized from nt].  nt is
-// derived from the byte size, so every entry point recovers the same carve
-// from (ws, ws_bytes) alone.
+// [tile_gt[nt] | tile_eq[nt]] [fast-path buffers sized from nt: sample keys,
+// per-wave candidate segments, dense candidates, 128 B of bit planes per
+// tile].  nt is derived from the byte size, so every entry point recovers
+// the same carve from (ws, ws_bytes) alone.
 constexpr int kHistEntries = 2 * kBinsBig + kBinsSmall;      // 8320
 constexpr int kHistStride = kHistEntries + 64;               // per-state stride
 constexpr size_t kSelFixedBytes =
