@@ -127,13 +127,13 @@ def replay_bench(G=8, W=32, seed=4):
         for c in cfgs:
             bnd = s % c.T == 0
             rz = s == 0 or (s - 1) % c.T == 0                # res is all zeros: no traffic for it
-            alg += ((0.0 if rz else 4.0) if bnd else 1.0) * n  # pass 1: res | sel
+            alg += ((0.0 if rz else 4.0) if bnd else 0.125) * n  # pass 1: res | sel (1 bit)
             # pass 3: m, v, w read+write; res read unless zero, written unless it stays zero
             alg += (24.0 + (0.0 if rz else 4.0) + (0.0 if (bnd and rz) else 4.0)
-                    + (0.0 if bnd else 1.0)) * n
+                    + (0.0 if bnd else 0.125)) * n
             if bnd and s > 0 and s + 1 < W:
                 per = (6.0 if c.score == "abs_g" else 18.0) - (4.0 if rz else 0.0)
-                alg += (per + 1.0) * n                       # one score sweep + the new mask
+                alg += (per + 0.125) * n                     # one score sweep + the new mask bits
                 n_resel += 1
     return {"metric": "replay config-steps/s", "value": G * W / dt, "unit": "config-steps/s",
             "ms_per_window": dt * 1e3, "G": G, "W": W, "n": n, "reselects": n_resel,

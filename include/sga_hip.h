@@ -304,14 +304,18 @@ int sga_state_repack(float* resid, float* p, float* m, float* v, float* state,
 
 /* One configuration's resident state for the current recorded step
  * (states[c][param] = {ms, vs, ws, res, sel}, replay_fused.py:1548-1567),
- * flattened over the shard.  sel / out_sel are byte masks (0/1). */
+ * flattened over the shard.  sel / out_sel are masks kept as BIT PLANES
+ * (sga_plane_words(n) uint32 each): per 1024-element chunk 32 words; element
+ * i = c*1024 + it*256 + lane*4 + e is bit (lane & 31) of word
+ * (i >> 8)*8 + 2*e + (lane >> 5) -- four wave64 ballots per 256 elements.
+ * sga_mask_to_planes / sga_planes_to_mask convert from and to byte masks. */
 typedef struct sga_replay_cfg {
   float* w;
   float* m;
   float* v;
   float* res;
-  const uint8_t* sel;
-  const uint8_t* out_sel; /* outgoing mask for the dual-lr split; NULL = sel */
+  const uint32_t* sel;
+  const uint32_t* out_sel; /* outgoing mask for the dual-lr split; NULL = sel */
   double lr_scale;        /* dual-lr scale, lr_inactive = lr * lr_scale      */
   int boundary;           /* si % T == 0                                     */
   int adams;              /* optimizer == "adams"                            */
@@ -356,7 +360,7 @@ int sga_replay_reselect(const void* g, int g_dtype, const float* res,
                         int64_t n, int64_t k, const sga_segment* segs,
                         int n_segs, int score_id, const float* coef_f,
                         float coef_dense, int adams, int packed, int res_zero,
-                        uint8_t* sel_out,
+                        uint32_t* sel_out,
                         sga_select_result* result, void* ws, size_t ws_bytes,
                         void* stream);
 
@@ -376,6 +380,13 @@ int sga_dense_replay_step(const void* g, int g_dtype, float* w, float* m, float*
                           float* lab, int64_t n, const sga_replay_segment* segs,
                           int n_segs, int adams, double coef_dense, double* partials,
                           double* recon2, void* stream);
+
+/* Bit-plane masks (layout above). */
+int64_t sga_plane_words(int64_t n);
+int sga_mask_to_planes(const uint8_t* mask, int64_t n, uint32_t* planes,
+                       void* stream);
+int sga_planes_to_mask(const uint32_t* planes, int64_t n, uint8_t* mask,
+                       void* stream);
 
 /* res /= T at fold boundaries (replay_fused.py:1632-1636), true division.
  * packed != 0: x is the run base of one array inside a packed state. */

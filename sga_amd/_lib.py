@@ -74,6 +74,9 @@ SIGNATURES = {
     "sga_replay_pass3": (I32, [P, I32, I64, F, P, I32, P, P, I32, P]),
     "sga_branch_score_f64": (I32, [I32, P, P, P, P, P, I64] + [C.c_double] * 6 + [I32, I32, P]),
     "sga_dense_replay_step": (I32, [P, I32, P, P, P, P, I64, P, I32, I32, C.c_double, P, P, P]),
+    "sga_plane_words": (I64, [I64]),
+    "sga_mask_to_planes": (I32, [P, I64, P, P]),
+    "sga_planes_to_mask": (I32, [P, I64, P, P]),
     "sga_div_inplace": (I32, [P, I64, F, I32, P]),
     "sga_sq_dist": (I32, [P, I32, P, I64, P, P, P]),
     "sga_calib_copy": (I32, [P, P, I64, P]),

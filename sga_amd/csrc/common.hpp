@@ -245,6 +245,42 @@ __device__ __forceinline__ void st_u8(uint8_t* base, int64_t i, int64_t n, const
   }
 }
 
+// Selection masks as bit planes: per 1024-element chunk c and 256-element
+// slab `it`, eight words; word 2e + h of the slab holds, for the element e of
+// each lane, the lanes [32h, 32h + 32) -- exactly four wave ballots.  Element
+// i = c*1024 + it*256 + lane*4 + e is bit (lane & 31) of word
+// planes[(i >> 8) * 8 + 2*e + (lane >> 5)].  i must be a multiple of 4.
+constexpr int kPlaneWordsPerChunk = 32;
+// UNIFORM promises that every lane of the wave addresses the same slab
+// (chunk- or workgroup-structured sweeps): the slab's eight words are then
+// fetched through one wave-uniform address.
+template <bool UNIFORM = false>
+__device__ __forceinline__ void plane_flags4(const uint32_t* __restrict__ planes, int64_t i,
+                                             uint32_t out[4]) {
+  const int l = (int)(i >> 2) & (kWave - 1);
+  int64_t slab = i >> 8;
+  if (UNIFORM) slab = __builtin_amdgcn_readfirstlane((int)slab);
+  const U4* w = reinterpret_cast<const U4*>(planes + slab * 8);
+  const U4 a = w[0], b = w[1];
+  const bool hi = l >= 32;
+  const uint32_t s = l & 31;
+  out[0] = ((hi ? a.y : a.x) >> s) & 1u;
+  out[1] = ((hi ? a.w : a.z) >> s) & 1u;
+  out[2] = ((hi ? b.y : b.x) >> s) & 1u;
+  out[3] = ((hi ? b.w : b.z) >> s) & 1u;
+}
+
+// Four ballots of a slab -> the lane's word of the chunk's 32 (lane 8*it + 2e + h).
+__device__ __forceinline__ void plane_collect(const uint32_t flag[4], int it, uint32_t& word) {
+  const uint64_t b0 = ballot64(flag[0] != 0), b1 = ballot64(flag[1] != 0);
+  const uint64_t b2 = ballot64(flag[2] != 0), b3 = ballot64(flag[3] != 0);
+  const int l = lane_id();
+  if ((l >> 3) == it) {
+    const uint64_t bb = (l & 4) ? ((l & 2) ? b3 : b2) : ((l & 2) ? b1 : b0);
+    word = (l & 1) ? (uint32_t)(bb >> 32) : (uint32_t)bb;
+  }
+}
+
 #endif  // __HIPCC__
 
 }  // namespace sga

@@ -25,8 +25,8 @@ struct RCfg {
   float* m;
   float* v;
   float* res;
-  const uint8_t* sel;       // current mask (bytes 0/1)
-  const uint8_t* out_sel;   // outgoing mask for the dual-lr split (may equal sel)
+  const uint32_t* sel;      // current mask, bit planes (common.hpp: plane_flags4)
+  const uint32_t* out_sel;  // outgoing mask for the dual-lr split (may equal sel)
   double lr_scale;          // dual-lr scale (lr_inactive = lr * lr_scale)
   int boundary;
   int adams;
@@ -109,13 +109,11 @@ __global__ __launch_bounds__(kBlock) void k_replay_pass1(const void* __restrict_
       uint32_t sl[NC][4];
 #pragma unroll
       for (int c = 0; c < NC; ++c) {
-        const uint8_t* sp = reinterpret_cast<const uint8_t*>(lst.ptr[c]);
+        const uint32_t* sp = reinterpret_cast<const uint32_t*>(lst.ptr[c]);
         if (!sp) {                       // no mask: every coordinate counts (q = gd)
           sl[c][0] = sl[c][1] = sl[c][2] = sl[c][3] = 1u;
-        } else if (full) {
-          ld_u8<true>(sp, i, n, sl[c], true);
         } else {
-          load4_u8(sp, i, n, sl[c], vec);
+          plane_flags4<true>(sp, i, sl[c]);    // bits past n are zero
         }
       }
 #pragma unroll
@@ -215,8 +213,8 @@ __device__ __forceinline__ void pass3_vec(const void* g, int64_t i, int64_t n, f
     ld_f32<FULL>(MM, i, n, mm, vec);
     if (!cf.adams) ld_f32<FULL>(VV, i, n, vv, vec);
     ld_f32<FULL>(WW, i, n, ww, vec);
-    if (!cf.boundary) ld_u8<FULL>(cf.sel, i, n, sl, vec);
-    if (cf.split) ld_u8<FULL>(cf.out_sel, i, n, so, vec);
+    if (!cf.boundary) plane_flags4<true>(cf.sel, i, sl);
+    if (cf.split) plane_flags4<true>(cf.out_sel, i, so);
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
       if (!FULL && i + e >= n) continue;
@@ -464,7 +462,7 @@ static bool group_aligned(const RGroup& grp) {
   for (int c = 0; c < grp.G; ++c) {
     const RCfg& d = grp.c[c];
     if (!aligned4(d.w, 4) || !aligned4(d.m, 4) || !aligned4(d.v, 4) || !aligned4(d.res, 4) ||
-        !aligned4(d.sel, 1) || !aligned4(d.out_sel, 1))
+        !aligned4(d.sel, 1) || !aligned4(d.out_sel, 1))   // 4-byte words
       return false;
   }
   return true;
@@ -562,15 +560,15 @@ template <bool BF16G, int SCORE>
 static int run_reselect(const void* g, const float* res, const float* w, const float* m,
                         const float* v, int64_t n, int64_t k, const sga_segment* segs, int n_segs,
                         const float* coef_f, float coef_dense, int adams, int packed, int res_zero,
-                        uint8_t* sel_out, sga_select_result* result, const SelWorkspace& ws,
+                        uint32_t* sel_out, sga_select_result* result, const SelWorkspace& ws,
                         hipStream_t s) {
   const bool vec = aligned4(g, BF16G ? 2 : 4) && aligned4(res, 4) && aligned4(w, 4) &&
                    aligned4(m, 4) && aligned4(v, 4);
   SrcReplay<BF16G, SCORE> src{g, res, w, m, v, coef_f, coef_dense, adams, vec, {},
                               packed ? kPackExtra : 0, res_zero};
   src.sc.init(segs, n_segs);
-  run_select(src, n, k, 0, true, ws, s, true);
-  finish_mask(src, n, 0, ws, sel_out, s);
+  run_select(src, n, k, 0, true, ws, s, sel_out);
+  finish_planes(src, n, 0, ws, sel_out, s);
   if (result) hipLaunchKernelGGL(k_sel_result, dim3(1), dim3(1), 0, s, ws.st, result);
   return check_launch("sga_replay_reselect");
 }
@@ -579,7 +577,7 @@ extern "C" int sga_replay_reselect(const void* g, int g_dtype, const float* res,
                                    const float* m, const float* v, int64_t n, int64_t k,
                                    const sga_segment* segs, int n_segs, int score_id,
                                    const float* coef_f, float coef_dense, int adams, int packed,
-                                   int res_zero, uint8_t* sel_out, sga_select_result* result, void* ws,
+                                   int res_zero, uint32_t* sel_out, sga_select_result* result, void* ws,
                                    size_t ws_bytes, void* stream) {
   if (!g || !res || !w || !m || !v || !segs || !coef_f || !sel_out || n < 1 || n >= (1ll << 31) ||
       k < 1 || k > n || n_segs < 1 || score_id < 0 || score_id > 3 ||
@@ -621,6 +619,27 @@ extern "C" int sga_dense_replay_step(const void* g, int g_dtype, float* w, float
   else hipLaunchKernelGGL((k_dense_step<false>), dim3(nb), dim3(kBlock), 0, s, g, n, w, m, v, lab, adams, coef_dense, rs, n_segs, partials, vec);
   hipLaunchKernelGGL(k_sqdist_stage2, dim3(1), dim3(kWave), 0, s, partials, (int)nb, recon2);
   return check_launch("sga_dense_replay_step");
+}
+
+extern "C" int64_t sga_plane_words(int64_t n) {
+  return n <= 0 ? 0 : cdiv64(n, kChunk) * kPlaneWordsPerChunk;
+}
+
+extern "C" int sga_mask_to_planes(const uint8_t* mask, int64_t n, uint32_t* planes, void* stream) {
+  if (n == 0) return SGA_OK;
+  if (!mask || !planes || n < 0) { set_error("sga_mask_to_planes: bad argument"); return SGA_ERR_ARG; }
+  hipLaunchKernelGGL(k_mask_to_planes, dim3(stream_grid(cdiv64(n, kChunk), kChunksPerBlock, 1 << 14)),
+                     dim3(kBlock), 0, (hipStream_t)stream, mask, n, planes, aligned4(mask, 1));
+  return check_launch("sga_mask_to_planes");
+}
+
+extern "C" int sga_planes_to_mask(const uint32_t* planes, int64_t n, uint8_t* mask, void* stream) {
+  if (n == 0) return SGA_OK;
+  if (!mask || !planes || n < 0) { set_error("sga_planes_to_mask: bad argument"); return SGA_ERR_ARG; }
+  hipLaunchKernelGGL(k_expand_mask, dim3(stream_grid(cdiv64(n, kChunk), kChunksPerBlock, 1 << 14)),
+                     dim3(kBlock), 0, (hipStream_t)stream, (const SelState*)nullptr, planes, n, mask,
+                     (reinterpret_cast<uintptr_t>(mask) & 15) == 0);
+  return check_launch("sga_planes_to_mask");
 }
 
 extern "C" int sga_div_inplace(float* x, int64_t n, float d, int packed, void* stream) {

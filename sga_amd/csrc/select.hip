@@ -268,7 +268,7 @@ extern "C" int sga_select_topk(const float* score, int64_t n, int64_t k, int tie
   hipStream_t s = (hipStream_t)stream;
   SrcF32 src{score, aligned4(score, 4)};
   const int tie_all = tie_mode == SGA_TIE_ALL;
-  run_select(src, n, k, tie_all, true, w, s, true);
+  run_select(src, n, k, tie_all, true, w, s, w.pbits);
   finish_mask(src, n, tie_all, w, mask_out, s);
   if (result) hipLaunchKernelGGL(k_sel_result, dim3(1), dim3(1), 0, s, w.st, result);
   return check_launch("sga_select_topk");

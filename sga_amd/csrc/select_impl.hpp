@@ -766,15 +766,8 @@ __device__ __forceinline__ void bracket_chunk(Src& src, int64_t n, int64_t c, ui
     if (PM) {
       // provisional mask as bit planes: everything above the bracket is
       // certainly selected; the few keys inside it are settled after the
-      // candidate descent.  Lane 8*it + 2e + h keeps the word with lanes
-      // [32h, 32h+32) of element e of slab `it`; one 128-byte store per chunk.
-      const uint64_t b0 = ballot64(above[0]), b1 = ballot64(above[1]);
-      const uint64_t b2 = ballot64(above[2]), b3 = ballot64(above[3]);
-      const int l = lane_id();
-      if ((l >> 3) == it) {
-        const uint64_t bb = (l & 4) ? ((l & 2) ? b3 : b2) : ((l & 2) ? b1 : b0);
-        pword = (l & 1) ? (uint32_t)(bb >> 32) : (uint32_t)bb;
-      }
+      // candidate descent.  One 128-byte store per chunk.
+      plane_collect(above, it, pword);
     }
     if (ballot64(mine != 0)) {
       const uint32_t incl = wave_incl_scan(mine);
@@ -917,7 +910,7 @@ static_assert(kChunk == 1024, "candidate -> chunk mapping uses idx >> 10");
 static __global__ __launch_bounds__(kBlock) void k_expand_mask(
     const SelState* __restrict__ st, const uint32_t* __restrict__ pbits, int64_t n,
     uint8_t* __restrict__ mask, bool mvec) {
-  if (!st->bracket_ok) return;
+  if (st && !st->bracket_ok) return;
   const int64_t n_chunks = cdiv64(n, kChunk);
   const int64_t wstride = (int64_t)gridDim.x * kChunksPerBlock;
   const int l = lane_id();
@@ -980,6 +973,96 @@ static __global__ __launch_bounds__(kBlock) void k_cand_mask(
   }
 }
 
+// The same settlement when the mask itself is kept as bit planes.
+static __global__ __launch_bounds__(kBlock) void k_cand_bits(
+    const SelState* __restrict__ st, const uint32_t* __restrict__ cand_idx,
+    const uint32_t* __restrict__ cand_key, const uint32_t* __restrict__ tile_eq,
+    int64_t n_tiles, int tie_all, uint32_t* __restrict__ planes) {
+  if (!st->bracket_ok) return;
+  const uint32_t T = st->thresh_bits, nc = st->cand_count, n_eq = st->n_eq;
+  const uint32_t need = tie_all ? 0xFFFFFFFFu : st->need;
+  for (uint32_t j = blockIdx.x * kBlock + threadIdx.x; j < nc; j += gridDim.x * kBlock) {
+    const uint32_t key = cand_key[j];
+    if (key < T) continue;
+    const uint32_t idx = cand_idx[j];
+    bool on = true;
+    if (key == T && need < n_eq) {
+      const uint32_t c = idx >> 10;
+      const uint32_t before = tile_eq[c];
+      const uint32_t upto = (int64_t)c + 1 < n_tiles ? tile_eq[c + 1] : n_eq;
+      if (before >= need) {
+        on = false;
+      } else if (upto > need) {
+        uint32_t rank = before;
+        for (uint32_t q = j; q > 0 && (cand_idx[q - 1] >> 10) == c; --q)
+          rank += cand_key[q - 1] == T;
+        on = rank < need;
+      }
+    }
+    if (on) {
+      const uint32_t lane = (idx >> 2) & 63u, e = idx & 3u;
+      atomicOr(&planes[(idx >> 8) * 8 + 2 * e + (lane >> 5)], 1u << (lane & 31));
+    }
+  }
+}
+
+// Ordered full pass that writes the mask as bit planes (the fallback of
+// k_cand_bits when the sampled bracket failed or was never tried).
+template <class Src>
+__global__ __launch_bounds__(kBlock) void k_write_bits(Src src, int64_t n, int tie_all,
+                                                       const SelState* __restrict__ st,
+                                                       const uint32_t* __restrict__ tile_sel,
+                                                       const uint32_t* __restrict__ tile_eq,
+                                                       uint32_t* __restrict__ planes) {
+  if (st->bracket_ok) return;
+  const uint32_t T = st->thresh_bits;
+  const uint32_t need = tie_all ? 0xFFFFFFFFu : st->need;
+  const int64_t n_chunks = cdiv64(n, kChunk);
+  const int64_t wstride = (int64_t)gridDim.x * kChunksPerBlock;
+  for (int64_t c = (int64_t)blockIdx.x * kChunksPerBlock + wave_id(); c < n_chunks; c += wstride) {
+    ChunkCursor cur;
+    cur.sel_run = tile_sel[c];
+    cur.eq_run = tile_eq[c];
+    const bool full = src.vec && (c + 1) * kChunk <= n;
+    uint32_t word = 0u;
+#pragma unroll
+    for (int it = 0; it < kChunkIters; ++it) {
+      const int64_t i = c * kChunk + it * (kWave * kVec) + lane_id() * kVec;
+      uint32_t key[4] = {0u, 0u, 0u, 0u};
+      if (full) src.template load<true>(i, n, key);
+      else if (i < n) src.template load<false>(i, n, key);
+      bool valid[4], sel[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) valid[e] = full || i + e < n;
+      uint32_t pos;
+      slab_select(key, valid, T, need, cur, sel, pos);
+      const uint32_t flag[4] = {sel[0], sel[1], sel[2], sel[3]};
+      plane_collect(flag, it, word);
+    }
+    if (lane_id() < 32) planes[c * kPlaneWordsPerChunk + lane_id()] = word;
+  }
+}
+
+// Byte mask -> bit planes (chunk-structured, planes sized for cdiv(n, 1024) chunks).
+static __global__ __launch_bounds__(kBlock) void k_mask_to_planes(const uint8_t* __restrict__ mask,
+                                                                  int64_t n,
+                                                                  uint32_t* __restrict__ planes,
+                                                                  bool mvec) {
+  const int64_t n_chunks = cdiv64(n, kChunk);
+  const int64_t wstride = (int64_t)gridDim.x * kChunksPerBlock;
+  for (int64_t c = (int64_t)blockIdx.x * kChunksPerBlock + wave_id(); c < n_chunks; c += wstride) {
+    uint32_t word = 0u;
+#pragma unroll
+    for (int it = 0; it < kChunkIters; ++it) {
+      const int64_t i = c * kChunk + it * (kWave * kVec) + lane_id() * kVec;
+      uint32_t mk[4] = {0u, 0u, 0u, 0u};
+      if (i < n) load4_u8(mask, i, n, mk, mvec);
+      plane_collect(mk, it, word);
+    }
+    if (lane_id() < 32) planes[c * kPlaneWordsPerChunk + lane_id()] = word;
+  }
+}
+
 // Persistent grid of the bracket sweep = exactly what the device holds at
 // once for THIS instantiation (a partial second round would idle most of the
 // chip).
@@ -1001,12 +1084,14 @@ static inline int sweep_grid() {
   return blocks;
 }
 
-// want_mask: the sweep also records, as bit planes, which keys lie above the
-// bracket, so a caller that only wants the mask can finish from those bits
-// and the candidates (finish_mask) instead of re-reading the data.
+// planes (optional): the sweep also records there, as bit planes, which keys
+// lie above the bracket, so a caller that only wants the mask can finish from
+// those bits and the candidates (finish_mask / finish_planes) instead of
+// re-reading the data.
 template <class Src>
 static inline void run_select(Src src, int64_t n, int64_t k, int tie_all, bool fast,
-                              const SelWorkspace& w, hipStream_t s, bool want_mask = false) {
+                              const SelWorkspace& w, hipStream_t s, uint32_t* planes = nullptr) {
+  const bool want_mask = planes != nullptr;
   const int64_t n_tiles = cdiv64(n, kChunk);
   launch_begin((uint32_t)k, w, s);
   if (fast && n >= kFastMinN && w.sample && n < (1ll << 32)) {
@@ -1028,7 +1113,7 @@ static inline void run_select(Src src, int64_t n, int64_t k, int tie_all, bool f
     if (want_mask)
       hipLaunchKernelGGL((k_bracket_sweep<Src, true>), dim3(sweep_blocks), dim3(kBlock), 0, s,
                          src, n, w.st, w.aux, w.tile_gt, w.tile_eq, w.seg_idx, w.seg_key, w.seg_cnt,
-                         (uint32_t)w.seg_cap, w.pbits);
+                         (uint32_t)w.seg_cap, planes);
     else
       hipLaunchKernelGGL((k_bracket_sweep<Src, false>), dim3(sweep_blocks), dim3(kBlock), 0, s,
                          src, n, w.st, w.aux, w.tile_gt, w.tile_eq, w.seg_idx, w.seg_key, w.seg_cnt,
@@ -1054,9 +1139,23 @@ static inline void run_select(Src src, int64_t n, int64_t k, int tie_all, bool f
   launch_tile_scan(n_tiles, tie_all, w, s);
 }
 
-// Mask of the selection after run_select(..., want_mask = true): the bit
-// planes and the candidates settle it when the bracket held, else the
-// ordered full pass writes it.
+// Bit-plane mask of the selection after run_select(..., planes): the
+// candidates settle the sweep's planes when the bracket held, else the
+// ordered full pass writes them.
+template <class Src>
+static inline void finish_planes(Src src, int64_t n, int tie_all, const SelWorkspace& w,
+                                 uint32_t* planes, hipStream_t s) {
+  const int64_t nc = cdiv64(n, kChunk);
+  if (w.cand_idx && n >= kFastMinN && n < (1ll << 32))
+    hipLaunchKernelGGL(k_cand_bits, dim3(256), dim3(kBlock), 0, s, w.st, w.cand_idx, w.cand_key,
+                       w.tile_eq, nc, tie_all, planes);
+  hipLaunchKernelGGL((k_write_bits<Src>), dim3(stream_grid(nc, kChunksPerBlock, 1 << 14)),
+                     dim3(kBlock), 0, s, src, n, tie_all, w.st, w.tile_gt, w.tile_eq, planes);
+}
+
+// Byte mask of the selection after run_select(..., w.pbits): the bit planes
+// and the candidates settle it when the bracket held, else the ordered full
+// pass writes it.
 template <class Src>
 static inline void finish_mask(Src src, int64_t n, int tie_all, const SelWorkspace& w,
                                uint8_t* mask, hipStream_t s) {

@@ -60,7 +60,8 @@ _ARRAY_SLOT = {"res": 0, "w": 1, "m": 2, "v": 3}
 class ConfigState:
     """One config's resident state: res / w / m / v interleaved in one packed
     buffer (64 KiB records, array order res, w, m, v) plus the byte masks.
-    ``state["w"]`` etc. return flat unpacked copies for inspection."""
+    ``state["w"]`` etc. return flat unpacked copies for inspection,
+    ``state["sel"]`` the mask expanded to bytes."""
 
     def __init__(self, n, w0, m0, v0, sel):
         dev = w0.device
@@ -69,16 +70,23 @@ class ConfigState:
                                 device=dev)
         L.call("sga_state_repack", None, L.ptr(w0), L.ptr(m0), L.ptr(v0), L.ptr(self.data), n, 0,
                L.stream())
-        self.sel = sel.reshape(-1).to(torch.uint8).clone()
-        self.spare = torch.empty(n, dtype=torch.uint8, device=dev)
+        # masks live as bit planes (four wave ballots per 256 elements): the
+        # re-selection writes them directly and the sweeps read 1 bit per element
+        words = int(L.raw("sga_plane_words", n))
+        self.sel = torch.zeros(words, dtype=torch.int32, device=dev)
+        self.spare = torch.zeros(words, dtype=torch.int32, device=dev)
+        m8 = sel.reshape(-1).to(torch.uint8).contiguous()
+        L.call("sga_mask_to_planes", L.ptr(m8), n, L.ptr(self.sel), L.stream())
 
     def base(self, name):
         """Device address of an array's first run inside the packed buffer."""
         return self.data.data_ptr() + 4 * _RUN * _ARRAY_SLOT[name]
 
     def __getitem__(self, name):
-        if name in ("sel", "spare"):
-            return getattr(self, name)
+        if name == "sel":
+            out = torch.empty(self.n, dtype=torch.uint8, device=self.data.device)
+            L.call("sga_planes_to_mask", L.ptr(self.sel), self.n, L.ptr(out), L.stream())
+            return out
         out = torch.empty(self.n, dtype=torch.float32, device=self.data.device)
         args = [None] * 4
         args[_ARRAY_SLOT[name]] = L.ptr(out)
