@@ -56,6 +56,21 @@ def _flat_views(views):
     return out
 
 
+def _flat_span(views):
+    """The views as ONE flat tensor when they are back-to-back slices of the
+    same storage (a bucket's per-param views usually are), else None."""
+    first = views[0]
+    store = first.untyped_storage()
+    end = first.data_ptr()
+    for g in views:
+        if g.untyped_storage().data_ptr() != store.data_ptr() or g.data_ptr() != end:
+            return None
+        end += g.numel() * 4
+    total = sum(g.numel() for g in views)
+    return torch.empty(0, dtype=torch.float32, device=first.device).set_(
+        store, first.storage_offset(), (total,), (1,))
+
+
 def select_exact_device(views, k, tie_mode, masks=None):
     """Exact top-k over a list of flat fp32 views; returns (result, masks).
     Views are laid out back to back in chunk space, each on a fresh
@@ -74,6 +89,18 @@ def select_exact_device(views, k, tie_mode, masks=None):
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
     res = torch.empty(8, dtype=torch.int32, device=dev)
     st = L.stream()
+    flat = _flat_span(views) if (masks is None and len(views) > 1) else None
+    if flat is not None:
+        # adjacent slices of one buffer: flat-index order is the view order, so
+        # the whole list is one array for the single-call entry point
+        fmask = torch.empty(n_total, dtype=torch.uint8, device=dev)
+        L.call("sga_select_topk", L.ptr(flat), n_total, k, tie_mode, L.ptr(fmask), L.ptr(res),
+               L.ptr(ws), ws_bytes, st)
+        out, off = [], 0
+        for g in views:
+            out.append(fmask[off:off + g.numel()])
+            off += g.numel()
+        return res, out
     if masks is None:
         masks = [torch.empty(g.numel(), dtype=torch.uint8, device=dev) for g in views]
     if len(views) == 1:

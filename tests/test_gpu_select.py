@@ -298,3 +298,34 @@ def test_adaptive_tau_trajectory_matches_oracle(dev):
     sel.select(SimpleNamespace(grad_views=[torch.zeros(64, device=dev)], comm_group=None,
                                warmup_target=0))
     assert sel.tau == OS.bin_edge_float(1, 19)
+
+
+def test_adjacent_views_take_the_flat_path(dev):
+    """Per-param views that are back-to-back slices of one buffer are selected
+    as one flat array (one sweep); the masks equal those of the same data held
+    in separate tensors (per-view passes) and the oracle's."""
+    from sga_amd import _lib as L
+    from sga_amd.selection import read_result, select_exact_device, select_masks_histogram
+    sizes = [300_001, 7, 1 << 20, 65_536, 1023]
+    n = sum(sizes)
+    flat = student_t(n, 4).to(torch.bfloat16).float()          # quantised: ties at the cut
+    buf = flat.to(dev)
+    views, clones, off = [], [], 0
+    for s in sizes:
+        views.append(buf[off:off + s])
+        clones.append(buf[off:off + s].clone())
+        off += s
+    for k in (n // 1000, n // 100, n // 7):
+        for tie in (L.TIE_LOWEST_INDEX, L.TIE_ALL):
+            ra, ma = select_exact_device(views, k, tie)
+            rb, mb = select_exact_device(clones, k, tie)
+            a, b = read_result(ra), read_result(rb)
+            assert a.path == 1 and b.path == 0             # one sweep vs the per-view passes
+            assert (a.thresh_bits, a.n_selected) == (b.thresh_bits, b.n_selected)
+            for x, y in zip(ma, mb):
+                assert torch.equal(x, y)
+        m_ref, t_ref = SEL.select_topk_flat(flat.abs(), k)
+        assert torch.equal(torch.cat(select_exact_device(views, k, L.TIE_LOWEST_INDEX)[1]).cpu().bool(),
+                           m_ref)
+        th, masks = select_masks_histogram(views, k, mode="exact")
+        assert th == t_ref and torch.equal(torch.cat(masks).cpu().bool(), flat.abs() >= t_ref)
