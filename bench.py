@@ -143,6 +143,48 @@ def replay_bench(G=8, W=32, seed=4):
                         "window, per-config fp32 w/m/v/res + u8 mask resident, clip 1.0"}
 
 
+def replay_cpu_baseline(G=8, W=8, seed=4, frac=24):
+    """The oracle's group loop (the reference's eager torch chain) on a 1/frac
+    prefix of the Qwen3-0.6B tensor list, same config draw as replay_bench, W
+    steps; the rate is scaled linearly to the full shard."""
+    import random
+    import torch
+    from oracle import replay as OR
+    from oracle import select as SEL
+    from sga_amd.shapes import qwen3_06b, segments_for
+    from tests.util import student_t
+    full_n = sum(n for _, n in qwen3_06b())
+    shapes, acc = [], 0
+    for name, n in qwen3_06b()[1:]:               # layer tensors, skipping the embedding
+        if acc + n > full_n // frac:
+            break
+        shapes.append((name, n))
+        acc += n
+    segs, n = segments_for(shapes)
+    entries = [{"a": s["start"], "n": s["n"], "b1": s["b1"], "b2": s["b2"], "eps": s["eps"],
+                "wd": s["wd"]} for s in segs]
+    rnd = random.Random(seed)
+    axes = [(sc, r, t) for sc in ("abs_g", "update", "coi") for r in (0.1, 1.0, 10.0)
+            for t in (1, 4, 16)]
+    cfgs = [OR.Config(*p) for p in rnd.sample(axes, G)]
+    gen = torch.Generator().manual_seed(1)
+    w0 = torch.randn(n, generator=gen) * 0.02
+    m0 = torch.randn(n, generator=gen) * 1e-4
+    v0 = torch.rand(n, generator=gen) * 1e-8
+    window = [(student_t(n, 500 + s) * (1.0 + 0.02 * s)).to(torch.bfloat16) for s in range(W)]
+    base = window[0].float().abs()
+    sel0 = [SEL.select_topk_flat(base, SEL.replay_k(n, c.ratio))[0] for c in cfgs]
+    metas = [{"clip_grad": 1.0, "grad_norm": float("nan"), "lr": 1e-4}] * W
+    t0 = time.perf_counter()
+    OR.group_replay(entries, w0, m0, v0, sel0, cfgs, window, metas, 100)
+    dt = time.perf_counter() - t0
+    return {"value": G * W / dt * n / full_n, "unit": "config-steps/s", "cores": torch.get_num_threads(),
+            "kind": "port",
+            "sample": f"{len(shapes)} layer tensors of the Qwen3-0.6B list ({n} elements = 1/"
+                      f"{full_n / n:.1f} of the shard), G={G}, W={W}, {dt:.1f} s; rate scaled "
+                      f"linearly to the full shard; host cpu_count={os.cpu_count()}"}
+
+
 def trace_io_bench(W=4, tmp=None):
     """Recorded-trace leg: writes a W-step bf16 trace of the Qwen3-0.6B shapes in
     the reference writer's layout under a temp dir, then streams it back through
@@ -402,6 +444,8 @@ def main():
         out["replay"] = replay_bench()
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(args.cpu_sample, 3, args.ratio)
+        if "replay" in out:
+            out["replay"]["cpu_baseline"] = replay_cpu_baseline()
     else:
         out["cpu_baseline"] = None
     print(json.dumps(out))
