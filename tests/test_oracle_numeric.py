@@ -341,3 +341,130 @@ def test_adams_grad_correct_vs_f64():
         ref = _f64_scores(p, m, v, g, b1, b2, eps, wd, 1.0, 1.0, adams=True)
         torch.testing.assert_close(g3.double(), ref[name], rtol=1e-5,
                                    atol=2e-6 if name == "coi" else 1e-7)
+
+
+def test_trace_dense_replay_against_fp64_recursion(tmp_path):
+    """oracle.trace.dense_replay (the dense reference pass over a recorded
+    window) against the textbook AdamW recursion in float64: weights, label
+    sum((lr*upd)^2), horizon norms ||w - w0|| and the pre-clip reconstruction
+    norm sqrt(sum((g/coef)^2))."""
+    import math
+    from oracle import trace as OT
+    from trace_fixture import make_trace
+    d = str(tmp_path)
+    W, t0 = 6, 10
+    make_trace(d, steps=W, clip=0.3)
+    cat, names, numel, s_files, g_files = OT.discover(d)
+    st = OT.load_file(s_files[t0])
+    entries = OT.entries_for(cat, names, numel, st["meta"])
+    n = sum(numel.values())
+    w0, m0, v0 = (OT.flat_slice(st["payload"][k], entries, n) for k in ("w", "m", "v"))
+    gs, metas = [], []
+    for s in range(t0, t0 + W):
+        f = OT.load_file(g_files[s])
+        gs.append(OT.flat_slice(f["payload"], entries, n))
+        metas.append(f["meta"])
+    lab, lab_total, den, recon, snaps = OT.dense_replay(entries, w0, m0, v0, gs, metas, t0, (3, 6))
+    w, m, v = w0.double(), m0.double(), v0.double()
+    lab64 = torch.zeros(n, dtype=torch.float64)
+    for si in range(W):
+        g = gs[si].double()
+        for e in entries:
+            a, b = e["a"], e["a"] + e["n"]
+            lr = metas[si]["lr"][e["group"]]
+            t = t0 + si + 1
+            m[a:b] = e["b1"] * m[a:b] + (1 - e["b1"]) * g[a:b]
+            v[a:b] = e["b2"] * v[a:b] + (1 - e["b2"]) * g[a:b] ** 2
+            upd = (m[a:b] / (1 - e["b1"] ** t)) / ((v[a:b] / (1 - e["b2"] ** t)).sqrt() + e["eps"])
+            w[a:b] = w[a:b] * (1 - lr * e["wd"]) - lr * upd
+            lab64[a:b] += (lr * upd) ** 2
+        coef = min(1.0, metas[si]["clip_grad"] / (metas[si]["grad_norm"] + 1e-6))
+        assert recon[si]["coef_dense"] == coef
+        ref_norm = math.sqrt(float(((g / coef) ** 2).sum()))
+        assert abs(recon[si]["recon_grad_norm"] - ref_norm) <= 1e-9 * ref_norm
+        # the fixture records post-clip gradients: g / coef is the pre-clip gradient
+        assert abs(ref_norm - metas[si]["grad_norm"]) <= 1e-5 * ref_norm
+        if si + 1 in (3, 6):
+            ref_den = math.sqrt(float(((w - w0.double()) ** 2).sum()))
+            assert abs(den[si + 1] - ref_den) <= 1e-4 * ref_den
+            assert float((snaps[si + 1].double() - w).abs().max()) <= 1e-6
+    assert float((lab.double() - lab64).abs().max()) <= 1e-5 * float(lab64.max())
+    assert abs(lab_total - float(lab64.sum())) <= 1e-5 * float(lab64.sum())
+
+
+def test_trace_branch_scores_against_fp64_closed_form():
+    """oracle.trace.branch_scores: |registry score| in double, rounded once to
+    fp32 -- against the formulas written out independently in float64."""
+    from oracle import trace as OT
+    gen = torch.Generator().manual_seed(3)
+    n = 50_000
+    w = torch.randn(n, generator=gen) * 0.02
+    m = torch.randn(n, generator=gen) * 1e-3
+    v = torch.rand(n, generator=gen) * 1e-5 + 1e-12
+    g = torch.randn(n, generator=gen) * 1e-2
+    e = {"a": 0, "n": n, "b1": 0.9, "b2": 0.95, "eps": 1e-8, "wd": 0.1}
+    t = 11
+    W, M, V, G = (x.double() for x in (w, m, v, g))
+    bc1, bc2 = 1 - 0.9 ** t, 1 - 0.95 ** t
+    def u(gg, vv, c1, c2):
+        return ((0.9 * M + 0.1 * gg) / c1) / (((0.95 * vv + 0.05 * gg * gg) / c2).sqrt() + 1e-8)
+    want = {("abs_g", "adamw"): G.abs(), ("abs_m", "adams"): M.abs(),
+            ("update", "adamw"): (0.1 * W + u(G, V, bc1, bc2)).abs(),
+            ("update", "adams"): (0.1 * W + u(G, M * M, 1.0, 1.0)).abs(),
+            ("coi", "adamw"): (u(G, V, bc1, bc2) - u(torch.zeros_like(G), V, bc1, bc2)).abs(),
+            ("coi", "adams"): (u(G, M * M, 1.0, 1.0) - u(torch.zeros_like(G), M * M, 1.0, 1.0)).abs()}
+    for (score, opt), ref in want.items():
+        got = OT.branch_scores(score, opt, [e], w, m, v, g, t).double()
+        # fp32 rounding of the result (2^-24) plus operand-scale cancellation for coi
+        scale = ref.abs() + (3.0 if score == "coi" else 0.0) * 1e-7
+        assert float(((got - ref).abs() / (scale + 1e-30)).max()) <= 2e-7, (score, opt)
+
+
+def test_clip_routes_against_closed_form():
+    """oracle.clip.masked_clip_grad_norm: norm = sqrt of the fp64 sum over the
+    contributing coordinates; coefficient clip/(norm+1e-6); each route scales
+    exactly the coordinates engine.py:1172-1216 scales."""
+    from types import SimpleNamespace
+    from oracle.clip import masked_clip_grad_norm
+
+    class Rec:
+        def __init__(self, grad, bucket, a, b):
+            self.grad, self.bucket_state, self.a, self.b = grad, bucket, a, b
+
+        def mask_u8(self):
+            m = self.bucket_state.active_mask_u8
+            return None if m is None else m[self.a:self.b]
+
+    def build(masked_tail=True):
+        gen = torch.Generator().manual_seed(2)
+        flat = torch.randn(3000, generator=gen)
+        mask = (torch.rand(3000, generator=gen) < 0.1).to(torch.uint8)
+        b = SimpleNamespace(active_mask_u8=mask)
+        b2 = SimpleNamespace(active_mask_u8=mask if masked_tail else None)
+        recs = [Rec(flat[0:1000], b, 0, 1000), Rec(flat[1000:3000], b2, 1000, 3000)]
+        return recs, flat, mask
+
+    recs, flat, mask = build()
+    before = flat.clone()
+    full = float(flat.double().pow(2).sum().sqrt())
+    sel = float(flat.double()[mask > 0].pow(2).sum().sqrt())
+    n, c = masked_clip_grad_norm(recs, 0.0, True)
+    assert abs(n - full) < 1e-5 * full and c == 1.0 and torch.equal(flat, before)
+    n, c = masked_clip_grad_norm(recs, 0.5 * full, True)          # full step: scaled in place
+    assert c == 1.0 and torch.allclose(flat, before * (0.5 * full / (n + 1e-6)), rtol=1e-6)
+    recs, flat, mask = build()
+    before = flat.clone()
+    n, c = masked_clip_grad_norm(recs, 0.5 * sel, False)          # sparse: coefficient handed on
+    assert abs(n - sel) < 1e-5 * sel and abs(c - 0.5 * sel / (n + 1e-6)) < 1e-12
+    assert torch.equal(flat, before)
+    n, c = masked_clip_grad_norm(recs, 0.5 * sel, False, trace_dumps=True)   # dump step
+    assert c == 1.0 and torch.equal(flat[mask == 0], before[mask == 0])
+    assert torch.allclose(flat[mask > 0], before[mask > 0] * (0.5 * sel / (n + 1e-6)), rtol=1e-6)
+    recs, flat, mask = build(masked_tail=False)                   # mask-less record counts whole
+    before = flat.clone()
+    mix = float((before.double()[:1000][mask[:1000] > 0].pow(2).sum()
+                 + before.double()[1000:].pow(2).sum()).sqrt())
+    n, c = masked_clip_grad_norm(recs, 0.5 * mix, False)
+    assert abs(n - mix) < 1e-5 * mix and c < 1.0
+    assert torch.equal(flat[:1000], before[:1000])
+    assert torch.allclose(flat[1000:], before[1000:] * c, rtol=1e-6)
