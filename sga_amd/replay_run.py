@@ -11,8 +11,8 @@ from .replay_dense import dense_replay_dev
 from .replay_fused import shard_select_balanced
 from .replay_group import Config, ReplayGroup
 from .scores import SCORE_MAP
-from .trace_io import (ShardParams, TraceFile, WindowReader, discover_trace, load_branch_state,
-                       lr_for_step, window_steps_for)
+from .trace_io import (ResidentWindow, ShardParams, TraceFile, WindowReader, discover_trace,
+                       load_branch_state, lr_for_step, window_steps_for)
 
 
 def branch_scores(score, optimizer, sp, w0, m0, v0, g0, count, include_wd=True):
@@ -68,10 +68,12 @@ def replay_window(trace_dir, t0, window, configs, horizons, device,
     cache = {}
     out = {"N": N, "window_steps": steps, "horizons": eff_h, "dense": {}, "configs": []}
     snaps = {}
+    # the trace is read once; every later pass iterates the device-resident copy
+    window = ResidentWindow(
+        lambda: WindowReader(g_files, steps, sp, device, depth=depth, index_cache=cache), W, N)
     for opt in sorted({c.optimizer for c in configs}):
-        reader = WindowReader(g_files, steps, sp, device, depth=depth, index_cache=cache)
         total, den_at, recon, snap, dense = dense_replay_dev(
-            sp.entries, w0, m0, v0, reader, t0, eff_h, optimizer=opt)
+            sp.entries, w0, m0, v0, window, t0, eff_h, optimizer=opt)
         out["dense"][opt] = {"label_total": total, "den_at": den_at, "recon_steps": recon,
                              "label": dense.label}
         snaps[opt] = snap
@@ -94,8 +96,7 @@ def replay_window(trace_dir, t0, window, configs, horizons, device,
     for opt, idxs in by_opt.items():
         group = ReplayGroup(sp.entries, w0, m0, v0, [sel0[i] for i in idxs],
                             [configs[i] for i in idxs], t0, W)
-        reader = WindowReader(g_files, steps, sp, device, depth=depth, index_cache=cache)
-        for _gstep, gmeta, g in reader:
+        for _gstep, gmeta, g in window:
             meta = {"clip_grad": gmeta.get("clip_grad", 0.0),
                     "grad_norm": gmeta.get("grad_norm", float("nan")),
                     "lr": (lambda e, gm=gmeta: lr_for_step(gm, e.get("group")))}

@@ -441,6 +441,32 @@ class WindowReader:
         self._free.put(None)
 
 
+class ResidentWindow:
+    """Keeps a window's gradients on the device after the first pass over a
+    ``WindowReader`` so that later passes (the dense reference pass, then one
+    streaming pass per optimizer family) re-read HBM instead of the trace: a
+    32-step bf16 window of a 0.6 B-element shard is 38 GB of the 288 GB.
+    Falls back to re-reading when the window would not fit ``budget_bytes``."""
+
+    def __init__(self, make_reader, n_steps, shard_elems, budget_bytes=96 << 30):
+        self._make_reader = make_reader
+        self._keep = n_steps * shard_elems * 4 <= budget_bytes      # worst case fp32
+        self._held = None
+
+    def __iter__(self):
+        if self._held is not None:
+            yield from self._held
+            return
+        held = []
+        for gstep, meta, g in self._make_reader():
+            if self._keep:
+                g = g.clone()
+                held.append((gstep, meta, g))
+            yield gstep, meta, g
+        if self._keep:
+            self._held = held
+
+
 # ------------------------------------------------------------------- writing
 def write_catalog(trace_dir, catalog, meta, g_dtype="fp32"):
     """``catalog.pt`` in the writer's layout (``sga/trace.py:770-799``):
