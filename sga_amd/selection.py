@@ -89,7 +89,14 @@ def select_exact_device(views, k, tie_mode, masks=None):
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
     res = torch.empty(8, dtype=torch.int32, device=dev)
     st = L.stream()
-    flat = _flat_span(views) if (masks is None and len(views) > 1) else None
+    flat = None
+    if masks is None and len(views) > 1:
+        flat = _flat_span(views)
+        if flat is None and n_total >= (1 << 20):
+            # scattered views: one staging copy (8 B/elem) buys the one-sweep
+            # select (5 B/elem) instead of five per-view passes (21 B/elem
+            # and five launches per view)
+            flat = torch.cat(views)
     if flat is not None:
         # adjacent slices of one buffer: flat-index order is the view order, so
         # the whole list is one array for the single-call entry point

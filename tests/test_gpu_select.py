@@ -302,8 +302,9 @@ def test_adaptive_tau_trajectory_matches_oracle(dev):
 
 def test_adjacent_views_take_the_flat_path(dev):
     """Per-param views that are back-to-back slices of one buffer are selected
-    as one flat array (one sweep); the masks equal those of the same data held
-    in separate tensors (per-view passes) and the oracle's."""
+    as one flat array (one sweep) in place; scattered tensors are staged into
+    one buffer first.  Both give the oracle's masks; explicit mask buffers keep
+    the per-view passes, which must agree too."""
     from sga_amd import _lib as L
     from sga_amd.selection import read_result, select_exact_device, select_masks_histogram
     sizes = [300_001, 7, 1 << 20, 65_536, 1023]
@@ -320,12 +321,15 @@ def test_adjacent_views_take_the_flat_path(dev):
             ra, ma = select_exact_device(views, k, tie)
             rb, mb = select_exact_device(clones, k, tie)
             a, b = read_result(ra), read_result(rb)
-            assert a.path == 1 and b.path == 0             # one sweep vs the per-view passes
+            assert a.path == 1 and b.path == 1             # both end up as one flat sweep
             assert (a.thresh_bits, a.n_selected) == (b.thresh_bits, b.n_selected)
             for x, y in zip(ma, mb):
                 assert torch.equal(x, y)
         m_ref, t_ref = SEL.select_topk_flat(flat.abs(), k)
         assert torch.equal(torch.cat(select_exact_device(views, k, L.TIE_LOWEST_INDEX)[1]).cpu().bool(),
                            m_ref)
+        own = [torch.empty(s, dtype=torch.uint8, device=dev) for s in sizes]
+        rc, mc = select_exact_device(clones, k, L.TIE_LOWEST_INDEX, masks=own)
+        assert read_result(rc).path == 0 and torch.equal(torch.cat(mc).cpu().bool(), m_ref)
         th, masks = select_masks_histogram(views, k, mode="exact")
         assert th == t_ref and torch.equal(torch.cat(masks).cpu().bool(), flat.abs() >= t_ref)
