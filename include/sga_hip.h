@@ -156,6 +156,30 @@ int sga_adamw_grad_correct(float* p, float* g, float* m, float* v,
                            float coeff, float interval, float lr_inactive,
                            int emit_mode, int flags, void* stream);
 
+/* The same commit over many records (one per parameter tensor) in ONE launch:
+ * what SgaAdamW's per-record loop (adamw.py:869-905) issues as one kernel per
+ * record.  recs: DEVICE table of n_recs records ordered by first_span; record
+ * r covers spans [first_span, first_span + ceil(n / 4096)), total_spans is the
+ * sum.  flags are per record (SGA_GC_*; a record without a mask carries none
+ * of HAS_MASK / APPLY_COEFF / CLEAR / FOLD / LR_SPLIT), with the same legality
+ * rules as sga_adamw_grad_correct -- checked by the host wrapper, the table
+ * being device memory.  bc1 / bc2 must be 1 for SGA_GC_ADAMS records. */
+typedef struct sga_gc_record {
+  float* p;
+  float* g;
+  float* m;
+  float* v;
+  const uint8_t* mask;     /* NULL when the record has no mask */
+  int64_t n;
+  int64_t first_span;
+  float lr, beta1, om1, beta2, om2, eps, wd, bc1, bc2, lr_inactive;
+  int flags;
+  int pad_;
+} sga_gc_record;
+int sga_adamw_grad_correct_multi(const sga_gc_record* recs, int n_recs,
+                                 int64_t total_spans, float coeff,
+                                 float interval, int emit_mode, void* stream);
+
 /* adamw_grad_correct_compact, adamw.py:217-322, 637-792: the commit reads its
  * gradient from the bucket-level sorted (idx, values) by merge-join.
  * flags: SGA_GC_APPLY_COEFF | SGA_GC_FOLD | SGA_GC_ADAMS (adams.py:507-654).

@@ -38,5 +38,6 @@ def _commit_compact(p, g, m, v, idx, values, rec_start, lr, b1, b2, eps, wd, ste
 
 class SgaAdamS(SgaAdamW):
     """``adams.py:657-850``: feature-identical to SgaAdamW, AdamS step math."""
+    _adams = True
     _commit = staticmethod(_commit)
     _commit_compact = staticmethod(_commit_compact)

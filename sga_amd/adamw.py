@@ -2,6 +2,7 @@
 (``sga/plugins/optimizer/adamw.py``): ``adamw_grad_correct``,
 ``adamw_grad_correct_compact``, ``build_dir_table`` and ``SgaAdamW`` with the
 reference's signatures, refusals and step order."""
+import ctypes as C
 import math
 from dataclasses import dataclass, field
 from types import SimpleNamespace
@@ -24,15 +25,10 @@ def _flat32(**named):
     L.require_contig(**named)
 
 
-def adamw_grad_correct(param_buffer, grad_buffer, exp_avg_buffer, exp_avg_sq_buffer,
-                       lr, beta1, beta2, eps, weight_decay, step, mask=None,
-                       emit_score: Optional[str] = None, coeff=1.0, clear=False,
-                       fold=False, interval=1.0, inactive_lr_scale=1.0, _adams=False):
-    """One fused commit on contiguous same-size 1-D fp32 buffers
-    (``adamw.py:502-634``).  ``emit_score=None`` is the sparse step; a score
-    name is the full step that also writes that score into ``grad_buffer``."""
-    bias_correction1 = 1.0 - beta1 ** step
-    bias_correction2 = 1.0 - beta2 ** step
+def _gc_prepare(param_buffer, grad_buffer, exp_avg_buffer, exp_avg_sq_buffer, mask,
+                emit_score, coeff, clear, fold, inactive_lr_scale, adams):
+    """The refusals of ``adamw.py:554-592`` and the launch flags; returns
+    ``(flags, mask_u8)``."""
     if emit_score is not None and emit_score not in SCORE_MAP:
         raise ValueError(
             f"emit_score '{emit_score}' has no _grad_correct_kernel branch "
@@ -59,7 +55,7 @@ def adamw_grad_correct(param_buffer, grad_buffer, exp_avg_buffer, exp_avg_sq_buf
             "the boundary split, or drop the mask for the mask-blind full step")
     n = param_buffer.numel()
     if n == 0:
-        return
+        return 0, None
     L.require_dev(param_buffer, grad_buffer, exp_avg_buffer, exp_avg_sq_buffer, mask)
     _flat32(param_buffer=param_buffer, grad_buffer=grad_buffer,
             exp_avg_buffer=exp_avg_buffer, exp_avg_sq_buffer=exp_avg_sq_buffer)
@@ -78,8 +74,25 @@ def adamw_grad_correct(param_buffer, grad_buffer, exp_avg_buffer, exp_avg_sq_buf
         flags |= L.GC_FOLD
     if inactive_lr_scale != 1.0:
         flags |= L.GC_LR_SPLIT
-    if _adams:
+    if adams:
         flags |= L.GC_ADAMS
+    return flags, mk
+
+
+def adamw_grad_correct(param_buffer, grad_buffer, exp_avg_buffer, exp_avg_sq_buffer,
+                       lr, beta1, beta2, eps, weight_decay, step, mask=None,
+                       emit_score: Optional[str] = None, coeff=1.0, clear=False,
+                       fold=False, interval=1.0, inactive_lr_scale=1.0, _adams=False):
+    """One fused commit on contiguous same-size 1-D fp32 buffers
+    (``adamw.py:502-634``).  ``emit_score=None`` is the sparse step; a score
+    name is the full step that also writes that score into ``grad_buffer``."""
+    bias_correction1 = 1.0 - beta1 ** step
+    bias_correction2 = 1.0 - beta2 ** step
+    flags, mk = _gc_prepare(param_buffer, grad_buffer, exp_avg_buffer, exp_avg_sq_buffer, mask,
+                            emit_score, coeff, clear, fold, inactive_lr_scale, _adams)
+    n = param_buffer.numel()
+    if n == 0:
+        return
     L.call("sga_adamw_grad_correct", L.ptr(param_buffer), L.ptr(grad_buffer),
            L.ptr(exp_avg_buffer), L.ptr(exp_avg_sq_buffer), L.ptr(mk), n, L.f32(lr),
            L.f32(beta1), L.f32(1.0 - beta1), L.f32(beta2), L.f32(1.0 - beta2),
@@ -87,6 +100,67 @@ def adamw_grad_correct(param_buffer, grad_buffer, exp_avg_buffer, exp_avg_sq_buf
            L.f32(bias_correction2), L.f32(coeff), L.f32(interval),
            L.f32(lr * inactive_lr_scale),
            SCORE_MAP[emit_score] if emit_score is not None else -1, flags, L.stream())
+
+
+class GcRecord(C.Structure):
+    """struct sga_gc_record"""
+    _fields_ = [("p", C.c_void_p), ("g", C.c_void_p), ("m", C.c_void_p), ("v", C.c_void_p),
+                ("mask", C.c_void_p), ("n", C.c_int64), ("first_span", C.c_int64)] + \
+               [(k, C.c_float) for k in ("lr", "beta1", "om1", "beta2", "om2", "eps", "wd",
+                                         "bc1", "bc2", "lr_inactive")] + \
+               [("flags", C.c_int), ("pad_", C.c_int)]
+
+
+_SPAN = 4096
+_uploaders = {}
+
+
+def adamw_grad_correct_multi(records, emit_score=None, coeff=1.0, interval=1.0, _adams=False):
+    """The commit of ``adamw_grad_correct`` over many records in one launch.
+
+    ``records``: dicts with the tensors ``p, g, m, v`` (flat fp32), ``mask``
+    (or None) and the scalars ``lr, beta1, beta2, eps, weight_decay, step``
+    plus the per-record knobs ``coeff_on, clear, fold, inactive_lr_scale``
+    (a record without a mask takes none of them).  Same refusals as the
+    single-record call, raised before anything is launched.
+    """
+    table, keep, spans = [], [], 0
+    for r in records:
+        c = coeff if r.get("coeff_on", True) else 1.0
+        flags, mk = _gc_prepare(r["p"], r["g"], r["m"], r["v"], r.get("mask"), emit_score, c,
+                                bool(r.get("clear", False)), bool(r.get("fold", False)),
+                                float(r.get("inactive_lr_scale", 1.0)), _adams)
+        n = r["p"].numel()
+        if n == 0:
+            continue
+        if c == 1.0:
+            flags &= ~L.GC_APPLY_COEFF
+        step = r["step"]
+        e = GcRecord()
+        e.p, e.g, e.m, e.v = (t.data_ptr() for t in (r["p"], r["g"], r["m"], r["v"]))
+        e.mask = mk.data_ptr() if mk is not None else None
+        e.n, e.first_span = n, spans
+        e.lr, e.beta1, e.om1 = L.f32(r["lr"]), L.f32(r["beta1"]), L.f32(1.0 - r["beta1"])
+        e.beta2, e.om2 = L.f32(r["beta2"]), L.f32(1.0 - r["beta2"])
+        e.eps, e.wd = L.f32(r["eps"]), L.f32(r["weight_decay"])
+        e.bc1 = 1.0 if _adams else L.f32(1.0 - r["beta1"] ** step)
+        e.bc2 = 1.0 if _adams else L.f32(1.0 - r["beta2"] ** step)
+        e.lr_inactive = L.f32(r["lr"] * float(r.get("inactive_lr_scale", 1.0)))
+        e.flags = flags
+        table.append(e)
+        keep.append(mk)
+        spans += -(-n // _SPAN)
+    if not table:
+        return
+    arr = (GcRecord * len(table))(*table)
+    dev = records[0]["p"].device
+    key = (dev, C.sizeof(arr))
+    up = _uploaders.get(key)
+    if up is None:
+        up = _uploaders[key] = L.TableUploader(C.sizeof(arr), dev)
+    up.upload(arr)
+    L.call("sga_adamw_grad_correct_multi", L.ptr(up.dev), len(table), spans, L.f32(coeff),
+           L.f32(interval), SCORE_MAP[emit_score] if emit_score is not None else -1, L.stream())
 
 
 def build_dir_table(idx, total_n):
@@ -237,19 +311,25 @@ class SgaAdamW:
             st["exp_avg_sq"] = torch.zeros_like(rec.main_param.data)
         return st
 
+    _adams = False            # SgaAdamS: the AdamS recursion in the same kernels
+
     def _records_pass(self, ctx, emit_score, use_mask, coeff=1.0, clear=False,
                       fold=False, interval=1.0, inactive_lr_scale=1.0):
+        # every record of the step in ONE launch (the reference issues one kernel
+        # per record, adamw.py:869-905); per-record knobs as in that loop
+        table = []
         for rec in ctx.records:
             st = self._state(rec)
             m = rec.mask_u8() if use_mask else None
-            self._commit(
-                rec.main_param.data.view(-1), rec.grad.data.view(-1),
-                st["exp_avg"].view(-1), st["exp_avg_sq"].view(-1), rec.lr, rec.beta1,
-                rec.beta2, rec.eps, rec.weight_decay, rec.step, mask=m,
-                emit_score=emit_score, coeff=coeff if m is not None else 1.0,
-                clear=clear and m is not None, fold=fold and m is not None,
-                interval=interval,
-                inactive_lr_scale=inactive_lr_scale if m is not None else 1.0)
+            table.append(dict(
+                p=rec.main_param.data.view(-1), g=rec.grad.data.view(-1),
+                m=st["exp_avg"].view(-1), v=st["exp_avg_sq"].view(-1), mask=m, lr=rec.lr,
+                beta1=rec.beta1, beta2=rec.beta2, eps=rec.eps, weight_decay=rec.weight_decay,
+                step=rec.step, coeff_on=m is not None, clear=clear and m is not None,
+                fold=fold and m is not None,
+                inactive_lr_scale=inactive_lr_scale if m is not None else 1.0))
+        adamw_grad_correct_multi(table, emit_score=emit_score, coeff=coeff, interval=interval,
+                                 _adams=self._adams)
 
     def _records_pass_compact(self, ctx, coeff=1.0, fold=False, interval=1.0):
         for rec in ctx.records:

@@ -13,60 +13,105 @@
 
 namespace sga {
 
+// One 4-element vector of the masked / full-step commit.
 // EMIT: -1 sparse step; 0 update, 1 |g|, 2 |m|, 3 coi -> written into g.
 template <int EMIT>
-__global__ __launch_bounds__(kBlock) void k_grad_correct(
-    float* __restrict__ p, float* __restrict__ g, float* __restrict__ m,
-    float* __restrict__ v, const uint8_t* __restrict__ mask, int64_t n, Hyper h,
-    float coeff, float interval, float lr_inactive, int flags, bool vec) {
+__device__ __forceinline__ void gc_vec(float* __restrict__ p, float* __restrict__ g,
+                                       float* __restrict__ m, float* __restrict__ v,
+                                       const uint8_t* __restrict__ mask, int64_t i, int64_t n,
+                                       const Hyper& h, float coeff, float interval,
+                                       float lr_inactive, int flags, bool vec) {
   const bool has_mask = flags & SGA_GC_HAS_MASK;
   const bool apply_coeff = flags & SGA_GC_APPLY_COEFF;
   const bool clear = flags & SGA_GC_CLEAR;
   const bool fold = flags & SGA_GC_FOLD;
   const bool split = flags & SGA_GC_LR_SPLIT;
   const bool adams = flags & SGA_GC_ADAMS;   // v basis = pre-commit m*m, h.bc1 = h.bc2 = 1
+  float pp[4], gg[4], mm[4], vv[4];
+  uint32_t mk[4] = {1, 1, 1, 1};
+  load4_f32(p, i, n, pp, vec);
+  load4_f32(g, i, n, gg, vec);
+  load4_f32(m, i, n, mm, vec);
+  if (adams) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) vv[e] = mm[e] * mm[e];
+  } else {
+    load4_f32(v, i, n, vv, vec);
+  }
+  if (has_mask) load4_u8(mask, i, n, mk, vec);
+  float gout[4];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const bool active = mk[e] != 0;
+    const float raw = gg[e];
+    float ge = raw;
+    if (EMIT < 0 && has_mask && !active) ge = 0.0f;
+    if (apply_coeff && active) ge = ge * coeff;
+    const Commit c = adamw_commit(pp[e], ge, mm[e], vv[e], h);
+    if (EMIT == 0) gout[e] = c.upd;
+    else if (EMIT == 1) gout[e] = fabsf(ge);
+    else if (EMIT == 2) gout[e] = fabsf(mm[e]);
+    else if (EMIT == 3) gout[e] = fabsf(c.u - coi_u0(mm[e], vv[e], h));
+    else {
+      float t = (clear && active) ? 0.0f : raw;
+      if (fold) t = __fdiv_rn(t, interval);
+      gout[e] = t;
+    }
+    const float lr_a = (split && !active) ? lr_inactive : h.lr;
+    pp[e] = pp[e] - lr_a * c.upd;
+    mm[e] = c.m_new;
+    vv[e] = c.v_new;
+  }
+  store4_f32(m, i, n, mm, vec);
+  store4_f32(v, i, n, vv, vec);
+  if (EMIT >= 0 || clear || fold) store4_f32(g, i, n, gout, vec);
+  store4_f32(p, i, n, pp, vec);
+}
+
+template <int EMIT>
+__global__ __launch_bounds__(kBlock) void k_grad_correct(
+    float* __restrict__ p, float* __restrict__ g, float* __restrict__ m,
+    float* __restrict__ v, const uint8_t* __restrict__ mask, int64_t n, Hyper h,
+    float coeff, float interval, float lr_inactive, int flags, bool vec) {
   const int64_t stride = (int64_t)gridDim.x * kBlock * kVec;
-  for (int64_t i = ((int64_t)blockIdx.x * kBlock + threadIdx.x) * kVec; i < n;
-       i += stride) {
-    float pp[4], gg[4], mm[4], vv[4];
-    uint32_t mk[4] = {1, 1, 1, 1};
-    load4_f32(p, i, n, pp, vec);
-    load4_f32(g, i, n, gg, vec);
-    load4_f32(m, i, n, mm, vec);
-    if (adams) {
+  for (int64_t i = ((int64_t)blockIdx.x * kBlock + threadIdx.x) * kVec; i < n; i += stride)
+    gc_vec<EMIT>(p, g, m, v, mask, i, n, h, coeff, interval, lr_inactive, flags, vec);
+}
+
+// The same commit over MANY records (one per parameter tensor) in one launch:
+// a workgroup owns one kBlockSpan-element span of one record, found by a
+// search over the records' first-span indices.
+struct GcRecord {           // sga_gc_record, see the header
+  float* p; float* g; float* m; float* v;
+  const uint8_t* mask;
+  int64_t n, first_span;
+  float lr, b1, om1, b2, om2, eps, wd, bc1, bc2, lr_inactive;
+  int flags, pad_;
+};
+
+template <int EMIT>
+__global__ __launch_bounds__(kBlock) void k_grad_correct_multi(const GcRecord* __restrict__ recs,
+                                                               int n_recs, float coeff,
+                                                               float interval) {
+  const int64_t span = blockIdx.x;
+  int a = 0, b = n_recs - 1;
+  while (a < b) {                       // last record whose first span is <= this one
+    const int mid = (a + b + 1) >> 1;
+    if (recs[mid].first_span <= span) a = mid; else b = mid - 1;
+  }
+  const GcRecord r = recs[a];
+  Hyper h;
+  h.lr = r.lr; h.b1 = r.b1; h.om1 = r.om1; h.b2 = r.b2; h.om2 = r.om2; h.eps = r.eps;
+  h.wd = r.wd; h.bc1 = r.bc1; h.bc2 = r.bc2;
+  const bool vec = aligned4(r.p, 4) && aligned4(r.g, 4) && aligned4(r.m, 4) && aligned4(r.v, 4) &&
+                   aligned4(r.mask, 1);
+  const int64_t base = (span - r.first_span) * kBlockSpan;
 #pragma unroll
-      for (int e = 0; e < 4; ++e) vv[e] = mm[e] * mm[e];
-    } else {
-      load4_f32(v, i, n, vv, vec);
-    }
-    if (has_mask) load4_u8(mask, i, n, mk, vec);
-    float gout[4];
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      const bool active = mk[e] != 0;
-      const float raw = gg[e];
-      float ge = raw;
-      if (EMIT < 0 && has_mask && !active) ge = 0.0f;
-      if (apply_coeff && active) ge = ge * coeff;
-      const Commit c = adamw_commit(pp[e], ge, mm[e], vv[e], h);
-      if (EMIT == 0) gout[e] = c.upd;
-      else if (EMIT == 1) gout[e] = fabsf(ge);
-      else if (EMIT == 2) gout[e] = fabsf(mm[e]);
-      else if (EMIT == 3) gout[e] = fabsf(c.u - coi_u0(mm[e], vv[e], h));
-      else {
-        float t = (clear && active) ? 0.0f : raw;
-        if (fold) t = __fdiv_rn(t, interval);
-        gout[e] = t;
-      }
-      const float lr_a = (split && !active) ? lr_inactive : h.lr;
-      pp[e] = pp[e] - lr_a * c.upd;
-      mm[e] = c.m_new;
-      vv[e] = c.v_new;
-    }
-    store4_f32(m, i, n, mm, vec);
-    store4_f32(v, i, n, vv, vec);
-    if (EMIT >= 0 || clear || fold) store4_f32(g, i, n, gout, vec);
-    store4_f32(p, i, n, pp, vec);
+  for (int it = 0; it < kBlockSpan / (kBlock * kVec); ++it) {
+    const int64_t i = base + ((int64_t)it * kBlock + threadIdx.x) * kVec;
+    if (i < r.n)
+      gc_vec<EMIT>(r.p, r.g, r.m, r.v, r.mask, i, r.n, h, coeff, interval, r.lr_inactive, r.flags,
+                   vec);
   }
 }
 
@@ -248,6 +293,34 @@ extern "C" int sga_adamw_grad_correct(float* p, float* g, float* m, float* v,
   }
 #undef SGA_GC_LAUNCH
   return check_launch("sga_adamw_grad_correct");
+}
+
+static_assert(sizeof(GcRecord) == sizeof(sga_gc_record), "commit record layout");
+
+extern "C" int sga_adamw_grad_correct_multi(const sga_gc_record* recs, int n_recs,
+                                            int64_t total_spans, float coeff, float interval,
+                                            int emit_mode, void* stream) {
+  if (n_recs == 0 || total_spans == 0) return SGA_OK;
+  if (!recs || n_recs < 0 || total_spans < 0 || total_spans >= (1ll << 31) || emit_mode < -1 ||
+      emit_mode > 3) {
+    set_error("sga_adamw_grad_correct_multi: bad argument (n_recs=%d spans=%lld emit_mode=%d)",
+              n_recs, (long long)total_spans, emit_mode);
+    return SGA_ERR_ARG;
+  }
+  const GcRecord* r = reinterpret_cast<const GcRecord*>(recs);
+  dim3 grid((unsigned)total_spans), block(kBlock);
+  hipStream_t st = (hipStream_t)stream;
+#define SGA_GCM_LAUNCH(E) \
+  hipLaunchKernelGGL((k_grad_correct_multi<E>), grid, block, 0, st, r, n_recs, coeff, interval)
+  switch (emit_mode) {
+    case -1: SGA_GCM_LAUNCH(-1); break;
+    case 0: SGA_GCM_LAUNCH(0); break;
+    case 1: SGA_GCM_LAUNCH(1); break;
+    case 2: SGA_GCM_LAUNCH(2); break;
+    default: SGA_GCM_LAUNCH(3); break;
+  }
+#undef SGA_GCM_LAUNCH
+  return check_launch("sga_adamw_grad_correct_multi");
 }
 
 extern "C" int sga_adamw_grad_correct_compact(

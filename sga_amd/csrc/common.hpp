@@ -42,7 +42,7 @@ static inline unsigned stream_grid(int64_t n_items, int64_t items_per_block,
 }
 
 // True when p is aligned for 4-element vector access of `elem` bytes each.
-static inline bool aligned4(const void* p, int elem) {
+__host__ __device__ static inline bool aligned4(const void* p, int elem) {
   return p == nullptr || (reinterpret_cast<uintptr_t>(p) % (4 * (size_t)elem)) == 0;
 }
 

@@ -281,3 +281,52 @@ def test_adams_compact_equals_masked(dev):
                                   coeff=0.5, dir_table=build_dir_table(idx, n))
     for x, y in zip(a, b):
         assert torch.equal(x, y)
+
+
+@pytest.mark.parametrize("mode", ["sparse", "full_update", "full_split", "adams_sparse"])
+def test_grad_correct_multi_equals_per_record_calls(dev, mode):
+    """One launch over a ragged list of records == the per-record kernel calls,
+    bit for bit, with per-record knobs (a record without a mask takes none)."""
+    from sga_amd.adamw import adamw_grad_correct, adamw_grad_correct_multi
+    gen = torch.Generator().manual_seed(17)
+    sizes = [5, 4096, 4097, 12_289, 1, 100_003, 8192]
+    adams = mode == "adams_sparse"
+    recs_a, recs_b = [], []
+    for j, n in enumerate(sizes):
+        t = {k: (torch.randn(n + 1, generator=gen) * s).to(dev)[1 if j % 3 == 0 else 0:][:n]
+             for k, s in (("p", 0.02), ("g", 1e-2), ("m", 1e-3))}
+        t["v"] = (torch.rand(n + 1, generator=gen) * 1e-5).to(dev)[:n]
+        mask = None if j == 4 else (torch.rand(n, generator=gen) < 0.3).to(torch.uint8).to(dev)
+        hp = dict(lr=1e-3 * (1 + j), beta1=0.9, beta2=0.95 if j % 2 else 0.999, eps=1e-8,
+                  weight_decay=0.1 if j % 2 else 0.0, step=3 + j)
+        recs_a.append((dict((k, v.clone()) for k, v in t.items()), mask, hp))
+        recs_b.append((dict((k, v.clone()) for k, v in t.items()), mask, hp))
+    if mode in ("sparse", "adams_sparse"):
+        emit, kn = None, dict(coeff=0.37, clear=True, fold=True, interval=4.0)
+    elif mode == "full_update":
+        emit, kn = "update", {}
+    else:
+        emit, kn = "abs_g", dict(inactive_lr_scale=0.25)
+    table = []
+    for t, mask, hp in recs_a:                    # reference: one call per record
+        use = mask if mode != "full_update" else None
+        kw = dict(kn) if use is not None else {}
+        if use is None:
+            kw.pop("inactive_lr_scale", None)
+        adamw_grad_correct(t["p"], t["g"], t["m"], t["v"], hp["lr"], hp["beta1"], hp["beta2"],
+                           hp["eps"], hp["weight_decay"], 1 if adams else hp["step"], mask=use,
+                           emit_score=emit, _adams=adams, **kw)
+    for t, mask, hp in recs_b:
+        use = mask if mode != "full_update" else None
+        table.append(dict(p=t["p"], g=t["g"], m=t["m"], v=t["v"], mask=use,
+                          coeff_on=use is not None, clear=kn.get("clear", False) and use is not None,
+                          fold=kn.get("fold", False) and use is not None,
+                          inactive_lr_scale=kn.get("inactive_lr_scale", 1.0) if use is not None
+                          else 1.0, **hp))
+    adamw_grad_correct_multi(table, emit_score=emit, coeff=kn.get("coeff", 1.0),
+                             interval=kn.get("interval", 1.0), _adams=adams)
+    for (ta, _, _), (tb, _, _) in zip(recs_a, recs_b):
+        for k in ("p", "g", "m", "v"):
+            assert torch.equal(ta[k].view(torch.int32), tb[k].view(torch.int32)), (mode, k)
+    with pytest.raises(ValueError, match="requires a sparse step"):
+        adamw_grad_correct_multi([dict(table[0], mask=None, clear=True)], emit_score=None)
