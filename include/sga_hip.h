@@ -194,6 +194,28 @@ int sga_adamw_grad_correct_compact(float* p, float* g, float* m, float* v,
                                    int flags, const int32_t* dir_table,
                                    int64_t n_table, void* stream);
 
+/* The compact commit over many records in ONE launch (the per-record loop of
+ * adamw.py:907-947).  recs: DEVICE table ordered by first_span; idx / values /
+ * table / k_total / n_table are the record's bucket's; flags:
+ * SGA_GC_APPLY_COEFF | SGA_GC_FOLD | SGA_GC_ADAMS per record; every record's
+ * values have the dtype values_dtype. */
+typedef struct sga_gcc_record {
+  float* p;
+  float* g;
+  float* m;
+  float* v;
+  const int32_t* idx;
+  const void* values;
+  const int32_t* table;    /* directory table or NULL */
+  int64_t rec_start, n, k_total, n_table, first_span;
+  float lr, beta1, om1, beta2, om2, eps, wd, bc1, bc2;
+  int flags;
+} sga_gcc_record;
+int sga_adamw_grad_correct_compact_multi(const sga_gcc_record* recs, int n_recs,
+                                         int64_t total_spans, int values_dtype,
+                                         float coeff, float interval,
+                                         void* stream);
+
 /* build_dir_table, adamw.py:325-349, 472-499:
  * table[j] = lower_bound(idx, j*1024), j < n_table. */
 int sga_build_dir_table(const int32_t* idx, int64_t k, int32_t* table,

@@ -47,6 +47,7 @@ SIGNATURES = {
     "sga_mask_fill": (I32, [P, I64, P, P, I64, P]),
     "sga_adamw_grad_correct": (I32, [P, P, P, P, P, I64] + [F] * 12 + [I32, I32, P]),
     "sga_adamw_grad_correct_multi": (I32, [P, I32, I64, F, F, I32, P]),
+    "sga_adamw_grad_correct_compact_multi": (I32, [P, I32, I64, I32, F, F, P]),
     "sga_adamw_grad_correct_compact": (I32, [P, P, P, P, P, P, I32, I64, I64, I64]
                                        + [F] * 11 + [I32, P, I64, P]),
     "sga_build_dir_table": (I32, [P, I64, P, I64, P]),

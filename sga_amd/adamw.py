@@ -180,20 +180,14 @@ def build_dir_table(idx, total_n):
     return table
 
 
-def adamw_grad_correct_compact(param_buffer, grad_buffer, exp_avg_buffer,
-                               exp_avg_sq_buffer, idx, values, rec_start, lr, beta1,
-                               beta2, eps, weight_decay, step, coeff=1.0, fold=False,
-                               interval=1.0, dir_table=None, _adams=False):
-    """Compact-emission commit: the gradient comes from the bucket-level sorted
-    ``(idx, values)`` by merge-join (``adamw.py:637-792``).  ``values`` may be
-    fp32 or bf16."""
+def _gcc_prepare(param_buffer, grad_buffer, exp_avg_buffer, exp_avg_sq_buffer, idx, values,
+                 rec_start, dir_table):
+    """The refusals of ``adamw.py:676-750``; returns ``(n, k_total, n_table)``."""
     if not idx.is_contiguous() or not values.is_contiguous():
         raise ValueError("adamw_grad_correct_compact requires contiguous idx/values")
-    bias_correction1 = 1.0 - beta1 ** step
-    bias_correction2 = 1.0 - beta2 ** step
     n = param_buffer.numel()
     if n == 0:
-        return
+        return 0, 0, 0
     k_total = idx.numel()
     assert k_total + _BLOCK_SIZE < 2 ** 31, (
         f"adamw_grad_correct_compact: k_total + BLOCK_SIZE = {k_total + _BLOCK_SIZE} "
@@ -215,6 +209,22 @@ def adamw_grad_correct_compact(param_buffer, grad_buffer, exp_avg_buffer,
             f"adamw_grad_correct_compact: dir_table has {dir_table.numel()} entries "
             f"but the record's last block needs >= {((rec_start + n - 1) >> 10) + 2}")
         n_table = dir_table.numel()
+    return n, k_total, n_table
+
+
+def adamw_grad_correct_compact(param_buffer, grad_buffer, exp_avg_buffer,
+                               exp_avg_sq_buffer, idx, values, rec_start, lr, beta1,
+                               beta2, eps, weight_decay, step, coeff=1.0, fold=False,
+                               interval=1.0, dir_table=None, _adams=False):
+    """Compact-emission commit: the gradient comes from the bucket-level sorted
+    ``(idx, values)`` by merge-join (``adamw.py:637-792``).  ``values`` may be
+    fp32 or bf16."""
+    bias_correction1 = 1.0 - beta1 ** step
+    bias_correction2 = 1.0 - beta2 ** step
+    n, k_total, n_table = _gcc_prepare(param_buffer, grad_buffer, exp_avg_buffer,
+                                       exp_avg_sq_buffer, idx, values, rec_start, dir_table)
+    if n == 0:
+        return
     flags = ((L.GC_APPLY_COEFF if coeff != 1.0 else 0) | (L.GC_FOLD if fold else 0)
              | (L.GC_ADAMS if _adams else 0))
     L.call("sga_adamw_grad_correct_compact", L.ptr(param_buffer), L.ptr(grad_buffer),
@@ -223,6 +233,54 @@ def adamw_grad_correct_compact(param_buffer, grad_buffer, exp_avg_buffer,
            L.f32(1.0 - beta1), L.f32(beta2), L.f32(1.0 - beta2), L.f32(eps),
            L.f32(weight_decay), L.f32(bias_correction1), L.f32(bias_correction2),
            L.f32(coeff), L.f32(interval), flags, L.ptr(dir_table), n_table, L.stream())
+
+
+class GccRecord(C.Structure):
+    """struct sga_gcc_record"""
+    _fields_ = [(k, C.c_void_p) for k in ("p", "g", "m", "v", "idx", "values", "table")] + \
+               [(k, C.c_int64) for k in ("rec_start", "n", "k_total", "n_table", "first_span")] + \
+               [(k, C.c_float) for k in ("lr", "beta1", "om1", "beta2", "om2", "eps", "wd",
+                                         "bc1", "bc2")] + [("flags", C.c_int)]
+
+
+def adamw_grad_correct_compact_multi(records, coeff=1.0, fold=False, interval=1.0, _adams=False):
+    """``adamw_grad_correct_compact`` over many records in one launch per values
+    dtype.  ``records``: dicts with ``p, g, m, v, idx, values, rec_start,
+    dir_table`` and ``lr, beta1, beta2, eps, weight_decay, step``."""
+    by_dtype = {}
+    for r in records:
+        n, k_total, n_table = _gcc_prepare(r["p"], r["g"], r["m"], r["v"], r["idx"], r["values"],
+                                           r["rec_start"], r.get("dir_table"))
+        if n == 0:
+            continue
+        lst = by_dtype.setdefault(r["values"].dtype, [])
+        e = GccRecord()
+        e.p, e.g, e.m, e.v = (t.data_ptr() for t in (r["p"], r["g"], r["m"], r["v"]))
+        e.idx, e.values = r["idx"].data_ptr(), r["values"].data_ptr()
+        e.table = r["dir_table"].data_ptr() if r.get("dir_table") is not None else None
+        e.rec_start, e.n, e.k_total, e.n_table = r["rec_start"], n, k_total, n_table
+        e.lr, e.beta1, e.om1 = L.f32(r["lr"]), L.f32(r["beta1"]), L.f32(1.0 - r["beta1"])
+        e.beta2, e.om2 = L.f32(r["beta2"]), L.f32(1.0 - r["beta2"])
+        e.eps, e.wd = L.f32(r["eps"]), L.f32(r["weight_decay"])
+        e.bc1 = 1.0 if _adams else L.f32(1.0 - r["beta1"] ** r["step"])
+        e.bc2 = 1.0 if _adams else L.f32(1.0 - r["beta2"] ** r["step"])
+        e.flags = ((L.GC_APPLY_COEFF if coeff != 1.0 else 0) | (L.GC_FOLD if fold else 0)
+                   | (L.GC_ADAMS if _adams else 0))
+        lst.append(e)
+    for dtype, lst in by_dtype.items():
+        spans = 0
+        for e in lst:
+            e.first_span = spans
+            spans += -(-e.n // _SPAN)
+        arr = (GccRecord * len(lst))(*lst)
+        dev = records[0]["p"].device
+        key = (dev, "gcc", C.sizeof(arr))
+        up = _uploaders.get(key)
+        if up is None:
+            up = _uploaders[key] = L.TableUploader(C.sizeof(arr), dev)
+        up.upload(arr)
+        L.call("sga_adamw_grad_correct_compact_multi", L.ptr(up.dev), len(lst), spans,
+               0 if dtype == torch.float32 else 1, L.f32(coeff), L.f32(interval), L.stream())
 
 
 @dataclass
@@ -332,23 +390,27 @@ class SgaAdamW:
                                  _adams=self._adams)
 
     def _records_pass_compact(self, ctx, coeff=1.0, fold=False, interval=1.0):
+        # records of buckets with communicated values: one merge-join launch;
+        # the others (no support in their bucket): one plain-commit launch
+        compact, plain = [], []
         for rec in ctx.records:
             st = self._state(rec)
             bs = rec.bucket_state
             values = ctx.compact_values.get(id(bs))
+            base = dict(p=rec.main_param.data.view(-1), g=rec.grad.data.view(-1),
+                        m=st["exp_avg"].view(-1), v=st["exp_avg_sq"].view(-1), lr=rec.lr,
+                        beta1=rec.beta1, beta2=rec.beta2, eps=rec.eps,
+                        weight_decay=rec.weight_decay, step=rec.step)
             if values is None:
-                self._commit(
-                    rec.main_param.data.view(-1), rec.grad.data.view(-1),
-                    st["exp_avg"].view(-1), st["exp_avg_sq"].view(-1), rec.lr,
-                    rec.beta1, rec.beta2, rec.eps, rec.weight_decay, rec.step)
+                plain.append(dict(base, mask=None, coeff_on=False))
                 continue
             bucket = ctx.support.buckets[bs.support_index]
             table = bucket.dir_table if self.compact_search == "table" else None
-            self._commit_compact(
-                rec.main_param.data.view(-1), rec.grad.data.view(-1),
-                st["exp_avg"].view(-1), st["exp_avg_sq"].view(-1), bucket.idx, values,
-                rec.start, rec.lr, rec.beta1, rec.beta2, rec.eps, rec.weight_decay,
-                rec.step, coeff=coeff, fold=fold, interval=interval, dir_table=table)
+            compact.append(dict(base, idx=bucket.idx, values=values, rec_start=rec.start,
+                                dir_table=table))
+        adamw_grad_correct_multi(plain, _adams=self._adams)
+        adamw_grad_correct_compact_multi(compact, coeff=coeff, fold=fold, interval=interval,
+                                         _adams=self._adams)
 
     @torch.no_grad()
     def full_step(self, ctx):

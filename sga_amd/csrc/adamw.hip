@@ -145,6 +145,87 @@ __device__ __forceinline__ int64_t coop_lower_bound(
   return lo;
 }
 
+// One kBlockSpan-element span of one record (all 256 threads of the workgroup).
+template <bool BF16>
+__device__ __forceinline__ void compact_span(
+    float* __restrict__ p, float* __restrict__ g, float* __restrict__ m,
+    float* __restrict__ v, const int32_t* __restrict__ idx,
+    const void* __restrict__ values, int64_t rec_start, int64_t n,
+    int64_t k_total, const Hyper& h, float coeff, float interval, int flags,
+    const int32_t* __restrict__ table, int64_t n_table, bool vec, int64_t span,
+    float* s_val, uint32_t* s_found, int64_t* s_bounds) {
+  const bool apply_coeff = flags & SGA_GC_APPLY_COEFF;
+  const bool fold = flags & SGA_GC_FOLD;
+  const bool adams = flags & SGA_GC_ADAMS;
+  const int64_t off0 = span * kBlockSpan;
+  const int64_t c0 = rec_start + off0;
+  int64_t c1 = c0 + kBlockSpan;
+  if (c1 > rec_start + n) c1 = rec_start + n;
+  for (int t = threadIdx.x; t < kBlockSpan; t += kBlock) s_val[t] = 0.0f;
+  if (threadIdx.x < kBlockSpan / 32) s_found[threadIdx.x] = 0u;
+  if (wave_id() < 2) {
+    const int64_t key = wave_id() == 0 ? c0 : c1;
+    int64_t lo = 0, hi = k_total;
+    if (table) {
+      const int64_t j = key >> 10;
+      if (j < n_table) {
+        lo = table[j];
+        hi = lo + (key & 1023);
+        if (hi > k_total) hi = k_total;
+        if (lo > k_total) lo = k_total;
+      }
+    }
+    const int64_t r = coop_lower_bound(idx, lo, hi, key);
+    if (lane_id() == 0) s_bounds[wave_id()] = r;
+  }
+  __syncthreads();
+  const int64_t lo = s_bounds[0], hi = s_bounds[1];
+  for (int64_t j = lo + threadIdx.x; j < hi; j += kBlock) {
+    const int64_t t = (int64_t)idx[j] - c0;
+    if (t >= 0 && t < kBlockSpan) {
+      float x = BF16 ? bf16_to_f32(reinterpret_cast<const uint16_t*>(values)[j])
+                     : reinterpret_cast<const float*>(values)[j];
+      s_val[t] = x;
+      atomicOr(&s_found[t >> 5], 1u << (t & 31));
+    }
+  }
+  __syncthreads();
+#pragma unroll
+  for (int it = 0; it < kChunkIters; ++it) {
+    const int t0 = it * (kBlock * kVec) + threadIdx.x * kVec;
+    const int64_t i = off0 + t0;
+    if (i < n) {
+      float pp[4], mm[4], vv[4], raw[4] = {0, 0, 0, 0};
+      load4_f32(p, i, n, pp, vec);
+      load4_f32(m, i, n, mm, vec);
+      if (adams) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) vv[e] = mm[e] * mm[e];
+      } else {
+        load4_f32(v, i, n, vv, vec);
+      }
+      if (fold) load4_f32(g, i, n, raw, vec);
+      const uint32_t fw = s_found[t0 >> 5] >> (t0 & 31);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const bool found = (fw >> e) & 1u;
+        float ge = s_val[t0 + e];
+        if (apply_coeff && found) ge = ge * coeff;
+        const Commit c = adamw_commit(pp[e], ge, mm[e], vv[e], h);
+        pp[e] = pp[e] - h.lr * c.upd;
+        mm[e] = c.m_new;
+        vv[e] = c.v_new;
+        if (fold && !found) raw[e] = __fdiv_rn(raw[e], interval);
+      }
+      store4_f32(m, i, n, mm, vec);
+      store4_f32(v, i, n, vv, vec);
+      if (fold) store4_f32(g, i, n, raw, vec);
+      store4_f32(p, i, n, pp, vec);
+    }
+  }
+  __syncthreads();
+}
+
 template <bool BF16>
 __global__ __launch_bounds__(kBlock) void k_grad_correct_compact(
     float* __restrict__ p, float* __restrict__ g, float* __restrict__ m,
@@ -155,79 +236,41 @@ __global__ __launch_bounds__(kBlock) void k_grad_correct_compact(
   __shared__ float s_val[kBlockSpan];
   __shared__ uint32_t s_found[kBlockSpan / 32];
   __shared__ int64_t s_bounds[2];
-  const bool apply_coeff = flags & SGA_GC_APPLY_COEFF;
-  const bool fold = flags & SGA_GC_FOLD;
-  const bool adams = flags & SGA_GC_ADAMS;
   const int64_t n_spans = cdiv64(n, kBlockSpan);
-  for (int64_t span = blockIdx.x; span < n_spans; span += gridDim.x) {
-    const int64_t off0 = span * kBlockSpan;
-    const int64_t c0 = rec_start + off0;
-    int64_t c1 = c0 + kBlockSpan;
-    if (c1 > rec_start + n) c1 = rec_start + n;
-    for (int t = threadIdx.x; t < kBlockSpan; t += kBlock) s_val[t] = 0.0f;
-    if (threadIdx.x < kBlockSpan / 32) s_found[threadIdx.x] = 0u;
-    if (wave_id() < 2) {
-      const int64_t key = wave_id() == 0 ? c0 : c1;
-      int64_t lo = 0, hi = k_total;
-      if (table) {
-        const int64_t j = key >> 10;
-        if (j < n_table) {
-          lo = table[j];
-          hi = lo + (key & 1023);
-          if (hi > k_total) hi = k_total;
-          if (lo > k_total) lo = k_total;
-        }
-      }
-      const int64_t r = coop_lower_bound(idx, lo, hi, key);
-      if (lane_id() == 0) s_bounds[wave_id()] = r;
-    }
-    __syncthreads();
-    const int64_t lo = s_bounds[0], hi = s_bounds[1];
-    for (int64_t j = lo + threadIdx.x; j < hi; j += kBlock) {
-      const int64_t t = (int64_t)idx[j] - c0;
-      if (t >= 0 && t < kBlockSpan) {
-        float x = BF16 ? bf16_to_f32(reinterpret_cast<const uint16_t*>(values)[j])
-                       : reinterpret_cast<const float*>(values)[j];
-        s_val[t] = x;
-        atomicOr(&s_found[t >> 5], 1u << (t & 31));
-      }
-    }
-    __syncthreads();
-#pragma unroll
-    for (int it = 0; it < kChunkIters; ++it) {
-      const int t0 = it * (kBlock * kVec) + threadIdx.x * kVec;
-      const int64_t i = off0 + t0;
-      if (i < n) {
-        float pp[4], mm[4], vv[4], raw[4] = {0, 0, 0, 0};
-        load4_f32(p, i, n, pp, vec);
-        load4_f32(m, i, n, mm, vec);
-        if (adams) {
-#pragma unroll
-          for (int e = 0; e < 4; ++e) vv[e] = mm[e] * mm[e];
-        } else {
-          load4_f32(v, i, n, vv, vec);
-        }
-        if (fold) load4_f32(g, i, n, raw, vec);
-        const uint32_t fw = s_found[t0 >> 5] >> (t0 & 31);
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const bool found = (fw >> e) & 1u;
-          float ge = s_val[t0 + e];
-          if (apply_coeff && found) ge = ge * coeff;
-          const Commit c = adamw_commit(pp[e], ge, mm[e], vv[e], h);
-          pp[e] = pp[e] - h.lr * c.upd;
-          mm[e] = c.m_new;
-          vv[e] = c.v_new;
-          if (fold && !found) raw[e] = __fdiv_rn(raw[e], interval);
-        }
-        store4_f32(m, i, n, mm, vec);
-        store4_f32(v, i, n, vv, vec);
-        if (fold) store4_f32(g, i, n, raw, vec);
-        store4_f32(p, i, n, pp, vec);
-      }
-    }
-    __syncthreads();
+  for (int64_t span = blockIdx.x; span < n_spans; span += gridDim.x)
+    compact_span<BF16>(p, g, m, v, idx, values, rec_start, n, k_total, h, coeff, interval, flags,
+                       table, n_table, vec, span, s_val, s_found, s_bounds);
+}
+
+// The compact commit over many records in one launch (one span per workgroup).
+struct GccRecord {          // sga_gcc_record, see the header
+  float* p; float* g; float* m; float* v;
+  const int32_t* idx; const void* values; const int32_t* table;
+  int64_t rec_start, n, k_total, n_table, first_span;
+  float lr, b1, om1, b2, om2, eps, wd, bc1, bc2;
+  int flags;
+};
+
+template <bool BF16>
+__global__ __launch_bounds__(kBlock) void k_grad_correct_compact_multi(
+    const GccRecord* __restrict__ recs, int n_recs, float coeff, float interval) {
+  __shared__ float s_val[kBlockSpan];
+  __shared__ uint32_t s_found[kBlockSpan / 32];
+  __shared__ int64_t s_bounds[2];
+  const int64_t span = blockIdx.x;
+  int a = 0, b = n_recs - 1;
+  while (a < b) {
+    const int mid = (a + b + 1) >> 1;
+    if (recs[mid].first_span <= span) a = mid; else b = mid - 1;
   }
+  const GccRecord r = recs[a];
+  Hyper h;
+  h.lr = r.lr; h.b1 = r.b1; h.om1 = r.om1; h.b2 = r.b2; h.om2 = r.om2; h.eps = r.eps;
+  h.wd = r.wd; h.bc1 = r.bc1; h.bc2 = r.bc2;
+  const bool vec = aligned4(r.p, 4) && aligned4(r.g, 4) && aligned4(r.m, 4) && aligned4(r.v, 4);
+  compact_span<BF16>(r.p, r.g, r.m, r.v, r.idx, r.values, r.rec_start, r.n, r.k_total, h, coeff,
+                     interval, r.flags, r.table, r.n_table, vec, span - r.first_span, s_val,
+                     s_found, s_bounds);
 }
 
 __global__ __launch_bounds__(kBlock) void k_dir_table(
@@ -357,6 +400,28 @@ extern "C" int sga_adamw_grad_correct_compact(
   else
     hipLaunchKernelGGL((k_grad_correct_compact<false>), grid, block, 0, st, p, g, m, v, idx, values, rec_start, n, k_total, h, coeff, interval, flags, dir_table, n_table, vec);
   return check_launch("sga_adamw_grad_correct_compact");
+}
+
+static_assert(sizeof(GccRecord) == sizeof(sga_gcc_record), "compact commit record layout");
+
+extern "C" int sga_adamw_grad_correct_compact_multi(const sga_gcc_record* recs, int n_recs,
+                                                    int64_t total_spans, int values_dtype,
+                                                    float coeff, float interval, void* stream) {
+  if (n_recs == 0 || total_spans == 0) return SGA_OK;
+  if (!recs || n_recs < 0 || total_spans < 0 || total_spans >= (1ll << 31) ||
+      (values_dtype != SGA_F32 && values_dtype != SGA_BF16)) {
+    set_error("sga_adamw_grad_correct_compact_multi: bad argument (n_recs=%d spans=%lld)", n_recs,
+              (long long)total_spans);
+    return SGA_ERR_ARG;
+  }
+  const GccRecord* r = reinterpret_cast<const GccRecord*>(recs);
+  dim3 grid((unsigned)total_spans), block(kBlock);
+  hipStream_t st = (hipStream_t)stream;
+  if (values_dtype == SGA_BF16)
+    hipLaunchKernelGGL((k_grad_correct_compact_multi<true>), grid, block, 0, st, r, n_recs, coeff, interval);
+  else
+    hipLaunchKernelGGL((k_grad_correct_compact_multi<false>), grid, block, 0, st, r, n_recs, coeff, interval);
+  return check_launch("sga_adamw_grad_correct_compact_multi");
 }
 
 extern "C" int sga_build_dir_table(const int32_t* idx, int64_t k, int32_t* table,

@@ -86,17 +86,20 @@ def test_header_is_plain_c_and_struct_sizes_agree(tmp_path):
     caller sees are the ones the ctypes mirrors use."""
     import subprocess
     from sga_amd import _lib as L
+    from sga_amd.adamw import GcRecord, GccRecord
     from sga_amd.replay_group import ReplayCfg, ReplaySegment
     from sga_amd.selection import SelectResult
     src = tmp_path / "sizes.c"
     src.write_text('#include <stdio.h>\n#include "sga_hip.h"\n'
-                   'int main(void) { printf("%zu %zu %zu %zu\\n", sizeof(sga_segment), '
+                   'int main(void) { printf("%zu %zu %zu %zu ", sizeof(sga_segment), '
                    'sizeof(sga_select_result), sizeof(sga_replay_cfg), '
-                   'sizeof(sga_replay_segment)); return 0; }\n')
+                   'sizeof(sga_replay_segment)); printf("%zu %zu\\n", sizeof(sga_gc_record), '
+                   'sizeof(sga_gcc_record)); return 0; }\n')
     exe = tmp_path / "sizes"
     subprocess.run(["gcc", "-std=c99", "-Wall", "-Werror", "-pedantic",
                     "-I", os.path.join(ROOT, "include"), str(src), "-o", str(exe)], check=True)
     got = [int(x) for x in subprocess.run([str(exe)], check=True, capture_output=True,
                                           text=True).stdout.split()]
     assert got == [ctypes.sizeof(L.Segment), ctypes.sizeof(SelectResult),
-                   ctypes.sizeof(ReplayCfg), ctypes.sizeof(ReplaySegment)]
+                   ctypes.sizeof(ReplayCfg), ctypes.sizeof(ReplaySegment),
+                   ctypes.sizeof(GcRecord), ctypes.sizeof(GccRecord)]

@@ -330,3 +330,46 @@ def test_grad_correct_multi_equals_per_record_calls(dev, mode):
             assert torch.equal(ta[k].view(torch.int32), tb[k].view(torch.int32)), (mode, k)
     with pytest.raises(ValueError, match="requires a sparse step"):
         adamw_grad_correct_multi([dict(table[0], mask=None, clear=True)], emit_score=None)
+
+
+@pytest.mark.parametrize("vdtype,adams", [(torch.float32, False), (torch.bfloat16, False),
+                                          (torch.float32, True)])
+def test_grad_correct_compact_multi_equals_per_record_calls(dev, vdtype, adams):
+    """One merge-join launch over every record of a bucket == the per-record
+    compact calls, bit for bit (with and without the directory table)."""
+    from sga_amd.adamw import (adamw_grad_correct_compact, adamw_grad_correct_compact_multi,
+                               build_dir_table)
+    gen = torch.Generator().manual_seed(23)
+    sizes = [1500, 4096, 5, 70_001, 8193, 1023]
+    n_total = sum(sizes)
+    mask = torch.rand(n_total, generator=gen) < 0.07
+    idx = mask.nonzero().reshape(-1).to(torch.int32).to(dev)
+    values = (torch.randn(idx.numel(), generator=gen) * 1e-2).to(vdtype).to(dev)
+    table = build_dir_table(idx, n_total)
+    for use_table in (True, False):
+        sets = []
+        for _ in range(2):
+            g2 = torch.Generator().manual_seed(5)
+            recs, off = [], 0
+            for j, n in enumerate(sizes):
+                recs.append(dict(
+                    p=(torch.randn(n, generator=g2) * 0.02).to(dev),
+                    g=(torch.randn(n, generator=g2) * 1e-2).to(dev),
+                    m=(torch.randn(n, generator=g2) * 1e-3).to(dev),
+                    v=(torch.rand(n, generator=g2) * 1e-5).to(dev),
+                    rec_start=off, lr=1e-3 * (j + 1), beta1=0.9, beta2=0.95, eps=1e-8,
+                    weight_decay=0.1 if j % 2 else 0.0, step=4 + j))
+                off += n
+            sets.append(recs)
+        tb = table if use_table else None
+        for r in sets[0]:
+            adamw_grad_correct_compact(r["p"], r["g"], r["m"], r["v"], idx, values, r["rec_start"],
+                                       r["lr"], r["beta1"], r["beta2"], r["eps"],
+                                       r["weight_decay"], 1 if adams else r["step"], coeff=0.6,
+                                       fold=True, interval=8.0, dir_table=tb, _adams=adams)
+        adamw_grad_correct_compact_multi(
+            [dict(r, idx=idx, values=values, dir_table=tb) for r in sets[1]], coeff=0.6,
+            fold=True, interval=8.0, _adams=adams)
+        for a, b in zip(*sets):
+            for k in ("p", "g", "m", "v"):
+                assert torch.equal(a[k].view(torch.int32), b[k].view(torch.int32)), (use_table, k)
