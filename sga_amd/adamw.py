@@ -140,12 +140,13 @@ def adamw_grad_correct_multi(records, emit_score=None, coeff=1.0, interval=1.0, 
         e.p, e.g, e.m, e.v = (t.data_ptr() for t in (r["p"], r["g"], r["m"], r["v"]))
         e.mask = mk.data_ptr() if mk is not None else None
         e.n, e.first_span = n, spans
-        e.lr, e.beta1, e.om1 = L.f32(r["lr"]), L.f32(r["beta1"]), L.f32(1.0 - r["beta1"])
-        e.beta2, e.om2 = L.f32(r["beta2"]), L.f32(1.0 - r["beta2"])
-        e.eps, e.wd = L.f32(r["eps"]), L.f32(r["weight_decay"])
-        e.bc1 = 1.0 if _adams else L.f32(1.0 - r["beta1"] ** step)
-        e.bc2 = 1.0 if _adams else L.f32(1.0 - r["beta2"] ** step)
-        e.lr_inactive = L.f32(r["lr"] * float(r.get("inactive_lr_scale", 1.0)))
+        # a Python float stored into a c_float field is rounded to nearest fp32
+        e.lr, e.beta1, e.om1 = r["lr"], r["beta1"], 1.0 - r["beta1"]
+        e.beta2, e.om2 = r["beta2"], 1.0 - r["beta2"]
+        e.eps, e.wd = r["eps"], r["weight_decay"]
+        e.bc1 = 1.0 if _adams else 1.0 - r["beta1"] ** step
+        e.bc2 = 1.0 if _adams else 1.0 - r["beta2"] ** step
+        e.lr_inactive = r["lr"] * float(r.get("inactive_lr_scale", 1.0))
         e.flags = flags
         table.append(e)
         keep.append(mk)
@@ -259,11 +260,11 @@ def adamw_grad_correct_compact_multi(records, coeff=1.0, fold=False, interval=1.
         e.idx, e.values = r["idx"].data_ptr(), r["values"].data_ptr()
         e.table = r["dir_table"].data_ptr() if r.get("dir_table") is not None else None
         e.rec_start, e.n, e.k_total, e.n_table = r["rec_start"], n, k_total, n_table
-        e.lr, e.beta1, e.om1 = L.f32(r["lr"]), L.f32(r["beta1"]), L.f32(1.0 - r["beta1"])
-        e.beta2, e.om2 = L.f32(r["beta2"]), L.f32(1.0 - r["beta2"])
-        e.eps, e.wd = L.f32(r["eps"]), L.f32(r["weight_decay"])
-        e.bc1 = 1.0 if _adams else L.f32(1.0 - r["beta1"] ** r["step"])
-        e.bc2 = 1.0 if _adams else L.f32(1.0 - r["beta2"] ** r["step"])
+        e.lr, e.beta1, e.om1 = r["lr"], r["beta1"], 1.0 - r["beta1"]
+        e.beta2, e.om2 = r["beta2"], 1.0 - r["beta2"]
+        e.eps, e.wd = r["eps"], r["weight_decay"]
+        e.bc1 = 1.0 if _adams else 1.0 - r["beta1"] ** r["step"]
+        e.bc2 = 1.0 if _adams else 1.0 - r["beta2"] ** r["step"]
         e.flags = ((L.GC_APPLY_COEFF if coeff != 1.0 else 0) | (L.GC_FOLD if fold else 0)
                    | (L.GC_ADAMS if _adams else 0))
         lst.append(e)
