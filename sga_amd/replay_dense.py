@@ -15,7 +15,7 @@ import torch
 
 from . import _lib as L
 from .replay import _bc_pair, coef_dense_for
-from .replay_group import ReplaySegment, _upload
+from .replay_group import ReplaySegment
 from .trace_io import lr_for_step
 
 
@@ -69,7 +69,7 @@ class DenseReplay:
             r.beta1, r.om1 = L.f32(e["b1"]), L.f32(1.0 - e["b1"])
             r.beta2, r.om2 = L.f32(e["b2"]), L.f32(1.0 - e["b2"])
             r.eps, r.wdf, r.bc1, r.bc2 = L.f32(e["eps"]), L.f32(e["wd"]), L.f32(bc1), L.f32(bc2)
-        _upload(self._seg_host, self._seg_up)
+        self._seg_up.upload(self._seg_host)
         st = L.stream()
         L.call("sga_dense_replay_step", L.ptr(g), L.dtype_code(g), L.ptr(self.w), L.ptr(self.m),
                L.ptr(self.v), L.ptr(self.label), self.N, L.ptr(self._seg_dev),

@@ -1,7 +1,10 @@
 """Fused offline-replay group step on MI355X: the per-recorded-step loop of
 ``sga/replay_fused.py:1607-1914`` at world == 1.  G configurations
 (score x ratio x cycle length x optimizer x fold x dual-lr) share one read of
-the recorded gradient per pass; state stays resident on the device."""
+the recorded gradient per pass.  State stays resident on the device: per
+config one packed buffer (res / w / m / v interleaved in 64 KiB records) and
+the selection mask as bit planes; the residual's traffic is skipped while it
+is known to be all zeros."""
 import ctypes as C
 import math
 
@@ -47,10 +50,6 @@ def coef_dense_for(clip_grad, grad_norm):
     if clip_grad <= 0.0 or not math.isfinite(grad_norm) or grad_norm <= 0.0:
         return 1.0
     return min(clip_grad / (grad_norm + 1.0e-6), 1.0)
-
-
-def _upload(struct_array, uploader):
-    uploader.upload(struct_array)
 
 
 _RUN = 4096                       # floats per array per packed record
@@ -101,6 +100,10 @@ class ReplayGroup:
               (ShardParams entries, ``replay_fused.py:251-271``)
     w0/m0/v0: flat fp32 device tensors, the branch-point state (copied per config)
     sel0    : per-config flat bool/uint8 device masks (branch selection)
+
+    ``state[ci]["w" | "m" | "v" | "res" | "sel"]`` returns flat copies for
+    inspection; ``dist_at[ci][H]`` holds ``||w - snapshot_H||`` after ``step``
+    was given the snapshots.
     """
 
     def __init__(self, entries, w0, m0, v0, sel0, configs, t0, window):
@@ -135,7 +138,7 @@ class ReplayGroup:
         self._rseg_dev = self._rseg_up.dev
         self._seg_host = (L.Segment * len(entries))()
         self._seg_up = L.TableUploader(C.sizeof(self._seg_host), dev)
-        self._seg_dev = {"adamw": self._seg_up.dev}
+        self._seg_dev = self._seg_up.dev
         self.dist_at = [dict() for _ in configs]
         # res is all zeros at the start and again after every boundary commit;
         # the kernels then skip its traffic (same values either way)
@@ -157,8 +160,8 @@ class ReplayGroup:
             s.start, s.n, s.lr = e["a"], e["n"], L.f32(lr_of(e))
             s.beta1, s.om1, s.beta2, s.om2 = r.beta1, r.om1, r.beta2, r.om2
             s.eps, s.wd, s.bc1, s.bc2 = r.eps, r.wdf, r.bc1, r.bc2
-        _upload(self._rseg_host, self._rseg_up)
-        _upload(self._seg_host, self._seg_up)
+        self._rseg_up.upload(self._rseg_host)
+        self._seg_up.upload(self._seg_host)
 
     def _fill_cfgs(self, bnd, out_sel):
         for ci, c in enumerate(self.configs):
@@ -204,7 +207,7 @@ class ReplayGroup:
             L.call("sga_replay_reselect", L.ptr(g), gd, C.c_void_p(s.base("res")),
                    C.c_void_p(s.base("w")), C.c_void_p(s.base("m")), C.c_void_p(s.base("v")), N,
                    self.ks[c.ratio],
-                   L.ptr(self._seg_dev["adamw"]), len(self.entries), SCORE_MAP[c.score],
+                   L.ptr(self._seg_dev), len(self.entries), SCORE_MAP[c.score],
                    C.c_void_p(self.coef_f.data_ptr() + 4 * ci), L.f32(coef_dense),
                    int(c.optimizer == "adams"), 1, int(self.res_zero[ci]), L.ptr(s.spare),
                    L.ptr(self.sel_result),
