@@ -185,6 +185,76 @@ def replay_cpu_baseline(G=8, W=8, seed=4, frac=24):
                       f"linearly to the full shard; host cpu_count={os.cpu_count()}"}
 
 
+def primitives_bench(n=1 << 28, ratio=1.0):
+    """The drop-in primitives on their own (one flat fp32 bucket of n elements,
+    k = ratio %): algorithmic bytes over wall time per call."""
+    import torch
+    from sga_amd import kernels as K
+    from sga_amd import replay_kernels as RK
+    from sga_amd.adamw import (adamw_grad_correct, adamw_grad_correct_compact, build_dir_table)
+    from sga_amd.replay import select_topk_flat
+    from sga_amd.selection import select_masks_histogram
+    from sga_amd.support import IndexPool, compact_mask_u8
+    dev = torch.device("cuda:0")
+    gen = torch.Generator(device=dev).manual_seed(0)
+    g = torch.randn(n, generator=gen, device=dev) * 1e-3
+    p = torch.randn(n, generator=gen, device=dev) * 0.02
+    m = torch.randn(n, generator=gen, device=dev) * 1e-4
+    v = torch.rand(n, generator=gen, device=dev) * 1e-8
+    k = max(1, int(round(n * ratio / 100.0)))
+    score = g.abs()
+    mask_b, _ = select_topk_flat(score, k)
+    mask = mask_b.view(torch.uint8)
+    pool = IndexPool()
+    idx = compact_mask_u8(mask, pool).clone()
+    values = torch.empty(k, device=dev)
+    total = torch.zeros(1, device=dev)
+    table = build_dir_table(idx, n)
+    out = torch.empty(n, device=dev)
+    rows = []
+
+    def timed(name, alg_bytes, fn, reps=5):
+        fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            fn()
+        torch.cuda.synchronize()
+        ms = (time.perf_counter() - t0) / reps * 1e3
+        rows.append({"op": name, "ms": ms, "alg_GB": alg_bytes / 1e9,
+                     "GBps": alg_bytes / ms / 1e6, "frac": alg_bytes / ms / 1e6 / 8000.0})
+
+    timed("select_topk_flat (exact, lowest-index ties, mask out)", n * 5.0,
+          lambda: select_topk_flat(score, k, check=False))
+    timed("select_masks_histogram exact (ties all)", n * 5.0,
+          lambda: select_masks_histogram([g], k, mode="exact"))
+    timed("select_masks_histogram balanced", n * (4.0 / 8 + 5.0),
+          lambda: select_masks_histogram([g], k, mode="balanced"))
+    timed("compact_mask_u8", n * 2.0 + k * 4.0, lambda: compact_mask_u8(mask, pool))
+    timed("pack_selected (fp32 values)", k * (4 + 32 + 32 + 4.0),
+          lambda: K.pack_selected(g, idx, values, 1.0))
+    timed("scatter_selected", k * (4 + 4 + 32.0), lambda: K.scatter_selected(g, idx, values))
+    timed("compact_norm_sq_contribution", k * 4.0,
+          lambda: K.compact_norm_sq_contribution(values, total))
+    timed("masked_norm_sq_contribution", n * 5.0,
+          lambda: K.masked_norm_sq_contribution(g, mask, total))
+    timed("adamw_grad_correct sparse (mask, clear)", n * 33.0,
+          lambda: adamw_grad_correct(p, g, m, v, 1e-4, 0.9, 0.95, 1e-8, 0.1, 3, mask=mask,
+                                     coeff=0.5, clear=True))
+    timed("adamw_grad_correct full (emit update)", n * 32.0,
+          lambda: adamw_grad_correct(p, g, m, v, 1e-4, 0.9, 0.95, 1e-8, 0.1, 3,
+                                     emit_score="update"))
+    timed("adamw_grad_correct_compact (dir table)", n * 24.0 + k * 8.0,
+          lambda: adamw_grad_correct_compact(p, g, m, v, idx, values, 0, 1e-4, 0.9, 0.95, 1e-8,
+                                             0.1, 3, coeff=0.5, dir_table=table))
+    timed("formula('update') score", n * 20.0,
+          lambda: RK.formula("update")(p, m, v, g, 0.9, 0.95, 1e-8, 0.1, 0.271, 0.143))   # w, m, v, g
+    timed("opt_step_inplace (replay commit)", n * 28.0,
+          lambda: RK.opt_step_inplace(g, m, v, p, None, 1e-4, 0.1, 0.9, 0.95, 0.271, 0.143, 1e-8))
+    return {"n": n, "k": k, "rows": rows,
+            "note": "pack/scatter bytes count a 32-byte sector per random 4-byte access"}
+
+
 def trace_io_bench(W=4, tmp=None):
     """Recorded-trace leg: writes a W-step bf16 trace of the Qwen3-0.6B shapes in
     the reference writer's layout under a temp dir, then streams it back through
@@ -267,6 +337,8 @@ def main():
     ap.add_argument("--trace-io", action="store_true",
                     help="run just the recorded-trace leg (writes a temporary trace, streams it "
                          "back through the pread reader and the dense pass) and print its JSON")
+    ap.add_argument("--primitives", action="store_true",
+                    help="time the drop-in primitives on their own and print their JSON")
     ap.add_argument("--only-replay", action="store_true",
                     help="run just the fused replay leg (for profiling) and print its JSON")
     ap.add_argument("--sweep", action="store_true",
@@ -290,6 +362,10 @@ def main():
     if args.trace_io:
         torch.cuda.set_device(0)
         print(json.dumps(trace_io_bench()))
+        return
+    if args.primitives:
+        torch.cuda.set_device(0)
+        print(json.dumps(primitives_bench()))
         return
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)

@@ -15,7 +15,9 @@ namespace sga {
 
 // One 4-element vector of the masked / full-step commit.
 // EMIT: -1 sparse step; 0 update, 1 |g|, 2 |m|, 3 coi -> written into g.
-template <int EMIT>
+// FULL: the whole workgroup span is in range and every array vector-aligned,
+// so all loads are unconditional and in flight together.
+template <int EMIT, bool FULL>
 __device__ __forceinline__ void gc_vec(float* __restrict__ p, float* __restrict__ g,
                                        float* __restrict__ m, float* __restrict__ v,
                                        const uint8_t* __restrict__ mask, int64_t i, int64_t n,
@@ -29,16 +31,15 @@ __device__ __forceinline__ void gc_vec(float* __restrict__ p, float* __restrict_
   const bool adams = flags & SGA_GC_ADAMS;   // v basis = pre-commit m*m, h.bc1 = h.bc2 = 1
   float pp[4], gg[4], mm[4], vv[4];
   uint32_t mk[4] = {1, 1, 1, 1};
-  load4_f32(p, i, n, pp, vec);
-  load4_f32(g, i, n, gg, vec);
-  load4_f32(m, i, n, mm, vec);
+  ld_f32<FULL>(p, i, n, pp, vec);
+  ld_f32<FULL>(g, i, n, gg, vec);
+  ld_f32<FULL>(m, i, n, mm, vec);
+  if (!adams) ld_f32<FULL>(v, i, n, vv, vec);
+  if (has_mask) ld_u8<FULL>(mask, i, n, mk, vec);
   if (adams) {
 #pragma unroll
     for (int e = 0; e < 4; ++e) vv[e] = mm[e] * mm[e];
-  } else {
-    load4_f32(v, i, n, vv, vec);
   }
-  if (has_mask) load4_u8(mask, i, n, mk, vec);
   float gout[4];
 #pragma unroll
   for (int e = 0; e < 4; ++e) {
@@ -62,10 +63,10 @@ __device__ __forceinline__ void gc_vec(float* __restrict__ p, float* __restrict_
     mm[e] = c.m_new;
     vv[e] = c.v_new;
   }
-  store4_f32(m, i, n, mm, vec);
-  store4_f32(v, i, n, vv, vec);
-  if (EMIT >= 0 || clear || fold) store4_f32(g, i, n, gout, vec);
-  store4_f32(p, i, n, pp, vec);
+  st_f32<FULL>(m, i, n, mm, vec);
+  st_f32<FULL>(v, i, n, vv, vec);
+  if (EMIT >= 0 || clear || fold) st_f32<FULL>(g, i, n, gout, vec);
+  st_f32<FULL>(p, i, n, pp, vec);
 }
 
 template <int EMIT>
@@ -74,8 +75,13 @@ __global__ __launch_bounds__(kBlock) void k_grad_correct(
     float* __restrict__ v, const uint8_t* __restrict__ mask, int64_t n, Hyper h,
     float coeff, float interval, float lr_inactive, int flags, bool vec) {
   const int64_t stride = (int64_t)gridDim.x * kBlock * kVec;
-  for (int64_t i = ((int64_t)blockIdx.x * kBlock + threadIdx.x) * kVec; i < n; i += stride)
-    gc_vec<EMIT>(p, g, m, v, mask, i, n, h, coeff, interval, lr_inactive, flags, vec);
+  for (int64_t base = (int64_t)blockIdx.x * kBlock * kVec; base < n; base += stride) {
+    const int64_t i = base + (int64_t)threadIdx.x * kVec;
+    if (vec && base + kBlock * kVec <= n)
+      gc_vec<EMIT, true>(p, g, m, v, mask, i, n, h, coeff, interval, lr_inactive, flags, true);
+    else if (i < n)
+      gc_vec<EMIT, false>(p, g, m, v, mask, i, n, h, coeff, interval, lr_inactive, flags, vec);
+  }
 }
 
 // The same commit over MANY records (one per parameter tensor) in one launch:
@@ -106,12 +112,16 @@ __global__ __launch_bounds__(kBlock) void k_grad_correct_multi(const GcRecord* _
   const bool vec = aligned4(r.p, 4) && aligned4(r.g, 4) && aligned4(r.m, 4) && aligned4(r.v, 4) &&
                    aligned4(r.mask, 1);
   const int64_t base = (span - r.first_span) * kBlockSpan;
+  const bool full = vec && base + kBlockSpan <= r.n;
 #pragma unroll
   for (int it = 0; it < kBlockSpan / (kBlock * kVec); ++it) {
     const int64_t i = base + ((int64_t)it * kBlock + threadIdx.x) * kVec;
-    if (i < r.n)
-      gc_vec<EMIT>(r.p, r.g, r.m, r.v, r.mask, i, r.n, h, coeff, interval, r.lr_inactive, r.flags,
-                   vec);
+    if (full)
+      gc_vec<EMIT, true>(r.p, r.g, r.m, r.v, r.mask, i, r.n, h, coeff, interval, r.lr_inactive,
+                         r.flags, true);
+    else if (i < r.n)
+      gc_vec<EMIT, false>(r.p, r.g, r.m, r.v, r.mask, i, r.n, h, coeff, interval, r.lr_inactive,
+                          r.flags, vec);
   }
 }
 
@@ -322,7 +332,7 @@ extern "C" int sga_adamw_grad_correct(float* p, float* g, float* m, float* v,
   const Hyper h = mk_hyper(lr, beta1, om1, beta2, om2, eps, wd, bc1, bc2);
   const bool vec = aligned4(p, 4) && aligned4(g, 4) && aligned4(m, 4) &&
                    aligned4(v, 4) && aligned4(mask, 1);
-  dim3 grid(stream_grid(n, (int64_t)kBlock * kVec)), block(kBlock);
+  dim3 grid(stream_grid(n, (int64_t)kBlock * kVec, 1 << 22)), block(kBlock);
   hipStream_t st = (hipStream_t)stream;
 #define SGA_GC_LAUNCH(E)                                                       \
   hipLaunchKernelGGL((k_grad_correct<E>), grid, block, 0, st, p, g, m, v, mask, \
@@ -393,7 +403,7 @@ extern "C" int sga_adamw_grad_correct_compact(
   if (flags & SGA_GC_ADAMS) { bc1 = 1.0f; bc2 = 1.0f; }
   const Hyper h = mk_hyper(lr, beta1, om1, beta2, om2, eps, wd, bc1, bc2);
   const bool vec = aligned4(p, 4) && aligned4(g, 4) && aligned4(m, 4) && aligned4(v, 4);
-  dim3 grid(stream_grid(n, kBlockSpan)), block(kBlock);
+  dim3 grid(stream_grid(n, kBlockSpan, 1 << 22)), block(kBlock);
   hipStream_t st = (hipStream_t)stream;
   if (values_dtype == SGA_BF16)
     hipLaunchKernelGGL((k_grad_correct_compact<true>), grid, block, 0, st, p, g, m, v, idx, values, rec_start, n, k_total, h, coeff, interval, flags, dir_table, n_table, vec);

@@ -12,28 +12,40 @@
 
 namespace sga {
 
+template <int SCORE, bool FULL>
+__device__ __forceinline__ void score_vec(const float* __restrict__ w, const float* __restrict__ m,
+                                          const float* __restrict__ v, const float* __restrict__ g,
+                                          float* __restrict__ out, int64_t i, int64_t n,
+                                          const Hyper& h, bool absolute, bool adams, bool vec) {
+  float ww[4] = {0, 0, 0, 0}, mm[4] = {0, 0, 0, 0}, vv[4] = {0, 0, 0, 0}, gg[4] = {0, 0, 0, 0};
+  if (SCORE != SGA_SCORE_ABS_M) ld_f32<FULL>(g, i, n, gg, vec);
+  if (SCORE != SGA_SCORE_ABS_G) ld_f32<FULL>(m, i, n, mm, vec);
+  if (SCORE == SGA_SCORE_UPDATE || SCORE == SGA_SCORE_COI) {
+    ld_f32<FULL>(w, i, n, ww, vec);
+    if (!adams) ld_f32<FULL>(v, i, n, vv, vec);
+  }
+  float o[4];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const float ve = adams ? mm[e] * mm[e] : vv[e];
+    const float s = score_value<SCORE>(gg[e], ww[e], mm[e], ve, h);
+    o[e] = absolute ? fabsf(s) : s;
+  }
+  st_f32<FULL>(out, i, n, o, vec);
+}
+
 template <int SCORE>
 __global__ __launch_bounds__(kBlock) void k_score_formula(
     const float* __restrict__ w, const float* __restrict__ m, const float* __restrict__ v,
     const float* __restrict__ g, float* __restrict__ out, int64_t n, Hyper h, bool absolute,
     bool adams, bool vec) {
   const int64_t stride = (int64_t)gridDim.x * kBlock * kVec;
-  for (int64_t i = ((int64_t)blockIdx.x * kBlock + threadIdx.x) * kVec; i < n; i += stride) {
-    float ww[4] = {0, 0, 0, 0}, mm[4] = {0, 0, 0, 0}, vv[4] = {0, 0, 0, 0}, gg[4] = {0, 0, 0, 0};
-    if (SCORE != SGA_SCORE_ABS_M) load4_f32(g, i, n, gg, vec);
-    if (SCORE != SGA_SCORE_ABS_G) load4_f32(m, i, n, mm, vec);
-    if (SCORE == SGA_SCORE_UPDATE || SCORE == SGA_SCORE_COI) {
-      load4_f32(w, i, n, ww, vec);
-      if (!adams) load4_f32(v, i, n, vv, vec);
-    }
-    float o[4];
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      const float ve = adams ? mm[e] * mm[e] : vv[e];
-      const float s = score_value<SCORE>(gg[e], ww[e], mm[e], ve, h);
-      o[e] = absolute ? fabsf(s) : s;
-    }
-    store4_f32(out, i, n, o, vec);
+  for (int64_t base = (int64_t)blockIdx.x * kBlock * kVec; base < n; base += stride) {
+    const int64_t i = base + (int64_t)threadIdx.x * kVec;
+    if (vec && base + kBlock * kVec <= n)
+      score_vec<SCORE, true>(w, m, v, g, out, i, n, h, absolute, adams, true);
+    else if (i < n)
+      score_vec<SCORE, false>(w, m, v, g, out, i, n, h, absolute, adams, vec);
   }
 }
 
@@ -89,44 +101,57 @@ struct StepK {
   float b1, om1, b2, om2, bc1, bc2, eps, omlwd, neglr, lr2, lr, lri, wd;
 };
 
+template <bool ADAMS, bool SPLIT, bool LAB, bool FULL>
+__device__ __forceinline__ void opt_step_vec(const float* __restrict__ q, float* __restrict__ m,
+                                             float* __restrict__ v, float* __restrict__ w,
+                                             float* __restrict__ lab,
+                                             const uint8_t* __restrict__ inactive, int64_t i,
+                                             int64_t n, const StepK& c, bool vec) {
+  float qq[4], mm[4], vv[4] = {0, 0, 0, 0}, ww[4], ll[4] = {0, 0, 0, 0};
+  uint32_t ina[4] = {0, 0, 0, 0};
+  ld_f32<FULL>(q, i, n, qq, vec);
+  ld_f32<FULL>(m, i, n, mm, vec);
+  if (!ADAMS) ld_f32<FULL>(v, i, n, vv, vec);
+  ld_f32<FULL>(w, i, n, ww, vec);
+  if (LAB) ld_f32<FULL>(lab, i, n, ll, vec);
+  if (SPLIT) ld_u8<FULL>(inactive, i, n, ina, vec);
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    float vb = ADAMS ? (mm[e] * mm[e]) * c.b2 : vv[e] * c.b2;
+    const float vn = __fmaf_rn(qq[e] * c.om2, qq[e], vb);
+    const float mn = __fmaf_rn(qq[e], c.om1, mm[e] * c.b1);
+    const float mh = __fdiv_rn(mn, c.bc1);
+    const float vh = __fsqrt_rn(__fdiv_rn(vn, c.bc2));
+    const float upd = __fdiv_rn(mh, vh + c.eps);
+    if (SPLIT) {
+      const float step = ina[e] ? c.lri : c.lr;
+      const float full = ww[e] * c.wd + upd;
+      ww[e] = __fmaf_rn(-full, step, ww[e]);
+    } else {
+      ww[e] = __fmaf_rn(upd, c.neglr, ww[e] * c.omlwd);
+    }
+    if (LAB) ll[e] = __fmaf_rn(upd * c.lr2, upd, ll[e]);
+    mm[e] = mn;
+    vv[e] = vn;
+  }
+  st_f32<FULL>(m, i, n, mm, vec);
+  st_f32<FULL>(v, i, n, vv, vec);
+  st_f32<FULL>(w, i, n, ww, vec);
+  if (LAB) st_f32<FULL>(lab, i, n, ll, vec);
+}
+
 template <bool ADAMS, bool SPLIT, bool LAB>
 __global__ __launch_bounds__(kBlock) void k_opt_step(
     const float* __restrict__ q, float* __restrict__ m, float* __restrict__ v,
     float* __restrict__ w, float* __restrict__ lab, const uint8_t* __restrict__ inactive,
     int64_t n, StepK c, bool vec) {
   const int64_t stride = (int64_t)gridDim.x * kBlock * kVec;
-  for (int64_t i = ((int64_t)blockIdx.x * kBlock + threadIdx.x) * kVec; i < n; i += stride) {
-    float qq[4], mm[4], vv[4] = {0, 0, 0, 0}, ww[4], ll[4] = {0, 0, 0, 0};
-    uint32_t ina[4] = {0, 0, 0, 0};
-    load4_f32(q, i, n, qq, vec);
-    load4_f32(m, i, n, mm, vec);
-    if (!ADAMS) load4_f32(v, i, n, vv, vec);
-    load4_f32(w, i, n, ww, vec);
-    if (LAB) load4_f32(lab, i, n, ll, vec);
-    if (SPLIT) load4_u8(inactive, i, n, ina, vec);
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      float vb = ADAMS ? (mm[e] * mm[e]) * c.b2 : vv[e] * c.b2;
-      const float vn = __fmaf_rn(qq[e] * c.om2, qq[e], vb);
-      const float mn = __fmaf_rn(qq[e], c.om1, mm[e] * c.b1);
-      const float mh = __fdiv_rn(mn, c.bc1);
-      const float vh = __fsqrt_rn(__fdiv_rn(vn, c.bc2));
-      const float upd = __fdiv_rn(mh, vh + c.eps);
-      if (SPLIT) {
-        const float step = ina[e] ? c.lri : c.lr;
-        const float full = ww[e] * c.wd + upd;
-        ww[e] = __fmaf_rn(-full, step, ww[e]);
-      } else {
-        ww[e] = __fmaf_rn(upd, c.neglr, ww[e] * c.omlwd);
-      }
-      if (LAB) ll[e] = __fmaf_rn(upd * c.lr2, upd, ll[e]);
-      mm[e] = mn;
-      vv[e] = vn;
-    }
-    store4_f32(m, i, n, mm, vec);
-    store4_f32(v, i, n, vv, vec);
-    store4_f32(w, i, n, ww, vec);
-    if (LAB) store4_f32(lab, i, n, ll, vec);
+  for (int64_t base = (int64_t)blockIdx.x * kBlock * kVec; base < n; base += stride) {
+    const int64_t i = base + (int64_t)threadIdx.x * kVec;
+    if (vec && base + kBlock * kVec <= n)
+      opt_step_vec<ADAMS, SPLIT, LAB, true>(q, m, v, w, lab, inactive, i, n, c, true);
+    else if (i < n)
+      opt_step_vec<ADAMS, SPLIT, LAB, false>(q, m, v, w, lab, inactive, i, n, c, vec);
   }
 }
 
@@ -153,7 +178,7 @@ extern "C" int sga_score_formula(int score_id, const float* w, const float* m, c
   const Hyper h = mk_hyper(0.0f, beta1, om1, beta2, om2, eps, wd, bc1, bc2);
   const bool vec = aligned4(w, 4) && aligned4(m, 4) && aligned4(v, 4) && aligned4(g, 4) &&
                    aligned4(out, 4);
-  dim3 grid(stream_grid(n, (int64_t)kBlock * kVec)), block(kBlock);
+  dim3 grid(stream_grid(n, (int64_t)kBlock * kVec, 1 << 22)), block(kBlock);
   hipStream_t st = (hipStream_t)stream;
 #define SGA_SF(S) hipLaunchKernelGGL((k_score_formula<S>), grid, block, 0, st, w, m, v, g, out, n, h, absolute != 0, adams != 0, vec)
   switch (score_id) {
@@ -185,7 +210,7 @@ extern "C" int sga_branch_score_f64(int score_id, const float* w, const float* m
   const BranchK c{beta1, 1.0 - beta1, beta2, 1.0 - beta2, eps, wd, bc1, bc2};
   const bool vec = aligned4(w, 4) && aligned4(m, 4) && aligned4(v, 4) && aligned4(g, 4) &&
                    aligned4(out, 4);
-  dim3 grid(stream_grid(n, (int64_t)kBlock * kVec)), block(kBlock);
+  dim3 grid(stream_grid(n, (int64_t)kBlock * kVec, 1 << 22)), block(kBlock);
   hipStream_t st = (hipStream_t)stream;
 #define SGA_BS(S) hipLaunchKernelGGL((k_branch_score<S>), grid, block, 0, st, w, m, v, g, out, n, c, adams != 0, include_wd != 0, vec)
   switch (score_id) {
@@ -213,7 +238,7 @@ extern "C" int sga_opt_step_inplace(const float* q, float* m, float* v, float* w
   StepK c{beta1, om1, beta2, om2, bc1, bc2, eps, omlwd, neglr, lr2, lr, lr_inactive, wd};
   const bool vec = aligned4(q, 4) && aligned4(m, 4) && aligned4(v, 4) && aligned4(w, 4) &&
                    aligned4(lab, 4) && aligned4(inactive, 1);
-  dim3 grid(stream_grid(n, (int64_t)kBlock * kVec)), block(kBlock);
+  dim3 grid(stream_grid(n, (int64_t)kBlock * kVec, 1 << 22)), block(kBlock);
   hipStream_t st = (hipStream_t)stream;
 #define SGA_OS(A, S, L) hipLaunchKernelGGL((k_opt_step<A, S, L>), grid, block, 0, st, q, m, v, w, lab, inactive, n, c, vec)
   const int sel = (adams ? 4 : 0) | (split ? 2 : 0) | (has_lab ? 1 : 0);

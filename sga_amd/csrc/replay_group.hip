@@ -548,7 +548,7 @@ extern "C" int sga_replay_pass3(const void* g, int g_dtype, int64_t n, float coe
   }
   const bool bg = g_dtype == SGA_BF16;
   const bool vec = aligned4(g, bg ? 2 : 4) && group_aligned(grp);
-  const unsigned nb = stream_grid(n, (int64_t)kBlock * kVec, kReplayBlocks);
+  const unsigned nb = stream_grid(n, (int64_t)kBlock * kVec, 1 << 22);   // one-shot: nothing to reduce
   hipStream_t s = (hipStream_t)stream;
   const RSeg* rs = reinterpret_cast<const RSeg*>(segs);
   if (bg) hipLaunchKernelGGL((k_replay_pass3<true>), dim3(nb), dim3(kBlock), 0, s, g, n, coef_dense, grp, coef_f, rs, n_segs, vec);
