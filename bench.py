@@ -251,6 +251,15 @@ def primitives_bench(n=1 << 28, ratio=1.0):
           lambda: RK.formula("update")(p, m, v, g, 0.9, 0.95, 1e-8, 0.1, 0.271, 0.143))   # w, m, v, g
     timed("opt_step_inplace (replay commit)", n * 28.0,
           lambda: RK.opt_step_inplace(g, m, v, p, None, 1e-4, 0.1, 0.9, 0.95, 0.271, 0.143, 1e-8))
+    from sga_amd.clip import scale_masked_
+    from sga_amd.selection import threshold_masks
+    tau = float(score.float().kthvalue(n - k + 1).values) if n <= (1 << 24) else 2.58e-3
+    timed("threshold_masks (|g| >= tau, mask + count)", n * 5.0, lambda: threshold_masks([g], tau))
+    timed("scale_masked_ (clip scale under a mask)", n * 1.0 + k * 64.0,
+          lambda: scale_masked_(g, mask, 1.0))
+    timed("scale_masked_ (whole tensor)", n * 8.0, lambda: scale_masked_(g, None, 1.0))
+    timed("gt_eq_counts (two masks + counts)", n * 6.0, lambda: RK.gt_eq_counts(score, tau))
+    timed("hist_top16 (incl. 256 KiB histogram to host)", n * 4.0, lambda: RK.hist_top16(score))
     return {"n": n, "k": k, "rows": rows,
             "note": "pack/scatter bytes count a 32-byte sector per random 4-byte access"}
 

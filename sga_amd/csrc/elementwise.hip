@@ -436,10 +436,13 @@ __global__ __launch_bounds__(kBlock) void k_scale_masked(float* __restrict__ g,
                                                          int64_t n, float coeff, bool vec) {
   const int64_t stride = (int64_t)gridDim.x * kBlock * kVec;
   for (int64_t i = ((int64_t)blockIdx.x * kBlock + threadIdx.x) * kVec; i < n; i += stride) {
+    uint32_t mk[4] = {1u, 1u, 1u, 1u};
+    if (MASKED) {
+      load4_u8(mask, i, n, mk, vec);
+      if (!(mk[0] | mk[1] | mk[2] | mk[3])) continue;   // untouched lanes move no gradient bytes
+    }
     float v[4];
     load4_f32(g, i, n, v, vec);
-    uint32_t mk[4] = {1u, 1u, 1u, 1u};
-    if (MASKED) load4_u8(mask, i, n, mk, vec);
 #pragma unroll
     for (int e = 0; e < 4; ++e) v[e] = mk[e] ? v[e] * coeff : v[e];
     store4_f32(g, i, n, v, vec);
@@ -450,7 +453,7 @@ extern "C" int sga_scale_masked(float* grad, const uint8_t* mask, int64_t n, flo
                                 void* stream) {
   if (n == 0) return SGA_OK;
   if (!grad || n < 0) { set_error("sga_scale_masked: bad argument"); return SGA_ERR_ARG; }
-  dim3 grid(stream_grid(n, (int64_t)kBlock * kVec * 4, 256 * 8)), block(kBlock);
+  dim3 grid(stream_grid(n, (int64_t)kBlock * kVec, 1 << 22)), block(kBlock);
   const bool vec = aligned4(grad, 4) && aligned4(mask, 1);
   if (mask)
     hipLaunchKernelGGL((k_scale_masked<true>), grid, block, 0, (hipStream_t)stream, grad, mask, n, coeff, vec);
@@ -523,7 +526,7 @@ extern "C" int sga_mask_count(const uint8_t* mask, int64_t n,
   hipStream_t st = (hipStream_t)stream;
   const int64_t nc = n_chunks_of(n);
   if (nc > 0)
-    hipLaunchKernelGGL(k_mask_count, dim3(stream_grid(nc, kChunksPerBlock)),
+    hipLaunchKernelGGL(k_mask_count, dim3(stream_grid(nc, kChunksPerBlock, 1 << 22)),
                        dim3(kBlock), 0, st, mask, n, chunk_counts, nc,
                        aligned4(mask, 1));
   int rc = exclusive_scan_u32(chunk_counts, nc, total, st);
@@ -541,7 +544,7 @@ extern "C" int sga_mask_fill(const uint8_t* mask, int64_t n,
     return SGA_ERR_ARG;
   }
   const int64_t nc = n_chunks_of(n);
-  hipLaunchKernelGGL(k_mask_fill, dim3(stream_grid(nc, kChunksPerBlock)),
+  hipLaunchKernelGGL(k_mask_fill, dim3(stream_grid(nc, kChunksPerBlock, 1 << 22)),
                      dim3(kBlock), 0, (hipStream_t)stream, mask, n,
                      chunk_offsets, idx_out, idx_capacity, nc,
                      aligned4(mask, 1));

@@ -628,7 +628,7 @@ extern "C" int64_t sga_plane_words(int64_t n) {
 extern "C" int sga_mask_to_planes(const uint8_t* mask, int64_t n, uint32_t* planes, void* stream) {
   if (n == 0) return SGA_OK;
   if (!mask || !planes || n < 0) { set_error("sga_mask_to_planes: bad argument"); return SGA_ERR_ARG; }
-  hipLaunchKernelGGL(k_mask_to_planes, dim3(stream_grid(cdiv64(n, kChunk), kChunksPerBlock, 1 << 14)),
+  hipLaunchKernelGGL(k_mask_to_planes, dim3(stream_grid(cdiv64(n, kChunk), kChunksPerBlock, 1 << 22)),
                      dim3(kBlock), 0, (hipStream_t)stream, mask, n, planes, aligned4(mask, 1));
   return check_launch("sga_mask_to_planes");
 }
@@ -636,7 +636,7 @@ extern "C" int sga_mask_to_planes(const uint8_t* mask, int64_t n, uint32_t* plan
 extern "C" int sga_planes_to_mask(const uint32_t* planes, int64_t n, uint8_t* mask, void* stream) {
   if (n == 0) return SGA_OK;
   if (!mask || !planes || n < 0) { set_error("sga_planes_to_mask: bad argument"); return SGA_ERR_ARG; }
-  hipLaunchKernelGGL(k_expand_mask, dim3(stream_grid(cdiv64(n, kChunk), kChunksPerBlock, 1 << 14)),
+  hipLaunchKernelGGL(k_expand_mask, dim3(stream_grid(cdiv64(n, kChunk), kChunksPerBlock, 1 << 22)),
                      dim3(kBlock), 0, (hipStream_t)stream, (const SelState*)nullptr, planes, n, mask,
                      (reinterpret_cast<uintptr_t>(mask) & 15) == 0);
   return check_launch("sga_planes_to_mask");
@@ -645,7 +645,7 @@ extern "C" int sga_planes_to_mask(const uint32_t* planes, int64_t n, uint8_t* ma
 extern "C" int sga_div_inplace(float* x, int64_t n, float d, int packed, void* stream) {
   if (n == 0) return SGA_OK;
   if (!x || n < 0) { set_error("sga_div_inplace: bad argument"); return SGA_ERR_ARG; }
-  hipLaunchKernelGGL(k_div_inplace, dim3(stream_grid(n, (int64_t)kBlock * kVec)), dim3(kBlock), 0,
+  hipLaunchKernelGGL(k_div_inplace, dim3(stream_grid(n, (int64_t)kBlock * kVec, 1 << 22)), dim3(kBlock), 0,
                      (hipStream_t)stream, x, n, d, aligned4(x, 4), packed ? kPackExtra : 0);
   return check_launch("sga_div_inplace");
 }

@@ -36,6 +36,47 @@ __global__ __launch_bounds__(kBlock) void k_hist_topbits(
   if (lane_id() == 0 && nf && nonfinite) atomicAdd(nonfinite, nf);
 }
 
+// Same histogram over every element of a 16-byte aligned array: 1024 lanes share one LDS table (the
+// 128 KiB of 32769 bins leave room for one workgroup per CU, so the workgroup is made as wide as it
+// can be), and each lane keeps two 16-byte loads in flight per trip.
+constexpr int kHistWide = 1024;
+__global__ __launch_bounds__(kHistWide) void k_hist_topbits_dense(
+    const float* __restrict__ x, int64_t n, int shift, unsigned long long* __restrict__ hist,
+    int nbins, uint32_t* __restrict__ nonfinite) {
+  extern __shared__ uint32_t s_h[];
+  for (int b = threadIdx.x; b < nbins; b += kHistWide) s_h[b] = 0u;
+  __syncthreads();
+  uint32_t nf = 0;
+  constexpr int64_t kSlab = (int64_t)kHistWide * kVec;
+  const int64_t step = (int64_t)gridDim.x * kSlab * 2;
+  // trip count is uniform over the workgroup: the ballots inside lds_hist_add need whole waves
+  for (int64_t base = (int64_t)blockIdx.x * kSlab * 2; base < n; base += step) {
+    float v[2][4];
+    const int64_t i0 = base + (int64_t)threadIdx.x * kVec;
+#pragma unroll
+    for (int u = 0; u < 2; ++u) load4_f32(x, i0 + u * kSlab, n, v[u], true);
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const bool ok = i0 + u * kSlab + e < n;
+        const uint32_t key = ok ? abs_key(v[u][e]) : 0u;
+        nf += (ok && key >= 0x7F800000u);
+        uint32_t bin = key >> shift;
+        if (bin >= (uint32_t)nbins) bin = nbins - 1;
+        lds_hist_add(s_h, bin, ok);
+      }
+    }
+  }
+  __syncthreads();
+  for (int b = threadIdx.x; b < nbins; b += kHistWide) {
+    const uint32_t c = s_h[b];
+    if (c) atomicAdd(&hist[b], (unsigned long long)c);
+  }
+  nf = wave_sum(nf);
+  if (lane_id() == 0 && nf && nonfinite) atomicAdd(nonfinite, nf);
+}
+
 __global__ __launch_bounds__(kBlock) void k_mask_topbits_ge(
     const float* __restrict__ x, int64_t n, int shift, uint32_t bin,
     uint8_t* __restrict__ mask, bool vec) {
@@ -105,27 +146,42 @@ __global__ __launch_bounds__(kBlock) void k_gt_eq(
     const float* __restrict__ x, int64_t n, float thresh, uint8_t* __restrict__ gt,
     uint8_t* __restrict__ eq, int32_t* __restrict__ counts, bool vec) {
   uint32_t cg = 0, ce = 0;
-  const int64_t stride = (int64_t)gridDim.x * kBlock * kVec;
-  for (int64_t i = ((int64_t)blockIdx.x * kBlock + threadIdx.x) * kVec; i < n; i += stride) {
-    float v[4];
-    load4_f32(x, i, n, v, vec);
-    uint32_t g4[4], e4[4];
+  // Capped grid (few count atomics), four independent loads per lane and trip.
+  constexpr int kUnroll = 4;
+  constexpr int64_t kSlab = (int64_t)kBlock * kVec;
+  const int64_t stride = (int64_t)gridDim.x * kSlab * kUnroll;
+  for (int64_t b = (int64_t)blockIdx.x * kSlab * kUnroll + (int64_t)threadIdx.x * kVec; b < n;
+       b += stride) {
+    float v[kUnroll][4];
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      const bool ok = i + e < n;
-      g4[e] = ok && v[e] > thresh;
-      e4[e] = ok && v[e] == thresh;
-      cg += g4[e];
-      ce += e4[e];
+    for (int u = 0; u < kUnroll; ++u) load4_f32(x, b + u * kSlab, n, v[u], vec);
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+      const int64_t i = b + u * kSlab;
+      if (i >= n) break;
+      uint32_t g4[4], e4[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const bool ok = i + e < n;
+        g4[e] = ok && v[u][e] > thresh;
+        e4[e] = ok && v[u][e] == thresh;
+        cg += g4[e];
+        ce += e4[e];
+      }
+      store4_u8(gt, i, n, g4, vec);
+      store4_u8(eq, i, n, e4, vec);
     }
-    store4_u8(gt, i, n, g4, vec);
-    store4_u8(eq, i, n, e4, vec);
   }
+  __shared__ uint32_t s_g[kChunksPerBlock], s_e[kChunksPerBlock];
   cg = wave_sum(cg);
   ce = wave_sum(ce);
-  if (lane_id() == 0) {
-    if (cg) atomicAdd(&counts[0], (int32_t)cg);
-    if (ce) atomicAdd(&counts[1], (int32_t)ce);
+  if (lane_id() == 0) { s_g[wave_id()] = cg; s_e[wave_id()] = ce; }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    const uint32_t tg = s_g[0] + s_g[1] + s_g[2] + s_g[3];
+    const uint32_t te = s_e[0] + s_e[1] + s_e[2] + s_e[3];
+    if (tg) atomicAdd(&counts[0], (int32_t)tg);
+    if (te) atomicAdd(&counts[1], (int32_t)te);
   }
 }
 
@@ -137,17 +193,28 @@ __global__ __launch_bounds__(kBlock) void k_mask_abs_ge(const float* __restrict_
                                                         bool vec) {
   __shared__ uint32_t s_w[kChunksPerBlock];
   uint32_t c = 0;
-  const int64_t stride = (int64_t)gridDim.x * kBlock * kVec;
-  for (int64_t i = ((int64_t)blockIdx.x * kBlock + threadIdx.x) * kVec; i < n; i += stride) {
-    float v[4];
-    load4_f32(x, i, n, v, vec);
-    uint32_t mk[4];
+  // Four independent 16-byte loads per lane and trip keep enough bytes in flight for a grid small
+  // enough that its one count atomic per block does not queue up on the single counter.
+  constexpr int kUnroll = 4;
+  constexpr int64_t kSlab = (int64_t)kBlock * kVec;
+  const int64_t stride = (int64_t)gridDim.x * kSlab * kUnroll;
+  for (int64_t b = (int64_t)blockIdx.x * kSlab * kUnroll + (int64_t)threadIdx.x * kVec; b < n;
+       b += stride) {
+    float v[kUnroll][4];
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      mk[e] = (i + e < n) && fabsf(v[e]) >= tau;
-      c += mk[e];
+    for (int u = 0; u < kUnroll; ++u) load4_f32(x, b + u * kSlab, n, v[u], vec);
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+      const int64_t i = b + u * kSlab;
+      if (i >= n) break;
+      uint32_t mk[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        mk[e] = (i + e < n) && fabsf(v[u][e]) >= tau;
+        c += mk[e];
+      }
+      store4_u8(mask, i, n, mk, vec);
     }
-    store4_u8(mask, i, n, mk, vec);
   }
   c = wave_sum(c);
   if (lane_id() == 0) s_w[wave_id()] = c;
@@ -241,7 +308,7 @@ extern "C" int sga_sel_mask(const float* score, int64_t n, int64_t tile_base, in
   if (!score || !mask_out || n < 0 || tile_base < 0) { set_error("sga_sel_mask: bad argument"); return SGA_ERR_ARG; }
   SrcF32 src{score, aligned4(score, 4)};
   const int64_t nc = cdiv64(n, kChunk);
-  hipLaunchKernelGGL((k_write_mask<SrcF32>), dim3(stream_grid(nc, kChunksPerBlock)), dim3(kBlock), 0,
+  hipLaunchKernelGGL((k_write_mask<SrcF32>), dim3(stream_grid(nc, kChunksPerBlock, 1 << 22)), dim3(kBlock), 0,
                      (hipStream_t)stream, src, n, tile_base, tie_mode == SGA_TIE_ALL, w.st,
                      w.tile_gt, w.tile_eq, mask_out, aligned4(mask_out, 1));
   return check_launch("sga_sel_mask");
@@ -285,6 +352,12 @@ extern "C" int sga_hist_topbits(const float* score, int64_t n, int shift, int st
   }
   const int64_t n_s = n <= phase ? 0 : (n - phase + stride - 1) / stride;
   if (n_s == 0) return SGA_OK;
+  if (stride == 1 && aligned4(score, 4)) {
+    hipLaunchKernelGGL(k_hist_topbits_dense, dim3(stream_grid(n, (int64_t)kHistWide * kVec * 2, 256)),
+                       dim3(kHistWide), (size_t)nbins * 4, (hipStream_t)stream, score, n, shift,
+                       reinterpret_cast<unsigned long long*>(hist), nbins, nonfinite);
+    return check_launch("sga_hist_topbits");
+  }
   hipLaunchKernelGGL(k_hist_topbits, dim3(stream_grid(n_s, (int64_t)kBlock * 16, 256 * 2)),
                      dim3(kBlock), (size_t)nbins * 4, (hipStream_t)stream, score, n, shift, stride,
                      phase, reinterpret_cast<unsigned long long*>(hist), nbins, nonfinite);
@@ -298,7 +371,7 @@ extern "C" int sga_mask_topbits_ge(const float* score, int64_t n, int shift, int
     set_error("sga_mask_topbits_ge: bad argument");
     return SGA_ERR_ARG;
   }
-  hipLaunchKernelGGL(k_mask_topbits_ge, dim3(stream_grid(n, (int64_t)kBlock * kVec)), dim3(kBlock),
+  hipLaunchKernelGGL(k_mask_topbits_ge, dim3(stream_grid(n, (int64_t)kBlock * kVec, 1 << 22)), dim3(kBlock),
                      0, (hipStream_t)stream, score, n, shift, (uint32_t)bin, mask_out,
                      aligned4(score, 4) && aligned4(mask_out, 1));
   return check_launch("sga_mask_topbits_ge");
@@ -308,7 +381,7 @@ extern "C" int sga_mask_abs_ge(const float* score, int64_t n, float tau, uint8_t
                                int64_t* count, void* stream) {
   if (n == 0) return SGA_OK;
   if (!score || !mask_out || n < 0) { set_error("sga_mask_abs_ge: bad argument"); return SGA_ERR_ARG; }
-  hipLaunchKernelGGL(k_mask_abs_ge, dim3(stream_grid(n, (int64_t)kBlock * kVec * 4, 256 * 8)),
+  hipLaunchKernelGGL(k_mask_abs_ge, dim3(stream_grid(n, (int64_t)kBlock * kVec * 4, 256 * 16)),
                      dim3(kBlock), 0, (hipStream_t)stream, score, n, tau, mask_out,
                      reinterpret_cast<unsigned long long*>(count),
                      aligned4(score, 4) && aligned4(mask_out, 1));
@@ -324,7 +397,7 @@ extern "C" int sga_cand_extract_count(const float* score, int64_t n, int32_t bin
   const int64_t nc = cdiv64(n, kChunk);
   hipStream_t st = (hipStream_t)stream;
   if (nc > 0)
-    hipLaunchKernelGGL(k_cand_count, dim3(stream_grid(nc, kChunksPerBlock)), dim3(kBlock), 0, st,
+    hipLaunchKernelGGL(k_cand_count, dim3(stream_grid(nc, kChunksPerBlock, 1 << 22)), dim3(kBlock), 0, st,
                        score, n, (uint32_t)bin, chunk_counts, nc, aligned4(score, 4));
   if (int rc = exclusive_scan_u32(chunk_counts, nc, total, st)) return rc;
   return check_launch("sga_cand_extract_count");
@@ -339,7 +412,7 @@ extern "C" int sga_cand_extract_fill(const float* score, int64_t n, int32_t bin,
     return SGA_ERR_ARG;
   }
   const int64_t nc = cdiv64(n, kChunk);
-  hipLaunchKernelGGL(k_cand_fill, dim3(stream_grid(nc, kChunksPerBlock)), dim3(kBlock), 0,
+  hipLaunchKernelGGL(k_cand_fill, dim3(stream_grid(nc, kChunksPerBlock, 1 << 22)), dim3(kBlock), 0,
                      (hipStream_t)stream, score, n, (uint32_t)bin, chunk_offsets, cand,
                      cand_capacity, nc, aligned4(score, 4));
   return check_launch("sga_cand_extract_fill");
@@ -354,7 +427,7 @@ extern "C" int sga_gt_eq(const float* score, int64_t n, float thresh, uint8_t* g
   hipStream_t st = (hipStream_t)stream;
   hipLaunchKernelGGL(k_zero_i32, dim3(1), dim3(64), 0, st, counts2, 2);
   if (n > 0)
-    hipLaunchKernelGGL(k_gt_eq, dim3(stream_grid(n, (int64_t)kBlock * kVec * 4, 256 * 8)),
+    hipLaunchKernelGGL(k_gt_eq, dim3(stream_grid(n, (int64_t)kBlock * kVec * 4, 256 * 16)),
                        dim3(kBlock), 0, st, score, n, thresh, gt, eq, counts2,
                        aligned4(score, 4) && aligned4(gt, 1) && aligned4(eq, 1));
   return check_launch("sga_gt_eq");

@@ -1161,7 +1161,7 @@ static inline void finish_mask(Src src, int64_t n, int tie_all, const SelWorkspa
                                uint8_t* mask, hipStream_t s) {
   const int64_t nc = cdiv64(n, kChunk);
   if (w.pbits && n >= kFastMinN && n < (1ll << 32)) {
-    hipLaunchKernelGGL(k_expand_mask, dim3(stream_grid(nc, kChunksPerBlock, 1 << 14)), dim3(kBlock),
+    hipLaunchKernelGGL(k_expand_mask, dim3(stream_grid(nc, kChunksPerBlock, 1 << 22)), dim3(kBlock),
                        0, s, w.st, w.pbits, n, mask, (reinterpret_cast<uintptr_t>(mask) & 15) == 0);
     hipLaunchKernelGGL(k_cand_mask, dim3(256), dim3(kBlock), 0, s, w.st, w.cand_idx, w.cand_key,
                        w.tile_eq, nc, tie_all, mask);
