@@ -67,9 +67,10 @@ struct SegCursor {
   const sga_segment* segs;
   int n_segs;
   int64_t lo, hi;
+  int at;                               // index of the cached segment (uniform seeks only)
   Hyper h;
   __host__ __device__ __forceinline__ void init(const sga_segment* s, int ns) {
-    segs = s; n_segs = ns; lo = 1; hi = 0;
+    segs = s; n_segs = ns; lo = 1; hi = 0; at = 0;
   }
   __device__ __forceinline__ void seek(int64_t i) {
     if (i >= lo && i < hi) return;
@@ -82,7 +83,70 @@ struct SegCursor {
     hi = lo + segs[a].n;
     h = hyper_of(segs[a]);
   }
+  // The same for an index every lane of the wave holds alike: the cursor and
+  // the hyper-parameters it caches live on the scalar unit.
+  __device__ __forceinline__ void take_uniform(int a) {
+    const sga_segment& s = segs[a];
+    at = a;
+    lo = uniform_i64(s.start);
+    hi = lo + uniform_i64(s.n);
+    h.lr = uniform_f32(s.lr); h.b1 = uniform_f32(s.beta1); h.om1 = uniform_f32(s.om1);
+    h.b2 = uniform_f32(s.beta2); h.om2 = uniform_f32(s.om2); h.eps = uniform_f32(s.eps);
+    h.wd = uniform_f32(s.wd); h.bc1 = uniform_f32(s.bc1); h.bc2 = uniform_f32(s.bc2);
+  }
+  __device__ __forceinline__ void seek_uniform(int64_t i) {
+    if (i >= lo && i < hi) return;
+    int a = 0, b = n_segs - 1;
+    while (a < b) {
+      const int mid = (a + b + 1) >> 1;
+      if (uniform_i64(segs[mid].start) <= i) a = mid; else b = mid - 1;
+    }
+    take_uniform(a);
+  }
+  // Steps to the segment that holds i, a little past the cached one (the
+  // next tensor of a slab that straddles a boundary).
+  __device__ __forceinline__ void advance_uniform(int64_t i) {
+    int a = at;
+    while (a + 1 < n_segs && uniform_i64(segs[a + 1].start) <= i) ++a;
+    take_uniform(a);
+  }
 };
+
+// Keys of one slab of a chunk-structured sweep: lane l holds the quad at
+// i = s0 + 4 l of the 256-element slab [s0, s0 + 256).  Hyper-parameters
+// change only at tensor boundaries, so the slab is scored once per segment
+// that intersects it (one, but for the few slabs that hold a boundary) with
+// that segment's hyper-parameters as scalar operands.  `sc` was placed on the
+// slab's chunk with seek_uniform and is only ever moved by the uniform seeks.  key[] comes in zeroed; quads past n stay zero.
+template <int SCORE, bool FULL>
+__device__ __forceinline__ void slab_score_keys(SegCursor& sc, int adams, int64_t i, int64_t n,
+                                                const float q[4], const float p[4],
+                                                const float m[4], const float v[4],
+                                                uint32_t key[4]) {
+  const int64_t s0 = uniform_i64(i);
+  int64_t s1 = s0 + kWave * kVec;
+  if (!FULL && s1 > n) s1 = n;
+  if (s0 >= sc.hi) sc.advance_uniform(s0);   // slabs of a chunk ascend from its seek_uniform
+  for (;;) {
+    Hyper h = sc.h;
+    if (adams) { h.bc1 = 1.0f; h.bc2 = 1.0f; }
+    uint32_t k4[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) k4[e] = score_key<SCORE>(q[e], p[e], m[e], v[e], h);
+    if (sc.lo <= s0 && sc.hi >= s1) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) key[e] = k4[e];
+      break;
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+      if (i + e >= sc.lo && i + e < sc.hi) key[e] = k4[e];
+    const int64_t pos = sc.hi;
+    if (pos >= s1) break;
+    sc.advance_uniform(pos);
+    if (sc.hi <= pos) break;              // the table does not tile [0, n): stop
+  }
+}
 #endif
 
 static inline Hyper mk_hyper(float lr, float b1, float om1, float b2, float om2, float eps,

@@ -81,6 +81,18 @@ __device__ __forceinline__ int64_t pack_shift(int64_t i, int64_t pack_extra) {
 }
 __device__ __forceinline__ int wave_id() { return threadIdx.x >> 6; }
 
+// Values every lane of the wave holds alike, moved to the scalar unit: what is
+// derived from them (addresses, hyper-parameters, branches) stays scalar too.
+__device__ __forceinline__ int uniform_i32(int x) { return __builtin_amdgcn_readfirstlane(x); }
+__device__ __forceinline__ float uniform_f32(float x) {
+  return __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(x)));
+}
+__device__ __forceinline__ int64_t uniform_i64(int64_t x) {
+  const uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)x);
+  const uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)((uint64_t)x >> 32));
+  return (int64_t)(((uint64_t)hi << 32) | lo);
+}
+
 // Number of set bits of `mask` strictly below the calling lane.
 __device__ __forceinline__ uint32_t lanes_below(uint64_t mask) {
   return __builtin_amdgcn_mbcnt_hi((uint32_t)(mask >> 32),
@@ -215,6 +227,41 @@ __device__ __forceinline__ void ld_bf16(const uint16_t* base, int64_t i, int64_t
     out[2] = bf16_to_f32(v.z); out[3] = bf16_to_f32(v.w);
   } else {
     load4_bf16(base, i, n, out, vec);
+  }
+}
+// Loads kept as the raw vectors that arrive from memory: nothing depends on
+// them until they are unpacked, so a sweep can issue the loads of several
+// slabs before it waits for the first.
+template <bool FULL>
+__device__ __forceinline__ F4 ldraw_f32(const float* base, int64_t i, int64_t n, bool vec) {
+  if (FULL) return ld4_nt(base + i);
+  float t[4];
+  load4_f32(base, i, n, t, vec);
+  return F4{t[0], t[1], t[2], t[3]};
+}
+__device__ __forceinline__ void unpack_f32(const F4& r, float out[4]) {
+  out[0] = r.x; out[1] = r.y; out[2] = r.z; out[3] = r.w;
+}
+struct RawG { H4 h; F4 f; };      // a gradient quad: bf16 bits (full vector path) or fp32
+template <bool BF16G, bool FULL>
+__device__ __forceinline__ void fetch_g(const void* g, int64_t i, int64_t n, bool vec, RawG& r) {
+  if (BF16G && FULL) {
+    r.h = ldh4_nt(reinterpret_cast<const uint16_t*>(g) + i);
+  } else if (BF16G) {
+    float t[4];
+    load4_bf16(reinterpret_cast<const uint16_t*>(g), i, n, t, vec);
+    r.f = F4{t[0], t[1], t[2], t[3]};
+  } else {
+    r.f = ldraw_f32<FULL>(reinterpret_cast<const float*>(g), i, n, vec);
+  }
+}
+template <bool BF16G, bool FULL>
+__device__ __forceinline__ void unpack_g(const RawG& r, float out[4]) {
+  if (BF16G && FULL) {
+    out[0] = bf16_to_f32(r.h.x); out[1] = bf16_to_f32(r.h.y);
+    out[2] = bf16_to_f32(r.h.z); out[3] = bf16_to_f32(r.h.w);
+  } else {
+    unpack_f32(r.f, out);
   }
 }
 template <bool FULL>

@@ -28,6 +28,54 @@ struct SrcFused {
   bool vec;
   SegCursor sc;        // per-thread cache of the current segment's hyper-parameters
   int64_t pack_extra;  // 0: separate arrays; else extra floats per kPackRun elements (packed state)
+  // Stepwise interface of the one-sweep select.
+  struct Raw { RawG g; F4 r, p, m, v; };
+  struct Chunk { int64_t sh; };
+  static constexpr bool kHyper = SCORE == SGA_SCORE_UPDATE || SCORE == SGA_SCORE_COI;
+  static constexpr int kAhead = kHyper ? 2 : kChunkIters;
+  __device__ __forceinline__ Chunk chunk_begin(int64_t c) {
+    const int64_t i0 = uniform_i64(c) * kChunk;
+    if (kHyper) sc.seek_uniform(i0);
+    return Chunk{(i0 >> kPackRunLog) * pack_extra};
+  }
+  template <bool FULL>
+  __device__ __forceinline__ void fetch(const Chunk& ck, int64_t i, int64_t n, Raw& w) {
+    fetch_g<BF16G, FULL>(g, i, n, vec, w.g);
+    w.r = ldraw_f32<FULL>(r + ck.sh, i, n, vec);
+    if (SCORE == SGA_SCORE_ABS_G) return;
+    w.m = ldraw_f32<FULL>(m + ck.sh, i, n, vec);
+    if (SCORE != SGA_SCORE_ABS_M) {
+      w.p = ldraw_f32<FULL>(p + ck.sh, i, n, vec);
+      w.v = ldraw_f32<FULL>(v + ck.sh, i, n, vec);
+    }
+  }
+  template <bool FULL>
+  __device__ __forceinline__ void keys(const Chunk& ck, int64_t i, int64_t n, const Raw& w,
+                                       uint32_t key[4]) {
+    float gg[4], rr[4];
+    unpack_g<BF16G, FULL>(w.g, gg);
+    unpack_f32(w.r, rr);
+    if (SCORE == SGA_SCORE_ABS_G) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) key[e] = abs_key(rr[e] + gg[e]);
+      return;
+    }
+    float pp[4] = {0, 0, 0, 0}, mm[4], vv[4] = {0, 0, 0, 0};
+    unpack_f32(w.m, mm);
+    if (SCORE == SGA_SCORE_ABS_M) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) key[e] = abs_key(mm[e]);
+      return;
+    }
+    if (SCORE != SGA_SCORE_ABS_M) {
+      unpack_f32(w.p, pp);
+      unpack_f32(w.v, vv);
+    }
+    float q[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) q[e] = rr[e] + gg[e];
+    slab_score_keys<SCORE, FULL>(sc, 0, i, n, q, pp, mm, vv, key);
+  }
   template <bool FULL = false>
   __device__ __forceinline__ void load(int64_t i, int64_t n, uint32_t key[4]) {
     const int64_t sh = pack_shift<FULL>(i, pack_extra);

@@ -353,6 +353,62 @@ struct SrcReplay {
   SegCursor sc;              // b1, b2, eps, wd, bc1, bc2 per tensor (cached per thread)
   int64_t pack_extra;        // 0 or kPackExtra (res/w/m/v of one packed state)
   int res_zero;              // res is known to be all zeros: not read
+  // Stepwise interface of the one-sweep select.
+  struct Raw { RawG g; F4 r, w, m, v; };
+  struct Chunk { int64_t sh; float coef; };
+  static constexpr bool kHyper = SCORE == SGA_SCORE_UPDATE || SCORE == SGA_SCORE_COI;
+  static constexpr int kAhead = kHyper ? 2 : kChunkIters;
+  __device__ __forceinline__ Chunk chunk_begin(int64_t c) {
+    const int64_t i0 = uniform_i64(c) * kChunk;
+    if (kHyper) sc.seek_uniform(i0);
+    return Chunk{(i0 >> kPackRunLog) * pack_extra, uniform_f32(coef_f[0])};
+  }
+  template <bool FULL>
+  __device__ __forceinline__ void fetch(const Chunk& ck, int64_t i, int64_t n, Raw& t) {
+    fetch_g<BF16G, FULL>(g, i, n, vec, t.g);
+    if (!res_zero) t.r = ldraw_f32<FULL>(res + ck.sh, i, n, vec);
+    if (SCORE == SGA_SCORE_ABS_G) return;
+    t.m = ldraw_f32<FULL>(m + ck.sh, i, n, vec);
+    if (SCORE != SGA_SCORE_ABS_M) {
+      t.w = ldraw_f32<FULL>(w + ck.sh, i, n, vec);
+      if (!adams) t.v = ldraw_f32<FULL>(v + ck.sh, i, n, vec);
+    }
+  }
+  template <bool FULL>
+  __device__ __forceinline__ void keys(const Chunk& ck, int64_t i, int64_t n, const Raw& t,
+                                       uint32_t key[4]) {
+    float gd[4], rr[4] = {0, 0, 0, 0};
+    unpack_g<BF16G, FULL>(t.g, gd);
+    if (coef_dense != 1.0f) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) gd[e] = __fdiv_rn(gd[e], coef_dense);
+    }
+    if (!res_zero) unpack_f32(t.r, rr);
+    float q[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) q[e] = (gd[e] + rr[e]) * ck.coef;
+    if (SCORE == SGA_SCORE_ABS_G) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) key[e] = abs_key(q[e]);
+      return;
+    }
+    float ww[4] = {0, 0, 0, 0}, mm[4], vv[4] = {0, 0, 0, 0};
+    unpack_f32(t.m, mm);
+    if (SCORE == SGA_SCORE_ABS_M) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) key[e] = abs_key(mm[e]);
+      return;
+    }
+    if (SCORE != SGA_SCORE_ABS_M) {
+      unpack_f32(t.w, ww);
+      if (!adams) unpack_f32(t.v, vv);
+    }
+    if (adams) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) vv[e] = mm[e] * mm[e];
+    }
+    slab_score_keys<SCORE, FULL>(sc, adams, i, n, q, ww, mm, vv, key);
+  }
   template <bool FULL = false>
   __device__ __forceinline__ void load(int64_t i, int64_t n, uint32_t key[4]) {
     const int64_t sh = pack_shift<FULL>(i, pack_extra);

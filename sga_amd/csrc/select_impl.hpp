@@ -163,9 +163,26 @@ static inline bool sel_ws_carve(void* ws, size_t bytes, int64_t n_tiles_needed,
 // ------------------------------------------------------------ key sources
 // A key source yields the 31-bit magnitude keys of 4 consecutive elements.
 // load<FULL>: FULL promises i + 4 <= n and vector alignment (see ld_f32).
+// The one-sweep select drives a source in three steps instead, so that the
+// loads of kAhead slabs of a chunk are in flight before the first key is
+// formed: chunk_begin (what is common to the chunk's 1024 elements, held on
+// the scalar unit), fetch (loads only), keys (arithmetic only).
+struct NoChunk {};
 struct SrcF32 {                 // |x| of an fp32 score array
   const float* x;
   bool vec;
+  using Raw = F4;
+  using Chunk = NoChunk;
+  static constexpr int kAhead = kChunkIters;
+  __device__ __forceinline__ Chunk chunk_begin(int64_t) { return Chunk{}; }
+  template <bool FULL>
+  __device__ __forceinline__ void fetch(const Chunk&, int64_t i, int64_t n, Raw& r) {
+    r = ldraw_f32<FULL>(x, i, n, vec);
+  }
+  template <bool FULL>
+  __device__ __forceinline__ void keys(const Chunk&, int64_t, int64_t, const Raw& r, uint32_t key[4]) {
+    key[0] = abs_key(r.x); key[1] = abs_key(r.y); key[2] = abs_key(r.z); key[3] = abs_key(r.w);
+  }
   template <bool FULL = false>
   __device__ __forceinline__ void load(int64_t i, int64_t n, uint32_t key[4]) {
     float v[4];
@@ -737,48 +754,64 @@ static __global__ void k_bracket_ranks(SelState* aux, uint32_t* hist, int nhist,
 // wave owns a private candidate segment, so no atomics are needed and the
 // candidates of a chunk stay in ascending index order.
 template <class Src, bool FULL, bool PM>
-__device__ __forceinline__ void bracket_chunk(Src& src, int64_t n, int64_t c, uint32_t T_LO,
+__device__ __forceinline__ void bracket_chunk(Src& src, const typename Src::Chunk& ck, int64_t n,
+                                              int64_t c, uint32_t T_LO,
                                               uint32_t T_HI, uint32_t& chi, uint32_t& tot_nf,
                                               uint32_t& mycnt, uint32_t seg_cap,
                                               uint32_t* __restrict__ my_idx,
                                               uint32_t* __restrict__ my_key,
                                               uint32_t* __restrict__ pbits) {
-  // one 256-element slab at a time: keeps the register footprint of
-  // expensive key sources (Adam-normalised scores) small enough for full
-  // occupancy; slabs of different waves overlap their loads
+  // The loads of kAhead slabs (256 elements each) are issued together, then
+  // their keys are formed slab by slab: expensive key sources (Adam-normalised
+  // scores) look fewer slabs ahead to stay within the register budget of four
+  // workgroups per CU.  The ragged path (last chunk, unaligned views) goes one
+  // slab at a time through a rolled loop: it only has to be small.
   uint32_t pword = 0u;
+  constexpr int kAhead = FULL ? Src::kAhead : 1;
+  static_assert(kChunkIters % kAhead == 0, "look-ahead divides the slabs of a chunk");
+  constexpr int kGroupUnroll = kAhead == kChunkIters ? kChunkIters : 1;
+#pragma unroll kGroupUnroll
+  for (int g0 = 0; g0 < kChunkIters; g0 += kAhead) {
+    typename Src::Raw raw[kAhead];
 #pragma unroll
-  for (int it = 0; it < kChunkIters; ++it) {
-    const int64_t i = c * kChunk + it * (kWave * kVec) + lane_id() * kVec;
-    uint32_t key[4] = {0u, 0u, 0u, 0u};
-    if (FULL || i < n) src.template load<FULL>(i, n, key);
-    bool cand[4];
-    uint32_t mine = 0, above[4];
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      const bool valid = FULL || i + e < n;
-      above[e] = (valid && key[e] >= T_HI);
-      chi += above[e];
-      tot_nf += (valid && key[e] >= 0x7F800000u);
-      cand[e] = valid && key[e] >= T_LO && key[e] < T_HI;
-      mine += cand[e];
+    for (int u = 0; u < kAhead; ++u) {
+      const int64_t i = c * kChunk + (g0 + u) * (kWave * kVec) + lane_id() * kVec;
+      if (FULL || i < n) src.template fetch<FULL>(ck, i, n, raw[u]);
     }
-    if (PM) {
-      // provisional mask as bit planes: everything above the bracket is
-      // certainly selected; the few keys inside it are settled after the
-      // candidate descent.  One 128-byte store per chunk.
-      plane_collect(above, it, pword);
-    }
-    if (ballot64(mine != 0)) {
-      const uint32_t incl = wave_incl_scan(mine);
-      uint32_t pos = mycnt + incl - mine;
 #pragma unroll
-      for (int e = 0; e < 4; ++e)
-        if (cand[e]) {
-          if (pos < seg_cap) { my_idx[pos] = (uint32_t)(i + e); my_key[pos] = key[e]; }
-          ++pos;
-        }
-      mycnt += __shfl(incl, kWave - 1, kWave);
+    for (int u = 0; u < kAhead; ++u) {
+      const int it = g0 + u;
+      const int64_t i = c * kChunk + it * (kWave * kVec) + lane_id() * kVec;
+      uint32_t key[4] = {0u, 0u, 0u, 0u};
+      if (FULL || i < n) src.template keys<FULL>(ck, i, n, raw[u], key);
+      bool cand[4];
+      uint32_t mine = 0, above[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const bool valid = FULL || i + e < n;
+        above[e] = (valid && key[e] >= T_HI);
+        chi += above[e];
+        tot_nf += (valid && key[e] >= 0x7F800000u);
+        cand[e] = valid && key[e] >= T_LO && key[e] < T_HI;
+        mine += cand[e];
+      }
+      if (PM) {
+        // provisional mask as bit planes: everything above the bracket is
+        // certainly selected; the few keys inside it are settled after the
+        // candidate descent.  One 128-byte store per chunk.
+        plane_collect(above, it, pword);
+      }
+      if (ballot64(mine != 0)) {
+        const uint32_t incl = wave_incl_scan(mine);
+        uint32_t pos = mycnt + incl - mine;
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          if (cand[e]) {
+            if (pos < seg_cap) { my_idx[pos] = (uint32_t)(i + e); my_key[pos] = key[e]; }
+            ++pos;
+          }
+        mycnt += __shfl(incl, kWave - 1, kWave);
+      }
     }
   }
   if (PM && lane_id() < 32) pbits[c * 32 + lane_id()] = pword;
@@ -804,10 +837,11 @@ __global__ __launch_bounds__(kBlock, 4) void k_bracket_sweep(
   uint32_t* my_key = seg_key + gw * seg_cap;
   for (int64_t c = gw; c < n_chunks; c += W) {
     uint32_t chi = 0;
+    const typename Src::Chunk ck = src.chunk_begin(c);
     if (src.vec && (c + 1) * kChunk <= n)
-      bracket_chunk<Src, true, PM>(src, n, c, T_LO, T_HI, chi, tot_nf, mycnt, seg_cap, my_idx, my_key, pbits);
+      bracket_chunk<Src, true, PM>(src, ck, n, c, T_LO, T_HI, chi, tot_nf, mycnt, seg_cap, my_idx, my_key, pbits);
     else
-      bracket_chunk<Src, false, PM>(src, n, c, T_LO, T_HI, chi, tot_nf, mycnt, seg_cap, my_idx, my_key, pbits);
+      bracket_chunk<Src, false, PM>(src, ck, n, c, T_LO, T_HI, chi, tot_nf, mycnt, seg_cap, my_idx, my_key, pbits);
     chi = wave_sum(chi);
     tot_hi += chi;
     if (lane_id() == 0) { tile_gt[c] = chi; tile_eq[c] = 0u; }
