@@ -32,7 +32,9 @@ struct SrcFused {
   struct Raw { RawG g; F4 r, p, m, v; };
   struct Chunk { int64_t sh; };
   static constexpr bool kHyper = SCORE == SGA_SCORE_UPDATE || SCORE == SGA_SCORE_COI;
-  static constexpr int kAhead = kHyper ? 2 : kChunkIters;
+  // measured: the |g + r| sweep is bound by DRAM and loses ~5 % with more slabs in flight; the
+  // Adam-normalised scores are bound by arithmetic and gain from hiding the load latency
+  static constexpr int kAhead = kHyper ? 2 : 1;
   __device__ __forceinline__ Chunk chunk_begin(int64_t c) {
     const int64_t i0 = uniform_i64(c) * kChunk;
     if (kHyper) sc.seek_uniform(i0);

@@ -6,6 +6,7 @@
 // per-chunk count so that ties at the threshold can be granted in ascending
 // index order without any float compare ambiguity.
 #pragma once
+#include <type_traits>
 #include "common.hpp"
 
 namespace sga {
@@ -268,11 +269,11 @@ __device__ __forceinline__ void level_scan_body(SelState* __restrict__ st,
   const uint32_t total = s_suf[0];
   if (LEVEL == 0 && t == 0) {
     st->total = total;
-    uint32_t nf = 0;
-    for (int b = 0xFF0; b < kBinsBig; ++b) nf += __atomic_load_n(&hist[b], __ATOMIC_RELAXED);
-    st->nonfinite = nf;                  // exponent 255: Inf / NaN
     if (krem < 1 || krem > total) st->status = 1;
   }
+  // exponent 255 (Inf / NaN) is bins 0xFF0..0xFFF: exactly the last thread's bins
+  static_assert(kBinsBig / kBlock == 16 && (kBlock - 1) * 16 == 0xFF0, "non-finite bins = last thread");
+  if (LEVEL == 0 && t == kBlock - 1) st->nonfinite = mine;
   const uint32_t above_me = s_suf[t + 1];
   if (krem >= 1 && above_me < krem && krem <= above_me + mine) {
     uint32_t above = above_me;
@@ -332,22 +333,37 @@ __global__ __launch_bounds__(kBlock) void k_level_hist(Src src, int64_t n,
   for (int q = 0; q < NS; ++q)
     for (int b = threadIdx.x; b < NB; b += kBlock) s_h[q][b] = 0u;
   __syncthreads();
-  const int64_t stride = (int64_t)gridDim.x * kBlock * kVec;
+  // Raw key buffers (sample, candidates) are short and sit in L2: what their passes cost is load
+  // latency, so each lane keeps kQuads 16-byte loads in flight per trip.  Key sources that compute
+  // (the radix passes over the data itself) go one quad at a time.
+  constexpr int kQuads = std::is_same<Src, SrcU32>::value ? 4 : 1;
+  constexpr int64_t kSlabKeys = (int64_t)kBlock * kVec;
+  const int64_t stride = (int64_t)gridDim.x * kSlabKeys * kQuads;
   // uniform trip count so the wave-level ballots inside lds_hist_add are safe
-  const int64_t first = ((int64_t)blockIdx.x * kBlock) * kVec;
+  const int64_t first = (int64_t)blockIdx.x * kSlabKeys * kQuads;
   for (int64_t base = first; base < n; base += stride) {
-    const int64_t i = base + (int64_t)threadIdx.x * kVec;
-    uint32_t key[4] = {0, 0, 0, 0};
-    const bool full = src.vec && base + kBlock * kVec <= n;   // whole workgroup span in range
-    if (full) src.template load<true>(i, n, key);
-    else if (i < n) src.template load<false>(i, n, key);
+    uint32_t key[kQuads][4];
+    bool full[kQuads];
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
+    for (int u = 0; u < kQuads; ++u) {
+      const int64_t bu = base + u * kSlabKeys;
+      const int64_t i = bu + (int64_t)threadIdx.x * kVec;
+      key[u][0] = key[u][1] = key[u][2] = key[u][3] = 0u;
+      full[u] = src.vec && bu + kSlabKeys <= n;   // whole workgroup span in range
+      if (full[u]) src.template load<true>(i, n, key[u]);
+      else if (i < n) src.template load<false>(i, n, key[u]);
+    }
 #pragma unroll
-      for (int q = 0; q < NS; ++q) {
-        uint32_t bin; bool part;
-        level_bin<LEVEL>(key[e], prefix[q], full || i + e < n, bin, part);
-        lds_hist_add(s_h[q], bin, part && on[q]);
+    for (int u = 0; u < kQuads; ++u) {
+      const int64_t i = base + u * kSlabKeys + (int64_t)threadIdx.x * kVec;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+#pragma unroll
+        for (int q = 0; q < NS; ++q) {
+          uint32_t bin; bool part;
+          level_bin<LEVEL>(key[u][e], prefix[q], full[u] || i + e < n, bin, part);
+          lds_hist_add(s_h[q], bin, part && on[q]);
+        }
       }
     }
   }
@@ -658,6 +674,11 @@ static __global__ void k_sel_result(const SelState* st, sga_select_result* out) 
 }
 
 // -------------------------------------------------------------- host drivers
+// Grid of the histogram passes over raw key buffers (<= 1M sample keys, ~1e6 candidates whose
+// count lives on the device).  What a workgroup costs there is fixed (zeroing and flushing its
+// LDS bins, the device-scope fence and ticket of the merged scan): measured, 256 or 1024
+// workgroups are 5 and 40 us slower per pass than 64.
+constexpr unsigned kRawKeyBlocks = 64;
 static inline dim3 hist_grid(int64_t n) {
   return dim3(stream_grid(n, (int64_t)kBlock * kVec * 4, 256 * 8));
 }
@@ -1140,9 +1161,7 @@ static inline void run_select(Src src, int64_t n, int64_t k, int tie_all, bool f
                        (uint32_t)k, (double)n, (double)ns);
     SrcU32 ssrc{w.sample};
     for (int level = 0; level < 3; ++level)
-      // <= 1M keys: 64 fat workgroups keep the histogram flush (one atomic per
-      // non-empty bin per workgroup) far below one atomic per key
-      launch_level<SrcU32, 2, true>(ssrc, ns, (const uint32_t*)nullptr, level, w.aux, w, s, 64);
+      launch_level<SrcU32, 2, true>(ssrc, ns, (const uint32_t*)nullptr, level, w.aux, w, s, kRawKeyBlocks);
     const int sweep_blocks = want_mask ? sweep_grid<Src, true>() : sweep_grid<Src, false>();
     if (want_mask)
       hipLaunchKernelGGL((k_bracket_sweep<Src, true>), dim3(sweep_blocks), dim3(kBlock), 0, s,
@@ -1159,9 +1178,7 @@ static inline void run_select(Src src, int64_t n, int64_t k, int tie_all, bool f
     SrcU32 csrc{w.cand_key};
     const int64_t cmax = (int64_t)kSegWaves * w.seg_cap;
     for (int level = 0; level < 3; ++level)
-      // the candidate count lives on the device (usually ~1e6): a small grid
-      // strides over it; a large grid would only add idle workgroups
-      launch_level<SrcU32, 1, true>(csrc, cmax, &w.st->cand_count, level, w.aux, w, s, 64);
+      launch_level<SrcU32, 1, true>(csrc, cmax, &w.st->cand_count, level, w.aux, w, s, kRawKeyBlocks);
     hipLaunchKernelGGL(k_cand_tiles, dim3(256), dim3(kBlock), 0, s, w.st, w.aux, w.cand_idx,
                        w.cand_key, w.tile_gt, w.tile_eq);
     // The radix passes below are no-ops unless the bracket failed
