@@ -11,18 +11,23 @@ from tests.util import rel_close, student_t, sub_scale
 pytestmark = pytest.mark.gpu
 
 
-def _segments(sizes, wd_every=2):
+def _segments(sizes, wd_every=2, vary=False):
     segs, off = [], 0
     for i, s in enumerate(sizes):
-        segs.append(dict(start=off, n=s, lr=1e-4, b1=0.9, b2=0.95, eps=1e-8,
-                         wd=0.1 if i % wd_every == 0 else 0.0))
+        seg = dict(start=off, n=s, lr=1e-4, b1=0.9, b2=0.95, eps=1e-8,
+                   wd=0.1 if i % wd_every == 0 else 0.0)
+        if vary:     # every hyper-parameter changes from tensor to tensor
+            seg.update(lr=1e-4 * (1 + i % 3), b1=(0.9, 0.8, 0.95)[i % 3], b2=(0.95, 0.99)[i % 2],
+                       eps=(1e-8, 1e-6, 1e-10)[(i + 1) % 3])
+        segs.append(seg)
         off += s
     return segs, off
 
 
-def _run(dev, sizes, steps, ratio, gdtype, vdtype, score="abs_g", seed0=0):
+def _run(dev, sizes, steps, ratio, gdtype, vdtype, score="abs_g", seed0=0, vary=False,
+         expect_path=None):
     from sga_amd.fused_step import FusedSparseStep
-    segs, n = _segments(sizes)
+    segs, n = _segments(sizes, vary=vary)
     gen = torch.Generator().manual_seed(1234)
     p = torch.randn(n, generator=gen) * 0.02
     m, v, r = torch.zeros(n), torch.zeros(n), torch.zeros(n)
@@ -52,6 +57,7 @@ def _run(dev, sizes, steps, ratio, gdtype, vdtype, score="abs_g", seed0=0):
         idx, vals = fs.step(g.to(dev), dr, dp, dm, dv, step, k=k, score=score)
         res = fs.read_result()
         assert res.status == 0 and res.nonfinite == 0 and res.n_selected == k
+        assert expect_path is None or res.path == expect_path
         assert res.thresh == th_ref, (step, res.thresh, th_ref)
         assert torch.equal(idx.cpu(), idx_ref), step
         assert torch.equal(fs.mask.cpu().bool(), mask_ref), step
@@ -91,6 +97,17 @@ def test_ragged_unaligned_segments(dev):
 @pytest.mark.parametrize("score", ["update", "coi", "abs_m"])
 def test_adam_normalised_scores(dev, score):
     _run(dev, [200_000, 1024, 100_000], 3, 1.0, torch.bfloat16, torch.bfloat16, score=score)
+
+
+@pytest.mark.parametrize("score", ["update", "coi"])
+def test_adam_scores_one_sweep_path_tensor_boundaries(dev, score):
+    """Above 2^20 elements the select is the one-sweep path, which scores a
+    256-element slab once per tensor that intersects it: tensors of 3..130
+    elements put several boundaries into one slab, none of them aligned, and
+    every hyper-parameter differs between neighbours."""
+    sizes = [300_000, 128, 37, 700_000, 3, 1024, 250_001, 130, 5, 60_000]
+    _run(dev, sizes, 2, 1.0, torch.bfloat16, torch.bfloat16, score=score, vary=True,
+         expect_path=1)
 
 
 def test_tie_heavy_gradients(dev):

@@ -86,7 +86,10 @@ def test_opt_step_inplace(dev, opt, lr, wd, count):
                            inactive=inactive.to(dev))
 
 
-def _fixture(n_sizes, W, seed=2026, bf16=False):
+_RAGGED = [600_000, 130, 37, 500_000, 3, 1024, 100_001, 5, 250]   # > 2^20: the one-sweep select
+
+
+def _fixture(n_sizes, W, seed=2026, bf16=False, vary=False):
     n = sum(n_sizes)
     gen = torch.Generator().manual_seed(seed)
     w0 = torch.randn(n, generator=gen) * 0.02
@@ -102,6 +105,9 @@ def _fixture(n_sizes, W, seed=2026, bf16=False):
     for i, s in enumerate(n_sizes):
         entries.append({"a": off, "n": s, "b1": 0.9, "b2": 0.95, "eps": 1e-8,
                         "wd": 0.1 if i % 2 == 0 else 0.0})
+        if vary:     # every hyper-parameter changes from tensor to tensor
+            entries[-1].update(b1=(0.9, 0.8, 0.95)[i % 3], b2=(0.95, 0.99)[i % 2],
+                               eps=(1e-8, 1e-6, 1e-10)[(i + 1) % 3])
         off += s
     return n, w0, m0, v0, grads, entries
 
@@ -153,6 +159,22 @@ def test_group_step_no_clip_bitwise(dev):
     assert float(grp.state[0]["res"].abs().max()) == 0.0       # T = 1: no residual survives
 
 
+def test_group_step_one_sweep_select(dev):
+    """More than 2^20 elements over ragged tensors: every boundary
+    re-selection of the group runs the one-sweep select and the commits go
+    through chunks that straddle tensors."""
+    specs = [("abs_g", 1.0, 1), ("abs_g", 10.0, 2), ("abs_m", 1.0, 2), ("abs_g", 0.1, 3, "adams")]
+    grp, out, w0 = _run_group(dev, specs, clip=0.0, W=5, bf16=True, sizes=_RAGGED)
+    assert grp.last_select().path == 1
+    for ci, o in enumerate(out):
+        s = grp.state[ci]
+        assert torch.equal(s["sel"].cpu().bool(), o["sel"]), ci
+        assert torch.equal(s["res"].cpu().view(torch.int32), o["res"].view(torch.int32)), ci
+        assert torch.equal(s["m"].cpu(), o["m"]) and torch.equal(s["v"].cpu(), o["v"]), ci
+        bad, worst = rel_close(s["w"], o["w"], 1e-6, atol=1e-6 * 5 * 5e-5 * 3)
+        assert bad == 0, (ci, worst)
+
+
 def test_group_step_with_clip(dev):
     specs = [("abs_g", 1.0, 1), ("abs_g", 10.0, 4), ("abs_g", 1.0, 4, "adams", True),
              ("abs_m", 0.1, 3, "adamw", False, 2.0)]
@@ -167,13 +189,17 @@ def test_group_step_with_clip(dev):
         assert bad == 0, (ci, worst)
 
 
+@pytest.mark.parametrize("sizes,vary,path", [([300_000, 1024, 200_000], False, 0),
+                                             (_RAGGED, True, 1)])
 @pytest.mark.parametrize("score", ["update", "coi"])
-def test_reselect_on_identical_score_bits(dev, score):
+def test_reselect_on_identical_score_bits(dev, score, sizes, vary, path):
     """Adam-normalised scores: the boundary re-selection is compared with the
-    oracle selector fed the device's own score bits."""
+    oracle selector fed the device's own score bits.  The ragged set runs the
+    one-sweep select, whose slabs hold several unaligned tensor boundaries with
+    different hyper-parameters on either side."""
     from sga_amd.replay_group import Config, ReplayGroup
     from sga_amd.scores import SCORE_MAP, device_formula
-    n, w0, m0, v0, grads, entries = _fixture([300_000, 1024, 200_000], 3)
+    n, w0, m0, v0, grads, entries = _fixture(sizes, 3, vary=vary)
     t0, lr = 5, 1e-4
     cfg = Config(score, 1.0, 1)
     k = SEL.replay_k(n, 1.0)
@@ -194,3 +220,4 @@ def test_reselect_on_identical_score_bits(dev, score):
     ref, th = SEL.select_topk_flat(sc, k)
     assert torch.equal(s["sel"].cpu().bool(), ref)
     assert grp.last_select().thresh == th
+    assert grp.last_select().path == path
