@@ -301,6 +301,17 @@ constexpr int kPlaneWordsPerChunk = 32;
 // UNIFORM promises that every lane of the wave addresses the same slab
 // (chunk- or workgroup-structured sweeps): the slab's eight words are then
 // fetched through one wave-uniform address.
+// For a wave whose lane l holds the quad at i = 256 * slab + 4 l (every
+// workgroup-structured sweep here): words 2e and 2e + 1 of the slab are the
+// 64-bit ballot of element e, so the flags are read back as lane masks with
+// no per-lane bit arithmetic at all.
+__device__ __forceinline__ void plane_wave_flags4(const uint32_t* __restrict__ planes, int64_t i,
+                                                  bool out[4]) {
+  const int64_t slab = uniform_i64(i >> 8);
+  const uint64_t* w = reinterpret_cast<const uint64_t*>(planes) + slab * 4;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) out[e] = __builtin_amdgcn_inverse_ballot_w64(w[e]);
+}
 template <bool UNIFORM = false>
 __device__ __forceinline__ void plane_flags4(const uint32_t* __restrict__ planes, int64_t i,
                                              uint32_t out[4]) {

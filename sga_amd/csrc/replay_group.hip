@@ -106,14 +106,14 @@ __global__ __launch_bounds__(kBlock) void k_replay_pass1(const void* __restrict_
       float gd2[4];
 #pragma unroll
       for (int e = 0; e < 4; ++e) gd2[e] = (full || i + e < n) ? gd[e] * gd[e] : 0.0f;
-      uint32_t sl[NC][4];
+      bool sl[NC][4];
 #pragma unroll
       for (int c = 0; c < NC; ++c) {
         const uint32_t* sp = reinterpret_cast<const uint32_t*>(lst.ptr[c]);
         if (!sp) {                       // no mask: every coordinate counts (q = gd)
-          sl[c][0] = sl[c][1] = sl[c][2] = sl[c][3] = 1u;
+          sl[c][0] = sl[c][1] = sl[c][2] = sl[c][3] = true;
         } else {
-          plane_flags4<true>(sp, i, sl[c]);    // bits past n are zero
+          plane_wave_flags4(sp, i, sl[c]);     // bits past n are zero
         }
       }
 #pragma unroll
@@ -207,14 +207,14 @@ __device__ __forceinline__ void pass3_vec(const void* g, int64_t i, int64_t n, f
     float* const VV = cf.v + sh;
     float* const WW = cf.w + sh;
     float rr[4], mm[4], vv[4] = {0, 0, 0, 0}, ww[4];
-    uint32_t sl[4] = {1, 1, 1, 1}, so[4] = {1, 1, 1, 1};
+    bool sl[4] = {true, true, true, true}, so[4] = {true, true, true, true};
     if (cf.res_zero) rr[0] = rr[1] = rr[2] = rr[3] = 0.0f;
     else ld_f32<FULL>(RES, i, n, rr, vec);
     ld_f32<FULL>(MM, i, n, mm, vec);
     if (!cf.adams) ld_f32<FULL>(VV, i, n, vv, vec);
     ld_f32<FULL>(WW, i, n, ww, vec);
-    if (!cf.boundary) plane_flags4<true>(cf.sel, i, sl);
-    if (cf.split) plane_flags4<true>(cf.out_sel, i, so);
+    if (!cf.boundary) plane_wave_flags4(cf.sel, i, sl);
+    if (cf.split) plane_wave_flags4(cf.out_sel, i, so);
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
       if (!FULL && i + e >= n) continue;
