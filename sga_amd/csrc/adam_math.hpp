@@ -132,7 +132,8 @@ struct SegCursor {
 // change only at tensor boundaries, so the slab is scored once per segment
 // that intersects it (one, but for the few slabs that hold a boundary) with
 // that segment's hyper-parameters as scalar operands.  `sc` was placed on the
-// slab's chunk with seek_uniform and is only ever moved by the uniform seeks.  key[] comes in zeroed; quads past n stay zero.
+// slab's chunk with seek_uniform and is only ever moved by the uniform seeks.
+// key[] comes in zeroed; quads past n stay zero.
 template <int SCORE, bool FULL>
 __device__ __forceinline__ void slab_score_keys(SegCursor& sc, int adams, int64_t i, int64_t n,
                                                 const float q[4], const float p[4],

@@ -298,9 +298,6 @@ __device__ __forceinline__ void st_u8(uint8_t* base, int64_t i, int64_t n, const
 // i = c*1024 + it*256 + lane*4 + e is bit (lane & 31) of word
 // planes[(i >> 8) * 8 + 2*e + (lane >> 5)].  i must be a multiple of 4.
 constexpr int kPlaneWordsPerChunk = 32;
-// UNIFORM promises that every lane of the wave addresses the same slab
-// (chunk- or workgroup-structured sweeps): the slab's eight words are then
-// fetched through one wave-uniform address.
 // For a wave whose lane l holds the quad at i = 256 * slab + 4 l (every
 // workgroup-structured sweep here): words 2e and 2e + 1 of the slab are the
 // 64-bit ballot of element e, so the flags are read back as lane masks with
@@ -311,21 +308,6 @@ __device__ __forceinline__ void plane_wave_flags4(const uint32_t* __restrict__ p
   const uint64_t* w = reinterpret_cast<const uint64_t*>(planes) + slab * 4;
 #pragma unroll
   for (int e = 0; e < 4; ++e) out[e] = __builtin_amdgcn_inverse_ballot_w64(w[e]);
-}
-template <bool UNIFORM = false>
-__device__ __forceinline__ void plane_flags4(const uint32_t* __restrict__ planes, int64_t i,
-                                             uint32_t out[4]) {
-  const int l = (int)(i >> 2) & (kWave - 1);
-  int64_t slab = i >> 8;
-  if (UNIFORM) slab = __builtin_amdgcn_readfirstlane((int)slab);
-  const U4* w = reinterpret_cast<const U4*>(planes + slab * 8);
-  const U4 a = w[0], b = w[1];
-  const bool hi = l >= 32;
-  const uint32_t s = l & 31;
-  out[0] = ((hi ? a.y : a.x) >> s) & 1u;
-  out[1] = ((hi ? a.w : a.z) >> s) & 1u;
-  out[2] = ((hi ? b.y : b.x) >> s) & 1u;
-  out[3] = ((hi ? b.w : b.z) >> s) & 1u;
 }
 
 // Four ballots of a slab -> the lane's word of the chunk's 32 (lane 8*it + 2e + h).

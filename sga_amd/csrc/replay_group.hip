@@ -25,7 +25,7 @@ struct RCfg {
   float* m;
   float* v;
   float* res;
-  const uint32_t* sel;      // current mask, bit planes (common.hpp: plane_flags4)
+  const uint32_t* sel;      // current mask, bit planes (common.hpp: plane_wave_flags4)
   const uint32_t* out_sel;  // outgoing mask for the dual-lr split (may equal sel)
   double lr_scale;          // dual-lr scale (lr_inactive = lr * lr_scale)
   int boundary;
