@@ -10,6 +10,7 @@ import math
 
 import torch
 
+from . import ieee
 from . import scores as S
 from . import select as SEL
 
@@ -54,7 +55,7 @@ def opt_step_inplace(q, m, v, w, lab, lr, wd, b1, b2, bc1c, bc2c, eps,
         m.mul_(b1).add_(q, alpha=1.0 - b1)
         v.mul_(b2).addcmul_(q, q, value=1.0 - b2)
     mh = m / bc1c
-    vh = torch.sqrt(v / bc2c)
+    vh = ieee.sqrt(v / bc2c)
     upd = mh / (vh + eps)
     if inactive is None:
         w.mul_(1.0 - lr * wd).add_(upd, alpha=-lr)

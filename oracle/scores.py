@@ -19,6 +19,8 @@ form in float64.
 """
 import torch
 
+from . import ieee
+
 SCORE_IDS = {"update": 0, "abs_g": 1, "abs_m": 2, "coi": 3}  # adamw.py:75-80
 
 
@@ -55,7 +57,7 @@ def update(w, m, v, g, b1, b2, eps, wd, bc1, bc2, update_includes_wd=True,
            optimizer="adamw"):
     """Signed materialized update ``wd*w + U(g)`` (scores.py:202-231)."""
     sa, sb = _moments(m, v, g, b1, b2, bc1, bc2, optimizer)
-    den = torch.sqrt(sb) + eps
+    den = ieee.sqrt(sb) + eps
     u = sa / den
     if update_includes_wd:
         return wd * w + u
@@ -72,8 +74,8 @@ def coi(w, m, v, g, b1, b2, eps, wd, bc1, bc2, update_includes_wd=True,
     else:
         num0 = (m * b1) / bc1
         den0 = (v * b2) / bc2
-    u0 = num0 / (torch.sqrt(den0) + eps)
-    ug = sa / (torch.sqrt(sb) + eps)
+    u0 = num0 / (ieee.sqrt(den0) + eps)
+    ug = sa / (ieee.sqrt(sb) + eps)
     return (ug - u0).abs()
 
 

@@ -35,7 +35,7 @@ __device__ __forceinline__ Commit adamw_commit(float p, float g, float m, float 
   c.v_new = sb;
   const float mh = __fdiv_rn(sa, h.bc1);
   const float vh = __fdiv_rn(sb, h.bc2);
-  const float den = __fsqrt_rn(vh) + h.eps;
+  const float den = sqrt_rn(vh) + h.eps;
   c.u = __fdiv_rn(mh, den);
   c.upd = h.wd * p + c.u;
   return c;
@@ -44,33 +44,20 @@ __device__ __forceinline__ Commit adamw_commit(float p, float g, float m, float 
 // U(0): the direction the same commit would take with a zero gradient.
 __device__ __forceinline__ float coi_u0(float m, float v, const Hyper& h) {
   const float num = __fdiv_rn(m * h.b1, h.bc1);
-  const float den = __fsqrt_rn(__fdiv_rn(v * h.b2, h.bc2)) + h.eps;
+  const float den = sqrt_rn(__fdiv_rn(v * h.b2, h.bc2)) + h.eps;
   return __fdiv_rn(num, den);
 }
 
-// Direction of a commit as the *scores* see it: the same chain with the three
-// divisions done by hardware reciprocals (about 1 ulp each, ~6 ulp on the
-// result), a third of the arithmetic of the separately rounded chain.  Every
-// kernel that ranks by an Adam-normalised score evaluates it here, so a
-// threshold found by one sweep means the same set in the next; the commit
-// itself (adamw_commit) keeps the exact chain.
-__device__ __forceinline__ float score_dir(float sa, float sb, const Hyper& h) {
-  const float mh = sa * __builtin_amdgcn_rcpf(h.bc1);
-  const float vh = sb * __builtin_amdgcn_rcpf(h.bc2);
-  const float den = __fsqrt_rn(vh) + h.eps;
-  return mh * __builtin_amdgcn_rcpf(den);
-}
-
 // Signed registry score.  SCORE: 0 update, 1 g, 2 m, 3 coi (already >= 0).
+// The Adam-normalised scores are the commit's own exact chain: every kernel
+// that ranks by them gets the same bits, the bits of the IEEE-754 evaluation.
 template <int SCORE>
 __device__ __forceinline__ float score_value(float q, float p, float m, float v, const Hyper& h) {
   if (SCORE == SGA_SCORE_ABS_G) return fabsf(q);
   if (SCORE == SGA_SCORE_ABS_M) return fabsf(m);
-  const float sa = m * h.b1 + q * h.om1;
-  const float sb = v * h.b2 + (q * h.om2) * q;
-  const float u = score_dir(sa, sb, h);
-  if (SCORE == SGA_SCORE_UPDATE) return h.wd * p + u;
-  return fabsf(u - score_dir(m * h.b1, v * h.b2, h));
+  const Commit c = adamw_commit(p, q, m, v, h);
+  if (SCORE == SGA_SCORE_UPDATE) return c.upd;
+  return fabsf(c.u - coi_u0(m, v, h));
 }
 template <int SCORE>
 __device__ __forceinline__ uint32_t score_key(float q, float p, float m, float v, const Hyper& h) {

@@ -81,6 +81,25 @@ __device__ __forceinline__ int64_t pack_shift(int64_t i, int64_t pack_extra) {
 }
 __device__ __forceinline__ int wave_id() { return threadIdx.x >> 6; }
 
+// Correctly rounded fp32 square root.  The hardware root is within 1 ulp, so
+// the answer is it or one of its neighbours: the exact residuals x - t*s of
+// the two neighbours t (one FMA each) say which.  Inputs below 2^-96 are
+// scaled by 2^32 first so the residuals stay normal.  (__fsqrt_rn compiles to
+// the bare hardware instruction on this toolchain.)
+__device__ __forceinline__ float sqrt_rn(float x) {
+  const bool small = x < 0x1p-96f;
+  const float xs = small ? x * 0x1p+32f : x;
+  float s = __builtin_amdgcn_sqrtf(xs);
+  const float sd = __uint_as_float(__float_as_uint(s) - 1u);
+  const float su = __uint_as_float(__float_as_uint(s) + 1u);
+  const float vd = __fmaf_rn(-sd, s, xs);
+  const float vu = __fmaf_rn(-su, s, xs);
+  s = vd <= 0.0f ? sd : s;
+  s = vu > 0.0f ? su : s;
+  s = small ? s * 0x1p-16f : s;
+  return (xs == 0.0f || xs == __builtin_huge_valf()) ? xs : s;
+}
+
 // Values every lane of the wave holds alike, moved to the scalar unit: what is
 // derived from them (addresses, hyper-parameters, branches) stays scalar too.
 __device__ __forceinline__ int uniform_i32(int x) { return __builtin_amdgcn_readfirstlane(x); }

@@ -111,25 +111,6 @@ struct SrcFused {
   }
 };
 
-// Commit used by the final sweep when the score does not depend on the
-// update itself (|g+r|, |m|): m' and v' are the exact separately-rounded
-// chain; the update direction uses reciprocal / hardware sqrt (about 1 ulp
-// each), which moves p by far less than 1e-6 of lr*|update|.
-struct FastHyper {
-  float inv_bc1, inv_bc2;
-};
-__device__ __forceinline__ void commit_fast(float& p, float g, float& m, float& v, const Hyper& h,
-                                            const FastHyper& f) {
-  const float sa = m * h.b1 + g * h.om1;
-  const float sb = v * h.b2 + (g * h.om2) * g;
-  const float den = __builtin_amdgcn_sqrtf(sb * f.inv_bc2) + h.eps;
-  const float u = (sa * f.inv_bc1) * __builtin_amdgcn_rcpf(den);
-  const float upd = h.wd * p + u;
-  p = p - h.lr * upd;
-  m = sa;
-  v = sb;
-}
-
 // Everything the final sweep needs besides the chunk index.
 struct FinalArgs {
   const void* g;
@@ -154,9 +135,7 @@ struct FinalArgs {
 // `cur` carries the running selected / tie counts across calls.
 template <bool BF16G, bool BF16V, int SCORE, bool FULL, int IT0, int NIT>
 __device__ __forceinline__ void final_chunk(const FinalArgs& a, int64_t c, ChunkCursor& cur,
-                                            SegCursor& sc, FastHyper& fh,
-                                            int64_t& fh_lo, int64_t& fh_hi) {
-  constexpr bool kFast = (SCORE == SGA_SCORE_ABS_G || SCORE == SGA_SCORE_ABS_M);
+                                            SegCursor& sc) {
   const int64_t n = a.n;
   const int64_t sh = pack_shift<true>(c << 10, a.pack_extra);     // c is wave-uniform
   float* const R = a.r + sh;
@@ -257,19 +236,10 @@ __device__ __forceinline__ void final_chunk(const FinalArgs& a, int64_t c, Chunk
           ++pos;
           if (a.apply_coeff) ge = ge * a.coeff;
         }
-        if (kFast) {
-          if (sc.lo != fh_lo || sc.hi != fh_hi) {
-            fh.inv_bc1 = __fdiv_rn(1.0f, sc.h.bc1);
-            fh.inv_bc2 = __fdiv_rn(1.0f, sc.h.bc2);
-            fh_lo = sc.lo; fh_hi = sc.hi;
-          }
-          commit_fast(pp[it][e], ge, mm[it][e], vv[it][e], sc.h, fh);
-        } else {
-          const Commit cm = adamw_commit(pp[it][e], ge, mm[it][e], vv[it][e], sc.h);
-          pp[it][e] = pp[it][e] - sc.h.lr * cm.upd;
-          mm[it][e] = cm.m_new;
-          vv[it][e] = cm.v_new;
-        }
+        const Commit cm = adamw_commit(pp[it][e], ge, mm[it][e], vv[it][e], sc.h);
+        pp[it][e] = pp[it][e] - sc.h.lr * cm.upd;
+        mm[it][e] = cm.m_new;
+        vv[it][e] = cm.v_new;
         rr[it][e] = sel[e] ? 0.0f : q[e];
       }
       st_f32<FULL>(R, i, n, rr[it], a.vec);
@@ -293,8 +263,6 @@ __global__ __launch_bounds__(kBlock) void k_fused_final(
   const int64_t wstride = (int64_t)gridDim.x * kChunksPerBlock;
   SegCursor sc;
   sc.init(segs, n_segs);
-  FastHyper fh{1.0f, 1.0f};
-  int64_t fh_lo = 1, fh_hi = 0;
   const bool can_full = a.vec && (a.mask_out == nullptr || a.mvec);
   for (int64_t c = (int64_t)blockIdx.x * kChunksPerBlock + wave_id(); c < n_chunks;
        c += wstride) {
@@ -304,12 +272,17 @@ __global__ __launch_bounds__(kBlock) void k_fused_final(
     if (can_full && (c + 1) * kChunk <= a.n) {
       // one 256-element slab at a time (5 loads in flight per lane): measured
       // as fast as batching all four slabs, at twice the occupancy
-      final_chunk<BF16G, BF16V, SCORE, true, 0, 1>(a, c, cur, sc, fh, fh_lo, fh_hi);
-      final_chunk<BF16G, BF16V, SCORE, true, 1, 1>(a, c, cur, sc, fh, fh_lo, fh_hi);
-      final_chunk<BF16G, BF16V, SCORE, true, 2, 1>(a, c, cur, sc, fh, fh_lo, fh_hi);
-      final_chunk<BF16G, BF16V, SCORE, true, 3, 1>(a, c, cur, sc, fh, fh_lo, fh_hi);
+      final_chunk<BF16G, BF16V, SCORE, true, 0, 1>(a, c, cur, sc);
+      final_chunk<BF16G, BF16V, SCORE, true, 1, 1>(a, c, cur, sc);
+      final_chunk<BF16G, BF16V, SCORE, true, 2, 1>(a, c, cur, sc);
+      final_chunk<BF16G, BF16V, SCORE, true, 3, 1>(a, c, cur, sc);
     } else {
-      final_chunk<BF16G, BF16V, SCORE, false, 0, kChunkIters>(a, c, cur, sc, fh, fh_lo, fh_hi);
+      // the ragged path too: holding four slabs at once would set the register count (and so
+      // the occupancy) of the whole kernel
+      final_chunk<BF16G, BF16V, SCORE, false, 0, 1>(a, c, cur, sc);
+      final_chunk<BF16G, BF16V, SCORE, false, 1, 1>(a, c, cur, sc);
+      final_chunk<BF16G, BF16V, SCORE, false, 2, 1>(a, c, cur, sc);
+      final_chunk<BF16G, BF16V, SCORE, false, 3, 1>(a, c, cur, sc);
     }
   }
 }

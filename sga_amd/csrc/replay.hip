@@ -121,7 +121,7 @@ __device__ __forceinline__ void opt_step_vec(const float* __restrict__ q, float*
     const float vn = __fmaf_rn(qq[e] * c.om2, qq[e], vb);
     const float mn = __fmaf_rn(qq[e], c.om1, mm[e] * c.b1);
     const float mh = __fdiv_rn(mn, c.bc1);
-    const float vh = __fsqrt_rn(__fdiv_rn(vn, c.bc2));
+    const float vh = sqrt_rn(__fdiv_rn(vn, c.bc2));
     const float upd = __fdiv_rn(mh, vh + c.eps);
     if (SPLIT) {
       const float step = ina[e] ? c.lri : c.lr;

@@ -233,7 +233,7 @@ __device__ __forceinline__ void pass3_vec(const void* g, int64_t i, int64_t n, f
       const float vn = __fmaf_rn(q * sc.s.om2, q, vb);
       const float mn = __fmaf_rn(q, sc.s.om1, mm[e] * sc.s.b1);
       const float mh = __fdiv_rn(mn, bc1);
-      const float vh = __fsqrt_rn(__fdiv_rn(vn, bc2));
+      const float vh = sqrt_rn(__fdiv_rn(vn, bc2));
       const float upd = __fdiv_rn(mh, vh + sc.s.eps);
       if (cf.split) {
         const float lri = (float)(sc.s.lr * cf.lr_scale);
@@ -297,7 +297,7 @@ __device__ __forceinline__ double dense_vec(const void* g, int64_t i, int64_t n,
     const float vn = __fmaf_rn(q[e] * sc.s.om2, q[e], vb);
     const float mn = __fmaf_rn(q[e], sc.s.om1, mm[e] * sc.s.b1);
     const float mh = __fdiv_rn(mn, bc1);
-    const float vh = __fsqrt_rn(__fdiv_rn(vn, bc2));
+    const float vh = sqrt_rn(__fdiv_rn(vn, bc2));
     const float upd = __fdiv_rn(mh, vh + sc.s.eps);
     ww[e] = __fmaf_rn(upd, sc.neglr, ww[e] * sc.omlwd);
     ll[e] = __fmaf_rn(upd * (float)(sc.s.lr * sc.s.lr), upd, ll[e]);

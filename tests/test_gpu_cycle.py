@@ -10,7 +10,7 @@ import torch
 from oracle import adamw as OA
 from oracle import kernels as OK
 from oracle import select as SEL
-from tests.util import rel_close, student_t
+from tests.util import same_bits, student_t
 
 pytestmark = pytest.mark.gpu
 HP = dict(lr=1e-3, beta1=0.9, beta2=0.95, eps=1e-8)
@@ -121,5 +121,4 @@ def test_full_then_sparse_cycle(dev, compact):
         assert torch.equal(dm, om) and torch.equal(dv, ov), it
         assert torch.equal(bucket.grad_data.cpu(), og), it
     dw = torch.cat([r.main_param.data for r in recs]).cpu()
-    bad, worst = rel_close(dw, ow, 1e-6, atol=1e-6 * 8 * 1e-3 * 3)
-    assert bad == 0, worst
+    assert same_bits(dw, ow)

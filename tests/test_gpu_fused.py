@@ -1,12 +1,14 @@
 """GPU parity of the fused per-rank sparse step vs the CPU oracle driver on
-the same seeded inputs: idx / mask / values / residual bit-exact, m and v
-bit-exact, p within 1e-6 relative."""
+the same seeded inputs, every output bit for bit: threshold, idx, mask,
+values, residual, m, v and p -- for the Adam-normalised scores too (the oracle
+selects on its own scores; the device evaluates the same correctly rounded
+chain)."""
 import pytest
 import torch
 
 from oracle import fused_step as OF
 from oracle import select as SEL
-from tests.util import rel_close, student_t, sub_scale
+from tests.util import same_bits, student_t
 
 pytestmark = pytest.mark.gpu
 
@@ -34,26 +36,10 @@ def _run(dev, sizes, steps, ratio, gdtype, vdtype, score="abs_g", seed0=0, vary=
     dp, dm, dv, dr = (t.to(dev) for t in (p, m, v, r))
     fs = FusedSparseStep(n, segs, dev, values_dtype=vdtype, want_mask=True)
     k = SEL.k_for(n, ratio)
-    travelled = p.abs()          # |p0| + sum of |applied steps| so far
     for step in range(1, steps + 1):
         g = student_t(n, seed0 + step - 1).to(gdtype)
-        given = None
-        if score != "abs_g":
-            # index parity for sqrt/div scores is asserted on identical score
-            # bits: feed the device's own score to the CPU selector
-            from sga_amd.scores import SCORE_MAP, device_formula
-            buf = dr + g.to(dev).float()
-            given = torch.empty(n)
-            for s in segs:
-                a, b = s["start"], s["start"] + s["n"]
-                given[a:b] = device_formula(
-                    SCORE_MAP[score], dp[a:b], dm[a:b], dv[a:b], buf[a:b], s["b1"], s["b2"],
-                    s["eps"], s["wd"], 1 - s["b1"] ** step, 1 - s["b2"] ** step,
-                    absolute=True).cpu()
-        p_old = p.clone()
         idx_ref, val_ref, mask_ref, th_ref = OF.fused_sparse_step(
-            g, r, p, m, v, segs, step, k=k, score=score, values_dtype=vdtype,
-            given_score=given)
+            g, r, p, m, v, segs, step, k=k, score=score, values_dtype=vdtype)
         idx, vals = fs.step(g.to(dev), dr, dp, dm, dv, step, k=k, score=score)
         res = fs.read_result()
         assert res.status == 0 and res.nonfinite == 0 and res.n_selected == k
@@ -63,14 +49,9 @@ def _run(dev, sizes, steps, ratio, gdtype, vdtype, score="abs_g", seed0=0, vary=
         assert torch.equal(fs.mask.cpu().bool(), mask_ref), step
         it = torch.int16 if vdtype == torch.bfloat16 else torch.int32
         assert torch.equal(vals.cpu().view(it), val_ref.view(it)), step
-        assert torch.equal(dr.cpu().view(torch.int32), r.view(torch.int32)), step
-        assert torch.equal(dm.cpu(), m) and torch.equal(dv.cpu(), v), step
-        # 1e-6 relative; where p' = p - lr*update cancels, relative to the
-        # operands of the subtractions applied so far (the device state is
-        # never re-synchronised from the oracle between steps)
-        travelled += (p - p_old).abs()
-        bad, worst = rel_close(dp, p, 1e-6, scale=travelled)
-        assert bad == 0, (step, worst)
+        # the device state is never re-synchronised from the oracle between steps
+        assert same_bits(dr, r) and same_bits(dm, m) and same_bits(dv, v), step
+        assert same_bits(dp, p), step
     return n, k
 
 

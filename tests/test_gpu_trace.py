@@ -8,7 +8,7 @@ import torch
 from oracle import replay as OR
 from oracle import select as SEL
 from oracle import trace as OT
-from tests.util import rel_close
+from tests.util import rel_close, same_bits
 from trace_fixture import make_trace
 
 pytestmark = pytest.mark.gpu
@@ -43,17 +43,8 @@ def test_branch_scores_fp64(dev, tmp_path, score, opt):
     assert torch.equal(dg.cpu(), g0)
     got = branch_scores(score, opt, sp, dw, dm, dv, dg, meta["step"] + 1).cpu()
     ref = OT.branch_scores(score, opt, entries, w0, m0, v0, g0, meta["step"] + 1)
-    if score in ("abs_g", "abs_m"):
-        assert torch.equal(got, ref)
-        return
-    # one fp64 op chain on each side; the host sqrt is 1 ulp low on some
-    # lanes, which can move the final fp32 rounding on a vanishing fraction
-    ulp = (got.view(torch.int32) - ref.view(torch.int32)).abs()
-    if score == "coi":                          # difference of two directions: operand scale
-        bad, worst = rel_close(got, ref, 1e-6, atol=1e-6 * 3)
-        assert bad == 0, worst
-    else:
-        assert int(ulp.max()) <= 1 and float((ulp > 0).float().mean()) < 1e-3
+    # one fp64 chain of correctly rounded operations on each side, rounded to fp32 once
+    assert same_bits(got, ref)
 
 
 @pytest.mark.parametrize("g_dtype,opt", [(None, "adamw"), (torch.bfloat16, "adamw"),
@@ -84,18 +75,14 @@ def test_dense_pass_matches_oracle(dev, tmp_path, g_dtype, opt):
                                 *OR.bc_pair(opt, t0 + si + 1, e["b1"], e["b2"]), e["eps"],
                                 optimizer=opt)
     assert torch.equal(dense.m.cpu(), om) and torch.equal(dense.v.cpu(), ov)
-    atol = 1e-6 * W * 5e-5 * 3
-    bad, worst = rel_close(dense.w, ow, 1e-6, atol=atol)
-    assert bad == 0, worst
+    assert same_bits(dense.w, ow)
     assert torch.equal(olab, lab)
-    bad, worst = rel_close(dense.label, lab, 1e-5, atol=1e-5 * float(lab.max()))
-    assert bad == 0, worst
+    assert same_bits(dense.label, lab)
     assert abs(total - lab_total) <= 1e-5 * lab_total
     assert set(dden) == {2, 6}
     for h in (2, 6):
         assert abs(dden[h] - den[h]) <= 1e-5 * den[h]
-        bad, worst = rel_close(dsnaps[h], snaps[h], 1e-6, atol=atol)
-        assert bad == 0, worst
+        assert same_bits(dsnaps[h], snaps[h])
     for a, b, mt in zip(drecon, recon, metas):
         assert a["coef_dense"] == b["coef_dense"]
         assert abs(a["recon_grad_norm"] - b["recon_grad_norm"]) <= 1e-9 * b["recon_grad_norm"]
@@ -141,9 +128,11 @@ def test_replay_window_end_to_end(dev, tmp_path, clip, g_dtype):
             assert torch.equal(s["sel"].cpu().bool(), o["sel"]), ci
             assert torch.equal(s["m"].cpu(), o["m"]) and torch.equal(s["v"].cpu(), o["v"]), ci
             assert torch.equal(s["res"].cpu(), o["res"]), ci
-            bad, worst = rel_close(s["w"], o["w"], 1e-6, atol=atol)
+            assert same_bits(s["w"], o["w"]), ci
         else:
+            # the clip coefficient comes from a double sum whose order differs between the two
+            # sides (1e-6 band): a last-bit change of the coefficient moves a few selections
             agree = float((s["sel"].cpu().bool() == o["sel"]).float().mean())
             assert agree > 0.9999, (ci, agree)
             bad, worst = rel_close(s["w"], o["w"], 1e-5, atol=10 * atol)
-        assert bad == 0, (ci, worst)
+            assert bad == 0, (ci, worst)

@@ -468,3 +468,29 @@ def test_clip_routes_against_closed_form():
     assert abs(n - mix) < 1e-5 * mix and c < 1.0
     assert torch.equal(flat[:1000], before[:1000])
     assert torch.allclose(flat[1000:], before[1000:] * c, rtol=1e-6)
+
+
+def test_ieee_sqrt_is_correctly_rounded():
+    """oracle.ieee.sqrt against the definition of round-to-nearest: the exact
+    value lies between the midpoints to the neighbouring floats.  s and ulp/2
+    have at most 25 significant bits, so the midpoints and their squares are
+    exact in float64 and the check involves no rounding at all."""
+    from oracle import ieee
+    gen = torch.Generator().manual_seed(5)
+    x = torch.cat([torch.rand(200_000, generator=gen) * 1e-6 + 1e-14,
+                   torch.rand(100_000, generator=gen) * 4.0,
+                   torch.rand(50_000, generator=gen) * 1e30,
+                   torch.tensor([1.0, 2.0, 4.0, 0.25, 1e-30, 3.0])])
+    x = x[x >= 2.0 ** -100]              # normal results, far from the subnormal range
+    s = ieee.sqrt(x)
+    assert s.dtype == torch.float32
+    nxt = (s.view(torch.int32) + 1).view(torch.float32)
+    half_ulp = (nxt.double() - s.double()) / 2
+    # going down across a power of two the spacing halves
+    prv = (s.view(torch.int32) - 1).view(torch.float32)
+    half_ulp_dn = (s.double() - prv.double()) / 2
+    lo, hi = s.double() - half_ulp_dn, s.double() + half_ulp
+    assert bool(((lo * lo <= x.double()) & (x.double() <= hi * hi)).all())
+    assert ieee.sqrt(torch.tensor([0.0, float("inf")])).tolist() == [0.0, float("inf")]
+    # and the reason it exists: the tensor library's own routine is not that
+    # (informational, never asserted): torch.sqrt may differ from it.

@@ -27,6 +27,16 @@ def student_t(n, seed, nu=3, scale=1e-3):
     return z / torch.sqrt(chi / nu) * scale
 
 
+def same_bits(a, b):
+    """Bitwise equality of two float tensors (signed zeros and NaN payloads
+    included): the device ran the same IEEE-754 chain as the oracle."""
+    a, b = a.detach().cpu().contiguous(), b.detach().cpu().contiguous()
+    if a.dtype != b.dtype or a.shape != b.shape:
+        return False
+    it = {torch.float32: torch.int32, torch.float64: torch.int64, torch.bfloat16: torch.int16}[a.dtype]
+    return bool(torch.equal(a.view(it), b.view(it)))
+
+
 def rel_close(a, b, rtol=1e-6, atol=0.0, scale=None):
     """|a-b| <= rtol*max(|a|,|b|,scale) + atol, elementwise.  ``scale`` carries
     the magnitude of the operands of a final subtraction (p' = p - lr*update):
