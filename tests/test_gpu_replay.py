@@ -1,7 +1,8 @@
 """GPU parity of the replay kernels: score formulas, in-place AdamW/AdamS
 commit (dual-lr, label accumulation) and the fused group step vs the CPU
-oracle.  Masks and thresholds bit-exact; m/v bit-exact (same FMA recipe);
-w within 1e-6 relative of the commit's operands; clip norms within the
+oracle.  Masks, thresholds, scores, m, v, w and the labels are bit-exact (the
+same chain of correctly rounded operations, FMAs where the reference's in-place
+ops have one); clip norms are double sums whose order differs: the
 reference's 1e-6 reordering band."""
 import pytest
 import torch
