@@ -173,3 +173,52 @@ def test_packed_state_is_bitwise_the_separate_layout(dev, score, gdtype):
                 assert torch.equal(a.view(torch.int32), b.view(torch.int32)), (sizes, step)
     with pytest.raises(ValueError):
         fb.step_packed(g, PackedState(n + 1, dev), 1, ratio_percent=1.0)
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_randomized_configurations(dev, seed):
+    """Seeded random draws of everything at once: tensor sizes (1 .. 700k
+    elements, shuffled), per-tensor hyper-parameters (beta1 = 0 and eps = 1e-15
+    included), score, gradient / value dtypes, ratio, and the magnitude of the
+    gradients, moments and residual (1e-12 .. 10, some all zero) -- three steps
+    each, every output bit for bit."""
+    import random
+    from sga_amd.fused_step import FusedSparseStep
+    rng = random.Random(seed)
+    total = rng.choice([70_001, 300_000, 1_100_000, 1_300_003])
+    sizes, left = [], total
+    while left > 0:
+        sz = min(left, rng.choice([1, 3, 37, 128, 130, 1000, 1024, 4099, 50_000, 300_001, 700_000]))
+        sizes.append(sz)
+        left -= sz
+    rng.shuffle(sizes)
+    score = ["abs_g", "update", "coi", "abs_m"][seed % 4]
+    gdtype = rng.choice([torch.bfloat16, torch.float32])
+    vdtype = rng.choice([torch.bfloat16, torch.float32])
+    gscale = 10.0 ** rng.uniform(-12, 1)
+    segs, off = [], 0
+    for sz in sizes:
+        segs.append(dict(start=off, n=sz, lr=10 ** rng.uniform(-5, -2),
+                         b1=rng.choice([0.9, 0.8, 0.95, 0.0]), b2=rng.choice([0.95, 0.99, 0.999]),
+                         eps=rng.choice([1e-8, 1e-6, 1e-10, 1e-15]), wd=rng.choice([0.0, 0.1, 0.01])))
+        off += sz
+    n = off
+    gen = torch.Generator().manual_seed(1000 + seed)
+    p = torch.randn(n, generator=gen) * 0.02
+    m = torch.randn(n, generator=gen) * gscale * rng.choice([0.0, 1.0, 1e-3])
+    v = torch.rand(n, generator=gen) * gscale * gscale * rng.choice([0.0, 1.0, 1e-6])
+    r = torch.randn(n, generator=gen) * gscale * rng.choice([0.0, 1.0])
+    dp, dm, dv, dr = (t.to(dev) for t in (p, m, v, r))
+    fs = FusedSparseStep(n, segs, dev, values_dtype=vdtype, want_mask=True)
+    k = SEL.k_for(n, rng.choice([0.1, 1.0, 10.0]))
+    for step in range(1, 4):
+        g = (student_t(n, seed * 10 + step) * (gscale / 1e-3)).to(gdtype)
+        idx_ref, val_ref, mask_ref, th_ref = OF.fused_sparse_step(
+            g, r, p, m, v, segs, step, k=k, score=score, values_dtype=vdtype)
+        idx, vals = fs.step(g.to(dev), dr, dp, dm, dv, step, k=k, score=score)
+        res = fs.read_result()
+        assert res.status == 0 and res.thresh == th_ref, (step, res.thresh, th_ref)
+        assert torch.equal(idx.cpu(), idx_ref) and torch.equal(fs.mask.cpu().bool(), mask_ref), step
+        it = torch.int16 if vdtype == torch.bfloat16 else torch.int32
+        assert torch.equal(vals.cpu().view(it), val_ref.view(it)), step
+        assert same_bits(dr, r) and same_bits(dm, m) and same_bits(dv, v) and same_bits(dp, p), step

@@ -210,3 +210,32 @@ def test_reselect_adam_scores(dev, score, sizes, vary, path):
     assert torch.equal(s["sel"].cpu().bool(), ref)
     assert grp.last_select().thresh == th
     assert grp.last_select().path == path
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_randomized_groups(dev, seed):
+    """Seeded random groups: ragged tensor sizes around 2^20 elements, 1..5
+    configs drawn over score x ratio x cycle length x optimizer x fold x
+    dual-lr, window length, gradient dtype, with and without clipping (the
+    device's clip coefficient is handed to the oracle) -- end state bit for bit."""
+    import random
+    rng = random.Random(100 + seed)
+    total = rng.choice([200_000, 900_000, 1_200_000, 1_500_007])
+    sizes, left = [], total
+    while left > 0:
+        sz = min(left, rng.choice([3, 37, 128, 130, 1024, 4099, 100_000, 400_001]))
+        sizes.append(sz)
+        left -= sz
+    if len(sizes) < 2:
+        sizes = [sizes[0] - 1000, 1000]
+    rng.shuffle(sizes)
+    specs = [(rng.choice(["abs_g", "abs_m", "abs_g"]), rng.choice([0.1, 1.0, 10.0]),
+              rng.choice([1, 2, 3, 4]), rng.choice(["adamw", "adams"]), rng.choice([False, True]),
+              rng.choice([1.0, 0.25, 2.0])) for _ in range(rng.randint(1, 5))]
+    grp, out, w0 = _run_group(dev, specs, clip=rng.choice([0.0, 0.3]), W=rng.choice([4, 6, 9]),
+                              bf16=rng.choice([True, False]), sizes=tuple(sizes))
+    for ci, o in enumerate(out):
+        s = grp.state[ci]
+        assert torch.equal(s["sel"].cpu().bool(), o["sel"]), (ci, specs[ci])
+        assert same_bits(s["res"], o["res"]) and same_bits(s["m"], o["m"]), (ci, specs[ci])
+        assert same_bits(s["v"], o["v"]) and same_bits(s["w"], o["w"]), (ci, specs[ci])
