@@ -274,12 +274,12 @@ __global__ __launch_bounds__(kBlock) void k_replay_pass3(const void* __restrict_
 
 // ------------------------------------------------------- dense reference step
 // One commit of the recorded (post-clip) gradient on the dense trajectory,
-// with the per-coordinate label lab += (lr*upd)^2 and the pre-clip
-// reconstruction sum((q / coef_dense)^2) in double.
+// with the per-coordinate label lab += (lr*upd)^2 and sum(q^2) in double for
+// the pre-clip reconstruction (the launcher divides the sum by coef_dense^2).
 template <bool BF16G, bool FULL>
 __device__ __forceinline__ double dense_vec(const void* g, int64_t i, int64_t n, float* w,
                                             float* m, float* v, float* lab, int adams,
-                                            double coef_dense, RSegCursor& sc, bool vec) {
+                                            RSegCursor& sc, bool vec) {
   float q[4], mm[4], vv[4] = {0, 0, 0, 0}, ww[4], ll[4] = {0, 0, 0, 0};
   if (BF16G) ld_bf16<FULL>(reinterpret_cast<const uint16_t*>(g), i, n, q, vec);
   else ld_f32<FULL>(reinterpret_cast<const float*>(g), i, n, q, vec);
@@ -303,8 +303,8 @@ __device__ __forceinline__ double dense_vec(const void* g, int64_t i, int64_t n,
     ll[e] = __fmaf_rn(upd * (float)(sc.s.lr * sc.s.lr), upd, ll[e]);
     mm[e] = mn;
     vv[e] = vn;
-    const double qd = (double)q[e] / coef_dense;
-    acc += qd * qd;
+    const double qd = (double)q[e];
+    acc += qd * qd;                       // exact product; the divisor is applied once, to the sum
   }
   st_f32<FULL>(m, i, n, mm, vec);
   st_f32<FULL>(v, i, n, vv, vec);
@@ -316,7 +316,7 @@ __device__ __forceinline__ double dense_vec(const void* g, int64_t i, int64_t n,
 template <bool BF16G>
 __global__ __launch_bounds__(kBlock) void k_dense_step(const void* __restrict__ g, int64_t n,
                                                        float* w, float* m, float* v, float* lab,
-                                                       int adams, double coef_dense,
+                                                       int adams,
                                                        const RSeg* __restrict__ segs, int n_segs,
                                                        double* __restrict__ partials, bool vec) {
   __shared__ double s_w[kChunksPerBlock];
@@ -327,9 +327,9 @@ __global__ __launch_bounds__(kBlock) void k_dense_step(const void* __restrict__ 
   for (int64_t base = (int64_t)blockIdx.x * kBlock * kVec; base < n; base += stride) {
     const int64_t i = base + (int64_t)threadIdx.x * kVec;
     if (vec && base + kBlock * kVec <= n)
-      acc += dense_vec<BF16G, true>(g, i, n, w, m, v, lab, adams, coef_dense, sc, true);
+      acc += dense_vec<BF16G, true>(g, i, n, w, m, v, lab, adams, sc, true);
     else if (i < n)
-      acc += dense_vec<BF16G, false>(g, i, n, w, m, v, lab, adams, coef_dense, sc, vec);
+      acc += dense_vec<BF16G, false>(g, i, n, w, m, v, lab, adams, sc, vec);
   }
   acc = wave_sum(acc);
   if (lane_id() == 0) s_w[wave_id()] = acc;
@@ -487,6 +487,23 @@ __global__ __launch_bounds__(kBlock) void k_sqdist_stage1(const float* __restric
   if (lane_id() == 0) s_w[wave_id()] = acc;
   __syncthreads();
   if (threadIdx.x == 0) partials[blockIdx.x] = s_w[0] + s_w[1] + s_w[2] + s_w[3];
+}
+// Fold of up to kReplayBlocks * kMaxCfg workgroup partials by one wide workgroup, fixed order:
+// lane t adds partials t, t + 1024, ... in turn, then a tree over the lanes.
+constexpr int kFoldThreads = 1024;
+__global__ __launch_bounds__(kFoldThreads) void k_fold_partials(const double* __restrict__ partials,
+                                                                int nb, double divisor,
+                                                                double* __restrict__ out) {
+  __shared__ double s_p[kFoldThreads];
+  double a = 0.0;
+  for (int b = threadIdx.x; b < nb; b += kFoldThreads) a += partials[b];
+  s_p[threadIdx.x] = a;
+  __syncthreads();
+  for (int o = kFoldThreads / 2; o > 0; o >>= 1) {
+    if ((int)threadIdx.x < o) s_p[threadIdx.x] += s_p[threadIdx.x + o];
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) out[0] = s_p[0] / divisor;
 }
 __global__ __launch_bounds__(kWave) void k_sqdist_stage2(const double* __restrict__ partials, int nb,
                                                          double* __restrict__ out) {
@@ -670,12 +687,15 @@ extern "C" int sga_dense_replay_step(const void* g, int g_dtype, float* w, float
   const bool bg = g_dtype == SGA_BF16;
   const bool vec = aligned4(g, bg ? 2 : 4) && aligned4(w, 4) && aligned4(m, 4) && aligned4(v, 4) &&
                    aligned4(lab, 4);
-  const unsigned nb = stream_grid(n, (int64_t)kBlock * kVec, kReplayBlocks);
+  // as close to one 1024-element slab per workgroup as the partials workspace allows (a capped
+  // grid-stride loop leaves a quarter of the bandwidth unused); the fold stays in a fixed order
+  const unsigned nb = stream_grid(n, (int64_t)kBlock * kVec, kReplayBlocks * kMaxCfg);
   hipStream_t s = (hipStream_t)stream;
   const RSeg* rs = reinterpret_cast<const RSeg*>(segs);
-  if (bg) hipLaunchKernelGGL((k_dense_step<true>), dim3(nb), dim3(kBlock), 0, s, g, n, w, m, v, lab, adams, coef_dense, rs, n_segs, partials, vec);
-  else hipLaunchKernelGGL((k_dense_step<false>), dim3(nb), dim3(kBlock), 0, s, g, n, w, m, v, lab, adams, coef_dense, rs, n_segs, partials, vec);
-  hipLaunchKernelGGL(k_sqdist_stage2, dim3(1), dim3(kWave), 0, s, partials, (int)nb, recon2);
+  if (bg) hipLaunchKernelGGL((k_dense_step<true>), dim3(nb), dim3(kBlock), 0, s, g, n, w, m, v, lab, adams, rs, n_segs, partials, vec);
+  else hipLaunchKernelGGL((k_dense_step<false>), dim3(nb), dim3(kBlock), 0, s, g, n, w, m, v, lab, adams, rs, n_segs, partials, vec);
+  hipLaunchKernelGGL(k_fold_partials, dim3(1), dim3(kFoldThreads), 0, s, partials, (int)nb,
+                     coef_dense * coef_dense, recon2);
   return check_launch("sga_dense_replay_step");
 }
 
