@@ -1,4 +1,4 @@
-"""Full-size runs of the BASELINE configurations checked through
+"""Full-size runs of the benchmark configurations checked through
 size-independent properties (the CPU oracle would take minutes at these
 sizes): exactly k selected, selected scores dominate unselected ones, ties
 form an index prefix, idx sorted and consistent with the mask, values are the
