@@ -22,7 +22,7 @@ from . import select as SEL
 
 def fused_sparse_step(g, resid, p, m, v, segments, step, ratio_percent=None,
                       k=None, score="abs_g", values_dtype=torch.float32,
-                      factor=1.0, coeff=1.0, given_score=None):
+                      factor=1.0, coeff=1.0):
     """One step over a flat bucket.
 
     g        : flat gradient (bf16 or fp32), read only
@@ -30,16 +30,12 @@ def fused_sparse_step(g, resid, p, m, v, segments, step, ratio_percent=None,
     p, m, v  : flat fp32 state, updated in place
     segments : list of dicts {"start","n","lr","b1","b2","eps","wd"}
     score    : "abs_g" (= |g+r|), "update", "coi", "abs_m"
-    given_score : optional precomputed non-negative score (used when index
-               parity must be asserted on identical score bits)
     Returns (idx int32[k], values[k], mask bool[N], thresh).
     """
     n = resid.numel()
     resid.add_(g.float())                      # buf = r + g (one fp32 add)
     buf = resid
-    if given_score is not None:
-        sc = given_score
-    elif score == "abs_g":
+    if score == "abs_g":
         sc = buf.abs()
     else:
         sc = torch.empty(n)
