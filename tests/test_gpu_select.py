@@ -142,6 +142,13 @@ def test_replay_select_building_blocks(dev):
     assert gt.dtype == torch.bool and torch.equal(gt.cpu(), sc > th)
     assert torch.equal(eq.cpu(), sc == th)
     assert counts.tolist() == [int((sc > th).sum()), int((sc == th).sum())]
+    # views that start off the 16-byte grid take the scalar paths of the same kernels
+    for off in (1, 3):
+        hv, _ = K.hist_top16(sd[off:])
+        assert torch.equal(hv, torch.bincount(top[off:], minlength=32769))
+        gv, ev, cv = K.gt_eq_counts(sd[off:], th)
+        assert torch.equal(gv.cpu(), sc[off:] > th) and torch.equal(ev.cpu(), sc[off:] == th)
+        assert cv.tolist() == [int((sc[off:] > th).sum()), int((sc[off:] == th).sum())]
     bad = sc.clone()
     bad[5] = float("nan")
     bad[6] = float("inf")
@@ -260,6 +267,11 @@ def test_adaptive_threshold_masks(dev):
     for a, b in zip(masks, ref):
         assert torch.equal(a.cpu(), b)
     assert cnt == sum(int(m.sum()) for m in ref)
+    big = torch.randn(1_000_003, generator=g)          # several trips of the unrolled loop, ragged end
+    for off in (0, 1):
+        mk, c = threshold_masks([big.to(dev)[off:]], tau)
+        assert torch.equal(mk[0].cpu(), (big[off:].abs() >= tau).to(torch.uint8))
+        assert c == int((big[off:].abs() >= tau).sum())
     assert adapt_threshold(2.0, 0.105, 0.10) == 2.0
     assert adapt_threshold(2.0, 0.4, 0.10) == 2.0 * 1.15
     assert abs(adapt_threshold(2.0, 0.12, 0.10, band=0.0) - 2.0 * 1.2 ** 0.5) < 1e-12
