@@ -93,6 +93,24 @@ int64_t sga_norm_partials(int64_t n);
 int sga_compact_norm_sq(const float* values, int64_t k, float* partials,
                         float* total, void* stream);
 
+/* Allocation-free variant of sga_compact_norm_sq.  It has no counterpart in
+ * the reference (whose compact_norm_sq_contribution allocates its partials on
+ * every call, kernels.py:264); it is for callers that cannot allocate device
+ * memory or carry a workspace: code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc.  The stage-1 partials live in an
+ * 8 KiB array inside the library's device image, one copy per GPU, kept until
+ * the process ends; the call allocates nothing and frees nothing.  Same
+ * kernels, same grid and the same bits in total[0] as sga_compact_norm_sq.
+ * k above SGA_NOALLOC_NORM_MAX_K is refused with SGA_ERR_ARG.  Every call on
+ * a GPU shares that GPU's array: calls that overlap on one GPU (two streams,
+ * two host threads) race; serialise them.  Nothing in the array has to be
+ * cleared between calls (each call overwrites the slots it reads).  The first
+ * call on a device looks the array's address up (hipGetSymbolAddress): make
+ * it before a graph capture starts. */
+#define SGA_NOALLOC_NORM_MAX_K 2147483647ll
+int sga_compact_norm_sq_noalloc(const float* values, int64_t k, float* total,
+                                void* stream);
+
 /* total[0] += sum(grad[mask]^2)
  *                 -- masked_norm_sq_contribution, kernels.py:284-302.
  * Deterministic two-stage reduction (the reference uses a float atomic). */

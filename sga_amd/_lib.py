@@ -36,6 +36,7 @@ SIGNATURES = {
     "sga_pack_selected": (I32, [P, P, P, I32, F, I64, I64, P]),
     "sga_norm_partials": (I64, [I64]),
     "sga_compact_norm_sq": (I32, [P, I64, P, P, P]),
+    "sga_compact_norm_sq_noalloc": (I32, [P, I64, P, P]),
     "sga_masked_norm_sq": (I32, [P, P, I64, P, P, P]),
     "sga_gather_selected_blocks": (I32, [P, P, P, P, I64, I32, F, I64, P]),
     "sga_scatter_selected_blocks": (I32, [P, P, P, P, I64, I32, I64, P]),

@@ -1,6 +1,8 @@
 // Scheme-agnostic masked ops: pack / scatter / norms / block gather-scatter /
 // mask compaction.  All are HBM-bound byte movers; nothing here is a
 // contraction.
+#include <mutex>
+
 #include "common.hpp"
 
 namespace sga {
@@ -347,6 +349,8 @@ extern "C" int sga_pack_selected(float* grad, const int32_t* idx, void* values,
 }
 
 static const int64_t kNormMaxBlocks = 2048;
+// largest k of the allocation-free norm: the int32 index domain of a bucket (kernels.py:154)
+static const int64_t kNoAllocNormMaxK = SGA_NOALLOC_NORM_MAX_K;
 
 static int xlog_of(int x);
 
@@ -409,6 +413,65 @@ extern "C" int sga_compact_norm_sq(const float* values, int64_t k,
   hipLaunchKernelGGL(k_norm_stage2, dim3(1), dim3(kBlock), 0, st, partials,
                      (int64_t)nb, total);
   return check_launch("sga_compact_norm_sq");
+}
+
+// The stage-1 partials of the allocation-free norm: one array per device,
+// held by every GPU the library runs on until the process ends (8 KiB).  In
+// host code the array's name is only a stand-in for the symbol; the device
+// address is resolved once per device and kept in g_norm_scratch_ptr.
+static __device__ __align__(256) float scratch[kNormMaxBlocks];
+
+static const int kNoAllocMaxDevices = 64;
+static std::mutex g_norm_scratch_mu;
+static float* g_norm_scratch_ptr[kNoAllocMaxDevices] = {};
+
+// Device address of `scratch` on the current device, or null with the error
+// text set.  The first call on a device resolves the symbol (no allocation).
+static float* norm_scratch_of_current_device(const char* who) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess || dev < 0 || dev >= kNoAllocMaxDevices) {
+    set_error("%s: cannot name the current device (%s, device %d, at most %d supported)", who,
+              hipGetErrorString(e), dev, kNoAllocMaxDevices);
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> lock(g_norm_scratch_mu);
+  if (!g_norm_scratch_ptr[dev]) {
+    void* ptr = nullptr;
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !ptr) {
+      set_error("%s: hipGetSymbolAddress(scratch) failed on device %d: %s", who, dev,
+                hipGetErrorString(e));
+      return nullptr;
+    }
+    g_norm_scratch_ptr[dev] = static_cast<float*>(ptr);
+  }
+  return g_norm_scratch_ptr[dev];
+}
+
+extern "C" int sga_compact_norm_sq_noalloc(const float* values, int64_t k, float* total,
+                                           void* stream) {
+  if (k == 0) return SGA_OK;
+  if (!values || !total || k < 0) {
+    set_error("sga_compact_norm_sq_noalloc: bad argument");
+    return SGA_ERR_ARG;
+  }
+  if (k > kNoAllocNormMaxK) {
+    set_error("sga_compact_norm_sq_noalloc: k=%lld exceeds the supported maximum %lld "
+              "(use sga_compact_norm_sq with a caller workspace)",
+              (long long)k, (long long)kNoAllocNormMaxK);
+    return SGA_ERR_ARG;
+  }
+  float* partials = norm_scratch_of_current_device("sga_compact_norm_sq_noalloc");
+  if (!partials) return SGA_ERR_LAUNCH;
+  // same two kernels, same grid as sga_compact_norm_sq: the result has the same bits.  Stage 1
+  // overwrites the nb slots stage 2 reads, so nothing in the array has to start at zero.
+  const unsigned nb = (unsigned)sga_norm_partials(k);
+  hipStream_t st = (hipStream_t)stream;
+  hipLaunchKernelGGL((k_norm_stage1<false>), dim3(nb), dim3(kBlock), 0, st, values,
+                     (const uint8_t*)nullptr, k, partials, aligned4(values, 4));
+  hipLaunchKernelGGL(k_norm_stage2, dim3(1), dim3(kBlock), 0, st, partials, (int64_t)nb, total);
+  return check_launch("sga_compact_norm_sq_noalloc");
 }
 
 extern "C" int sga_masked_norm_sq(const float* grad, const uint8_t* mask,
