@@ -90,3 +90,26 @@ def mask_layout_unpack(grad, mask_u8, payloads, slices=2):
     bounds = [i * (n // slices) for i in range(slices)] + [n]
     for (s, e), p in zip(zip(bounds[:-1], bounds[1:]), payloads):
         grad[s:e][mask_u8[s:e].bool()] = p
+
+
+def index_layout_bounds(idx, n, slices=2):
+    """(lo, hi) ranges of the sorted idx per pipeline slice: bucket-midpoint
+    split for the default two slices (``support.split``, support.py:345-351),
+    even split of the selected set otherwise
+    (``torch_pipelined_index.py:314-325``)."""
+    k = idx.numel()
+    if slices == 2:
+        n0 = int((idx.long() < n // 2).sum())
+        return [(0, n0), (n0, k)]
+    return [(i * k // slices, (i + 1) * k // slices) for i in range(slices)]
+
+
+def index_layout_pack(grad, idx, values, factor, slices=2):
+    """Compact emission of the index backend: slice by slice
+    ``pack_selected(grad, idx[lo:hi], values[lo:hi], factor)``
+    (``torch_pipelined_index.py:508-520``)."""
+    out = index_layout_bounds(idx, grad.numel(), slices)
+    for lo, hi in out:
+        if hi > lo:
+            pack_selected(grad, idx[lo:hi], values[lo:hi], factor)
+    return out

@@ -9,18 +9,28 @@ from . import kernels as K
 from .support import compact_mask_u8
 
 
+def index_layout_bounds(idx, n, slices=2):
+    """Per-slice (lo, hi) ranges into the sorted ``idx``: with the default two
+    slices the split sits at the bucket midpoint (``support.split`` =
+    ``searchsorted(idx, n // 2)``, ``sga/support.py:345-351``), any other count
+    splits the selected set evenly (``torch_pipelined_index.py:314-325``)."""
+    k = idx.numel()
+    if slices == 2:
+        mid = torch.tensor([n // 2], dtype=idx.dtype, device=idx.device)
+        n0 = int(torch.searchsorted(idx, mid).item())
+        return [(0, n0), (n0, k)]
+    return [(i * k // slices, (i + 1) * k // slices) for i in range(slices)]
+
+
 def index_layout_pack(grad, idx, values, factor=1.0, slices=2):
     """Index layout: ``values[k]`` in ``grad``'s order of the sorted int32
-    ``idx``, packed slice by slice at the midpoint-style split the reference
-    pipelines (``torch_pipelined_index.py:508-520``); the packed positions of
-    ``grad`` are zeroed.  Returns the per-slice (lo, hi) ranges of ``values``."""
-    k = idx.numel()
-    bounds = [k * i // slices for i in range(slices)] + [k]
-    out = []
-    for lo, hi in zip(bounds[:-1], bounds[1:]):
+    ``idx``, packed slice by slice as the reference pipelines it
+    (``torch_pipelined_index.py:508-520``); the packed positions of ``grad``
+    are zeroed.  Returns the per-slice (lo, hi) ranges of ``values``."""
+    out = index_layout_bounds(idx, grad.numel(), slices)
+    for lo, hi in out:
         if hi > lo:
             K.pack_selected(grad, idx[lo:hi], values[lo:hi], factor)
-        out.append((lo, hi))
     return out
 
 

@@ -212,6 +212,42 @@ def test_reselect_adam_scores(dev, score, sizes, vary, path):
     assert grp.last_select().path == path
 
 
+def _assert_group_equal(grp, out, specs):
+    for ci, o in enumerate(out):
+        s = grp.state[ci]
+        assert torch.equal(s["sel"].cpu().bool(), o["sel"]), (ci, specs[ci])
+        assert same_bits(s["res"], o["res"]) and same_bits(s["m"], o["m"]), (ci, specs[ci])
+        assert same_bits(s["v"], o["v"]) and same_bits(s["w"], o["w"]), (ci, specs[ci])
+
+
+@pytest.mark.parametrize("opt", ["adamw", "adams"])
+@pytest.mark.parametrize("clip", [0.0, 0.3])
+def test_group_adam_scores_live_residual(dev, opt, clip):
+    """Boundary re-selection by the Adam-normalised scores with a LIVE residual
+    (T > 1), a clip coefficient below one, a dense-run coefficient below one
+    (the recorded norm is finite), fold and dual-lr arms, under AdamW and AdamS
+    (v := m*m, bc := 1: replay.py:486-505): score = |formula(w, m, v,
+    (g / coef_dense + res) * coef)| as replay_fused.py:1752-1825 forms it.  The
+    oracle selects on its own scores; masks and state must agree bit for bit."""
+    specs = [("update", 1.0, 2, opt), ("coi", 10.0, 4, opt), ("update", 0.1, 4, opt, True),
+             ("coi", 1.0, 2, opt, False, 0.25), ("update", 10.0, 3, opt, True, 2.0),
+             ("coi", 0.1, 3, opt)]
+    grp, out, w0 = _run_group(dev, specs, clip=clip, W=9, bf16=True)
+    assert float(grp.state[5]["res"].abs().max()) > 0.0          # T = 3 ends two steps past a boundary
+    _assert_group_equal(grp, out, specs)
+
+
+@pytest.mark.parametrize("opt", ["adamw", "adams"])
+def test_group_adam_scores_one_sweep_long_cycle(dev, opt):
+    """The same cell above 2^20 elements on ragged tensors (one-sweep select,
+    slabs that straddle tensors) with a T = 16 arm that re-selects at si = 16
+    after 15 masked steps of residual accumulation, f32 gradients, clip on."""
+    specs = [("update", 1.0, 16, opt), ("coi", 1.0, 4, opt), ("update", 0.1, 2, opt, True, 0.25)]
+    grp, out, w0 = _run_group(dev, specs, clip=0.3, W=18, bf16=False, sizes=_RAGGED)
+    assert grp.last_select().path == 1
+    _assert_group_equal(grp, out, specs)
+
+
 @pytest.mark.parametrize("seed", range(6))
 def test_randomized_groups(dev, seed):
     """Seeded random groups: ragged tensor sizes around 2^20 elements, 1..5
@@ -229,7 +265,7 @@ def test_randomized_groups(dev, seed):
     if len(sizes) < 2:
         sizes = [sizes[0] - 1000, 1000]
     rng.shuffle(sizes)
-    specs = [(rng.choice(["abs_g", "abs_m", "abs_g"]), rng.choice([0.1, 1.0, 10.0]),
+    specs = [(rng.choice(["abs_g", "abs_m", "update", "coi"]), rng.choice([0.1, 1.0, 10.0]),
               rng.choice([1, 2, 3, 4]), rng.choice(["adamw", "adams"]), rng.choice([False, True]),
               rng.choice([1.0, 0.25, 2.0])) for _ in range(rng.randint(1, 5))]
     grp, out, w0 = _run_group(dev, specs, clip=rng.choice([0.0, 0.3]), W=rng.choice([4, 6, 9]),

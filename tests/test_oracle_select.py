@@ -165,6 +165,41 @@ def test_compact_mask_kats():
     assert OK.compact_mask_u8(m).tolist() == [i for i, b in enumerate(m.tolist()) if b]
 
 
+def test_layout_oracles_against_element_loops():
+    """The two sparse-sync layouts of the oracle against plain Python loops on
+    small inputs: mask layout = per slice [i*(n//s), ...) the set coordinates
+    in index order times factor, written back in place; index layout = gather,
+    scale, zero, with the bucket-midpoint split for two slices (the KAT's
+    split_at_mid) and the even split otherwise."""
+    g = torch.Generator().manual_seed(9)
+    for n, s in ((11, 2), (11, 3), (10, 1), (7, 4), (1, 2)):
+        grad = torch.randn(n, generator=g)
+        mask = (torch.rand(n, generator=g) < 0.5).to(torch.uint8)
+        cuts = [i * (n // s) for i in range(s)] + [n]
+        want = [[grad[i].item() * 0.5 for i in range(a, b) if mask[i]]
+                for a, b in zip(cuts[:-1], cuts[1:])]
+        got = OK.mask_layout_pack(grad, mask, 0.5, s)
+        assert [p.tolist() for p in got] == want
+        back = torch.zeros(n)
+        OK.mask_layout_unpack(back, mask, got, s)
+        assert back.tolist() == [grad[i].item() * 0.5 if mask[i] else 0.0 for i in range(n)]
+        idx = OK.compact_mask_u8(mask)
+        k = idx.numel()
+        bounds = OK.index_layout_bounds(idx, n, s)
+        if s == 2:
+            n0 = sum(1 for i in idx.tolist() if i < n // 2)
+            assert bounds == [(0, n0), (n0, k)]
+        else:
+            assert bounds == [(i * k // s, (i + 1) * k // s) for i in range(s)]
+        g2, vals = grad.clone(), torch.empty(k)
+        assert OK.index_layout_pack(g2, idx, vals, 0.5, s) == bounds
+        assert vals.tolist() == [grad[i].item() * 0.5 for i in idx.tolist()]
+        assert g2.tolist() == [0.0 if mask[i] else grad[i].item() for i in range(n)]
+    kat = KATS["compact_mask"][0]
+    idx = torch.tensor(kat["idx"], dtype=torch.int32)
+    assert OK.index_layout_bounds(idx, len(kat["mask"]), 2)[0][1] == kat["split_at_mid"]
+
+
 def test_block_helpers_kats():
     """Literal block KATs: ANY rule, short tail blocks, x == 1 == compaction."""
     m = torch.tensor([0, 1, 0, 0, 0, 0, 1, 1, 0, 0, 1], dtype=torch.uint8)
