@@ -143,3 +143,157 @@ def test_qwen06b_set_mask_layout_per_bucket(dev):
         dst = torch.zeros(nb, device=dev)
         backends.mask_layout_unpack(dst, idx2, payloads)
         assert torch.equal(dst, torch.where(fs.mask.bool(), buf, torch.zeros((), device=dev)))
+
+
+def _dev_scalar(x, dev):
+    return torch.tensor(x, dtype=torch.float32, device=dev)
+
+
+def _update_score_torch(segs, p, m, v, q, step):
+    """|wd*p + U(q)| with plain torch ops on the device, one separately rounded
+    fp32 kernel per operation in the order of scores.py:183-226.  Divisions go
+    through 0-dim device tensors: torch divides a device tensor by a Python
+    scalar as a multiplication by the reciprocal, by a tensor as a division."""
+    dev = q.device
+    out = torch.empty_like(q)
+    for s in segs:
+        a, b = s["start"], s["start"] + s["n"]
+        b1, b2 = s["b1"], s["b2"]
+        sa = (m[a:b] * b1 + q[a:b] * (1.0 - b1)) / _dev_scalar(1.0 - b1 ** step, dev)
+        sb = (v[a:b] * b2 + (q[a:b] * (1.0 - b2)) * q[a:b]) / _dev_scalar(1.0 - b2 ** step, dev)
+        out[a:b] = (s["wd"] * p[a:b] + sa / (torch.sqrt(sb) + s["eps"])).abs()
+    return out
+
+
+@pytest.mark.parametrize("ratio", [0.1, 1.0, 10.0])
+def test_llama1b_set_update_score(dev, ratio):
+    """Config 3 as worded: Llama-3.2-1B set, bf16 Student-t grads, the
+    Adam-normalised score (`update`, scores.py:202-231) at 0.1 / 1 / 10 %,
+    index pack int32 + bf16.  The score is rebuilt with torch ops on the device
+    from the pre-step state; the one-sweep select scores slabs that straddle
+    the 146 tensors with per-tensor weight decay."""
+    from sga_amd.fused_step import FusedSparseStep, k_for
+    from sga_amd.shapes import llama32_1b, segments_for
+    segs, n = segments_for(llama32_1b())
+    step = 5
+    g = _student_t(n, 3, dev).to(torch.bfloat16)
+    gen = torch.Generator(device=dev).manual_seed(2)
+    p = torch.randn(n, generator=gen, device=dev) * 0.02
+    m = torch.randn(n, generator=gen, device=dev) * 1e-4
+    v = torch.rand(n, generator=gen, device=dev) * 1e-8
+    r = _student_t(n, 4, dev, scale=3e-4)
+    buf = r + g.float()
+    score = _update_score_torch(segs, p, m, v, buf, step)
+    m0 = m.clone()
+    k = k_for(n, ratio)
+    fs = FusedSparseStep(n, segs, dev, values_dtype=torch.bfloat16, max_k=k, want_mask=True)
+    idx, vals = fs.step(g, r, p, m, v, step, k=k, score="update")
+    res = fs.read_result()
+    assert res.status == 0 and res.n_selected == k and res.path == 1 and res.nonfinite == 0
+    mask = fs.mask.bool()
+    _check_select(score, mask, k, res.thresh)
+    assert torch.equal(idx.long(), torch.nonzero(mask).reshape(-1))
+    assert torch.equal(vals, buf[mask].to(torch.bfloat16))
+    assert torch.equal(r, torch.where(mask, torch.zeros((), device=dev), buf))
+    gq = torch.where(mask, buf.to(torch.bfloat16).float(), torch.zeros((), device=dev))
+    assert torch.equal(m, m0 * 0.9 + gq * (1.0 - 0.9))
+
+
+def _select_ok(score, mask, k):
+    """Exact-k, dominance and lowest-index ties of a mask against a score."""
+    assert int(mask.sum()) == k
+    th = float(score[mask].min())
+    _check_select(score, mask, k, th)
+
+
+def test_qwen06b_replay_group_full_window(dev):
+    """Config 4 at full size: Qwen3-0.6B shapes (596,049,920 elements, 310
+    tensors), G = 8 configs over score x ratio x cycle length, window of 32
+    recorded bf16 steps, clip 1.0.  Size-independent properties:
+    * every config's mask holds exactly k coordinates at every step end checked;
+    * T = 1 configs never keep a residual;
+    * off a boundary the residual is zero on the mask and the running fp32 sum
+      of the recorded gradient since the last boundary elsewhere;
+    * the re-selection at si = 16 of the T = 16 arm (15 masked steps of
+      residual behind it) and at si = 28 of a T = 4 `update` arm equal the exact
+      top-k of the score rebuilt from the state just before that step;
+    * with clipping off, a T = 1 arm is the dense reference trajectory
+      (sga_dense_replay_step) bit for bit."""
+    from sga_amd.replay import score_formula, select_topk_flat
+    from sga_amd.replay_dense import DenseReplay
+    from sga_amd.replay_group import Config, ReplayGroup
+    from sga_amd.shapes import qwen3_06b, segments_for
+    segs, n = segments_for(qwen3_06b())
+    assert n == 596_049_920 and len(segs) == 310
+    W, t0, lr = 32, 100, 1e-4
+    entries = [{"a": s["start"], "n": s["n"], "b1": s["b1"], "b2": s["b2"], "eps": s["eps"],
+                "wd": s["wd"]} for s in segs]
+    specs = [("abs_g", 1.0, 1), ("abs_g", 0.1, 4), ("abs_g", 10.0, 16), ("update", 1.0, 4),
+             ("update", 10.0, 1), ("coi", 1.0, 16), ("coi", 0.1, 4), ("update", 0.1, 16)]
+    cfgs = [Config(*sp) for sp in specs]
+    gen = torch.Generator(device=dev).manual_seed(1)
+    w0 = torch.randn(n, generator=gen, device=dev) * 0.02
+    m0 = torch.randn(n, generator=gen, device=dev) * 1e-4
+    v0 = torch.rand(n, generator=gen, device=dev) * 1e-8
+    window = [_student_t(n, 500 + s, dev, scale=1e-3 * (1.0 + 0.02 * s)).to(torch.bfloat16)
+              for s in range(W)]
+    ks = [max(1, int(round(c.ratio / 100.0 * n))) for c in cfgs]
+    base = window[0].float().abs()
+    sel0 = [select_topk_flat(base, k)[0] for k in ks]
+    del base
+    grp = ReplayGroup(entries, w0, m0, v0, sel0, cfgs, t0, W)
+    del sel0
+    meta = {"clip_grad": 1.0, "grad_norm": float("nan"), "lr": lr}
+    probes = {16: 2, 28: 3}                       # si -> config whose re-selection is rebuilt
+    for si in range(W):
+        pre = None
+        if si in probes:
+            s = grp.state[probes[si]]
+            pre = {x: s[x].clone() for x in ("w", "m", "v", "res")}
+        grp.step(window[si], meta)
+        if pre is not None:
+            ci = probes[si]
+            c = cfgs[ci]
+            coef = grp.coef_f[ci:ci + 1]
+            assert 0.0 < float(coef) < 1.0                     # the clip is live
+            q = (window[si].float() + pre["res"]) * coef       # coef_dense == 1 (no recorded norm)
+            if c.score == "abs_g":
+                score = q.abs()
+            else:
+                score = torch.empty_like(q)
+                count = t0 + si + 1
+                for e in entries:
+                    a, b = e["a"], e["a"] + e["n"]
+                    score[a:b] = score_formula(c.score, pre["w"][a:b], pre["m"][a:b],
+                                               pre["v"][a:b], q[a:b], e["b1"], e["b2"], e["eps"],
+                                               e["wd"], 1 - e["b1"] ** count, 1 - e["b2"] ** count,
+                                               "adamw", update_includes_wd=True).abs()
+            _select_ok(score, grp.state[ci]["sel"].bool(), ks[ci])
+            del pre, q, score
+    for ci, c in enumerate(cfgs):
+        s = grp.state[ci]
+        mask = s["sel"].bool()
+        assert int(mask.sum()) == ks[ci], ci
+        res = s["res"]
+        if c.T == 1:
+            assert float(res.abs().max()) == 0.0, ci
+            continue
+        last_b = ((W - 1) // c.T) * c.T                        # res was zeroed there
+        acc = torch.zeros(n, device=dev)
+        for si in range(last_b + 1, W):
+            acc += window[si].float()
+        assert torch.equal(res, torch.where(mask, torch.zeros((), device=dev), acc)), ci
+        del acc
+    del grp
+    torch.cuda.empty_cache()
+    # clipping off: a T = 1 arm IS the dense trajectory
+    steps = 6
+    sel = torch.zeros(n, dtype=torch.bool, device=dev)
+    grp = ReplayGroup(entries, w0, m0, v0, [sel], [Config("abs_g", 1.0, 1)], t0, steps)
+    dense = DenseReplay(entries, w0, m0, v0, t0)
+    for si in range(steps):
+        grp.step(window[si], {"clip_grad": 0.0, "lr": lr})
+        dense.step(t0 + si, window[si], {"clip_grad": 0.0, "lr": [lr]})
+    s = grp.state[0]
+    for name, ref in (("w", dense.w), ("m", dense.m), ("v", dense.v)):
+        assert torch.equal(s[name].view(torch.int32), ref.view(torch.int32)), name
