@@ -1,20 +1,20 @@
 #!/usr/bin/env python3
 """Benchmark of the fused per-rank sparse step on one MI355X.
 
-One "step" = score |g+r| -> exact top-k (1 %, lowest-index ties) -> index pack
-(int32 idx + bf16 values) -> residual update -> residual-aware AdamW over the
+One "step" = score -> exact top-k (lowest-index ties) -> index pack (int32 idx
++ bf16 values) -> residual update -> residual-aware AdamW over the
 Llama-3.2-1B-shaped gradient set (1,235,814,400 elements, 146 tensors, bf16
 Student-t(3) gradients, fp32 p/m/v/residual) with every input resident in HBM.
 
-The step is timed on both state layouts: the library-owned packed layout
-(resid/p/m/v interleaved in 64 KiB records -- the headline) and the drop-in
-one (four flat tensors, as the reference's buffers are); both run the same
-arithmetic and produce the same bits.
-
-Prints ONE JSON line: whole-job elements/s, the roofline of the dominant
-kernel (the final sweep, timed live with HIP events on its launch stream),
-both layouts under "layouts", the fused replay leg and the CPU oracle timed on
-a bounded sample of the same workload.
+The headline is the drop-in entry point (resid / p / m / v as the caller's four
+flat tensors, as the reference's buffers are) with the Adam-normalised score
+(`update`) at 1 %.  The same JSON line carries the whole sweep of the
+benchmark configuration -- scores {update, abs_g} x ratios {0.1, 1, 10} % x
+state layouts {separate, packed (library-owned 64 KiB records)} -- with each
+leg's own algorithmic bytes, one row for the Qwen3-0.6B per-bucket mask-layout
+configuration, one for the 1e9-element stress buffer, the fused replay leg and
+the CPU oracle timed on a bounded sample of the headline workload.  The
+dominant kernels are timed live with HIP events on their launch stream.
 """
 import argparse
 import ctypes
@@ -27,8 +27,27 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK = 8.0e12          # MI355X HBM3E, B/s
-ALG_BYTES_STEP = 40.0      # 2*(2+4) + 4 + 24  (bf16 g, two-buffer contract)
 ALG_BYTES_FINAL = 34.0     # final sweep: read g,r,p,m,v (18) + write r,p,m,v (16)
+PROF_FINAL, PROF_SWEEP, PROF_PASS3, PROF_PASS1 = 0, 1, 2, 3     # include/sga_hip_bench.h
+
+
+def sweep_bytes_per_elem(score, g_bytes=2.0):
+    """Algorithmic bytes per element of the select's one data sweep: it reads
+    the gradient and the residual, and for the Adam-normalised scores p, m, v
+    as well."""
+    return g_bytes + 4.0 + (12.0 if score in ("update", "coi") else 0.0)
+
+
+def step_bytes_per_elem(score, g_bytes=2.0):
+    """Whole step: the select sweep + the final sweep (reads g, r, p, m, v,
+    writes r, p, m, v)."""
+    return sweep_bytes_per_elem(score, g_bytes) + g_bytes + 32.0
+
+
+def prof_read(L, tag):
+    tot, cnt = ctypes.c_double(0), ctypes.c_int(0)
+    L.call("sga_prof_read", tag, ctypes.byref(tot), ctypes.byref(cnt))
+    return tot.value, cnt.value
 
 
 def student_t_dev(n, seed, dev, scale=1e-3, nu=3, chunk=1 << 26):
@@ -45,7 +64,7 @@ def student_t_dev(n, seed, dev, scale=1e-3, nu=3, chunk=1 << 26):
     return out
 
 
-def cpu_baseline(sample_n, steps, ratio):
+def cpu_baseline(sample_n, steps, ratio, score="abs_g"):
     """Oracle (torch CPU restatement of the reference's pure-torch path) on the
     first ``sample_n`` elements of the same tensor list."""
     import torch
@@ -63,17 +82,17 @@ def cpu_baseline(sample_n, steps, ratio):
     p = torch.randn(n, generator=gen) * 0.02
     m, v, r = torch.zeros(n), torch.zeros(n), torch.zeros(n)
     grads = [student_t(n, 100 + s).to(torch.bfloat16) for s in range(steps)]
-    OF.fused_sparse_step(grads[0], r, p, m, v, segs, 1, ratio_percent=ratio,
+    OF.fused_sparse_step(grads[0], r, p, m, v, segs, 1, ratio_percent=ratio, score=score,
                          values_dtype=torch.bfloat16)             # warm-up step
     t0 = time.perf_counter()
     for s in range(steps):
-        OF.fused_sparse_step(grads[s], r, p, m, v, segs, s + 2, ratio_percent=ratio,
+        OF.fused_sparse_step(grads[s], r, p, m, v, segs, s + 2, ratio_percent=ratio, score=score,
                              values_dtype=torch.bfloat16)
     dt = time.perf_counter() - t0
     return {"value": n * steps / dt, "unit": "elem/s", "cores": torch.get_num_threads(),
             "kind": "port",
             "sample": f"{len(shapes)} layer tensors of the Llama-3.2-1B list "
-                      f"({n} elements), {steps} steps at {ratio}% after 1 warm-up step, "
+                      f"({n} elements), score {score}, {steps} steps at {ratio}% after 1 warm-up step, "
                       f"{dt:.1f} s; host cpu_count={os.cpu_count()}"}
 
 
@@ -114,31 +133,51 @@ def replay_bench(G=8, W=32, seed=4):
     del sel0
     meta = {"clip_grad": 1.0, "grad_norm": float("nan"), "lr": 1e-4}
     torch.cuda.synchronize()
+    L.raw("sga_prof_enable", 1)
     t0 = time.perf_counter()
     for s in range(W):
         grp.step(window[s], meta)
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
+    p3_ms, p3_n = prof_read(L, PROF_PASS3)
+    p1_ms, p1_n = prof_read(L, PROF_PASS1)
+    sw_ms, sw_n = prof_read(L, PROF_SWEEP)
+    L.raw("sga_prof_enable", 0)
     # algorithmic bytes of this calendar (bf16 g read once per pass for the group)
-    alg = 0.0
+    alg = alg_p1 = alg_p3 = alg_sw = 0.0
     n_resel = 0
     for s in range(W):
-        alg += 2 * 2.0 * n                                   # g in pass 1 and pass 3
+        alg_p1 += 2.0 * n                                    # g in pass 1
+        alg_p3 += 2.0 * n                                    # g in pass 3
         for c in cfgs:
             bnd = s % c.T == 0
             rz = s == 0 or (s - 1) % c.T == 0                # res is all zeros: no traffic for it
-            alg += ((0.0 if rz else 4.0) if bnd else 0.125) * n  # pass 1: res | sel (1 bit)
+            alg_p1 += ((0.0 if rz else 4.0) if bnd else 0.125) * n  # pass 1: res | sel (1 bit)
             # pass 3: m, v, w read+write; res read unless zero, written unless it stays zero
-            alg += (24.0 + (0.0 if rz else 4.0) + (0.0 if (bnd and rz) else 4.0)
-                    + (0.0 if bnd else 0.125)) * n
+            alg_p3 += (24.0 + (0.0 if rz else 4.0) + (0.0 if (bnd and rz) else 4.0)
+                       + (0.0 if bnd else 0.125)) * n
             if bnd and s > 0 and s + 1 < W:
-                per = (6.0 if c.score == "abs_g" else 18.0) - (4.0 if rz else 0.0)
-                alg += (per + 0.125) * n                     # one score sweep + the new mask bits
+                per = (6.0 if c.score in ("abs_g", "abs_g_blind") else 18.0) - (4.0 if rz else 0.0)
+                alg_sw += (per + 0.125) * n                  # one score sweep + the new mask bits
                 n_resel += 1
+    alg = alg_p1 + alg_p3 + alg_sw
+    kernels = {}
+    for name, ms, cnt, b in (("k_replay_pass3", p3_ms, p3_n, alg_p3),
+                             ("k_replay_pass1 (launches of one step)", p1_ms, p1_n, alg_p1),
+                             ("k_bracket_sweep<SrcReplay>", sw_ms, sw_n, alg_sw)):
+        if cnt:
+            kernels[name] = {"launches": cnt, "total_ms": ms, "avg_ms": ms / cnt, "alg_bytes": b,
+                             "frac": b / (ms * 1e-3) / HBM_PEAK if ms > 0 else None}
     return {"metric": "replay config-steps/s", "value": G * W / dt, "unit": "config-steps/s",
             "ms_per_window": dt * 1e3, "G": G, "W": W, "n": n, "reselects": n_resel,
             "configs": [list(p) for p in picks],
             "alg_bytes": alg, "achieved_GBps": alg / dt / 1e9, "frac": alg / dt / HBM_PEAK,
+            "roofline": {"bound": "hbm", "kernel": "k_replay_pass3",
+                         "achieved": alg_p3 / (p3_ms * 1e-3) / 1e9 if p3_ms > 0 else None,
+                         "peak": HBM_PEAK / 1e9, "unit": "GB/s",
+                         "frac": alg_p3 / (p3_ms * 1e-3) / HBM_PEAK if p3_ms > 0 else None,
+                         "avg_ms": p3_ms / max(p3_n, 1), "traffic": None},
+            "kernels": kernels,
             "workload": "Qwen3-0.6B shapes (596,049,920 elems, 310 tensors), bf16 Student-t(3) "
                         "window, per-config fp32 w/m/v/res + u8 mask resident, clip 1.0"}
 
@@ -327,22 +366,158 @@ def trace_io_bench(W=4, tmp=None):
         shutil.rmtree(d, ignore_errors=True)
 
 
+def qwen_mask_layout_row(steps=5, warmup=2):
+    """Qwen3-0.6B-shaped set, bf16 Gaussian grads with per-tensor std
+    log-uniform in [1e-5, 1e-2], per-bucket exact top-k at 1 % (the embedding,
+    then seven buckets of four layers), mask backend layout: the step's outputs
+    are the uint8 mask and the ordered payload (what `torch_pipelined_mask`
+    hands to the all-reduce), fp32 values."""
+    import torch
+    from sga_amd.fused_step import FusedSparseStep, k_for
+    from sga_amd.shapes import qwen3_06b, segments_for
+    dev = torch.device("cuda:0")
+    segs, n = segments_for(qwen3_06b())
+    gen = torch.Generator(device=dev).manual_seed(5)
+    cpu_gen = torch.Generator().manual_seed(5)
+    grads = []
+    for rep in range(2):
+        g = torch.empty(n, dtype=torch.bfloat16, device=dev)
+        for s in segs:
+            std = 10 ** (-5 + 3 * float(torch.rand(1, generator=cpu_gen)))
+            g[s["start"]:s["start"] + s["n"]] = (
+                torch.randn(s["n"], generator=gen, device=dev) * std).to(torch.bfloat16)
+        grads.append(g)
+    cuts = [0, segs[1]["start"]] + [segs[1 + 11 * j]["start"] for j in range(4, 28, 4)] + [n]
+    p = torch.randn(n, generator=gen, device=dev) * 0.02
+    m, v, r = (torch.zeros(n, device=dev) for _ in range(3))
+    buckets = []
+    for lo, hi in zip(cuts[:-1], cuts[1:]):
+        bsegs = [dict(s, start=s["start"] - lo) for s in segs if lo <= s["start"] < hi]
+        k = k_for(hi - lo, 1.0)
+        buckets.append((lo, hi, k, FusedSparseStep(hi - lo, bsegs, dev, values_dtype=torch.float32,
+                                                   max_k=k, want_mask=True)))
+
+    def one(t):
+        g = grads[t % 2]
+        for lo, hi, k, fs in buckets:
+            fs.step(g[lo:hi], r[lo:hi], p[lo:hi], m[lo:hi], v[lo:hi], t + 1, k=k)
+
+    for t in range(warmup):
+        one(t)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for t in range(warmup, warmup + steps):
+        one(t)
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / steps
+    for lo, hi, k, fs in buckets:
+        res = fs.read_result()
+        assert res.status == 0 and res.n_selected == k, vars(res)
+    ktot = sum(b[2] for b in buckets)
+    alg = n * (step_bytes_per_elem("abs_g") + 1.0) + ktot * 8.0       # + u8 mask, idx + fp32 payload
+    return {"workload": "Qwen3-0.6B-shaped set (596,049,920 elems, 310 tensors), bf16 Gaussian grads "
+                        "with per-tensor std log-uniform in [1e-5, 1e-2], per-bucket exact top-k 1 % "
+                        f"over {len(buckets)} buckets, score abs_g, mask layout (u8 mask + ordered "
+                        "fp32 payload), four flat state tensors",
+            "n": n, "buckets": len(buckets), "k_total": ktot, "ms_per_step": dt * 1e3,
+            "elem_per_s": n / dt, "alg_bytes_per_step": alg,
+            "step_frac": alg / dt / HBM_PEAK}
+
+
+def stress_row(steps=3):
+    """One contiguous 1.0e9-element fp32 gradient buffer, heavy-tailed with
+    5 % duplicated magnitudes: the exact global top-k alone at 0.01 % and 1 %
+    (mask out), then the fused residual-aware AdamW step at 1 % (fp32 grads,
+    index pack int32 + fp32)."""
+    import torch
+    from sga_amd.fused_step import FusedSparseStep, k_for
+    from sga_amd.replay import select_topk_flat
+    dev = torch.device("cuda:0")
+    n = 1_000_000_000
+    g = student_t_dev(n, 7, dev).float()
+    gen = torch.Generator(device=dev).manual_seed(1)
+    dup = torch.randint(0, n, (n // 20,), generator=gen, device=dev)
+    g[dup] = g[dup.roll(1)]
+    del dup
+    score = g.abs()
+    sel = {}
+    for ratio in (0.01, 1.0):
+        k = k_for(n, ratio)
+        select_topk_flat(score, k, check=False)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            mask, th = select_topk_flat(score, k, check=False)
+        torch.cuda.synchronize()
+        dt = (time.perf_counter() - t0) / steps
+        assert int(mask.sum()) == k
+        sel[str(ratio)] = {"k": k, "ms": dt * 1e3, "elem_per_s": n / dt,
+                           "frac": n * (4.0 + 0.125 + 1.0) / dt / HBM_PEAK}
+        del mask
+    del score
+    segs = [dict(start=0, n=n, lr=1e-4, b1=0.9, b2=0.95, eps=1e-8, wd=0.1)]
+    p = torch.randn(n, generator=gen, device=dev) * 0.02
+    m, v, r = (torch.zeros(n, device=dev) for _ in range(3))
+    k = k_for(n, 1.0)
+    fs = FusedSparseStep(n, segs, dev, values_dtype=torch.float32, max_k=k)
+    fs.step(g, r, p, m, v, 1, k=k)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for t in range(steps):
+        fs.step(g, r, p, m, v, t + 2, k=k)
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / steps
+    res = fs.read_result()
+    assert res.status == 0 and res.n_selected == k, vars(res)
+    alg = n * step_bytes_per_elem("abs_g", 4.0) + k * 8.0
+    return {"workload": "one contiguous 1.0e9-element fp32 buffer, Student-t(3) with 5 % duplicated "
+                        "magnitudes; select_topk_flat alone (mask out; bytes = 4 read + 1/8 bit planes "
+                        "+ 1 mask) and the fused step at 1 % (fp32 grads, idx int32 + fp32 values)",
+            "n": n, "select_only": sel,
+            "fused_step": {"k": k, "ms_per_step": dt * 1e3, "elem_per_s": n / dt,
+                           "alg_bytes_per_step": alg, "step_frac": alg / dt / HBM_PEAK,
+                           "path": res.path}}
+
+
+def load_traffic(layout, score, ratio):
+    """HBM bytes per launch of the final sweep from the committed counter
+    profile -- only when that profile was taken on this very configuration."""
+    tpath = os.path.join(ROOT, "profiles", "fused_final_llama1b_traffic.json")
+    try:
+        entries = json.load(open(tpath))
+    except Exception:
+        return None, None
+    if isinstance(entries, dict):
+        entries = [entries]
+    for e in entries:
+        c = e.get("config", {})
+        if (c.get("layout"), c.get("score"), c.get("ratio_percent")) == (layout, score, ratio):
+            return e.get("hbm_bytes_per_launch"), "profiles/fused_final_llama1b_traffic.json"
+    return None, None
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--ratio", type=float, default=1.0)
-    ap.add_argument("--score", default="abs_g")
-    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--cpu-sample", type=int, default=1 << 29)
+    ap.add_argument("--score", default="update",
+                    help="headline score: update (the Adam-normalised score of the benchmark "
+                         "configuration) or abs_g (|g + residual|)")
+    ap.add_argument("--layout", choices=("separate", "packed"), default="separate",
+                    help="headline state layout: separate = the drop-in entry point on four flat "
+                         "tensors; packed = the library-owned 64 KiB records")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
+    ap.add_argument("--cpu-sample", type=int, default=1 << 28)
     ap.add_argument("--calib", action="store_true",
-                    help="also launch one plain copy of 2^30 fp32 (k_calib_copy) so counter "
-                         "runs can be scaled against a kernel of known traffic")
+                    help="also launch one plain copy of 2^30 fp32 (k_calib_copy) and the math-free "
+                         "stream stand-in so counter runs can be scaled against known traffic")
     ap.add_argument("--no-replay", action="store_true", help="skip the fused replay leg")
-    ap.add_argument("--layout", choices=("both", "packed", "separate"), default="both",
-                    help="state layout(s) to time; the headline is the packed layout unless "
-                         "only the separate one runs")
+    ap.add_argument("--no-sweep", action="store_true",
+                    help="time only the headline configuration of the fused step")
+    ap.add_argument("--no-rows", action="store_true",
+                    help="skip the Qwen3-0.6B mask-layout row and the 1e9 stress row")
     ap.add_argument("--trace-io", action="store_true",
                     help="run just the recorded-trace leg (writes a temporary trace, streams it "
                          "back through the pread reader and the dense pass) and print its JSON")
@@ -350,8 +525,6 @@ def main():
                     help="time the drop-in primitives on their own and print their JSON")
     ap.add_argument("--only-replay", action="store_true",
                     help="run just the fused replay leg (for profiling) and print its JSON")
-    ap.add_argument("--sweep", action="store_true",
-                    help="also time ratios 0.1/1/10 % and the update score")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs one data-parallel rank's share on ONE GPU; "
@@ -360,7 +533,7 @@ def main():
 
     import torch
     from sga_amd import _lib as L
-    from sga_amd.fused_step import FusedSparseStep, k_for
+    from sga_amd.fused_step import FusedSparseStep, PackedState, k_for
     from sga_amd.shapes import llama32_1b, segments_for
 
     L.load()
@@ -418,67 +591,76 @@ def main():
         calib["streams"] = {"kernel": "k_calib_streams", "bytes": n * 34, "avg_ms": ms,
                             "GBps": n * 34 / ms / 1e6}
         del sg, sc
-    k = k_for(n, args.ratio)
-    final_bytes = n * ALG_BYTES_FINAL + k * 6.0
 
-    def time_leg(step_fn, step0):
-        """W warm-up + K timed steps of one layout; returns (seconds, final-sweep ms)."""
-        for s in range(args.warmup):
-            step_fn(step0 + s)
+    state = {"t": 0, "packed": None}
+
+    def time_leg(layout, score, ratio, warmup, steps):
+        """`warmup` untimed + exactly `steps` timed steps of one configuration."""
+        k = k_for(n, ratio)
+        if layout == "packed" and state["packed"] is None:
+            state["packed"] = PackedState(n, dev).pack(r, p, m, v)
+
+        def step_fn(t):
+            if layout == "packed":
+                fs.step_packed(grads[t % 2], state["packed"], t + 1, k=k, score=score)
+            else:
+                fs.step(grads[t % 2], r, p, m, v, t + 1, k=k, score=score)
+        for _ in range(warmup):
+            step_fn(state["t"])
+            state["t"] += 1
         torch.cuda.synchronize()
         L.raw("sga_prof_enable", 1)
         t0 = time.perf_counter()
-        for s in range(args.steps):
-            step_fn(step0 + args.warmup + s)
+        for _ in range(steps):
+            step_fn(state["t"])
+            state["t"] += 1
         torch.cuda.synchronize()
         dt = time.perf_counter() - t0
-        tot_ms, cnt = ctypes.c_double(0), ctypes.c_int(0)
-        L.call("sga_prof_read", ctypes.byref(tot_ms), ctypes.byref(cnt))
+        fin_ms, fin_n = prof_read(L, PROF_FINAL)
+        sw_ms, sw_n = prof_read(L, PROF_SWEEP)
         L.raw("sga_prof_enable", 0)
         res = fs.read_result()
         assert res.status == 0 and res.n_selected == k, vars(res)
-        return dt, tot_ms.value / max(cnt.value, 1), res
+        final_bytes = n * ALG_BYTES_FINAL + k * 6.0
+        sweep_bytes = n * sweep_bytes_per_elem(score)
+        step_bytes = n * step_bytes_per_elem(score) + k * 6.0
+        fin_avg, sw_avg = fin_ms / max(fin_n, 1), sw_ms / max(sw_n, 1)
+        return {"layout": layout, "score": score, "ratio_percent": ratio, "k": k, "steps": steps,
+                "seconds": dt, "ms_per_step": dt / steps * 1e3, "elem_per_s": n * steps / dt,
+                "alg_bytes_per_elem": step_bytes_per_elem(score),
+                "alg_bytes_per_step": step_bytes,
+                "step_frac": step_bytes * steps / dt / HBM_PEAK,
+                "final_avg_ms": fin_avg, "final_bytes": final_bytes,
+                "final_frac": final_bytes / (fin_avg * 1e-3) / HBM_PEAK if fin_avg > 0 else None,
+                "sweep_avg_ms": sw_avg, "sweep_bytes": sweep_bytes,
+                "sweep_frac": sweep_bytes / (sw_avg * 1e-3) / HBM_PEAK if sw_avg > 0 else None,
+                "select": {"thresh": res.thresh, "n_gt": res.n_gt, "n_eq": res.n_eq,
+                           "path": res.path}}
 
-    def leg_summary(dt, final_ms):
-        return {"value": n * args.steps / dt, "ms_per_step": dt / args.steps * 1e3,
-                "step_frac": n * args.steps / dt * ALG_BYTES_STEP / HBM_PEAK,
-                "final_avg_ms": final_ms,
-                "final_frac": final_bytes / (final_ms * 1e-3) / HBM_PEAK}
-
-    legs, step0 = {}, 0
-    if args.layout in ("separate", "both"):
-        # the drop-in entry point: resid / p / m / v are the caller's four flat tensors
-        dt_s, ms_s, res = time_leg(
-            lambda t: fs.step(grads[t % 2], r, p, m, v, t + 1, k=k, score=args.score), step0)
-        legs["separate"] = (dt_s, ms_s)
-        step0 += args.warmup + args.steps
-    if args.layout in ("packed", "both"):
-        # the library-owned state layout: the same four arrays interleaved in 64 KiB
-        # records; identical arithmetic and outputs (asserted bitwise by the tests)
-        from sga_amd.fused_step import PackedState
-        st = PackedState(n, dev).pack(r, p, m, v)
-        dt_p, ms_p, res = time_leg(
-            lambda t: fs.step_packed(grads[t % 2], st, t + 1, k=k, score=args.score), step0)
-        legs["packed"] = (dt_p, ms_p)
-        step0 += args.warmup + args.steps
-    head = "packed" if "packed" in legs else "separate"
-    dt, final_ms = legs[head]
-    achieved = final_bytes / (final_ms * 1e-3) if final_ms > 0 else 0.0
-    traffic = None
-    tpath = os.path.join(ROOT, "profiles", "fused_final_llama1b_traffic.json")
-    if os.path.exists(tpath):
-        try:
-            traffic = json.load(open(tpath)).get("hbm_bytes_per_launch")
-        except Exception:
-            traffic = None
-    value = n * args.steps / dt
+    head = time_leg(args.layout, args.score, args.ratio, args.warmup, args.steps)
+    sweep = []
+    if not args.no_sweep:
+        for layout in ("separate", "packed"):
+            for score in ("update", "abs_g"):
+                for ratio in (0.1, 1.0, 10.0):
+                    if (layout, score, ratio) == (args.layout, args.score, args.ratio):
+                        sweep.append(head)
+                    else:
+                        sweep.append(time_leg(layout, score, ratio, 1, 5))
+    if state["packed"] is not None:
+        state["packed"].unpack(r, p, m, v)
+        state["packed"] = None
+    traffic, traffic_src = load_traffic(args.layout, args.score, args.ratio)
+    k = head["k"]
+    value = n * args.steps / head["seconds"]
     layout_txt = ("resid/p/m/v interleaved in 64 KiB records (sga_fused_sparse_step_packed)"
-                  if head == "packed" else
-                  "resid/p/m/v as four flat tensors (sga_fused_sparse_step)")
+                  if args.layout == "packed" else
+                  "resid/p/m/v as the caller's four flat tensors (sga_fused_sparse_step, the "
+                  "drop-in entry point)")
     out = {
         "metric": "grad elems/s (score+top-k+resid AdamW)",
         "value": value, "unit": "elem/s", "n_gpus": 1, "steps": args.steps,
-        "warmup": args.warmup, "ms_per_step": dt / args.steps * 1e3,
+        "warmup": args.warmup, "ms_per_step": head["ms_per_step"],
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
         "config": {"workload": "Llama-3.2-1B-shaped set, 1,235,814,400 elems / 146 tensors, "
@@ -486,49 +668,36 @@ def main():
                                f"{args.score}, exact top-k {args.ratio}% (k={k}), index pack "
                                "int32+bf16, residual-aware AdamW; state layout: " + layout_txt,
                    "ratio_percent": args.ratio, "score": args.score, "k": k,
-                   "state_layout": head},
-        "roofline": {"bound": "hbm", "achieved": achieved / 1e9, "peak": HBM_PEAK / 1e9,
-                     "unit": "GB/s", "frac": achieved / HBM_PEAK, "traffic": traffic,
-                     "kernel": "k_fused_final", "avg_ms": final_ms,
-                     "alg_bytes_per_launch": final_bytes},
-        "step_roofline": {"alg_bytes_per_elem": ALG_BYTES_STEP,
-                          "achieved_GBps": value * ALG_BYTES_STEP / 1e9,
-                          "frac": value * ALG_BYTES_STEP / HBM_PEAK},
-        "select": {"thresh": res.thresh, "n_gt": res.n_gt, "n_eq": res.n_eq, "path": res.path},
-        "layouts": {name: leg_summary(*v) for name, v in legs.items()},
+                   "state_layout": args.layout, "grad_dtype": "bf16", "values_dtype": "bf16",
+                   "state_dtype": "f32", "arithmetic": "f32"},
+        "roofline": {"bound": "hbm", "achieved": head["final_bytes"] / (head["final_avg_ms"] * 1e-3) / 1e9,
+                     "peak": HBM_PEAK / 1e9, "unit": "GB/s", "frac": head["final_frac"],
+                     "traffic": traffic, "traffic_source": traffic_src,
+                     "kernel": "k_fused_final", "avg_ms": head["final_avg_ms"],
+                     "alg_bytes_per_launch": head["final_bytes"]},
+        "step_roofline": {"alg_bytes_per_elem": head["alg_bytes_per_elem"],
+                          "achieved_GBps": head["alg_bytes_per_step"] / (head["ms_per_step"] * 1e-3) / 1e9,
+                          "frac": head["step_frac"],
+                          "select_sweep": {"kernel": "k_bracket_sweep", "avg_ms": head["sweep_avg_ms"],
+                                           "alg_bytes_per_launch": head["sweep_bytes"],
+                                           "frac": head["sweep_frac"]}},
+        "select": head["select"],
+        "sweep": sweep,
     }
     if calib:
         out["copy_calibration"] = calib
-    if args.sweep:
-        sw = []
-        def run(steps, t0_, ratio, score):          # on the headline layout
-            kk = k_for(n, ratio)
-            for t in range(t0_, t0_ + steps):
-                if head == "packed":
-                    fs.step_packed(grads[t % 2], st, t + 1, k=kk, score=score)
-                else:
-                    fs.step(grads[t % 2], r, p, m, v, t + 1, k=kk, score=score)
-        for score, ratio in (("abs_g", 0.1), ("abs_g", 10.0), ("update", 0.1),
-                             ("update", 1.0), ("update", 10.0)):
-            run(1, step0, ratio, score)
-            torch.cuda.synchronize()
-            t1 = time.perf_counter()
-            run(3, step0 + 1, ratio, score)
-            torch.cuda.synchronize()
-            d = (time.perf_counter() - t1) / 3
-            step0 += 4
-            sw.append({"score": score, "ratio_percent": ratio, "elem_per_s": n / d,
-                       "ms_per_step": d * 1e3})
-        out["sweep"] = sw
-    if head == "packed":
-        st.unpack(r, p, m, v)
-        del st
-    if not args.no_replay:
-        del p, m, v, r, grads, fs
+    del p, m, v, r, grads, fs
+    torch.cuda.empty_cache()
+    if not args.no_rows:
+        out["qwen06b_mask_layout"] = qwen_mask_layout_row()
         torch.cuda.empty_cache()
+        out["stress_1e9"] = stress_row()
+        torch.cuda.empty_cache()
+    if not args.no_replay:
         out["replay"] = replay_bench()
+        torch.cuda.empty_cache()
     if not args.no_cpu:
-        out["cpu_baseline"] = cpu_baseline(args.cpu_sample, 3, args.ratio)
+        out["cpu_baseline"] = cpu_baseline(args.cpu_sample, 3, args.ratio, args.score)
         if "replay" in out:
             out["replay"]["cpu_baseline"] = replay_cpu_baseline()
     else:

@@ -298,12 +298,17 @@ int sga_gt_eq(const float* score, int64_t n, float thresh, uint8_t* gt,
 /* ---- score formulas and replay commit (sga/replay_kernels.py) ----------- */
 
 /* formula(name): out = score(w,m,v,g); absolute != 0 stores |score|.
- * scores.py:147-269 / replay_kernels.py:109-160.  adams != 0 substitutes
- * v := m*m and bc := 1 (replay.py:486-505). */
+ * scores.py:147-269 / replay_kernels.py:109-160.  flags: SGA_SF_ADAMS
+ * substitutes v := m*m and bc := 1 (replay.py:486-505); SGA_SF_NO_WD leaves
+ * the wd*w term of `update` out altogether (update_includes_wd=False,
+ * scores.py:227-230: the score is then U(g) itself, also for -0 and for
+ * non-finite w). */
+#define SGA_SF_ADAMS 1
+#define SGA_SF_NO_WD 2
 int sga_score_formula(int score_id, const float* w, const float* m,
                       const float* v, const float* g, float* out, int64_t n,
                       float beta1, float om1, float beta2, float om2, float wd,
-                      float bc1, float bc2, float eps, int absolute, int adams,
+                      float bc1, float bc2, float eps, int absolute, int flags,
                       void* stream);
 
 /* Branch-point score of the replay front select (replay_fused.py:1236-1265):
@@ -461,23 +466,6 @@ int sga_div_inplace(float* x, int64_t n, float d, int packed, void* stream);
  * inside a packed state; b is always flat. */
 int sga_sq_dist(const float* a, int a_packed, const float* b, int64_t n,
                 double* partials, double* out, void* stream);
-
-/* Live timing of the fused step's final sweep with HIP events recorded on the
- * launch stream (no counterpart in the reference; used by the benchmark).
- * enable(1) resets and arms up to 512 launches; read() waits for the recorded
- * events and returns their summed duration in ms and their number. */
-int sga_prof_enable(int on);
-/* dst[0..n) = src[0..n), fp32, n % 4 == 0: plain copy of known size used to
- * calibrate the HBM traffic counters (no counterpart in the reference). */
-int sga_calib_copy(float* dst, const float* src, int64_t n, void* stream);
-
-/* Math-free kernel with the fused final sweep's stream structure (reads bf16
- * g and fp32 r/p/m/v, rewrites r/p/m/v: 34 B per element), to measure what that
- * mix of streams reaches on the device (no counterpart in the reference).
- * Overwrites r/p/m/v with meaningless values: use scratch buffers. */
-int sga_calib_streams(const void* g_bf16, float* r, float* p, float* m, float* v,
-                      int64_t n, void* stream);
-int sga_prof_read(double* total_ms, int* launches);
 
 #ifdef __cplusplus
 }

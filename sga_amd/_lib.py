@@ -85,7 +85,7 @@ SIGNATURES = {
     "sga_calib_copy": (I32, [P, P, I64, P]),
     "sga_calib_streams": (I32, [P, P, P, P, P, I64, P]),
     "sga_prof_enable": (I32, [I32]),
-    "sga_prof_read": (I32, [P, P]),
+    "sga_prof_read": (I32, [I32, P, P]),
     "sga_fused_workspace_bytes": (SZ, [I64]),
     "sga_fused_sparse_step": (I32, [P, I32, P, P, P, P, I64, I64, P, I32, I32, P, P,
                                     I32, P, F, F, I32, P, P, SZ, P]),

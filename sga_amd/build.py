@@ -14,7 +14,8 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libsga_hip.so")
 SOURCES = ["runtime.hip", "scan.hip", "elementwise.hip", "adamw.hip",
-           "select.hip", "fused_step.hip", "replay.hip", "replay_group.hip"]
+           "select.hip", "fused_step.hip", "replay.hip", "replay_group.hip",
+           "bench_hooks.hip"]
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
          "-ffp-contract=off", "-fno-fast-math",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",

@@ -29,6 +29,16 @@ static_assert(kPackRun % kChunk == 0 && kChunk == 1024, "a chunk never straddles
 void set_error(const char* fmt, ...);
 int check_launch(const char* what);
 
+// Benchmark timing hook (bench_hooks.hip): when armed through sga_prof_enable, brackets a launch
+// with two HIP events on its stream; a single relaxed load and a null return otherwise.
+struct ProfPair { hipEvent_t a, b; int tag; int closed; };
+ProfPair* prof_begin(int tag, hipStream_t s);
+void prof_end(ProfPair* pp, hipStream_t s);
+constexpr int SGA_PROF_FUSED_FINAL = 0;   // k_fused_final
+constexpr int SGA_PROF_SELECT_SWEEP = 1;  // k_bracket_sweep (any key source)
+constexpr int SGA_PROF_REPLAY_PASS3 = 2;  // k_replay_pass3
+constexpr int SGA_PROF_REPLAY_PASS1 = 3;  // k_replay_pass1 launches of one step
+
 __host__ __device__ static inline int64_t cdiv64(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
 // Grid for streaming kernels that loop grid-stride: enough workgroups to fill

@@ -19,43 +19,6 @@ __global__ __launch_bounds__(kBlock) void k_scatter(float* __restrict__ dst,
   }
 }
 
-// Plain 128-bit copy of known size: the yardstick the HBM traffic counters
-// and the achievable streaming bandwidth are calibrated against.
-__global__ __launch_bounds__(kBlock) void k_calib_copy(float* __restrict__ dst,
-                                                       const float* __restrict__ src,
-                                                       int64_t n4) {
-  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n4;
-       i += (int64_t)gridDim.x * kBlock)
-    reinterpret_cast<F4*>(dst)[i] = reinterpret_cast<const F4*>(src)[i];
-}
-
-// Math-free stand-in with the final sweep's stream structure (reads bf16 g
-// and fp32 r, p, m, v; writes r, p, m, v; 34 B per element): what this mix of
-// five read and four write streams can reach, as opposed to a plain copy.
-__global__ __launch_bounds__(kBlock) void k_calib_streams(const uint16_t* __restrict__ g,
-                                                          float* __restrict__ r,
-                                                          float* __restrict__ p,
-                                                          float* __restrict__ m,
-                                                          float* __restrict__ v, int64_t n) {
-  const int64_t i = ((int64_t)blockIdx.x * kBlock + threadIdx.x) * kVec;
-  if (i + kVec > n) return;
-  const H4 gh = ldh4_nt(g + i);
-  F4 rr = ld4_nt(r + i), pp = ld4_nt(p + i), mm = ld4_nt(m + i), vv = ld4_nt(v + i);
-  const float gf[4] = {bf16_to_f32(gh.x), bf16_to_f32(gh.y), bf16_to_f32(gh.z), bf16_to_f32(gh.w)};
-  float* rp = &rr.x; float* ppp = &pp.x; float* mp = &mm.x; float* vp = &vv.x;
-#pragma unroll
-  for (int e = 0; e < 4; ++e) {
-    rp[e] += gf[e];
-    mp[e] = mp[e] * 0.5f + rp[e];
-    vp[e] = vp[e] * 0.5f + rp[e] * rp[e];
-    ppp[e] -= mp[e] * 0.5f;
-  }
-  st4_nt(r + i, rr);
-  st4_nt(p + i, pp);
-  st4_nt(m + i, mm);
-  st4_nt(v + i, vv);
-}
-
 // ------------------------------------------------------------------- pack
 template <bool BF16, bool SCALE>
 __global__ __launch_bounds__(kBlock) void k_pack(float* __restrict__ grad,
@@ -298,31 +261,6 @@ extern "C" int sga_scatter_selected(float* dst, const int32_t* idx,
   hipLaunchKernelGGL(k_scatter, dim3(stream_grid(k, kBlock)), dim3(kBlock), 0,
                      (hipStream_t)stream, dst, idx, src, k, n_dst);
   return check_launch("sga_scatter_selected");
-}
-
-extern "C" int sga_calib_copy(float* dst, const float* src, int64_t n, void* stream) {
-  if (!dst || !src || n < 0 || (n & 3) || !aligned4(dst, 4) || !aligned4(src, 4)) {
-    set_error("sga_calib_copy: needs 16-byte aligned buffers and n %% 4 == 0");
-    return SGA_ERR_ARG;
-  }
-  if (n == 0) return SGA_OK;
-  hipLaunchKernelGGL(k_calib_copy, dim3(stream_grid(n / 4, kBlock, 1 << 20)), dim3(kBlock), 0,
-                     (hipStream_t)stream, dst, src, n / 4);
-  return check_launch("sga_calib_copy");
-}
-
-extern "C" int sga_calib_streams(const void* g_bf16, float* r, float* p, float* m, float* v,
-                                 int64_t n, void* stream) {
-  if (!g_bf16 || !r || !p || !m || !v || n < 0 || (n & 3) || !aligned4(g_bf16, 2) ||
-      !aligned4(r, 4) || !aligned4(p, 4) || !aligned4(m, 4) || !aligned4(v, 4)) {
-    set_error("sga_calib_streams: needs aligned buffers and n a multiple of 4");
-    return SGA_ERR_ARG;
-  }
-  if (n == 0) return SGA_OK;
-  hipLaunchKernelGGL(k_calib_streams, dim3((unsigned)cdiv64(n, (int64_t)kBlock * kVec)),
-                     dim3(kBlock), 0, (hipStream_t)stream,
-                     reinterpret_cast<const uint16_t*>(g_bf16), r, p, m, v, n);
-  return check_launch("sga_calib_streams");
 }
 
 extern "C" int sga_pack_selected(float* grad, const int32_t* idx, void* values,

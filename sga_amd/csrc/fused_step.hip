@@ -287,23 +287,6 @@ __global__ __launch_bounds__(kBlock) void k_fused_final(
   }
 }
 
-// Optional live timing of the final sweep (HIP events on the launch stream),
-// switched on by sga_prof_enable; read back with sga_prof_read after a sync.
-struct ProfPair { hipEvent_t a, b; };
-static bool g_prof_on = false;
-static ProfPair g_prof[512];
-static int g_prof_made = 0, g_prof_used = 0;
-
-static ProfPair* prof_next() {
-  if (!g_prof_on || g_prof_used >= 512) return nullptr;
-  if (g_prof_used >= g_prof_made) {
-    if (hipEventCreate(&g_prof[g_prof_made].a) != hipSuccess) return nullptr;
-    if (hipEventCreate(&g_prof[g_prof_made].b) != hipSuccess) return nullptr;
-    ++g_prof_made;
-  }
-  return &g_prof[g_prof_used++];
-}
-
 template <bool BF16G, bool BF16V, int SCORE>
 static int run_fused(const void* g, float* resid, float* p, float* m, float* v, int64_t n,
                      int64_t k, const sga_segment* segs, int n_segs, int32_t* idx_out,
@@ -316,8 +299,7 @@ static int run_fused(const void* g, float* resid, float* p, float* m, float* v, 
   src.sc.init(segs, n_segs);
   run_select(src, n, k, 0, fast != 0, w, s);
   const int64_t n_tiles = cdiv64(n, kChunk);
-  ProfPair* pp = prof_next();
-  if (pp) (void)hipEventRecord(pp->a, s);
+  ProfPair* pp = prof_begin(SGA_PROF_FUSED_FINAL, s);
   FinalArgs fa;
   fa.g = g; fa.r = resid; fa.p = p; fa.m = m; fa.v = v; fa.n = n; fa.k = k;
   fa.idx_out = idx_out; fa.values_out = values_out; fa.mask_out = mask_out;
@@ -328,7 +310,7 @@ static int run_fused(const void* g, float* resid, float* p, float* m, float* v, 
   hipLaunchKernelGGL((k_fused_final<BF16G, BF16V, SCORE>),
                      dim3(stream_grid(n_tiles, kChunksPerBlock, 1 << 20)), dim3(kBlock), 0, s, fa,
                      segs, n_segs, w.st, w.tile_gt, w.tile_eq);
-  if (pp) (void)hipEventRecord(pp->b, s);
+  prof_end(pp, s);
   if (result) hipLaunchKernelGGL(k_sel_result, dim3(1), dim3(1), 0, s, w.st, result);
   return check_launch("sga_fused_sparse_step");
 }
@@ -336,31 +318,6 @@ static int run_fused(const void* g, float* resid, float* p, float* m, float* v, 
 }  // namespace sga
 
 using namespace sga;
-
-extern "C" int sga_prof_enable(int on) {
-  g_prof_on = on != 0;
-  g_prof_used = 0;
-  return SGA_OK;
-}
-
-extern "C" int sga_prof_read(double* total_ms, int* launches) {
-  if (!total_ms || !launches) { set_error("sga_prof_read: null output"); return SGA_ERR_ARG; }
-  double tot = 0.0;
-  int cnt = 0;
-  for (int i = 0; i < g_prof_used; ++i) {
-    float ms = 0.0f;
-    if (hipEventSynchronize(g_prof[i].b) != hipSuccess ||
-        hipEventElapsedTime(&ms, g_prof[i].a, g_prof[i].b) != hipSuccess) {
-      set_error("sga_prof_read: event %d not ready", i);
-      return SGA_ERR_LAUNCH;
-    }
-    tot += ms;
-    ++cnt;
-  }
-  *total_ms = tot;
-  *launches = cnt;
-  return SGA_OK;
-}
 
 extern "C" size_t sga_fused_workspace_bytes(int64_t n) { return sel_ws_bytes(n < 0 ? 0 : n); }
 

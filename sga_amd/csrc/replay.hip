@@ -16,7 +16,8 @@ template <int SCORE, bool FULL>
 __device__ __forceinline__ void score_vec(const float* __restrict__ w, const float* __restrict__ m,
                                           const float* __restrict__ v, const float* __restrict__ g,
                                           float* __restrict__ out, int64_t i, int64_t n,
-                                          const Hyper& h, bool absolute, bool adams, bool vec) {
+                                          const Hyper& h, bool absolute, bool adams, bool no_wd,
+                                          bool vec) {
   float ww[4] = {0, 0, 0, 0}, mm[4] = {0, 0, 0, 0}, vv[4] = {0, 0, 0, 0}, gg[4] = {0, 0, 0, 0};
   if (SCORE != SGA_SCORE_ABS_M) ld_f32<FULL>(g, i, n, gg, vec);
   if (SCORE != SGA_SCORE_ABS_G) ld_f32<FULL>(m, i, n, mm, vec);
@@ -28,7 +29,9 @@ __device__ __forceinline__ void score_vec(const float* __restrict__ w, const flo
 #pragma unroll
   for (int e = 0; e < 4; ++e) {
     const float ve = adams ? mm[e] * mm[e] : vv[e];
-    const float s = score_value<SCORE>(gg[e], ww[e], mm[e], ve, h);
+    float s;
+    if (SCORE == SGA_SCORE_UPDATE && no_wd) s = adamw_commit(ww[e], gg[e], mm[e], ve, h).u;   // U(g) alone
+    else s = score_value<SCORE>(gg[e], ww[e], mm[e], ve, h);
     o[e] = absolute ? fabsf(s) : s;
   }
   st_f32<FULL>(out, i, n, o, vec);
@@ -38,14 +41,14 @@ template <int SCORE>
 __global__ __launch_bounds__(kBlock) void k_score_formula(
     const float* __restrict__ w, const float* __restrict__ m, const float* __restrict__ v,
     const float* __restrict__ g, float* __restrict__ out, int64_t n, Hyper h, bool absolute,
-    bool adams, bool vec) {
+    bool adams, bool no_wd, bool vec) {
   const int64_t stride = (int64_t)gridDim.x * kBlock * kVec;
   for (int64_t base = (int64_t)blockIdx.x * kBlock * kVec; base < n; base += stride) {
     const int64_t i = base + (int64_t)threadIdx.x * kVec;
     if (vec && base + kBlock * kVec <= n)
-      score_vec<SCORE, true>(w, m, v, g, out, i, n, h, absolute, adams, true);
+      score_vec<SCORE, true>(w, m, v, g, out, i, n, h, absolute, adams, no_wd, true);
     else if (i < n)
-      score_vec<SCORE, false>(w, m, v, g, out, i, n, h, absolute, adams, vec);
+      score_vec<SCORE, false>(w, m, v, g, out, i, n, h, absolute, adams, no_wd, vec);
   }
 }
 
@@ -162,7 +165,9 @@ using namespace sga;
 extern "C" int sga_score_formula(int score_id, const float* w, const float* m, const float* v,
                                  const float* g, float* out, int64_t n, float beta1, float om1,
                                  float beta2, float om2, float wd, float bc1, float bc2,
-                                 float eps, int absolute, int adams, void* stream) {
+                                 float eps, int absolute, int flags, void* stream) {
+  const int adams = flags & SGA_SF_ADAMS;
+  const bool no_wd = (flags & SGA_SF_NO_WD) != 0;
   if (n == 0) return SGA_OK;
   if (!out || n < 0 || score_id < 0 || score_id > 3) {
     set_error("sga_score_formula: bad argument (score_id=%d)", score_id);
@@ -180,7 +185,7 @@ extern "C" int sga_score_formula(int score_id, const float* w, const float* m, c
                    aligned4(out, 4);
   dim3 grid(stream_grid(n, (int64_t)kBlock * kVec, 1 << 22)), block(kBlock);
   hipStream_t st = (hipStream_t)stream;
-#define SGA_SF(S) hipLaunchKernelGGL((k_score_formula<S>), grid, block, 0, st, w, m, v, g, out, n, h, absolute != 0, adams != 0, vec)
+#define SGA_SF(S) hipLaunchKernelGGL((k_score_formula<S>), grid, block, 0, st, w, m, v, g, out, n, h, absolute != 0, adams != 0, no_wd, vec)
   switch (score_id) {
     case 0: SGA_SF(0); break;
     case 1: SGA_SF(1); break;

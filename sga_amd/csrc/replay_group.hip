@@ -606,8 +606,10 @@ extern "C" int sga_replay_pass1(const void* g, int g_dtype, int64_t n, float coe
     }
   }
   for (int c = G; c < kMaxCfg; ++c) al.src[c] = 0;
+  ProfPair* pp = prof_begin(SGA_PROF_REPLAY_PASS1, s);
   launch_pass1<true>(bg, n_b, nb, s, g, n, coef_dense, lb, partials, vec, grp.pack_extra);
   launch_pass1<false>(bg, n_m, nb, s, g, n, coef_dense, lm, partials, vec, 0);
+  prof_end(pp, s);
   hipLaunchKernelGGL(k_replay_coef, dim3(1), dim3(kBlock), 0, s, partials, (int)nb, G, clip, qn2, coef_d, coef_f, al);
   return check_launch("sga_replay_pass1");
 }
@@ -626,8 +628,10 @@ extern "C" int sga_replay_pass3(const void* g, int g_dtype, int64_t n, float coe
   const unsigned nb = stream_grid(n, (int64_t)kBlock * kVec, 1 << 22);   // one-shot: nothing to reduce
   hipStream_t s = (hipStream_t)stream;
   const RSeg* rs = reinterpret_cast<const RSeg*>(segs);
+  ProfPair* pp = prof_begin(SGA_PROF_REPLAY_PASS3, s);
   if (bg) hipLaunchKernelGGL((k_replay_pass3<true>), dim3(nb), dim3(kBlock), 0, s, g, n, coef_dense, grp, coef_f, rs, n_segs, vec);
   else hipLaunchKernelGGL((k_replay_pass3<false>), dim3(nb), dim3(kBlock), 0, s, g, n, coef_dense, grp, coef_f, rs, n_segs, vec);
+  prof_end(pp, s);
   return check_launch("sga_replay_pass3");
 }
 

@@ -6,6 +6,7 @@
 // per-chunk count so that ties at the threshold can be granted in ascending
 // index order without any float compare ambiguity.
 #pragma once
+#include <atomic>
 #include <type_traits>
 #include "common.hpp"
 
@@ -1123,11 +1124,15 @@ static __global__ __launch_bounds__(kBlock) void k_mask_to_planes(const uint8_t*
 // chip).
 template <class Src, bool PM>
 static inline int sweep_grid() {
-  static int blocks = 0;
+  constexpr int kMaxDev = 64;
+  static std::atomic<int> cache[kMaxDev];     // per device; 0 = not asked yet
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDev) dev = -1;
+  int blocks = dev >= 0 ? cache[dev].load(std::memory_order_relaxed) : 0;
   if (blocks == 0) {
-    int per_cu = 0, dev = 0;
+    int per_cu = 0;
     hipDeviceProp_t prop;
-    if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess &&
+    if (dev >= 0 && hipGetDeviceProperties(&prop, dev) == hipSuccess &&
         hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, k_bracket_sweep<Src, PM>, kBlock, 0) ==
             hipSuccess && per_cu > 0) {
       blocks = per_cu * prop.multiProcessorCount;
@@ -1135,6 +1140,7 @@ static inline int sweep_grid() {
       blocks = 1024;
     }
     if (blocks > kSegWaves / kChunksPerBlock) blocks = kSegWaves / kChunksPerBlock;
+    if (dev >= 0) cache[dev].store(blocks, std::memory_order_relaxed);
   }
   return blocks;
 }
@@ -1163,6 +1169,7 @@ static inline void run_select(Src src, int64_t n, int64_t k, int tie_all, bool f
     for (int level = 0; level < 3; ++level)
       launch_level<SrcU32, 2, true>(ssrc, ns, (const uint32_t*)nullptr, level, w.aux, w, s, kRawKeyBlocks);
     const int sweep_blocks = want_mask ? sweep_grid<Src, true>() : sweep_grid<Src, false>();
+    ProfPair* pp = prof_begin(SGA_PROF_SELECT_SWEEP, s);
     if (want_mask)
       hipLaunchKernelGGL((k_bracket_sweep<Src, true>), dim3(sweep_blocks), dim3(kBlock), 0, s,
                          src, n, w.st, w.aux, w.tile_gt, w.tile_eq, w.seg_idx, w.seg_key, w.seg_cnt,
@@ -1171,6 +1178,7 @@ static inline void run_select(Src src, int64_t n, int64_t k, int tie_all, bool f
       hipLaunchKernelGGL((k_bracket_sweep<Src, false>), dim3(sweep_blocks), dim3(kBlock), 0, s,
                          src, n, w.st, w.aux, w.tile_gt, w.tile_eq, w.seg_idx, w.seg_key, w.seg_cnt,
                          (uint32_t)w.seg_cap, (uint32_t*)nullptr);
+    prof_end(pp, s);
     hipLaunchKernelGGL(k_bracket_check, dim3(1), dim3(kBlock), 0, s, w.st, w.aux, w.seg_cnt, w.hist,
                        kHistStride * 2, sweep_blocks * kChunksPerBlock);
     hipLaunchKernelGGL(k_cand_compact, dim3(256), dim3(kBlock), 0, s, w.aux, w.seg_cnt, w.seg_idx,

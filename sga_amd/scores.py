@@ -44,11 +44,11 @@ def device_formula(score_id, w, m, v, g, b1, b2, eps, wd, bc1, bc2, absolute=Fal
             L.require_contig(t=t)
     if out is None:
         out = torch.empty(n, dtype=torch.float32, device=ref.device)
-    wdv = wd if update_includes_wd else 0.0
+    flags = (1 if optimizer == "adams" else 0) | (0 if update_includes_wd else 2)   # SGA_SF_*
     L.call("sga_score_formula", score_id, L.ptr(flat[0]), L.ptr(flat[1]), L.ptr(flat[2]),
            L.ptr(flat[3]), L.ptr(out), n, L.f32(b1), L.f32(1.0 - b1), L.f32(b2),
-           L.f32(1.0 - b2), L.f32(wdv), L.f32(bc1), L.f32(bc2), L.f32(eps),
-           1 if absolute else 0, 1 if optimizer == "adams" else 0, L.stream())
+           L.f32(1.0 - b2), L.f32(wd), L.f32(bc1), L.f32(bc2), L.f32(eps),
+           1 if absolute else 0, flags, L.stream())
     return out.view(shape)
 
 

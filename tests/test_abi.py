@@ -12,7 +12,8 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
 def _declared():
-    txt = open(os.path.join(ROOT, "include", "sga_hip.h")).read()
+    txt = (open(os.path.join(ROOT, "include", "sga_hip.h")).read()
+           + open(os.path.join(ROOT, "include", "sga_hip_bench.h")).read())
     txt = re.sub(r"/\*.*?\*/", "", txt, flags=re.S)
     return sorted(set(re.findall(r"\b(sga_[a-z0-9_]+)\s*\(", txt)))
 

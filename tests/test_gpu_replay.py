@@ -44,6 +44,24 @@ def test_score_formulas(dev, name, opt):
 
 
 @pytest.mark.parametrize("opt", ["adamw", "adams"])
+def test_update_without_weight_decay_term(dev, opt):
+    """update_includes_wd=False returns U(g) itself (scores.py:227-230), not
+    0*w + U(g): lanes whose w is Inf / NaN or whose U is -0 keep U's bits."""
+    from sga_amd.replay import score_formula
+    b1, b2, eps, wd, step = 0.9, 0.95, 1e-8, 1e-2, 7
+    bc1, bc2 = 1 - b1 ** step, 1 - b2 ** step
+    w, m, v, g = _state(10_007, 5)
+    w[:4] = torch.tensor([float("inf"), float("-inf"), float("nan"), -1.0])
+    m[4:8] = torch.tensor([-0.0, 0.0, -0.0, 0.0])
+    g[4:8] = torch.tensor([-0.0, -0.0, 0.0, 0.0])              # U = -0 / +0 lanes
+    ref = OS.score_formula("update", w, m, v, g, b1, b2, eps, wd, bc1, bc2, opt,
+                           update_includes_wd=False)
+    got = score_formula("update", *(t.to(dev) for t in (w, m, v, g)), b1, b2, eps, wd, bc1, bc2,
+                        opt, update_includes_wd=False)
+    assert bool(torch.isfinite(ref[:4]).all()) and same_bits(got, ref)
+
+
+@pytest.mark.parametrize("opt", ["adamw", "adams"])
 @pytest.mark.parametrize("lr,wd,count", [(1e-3, .01, 7), (3e-4, .01, 1), (1e-3, 0.0, 100)])
 def test_opt_step_inplace(dev, opt, lr, wd, count):
     from sga_amd import replay_kernels as K

@@ -494,3 +494,65 @@ def test_ieee_sqrt_is_correctly_rounded():
     assert ieee.sqrt(torch.tensor([0.0, float("inf")])).tolist() == [0.0, float("inf")]
     # and the reason it exists: the tensor library's own routine is not that
     # (informational, never asserted): torch.sqrt may differ from it.
+
+
+def test_torch_sqrt_deviation_is_bounded(monkeypatch):
+    """The oracle's one deliberate departure from a literal torch-CPU run of
+    the reference: square roots come from oracle.ieee (correctly rounded), the
+    reference calls torch.sqrt (scores.py:216-226, replay.py:695-705), which on
+    the CPU is a vector-library routine that may be one ulp off.  This test
+    runs every chain that holds a square root both ways on config-1-sized
+    inputs (2^22 Student-t gradients, p ~ N(0, 0.02)) and bounds the gap:
+    p / w / scores agree within the 1e-6 the parity bar allows (relative to the
+    operands of the final subtraction), m and v do not depend on the root at
+    all, and the top-k sets by `update` / `coi` differ by a handful of
+    threshold neighbours at most."""
+    from oracle import ieee
+    from tests.util import rel_close, student_t, sub_scale
+    n = 1 << 22
+    gen = torch.Generator().manual_seed(0)
+    p0 = torch.randn(n, generator=gen) * 0.02
+    m0 = torch.randn(n, generator=gen) * 1e-4
+    v0 = torch.rand(n, generator=gen) * 1e-8
+    g = student_t(n, 1)
+    b1, b2, eps, wd, lr, step = 0.9, 0.95, 1e-8, 0.1, 1e-4, 3
+    bc1, bc2 = 1 - b1 ** step, 1 - b2 ** step
+    k = SEL.k_for(n, 1.0)
+
+    def run_all():
+        out = {}
+        for name in ("update", "coi"):
+            out[name] = S.score_formula(name, p0, m0, v0, g, b1, b2, eps, wd, bc1, bc2, "adamw",
+                                        update_includes_wd=True)
+            out[name + "_sel"] = SEL.select_topk_flat(out[name].abs(), k)[0]
+        p, gg, m, v = p0.clone(), g.clone(), m0.clone(), v0.clone()
+        A.grad_correct(p, gg, m, v, lr, b1, b2, eps, wd, bc1, bc2, None, "update")
+        out.update(gc_p=p, gc_m=m, gc_v=v, gc_score=gg)
+        w, m, v = p0.clone(), m0.clone(), v0.clone()
+        R.opt_step_inplace(g, m, v, w, None, lr, wd, b1, b2, bc1, bc2, eps)
+        out.update(rp_w=w, rp_m=m, rp_v=v)
+        return out
+
+    exact = run_all()
+    monkeypatch.setattr(ieee, "sqrt", torch.sqrt)
+    literal = run_all()
+    monkeypatch.undo()
+    lanes = int((exact["update"] != literal["update"]).sum())
+    for key in ("gc_m", "gc_v", "rp_m", "rp_v"):                 # no square root upstream
+        assert torch.equal(exact[key], literal[key]), key
+    for key in ("gc_p", "rp_w"):
+        bad, worst = rel_close(exact[key], literal[key], rtol=1e-6,
+                               scale=sub_scale(p0, exact[key]))
+        assert bad == 0, (key, bad, worst)
+    for key in ("update", "coi", "gc_score"):
+        # one ulp of the root moves U by at most ~2 ulp (one for the root, one for the quotient's
+        # rounding): 2^-22 relative to |U|, the larger operand of wd*w + U and of U(g) - U(0)
+        bad, worst = rel_close(exact[key], literal[key], rtol=1e-6,
+                               scale=exact["update"] - wd * p0)
+        assert bad == 0, (key, bad, worst)
+    moved = {}
+    for name in ("update", "coi"):
+        moved[name] = int((exact[name + "_sel"] ^ literal[name + "_sel"]).sum())
+        assert moved[name] <= max(16, k // 1000), (name, moved[name], k)
+    print(f"torch.sqrt vs correctly rounded sqrt at n=2^22: {lanes} score lanes differ in the "
+          f"last bits; top-{k} sets differ by {moved} coordinates (symmetric difference)")
