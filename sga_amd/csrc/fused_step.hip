@@ -34,11 +34,21 @@ struct SrcFused {
   static constexpr bool kHyper = SCORE == SGA_SCORE_UPDATE || SCORE == SGA_SCORE_COI;
   // measured: the |g + r| sweep is bound by DRAM and loses ~5 % with more slabs in flight; the
   // Adam-normalised scores are bound by arithmetic and gain from hiding the load latency
-  static constexpr int kAhead = kHyper ? 2 : 1;
+  #ifndef SGA_AHEAD_ABSG
+#define SGA_AHEAD_ABSG 1
+#endif
+#ifndef SGA_AHEAD_HYPER
+#define SGA_AHEAD_HYPER 2
+#endif
+  static constexpr int kAhead = kHyper ? SGA_AHEAD_HYPER : SGA_AHEAD_ABSG;
   __device__ __forceinline__ Chunk chunk_begin(int64_t c) {
     const int64_t i0 = uniform_i64(c) * kChunk;
-    if (kHyper) sc.seek_uniform(i0);
     return Chunk{(i0 >> kPackRunLog) * pack_extra};
+  }
+  // The tensor of the chunk's first element: a search over the segment table, placed by the
+  // sweep behind the chunk's first loads so that their latencies overlap.
+  __device__ __forceinline__ void chunk_hyper(int64_t c) {
+    if (kHyper) sc.seek_uniform(uniform_i64(c) * kChunk);
   }
   template <bool FULL>
   __device__ __forceinline__ void fetch(const Chunk& ck, int64_t i, int64_t n, Raw& w) {
@@ -126,6 +136,7 @@ struct FinalArgs {
   uint32_t T, need;
   bool vec, mvec, scale, apply_coeff;
   int64_t pack_extra;
+  const uint32_t* planes;   // the settled selection as bit planes (PLANES mode), else unused
 };
 
 // One 1024-element chunk of the final sweep, owned by one wave.  FULL: the
@@ -133,9 +144,12 @@ struct FinalArgs {
 // loads are unconditional and issued before the first use.
 // IT0 / NIT: the slabs [IT0, IT0+NIT) of the chunk are handled by this call;
 // `cur` carries the running selected / tie counts across calls.
-template <bool BF16G, bool BF16V, int SCORE, bool FULL, int IT0, int NIT>
+// PLANES: the selection was already settled as bit planes (bracket sweep +
+// candidates): the slab's four 64-bit ballots are read on the scalar unit and
+// the keys are not formed again; SCORE is then irrelevant.
+template <bool BF16G, bool BF16V, int SCORE, bool FULL, int IT0, int NIT, bool PLANES>
 __device__ __forceinline__ void final_chunk(const FinalArgs& a, int64_t c, ChunkCursor& cur,
-                                            SegCursor& sc) {
+                                            SegCursor& sc, SegCursor& lc) {
   const int64_t n = a.n;
   const int64_t sh = pack_shift<true>(c << 10, a.pack_extra);     // c is wave-uniform
   float* const R = a.r + sh;
@@ -193,53 +207,92 @@ __device__ __forceinline__ void final_chunk(const FinalArgs& a, int64_t c, Chunk
   for (int it = IT0; it < IT0 + NIT; ++it) {
     const int64_t i = c * kChunk + it * (kWave * kVec) + lane_id() * kVec;
     float q[4];
-    uint32_t key[4];
     bool valid[4], sel[4];
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      valid[e] = FULL || i + e < n;
-      q[e] = rr[it][e] + gg[it][e];
-      if (SCORE == SGA_SCORE_ABS_G) key[e] = abs_key(q[e]);
-      else if (SCORE == SGA_SCORE_ABS_M) key[e] = abs_key(mm[it][e]);
-      else {
-        if (valid[e]) sc.seek(i + e);
-        key[e] = valid[e] ? score_key<SCORE>(q[e], pp[it][e], mm[it][e], vv[it][e], sc.h) : 0u;
-      }
-    }
     uint32_t pos;
-    slab_select(key, valid, a.T, a.need, cur, sel, pos);
+    if (PLANES) {
+      // words 2e, 2e + 1 of the slab are the ballot of element e over the 64 lanes; lanes are in
+      // index order, so the selected coordinates before (lane, e) are the mask bits below the
+      // lane over all four ballots plus the lane's own earlier elements
+      const uint64_t* pw = reinterpret_cast<const uint64_t*>(a.planes) + (uniform_i64(c) * kChunkIters + it) * 4;
+      uint32_t below = 0, total = 0;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const uint64_t mk = pw[e];
+        valid[e] = FULL || i + e < n;
+        q[e] = rr[it][e] + gg[it][e];
+        sel[e] = __builtin_amdgcn_inverse_ballot_w64(mk);
+        below += lanes_below(mk);
+        total += (uint32_t)__popcll(mk);
+      }
+      pos = cur.sel_run + below;
+      cur.sel_run += total;
+    } else {
+      uint32_t key[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        valid[e] = FULL || i + e < n;
+        q[e] = rr[it][e] + gg[it][e];
+        if (SCORE == SGA_SCORE_ABS_G) key[e] = abs_key(q[e]);
+        else if (SCORE == SGA_SCORE_ABS_M) key[e] = abs_key(mm[it][e]);
+        else {
+          // only when the one-sweep select is off or failed: a per-lane cursor
+          if (valid[e]) lc.seek(i + e);
+          key[e] = valid[e] ? score_key<SCORE>(q[e], pp[it][e], mm[it][e], vv[it][e], lc.h) : 0u;
+        }
+      }
+      slab_select(key, valid, a.T, a.need, cur, sel, pos);
+    }
     if (FULL || i < n) {
       uint32_t mk[4];
+      float ge[4];
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         mk[e] = sel[e];
-        if (!valid[e]) continue;
-        sc.seek(i + e);
-        float ge = 0.0f;
-        if (sel[e]) {
-          float val = q[e];
-          if (a.scale) val = val * a.factor;
-          if (BF16V) {
-            const uint16_t hb = f32_to_bf16(val);
-            if ((int64_t)pos < a.k) {
-              a.idx_out[pos] = (int32_t)(i + e);
-              reinterpret_cast<uint16_t*>(a.values_out)[pos] = hb;
-            }
-            ge = bf16_to_f32(hb);
-          } else {
-            if ((int64_t)pos < a.k) {
-              a.idx_out[pos] = (int32_t)(i + e);
-              reinterpret_cast<float*>(a.values_out)[pos] = val;
-            }
-            ge = val;
+        ge[e] = 0.0f;
+        if (!valid[e] || !sel[e]) continue;
+        float val = q[e];
+        if (a.scale) val = val * a.factor;
+        if (BF16V) {
+          const uint16_t hb = f32_to_bf16(val);
+          if ((int64_t)pos < a.k) {
+            a.idx_out[pos] = (int32_t)(i + e);
+            reinterpret_cast<uint16_t*>(a.values_out)[pos] = hb;
           }
-          ++pos;
-          if (a.apply_coeff) ge = ge * a.coeff;
+          ge[e] = bf16_to_f32(hb);
+        } else {
+          if ((int64_t)pos < a.k) {
+            a.idx_out[pos] = (int32_t)(i + e);
+            reinterpret_cast<float*>(a.values_out)[pos] = val;
+          }
+          ge[e] = val;
         }
-        const Commit cm = adamw_commit(pp[it][e], ge, mm[it][e], vv[it][e], sc.h);
-        pp[it][e] = pp[it][e] - sc.h.lr * cm.upd;
-        mm[it][e] = cm.m_new;
-        vv[it][e] = cm.v_new;
+        ++pos;
+        if (a.apply_coeff) ge[e] = ge[e] * a.coeff;
+      }
+      // The commit takes its hyper-parameters from the scalar unit: the slab lies inside one
+      // tensor but for the few that hold a boundary, which are committed once per tensor piece.
+      const int64_t s0 = uniform_i64(c) * kChunk + it * (kWave * kVec);
+      int64_t s1 = s0 + kWave * kVec;
+      if (!FULL && s1 > n) s1 = n;
+      if (s0 < sc.lo || s0 >= sc.hi) sc.seek_uniform(s0);
+      float pn[4], mn[4], vn[4];
+      for (;;) {
+        const bool whole = sc.lo <= s0 && sc.hi >= s1;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const Commit cm = adamw_commit(pp[it][e], ge[e], mm[it][e], vv[it][e], sc.h);
+          const float pe = pp[it][e] - sc.h.lr * cm.upd;
+          if (whole || (i + e >= sc.lo && i + e < sc.hi)) { pn[e] = pe; mn[e] = cm.m_new; vn[e] = cm.v_new; }
+        }
+        const int64_t nxt = sc.hi;
+        if (whole || nxt >= s1) break;
+        sc.advance_uniform(nxt);
+        if (sc.hi <= nxt) break;              // the table does not tile [0, n): stop
+      }
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        if (!valid[e]) continue;
+        pp[it][e] = pn[e]; mm[it][e] = mn[e]; vv[it][e] = vn[e];
         rr[it][e] = sel[e] ? 0.0f : q[e];
       }
       st_f32<FULL>(R, i, n, rr[it], a.vec);
@@ -252,37 +305,44 @@ __device__ __forceinline__ void final_chunk(const FinalArgs& a, int64_t c, Chunk
 }
 
 // Final sweep: select flags in index order, pack, residual, commit.
-template <bool BF16G, bool BF16V, int SCORE>
-__global__ __launch_bounds__(kBlock) void k_fused_final(
+// `when`: 0 run always; 1 only if the sampled bracket held (the planes are
+// settled); 2 only if it failed (the radix passes fixed the threshold and the
+// keys are formed again here).
+// (five waves per SIMD wherever the key is not an Adam-normalised chain formed in this kernel)
+template <bool BF16G, bool BF16V, int SCORE, bool PLANES>
+__global__ __launch_bounds__(kBlock, (PLANES || SCORE == SGA_SCORE_ABS_G || SCORE == SGA_SCORE_ABS_M) ? 5 : 1)
+void k_fused_final(
     FinalArgs a, const sga_segment* __restrict__ segs, int n_segs,
     const SelState* __restrict__ st, const uint32_t* __restrict__ tile_sel,
-    const uint32_t* __restrict__ tile_eq) {
+    const uint32_t* __restrict__ tile_eq, int when) {
+  if (when != 0 && (st->bracket_ok != 0) != (when == 1)) return;
   a.T = st->thresh_bits;
   a.need = st->need;
   const int64_t n_chunks = cdiv64(a.n, kChunk);
   const int64_t wstride = (int64_t)gridDim.x * kChunksPerBlock;
-  SegCursor sc;
+  SegCursor sc, lc;              // sc: wave-uniform (scalar unit); lc: per lane, key forming only
   sc.init(segs, n_segs);
+  lc.init(segs, n_segs);
   const bool can_full = a.vec && (a.mask_out == nullptr || a.mvec);
   for (int64_t c = (int64_t)blockIdx.x * kChunksPerBlock + wave_id(); c < n_chunks;
        c += wstride) {
     ChunkCursor cur;
     cur.sel_run = tile_sel[c];
-    cur.eq_run = tile_eq[c];
+    cur.eq_run = PLANES ? 0u : tile_eq[c];
     if (can_full && (c + 1) * kChunk <= a.n) {
       // one 256-element slab at a time (5 loads in flight per lane): measured
       // as fast as batching all four slabs, at twice the occupancy
-      final_chunk<BF16G, BF16V, SCORE, true, 0, 1>(a, c, cur, sc);
-      final_chunk<BF16G, BF16V, SCORE, true, 1, 1>(a, c, cur, sc);
-      final_chunk<BF16G, BF16V, SCORE, true, 2, 1>(a, c, cur, sc);
-      final_chunk<BF16G, BF16V, SCORE, true, 3, 1>(a, c, cur, sc);
+      final_chunk<BF16G, BF16V, SCORE, true, 0, 1, PLANES>(a, c, cur, sc, lc);
+      final_chunk<BF16G, BF16V, SCORE, true, 1, 1, PLANES>(a, c, cur, sc, lc);
+      final_chunk<BF16G, BF16V, SCORE, true, 2, 1, PLANES>(a, c, cur, sc, lc);
+      final_chunk<BF16G, BF16V, SCORE, true, 3, 1, PLANES>(a, c, cur, sc, lc);
     } else {
       // the ragged path too: holding four slabs at once would set the register count (and so
       // the occupancy) of the whole kernel
-      final_chunk<BF16G, BF16V, SCORE, false, 0, 1>(a, c, cur, sc);
-      final_chunk<BF16G, BF16V, SCORE, false, 1, 1>(a, c, cur, sc);
-      final_chunk<BF16G, BF16V, SCORE, false, 2, 1>(a, c, cur, sc);
-      final_chunk<BF16G, BF16V, SCORE, false, 3, 1>(a, c, cur, sc);
+      final_chunk<BF16G, BF16V, SCORE, false, 0, 1, PLANES>(a, c, cur, sc, lc);
+      final_chunk<BF16G, BF16V, SCORE, false, 1, 1, PLANES>(a, c, cur, sc, lc);
+      final_chunk<BF16G, BF16V, SCORE, false, 2, 1, PLANES>(a, c, cur, sc, lc);
+      final_chunk<BF16G, BF16V, SCORE, false, 3, 1, PLANES>(a, c, cur, sc, lc);
     }
   }
 }
@@ -297,8 +357,17 @@ static int run_fused(const void* g, float* resid, float* p, float* m, float* v, 
                    aligned4(m, 4) && aligned4(v, 4);
   SrcFused<BF16G, SCORE> src{g, resid, p, m, v, vec, {}, pack_extra};
   src.sc.init(segs, n_segs);
-  run_select(src, n, k, 0, fast != 0, w, s);
+  // Adam-normalised scores with the one-sweep select armed: the sweep leaves the selection as bit
+  // planes (settled by the candidates) and the final sweep reads one bit per coordinate instead of
+  // evaluating the score chain a second time; if the bracket fails on the device, the key-forming
+  // final sweep runs instead.  For |g + r| and |m| the key is one instruction and re-forming it is
+  // cheaper than writing and reading the planes (measured: 0.3 ms per step at 1.2e9 elements).
+  const bool planes = SrcFused<BF16G, SCORE>::kHyper && fast != 0 && n >= kFastMinN && w.pbits != nullptr;
+  run_select(src, n, k, 0, fast != 0, w, s, planes ? w.pbits : nullptr);
   const int64_t n_tiles = cdiv64(n, kChunk);
+  if (planes)
+    hipLaunchKernelGGL(k_cand_bits, dim3(256), dim3(kBlock), 0, s, w.st, w.cand_idx, w.cand_key,
+                       w.tile_eq, n_tiles, 0, w.pbits);
   ProfPair* pp = prof_begin(SGA_PROF_FUSED_FINAL, s);
   FinalArgs fa;
   fa.g = g; fa.r = resid; fa.p = p; fa.m = m; fa.v = v; fa.n = n; fa.k = k;
@@ -307,9 +376,19 @@ static int run_fused(const void* g, float* resid, float* p, float* m, float* v, 
   fa.vec = vec; fa.mvec = aligned4(mask_out, 1);
   fa.scale = factor != 1.0f; fa.apply_coeff = coeff != 1.0f;
   fa.pack_extra = pack_extra;
-  hipLaunchKernelGGL((k_fused_final<BF16G, BF16V, SCORE>),
-                     dim3(stream_grid(n_tiles, kChunksPerBlock, 1 << 20)), dim3(kBlock), 0, s, fa,
-                     segs, n_segs, w.st, w.tile_gt, w.tile_eq);
+  fa.planes = w.pbits;
+  const dim3 one_shot(stream_grid(n_tiles, kChunksPerBlock, 1 << 20));
+  if (planes) {
+    hipLaunchKernelGGL((k_fused_final<BF16G, BF16V, SGA_SCORE_ABS_G, true>), one_shot, dim3(kBlock), 0, s,
+                       fa, segs, n_segs, w.st, w.tile_gt, w.tile_eq, 1);
+    // the rare other outcome: a small grid that strides over the chunks (returns at once otherwise)
+    hipLaunchKernelGGL((k_fused_final<BF16G, BF16V, SCORE, false>),
+                       dim3(stream_grid(n_tiles, kChunksPerBlock, 2048)), dim3(kBlock), 0, s, fa,
+                       segs, n_segs, w.st, w.tile_gt, w.tile_eq, 2);
+  } else {
+    hipLaunchKernelGGL((k_fused_final<BF16G, BF16V, SCORE, false>), one_shot, dim3(kBlock), 0, s, fa,
+                       segs, n_segs, w.st, w.tile_gt, w.tile_eq, 0);
+  }
   prof_end(pp, s);
   if (result) hipLaunchKernelGGL(k_sel_result, dim3(1), dim3(1), 0, s, w.st, result);
   return check_launch("sga_fused_sparse_step");

@@ -362,8 +362,10 @@ struct SrcReplay {
   static constexpr int kAhead = kHyper ? 2 : kChunkIters;
   __device__ __forceinline__ Chunk chunk_begin(int64_t c) {
     const int64_t i0 = uniform_i64(c) * kChunk;
-    if (kHyper) sc.seek_uniform(i0);
     return Chunk{(i0 >> kPackRunLog) * pack_extra, uniform_f32(coef_f[0])};
+  }
+  __device__ __forceinline__ void chunk_hyper(int64_t c) {
+    if (kHyper) sc.seek_uniform(uniform_i64(c) * kChunk);
   }
   template <bool FULL>
   __device__ __forceinline__ void fetch(const Chunk& ck, int64_t i, int64_t n, Raw& t) {

@@ -68,7 +68,8 @@ struct SelWorkspace {
   int64_t seg_cap;     // per-wave candidate capacity
 };
 
-constexpr int kSegWaves = 8192;            // persistent waves of the bracket sweep
+constexpr int kSegWaves = 8192;            // candidate segments the sweep's chunks hash to
+constexpr int kSweepParts = 256;            // partial counters of the sweep's two totals
 constexpr int64_t kFastMinN = 1 << 20;     // below this the radix passes are cheap enough
 
 static inline int64_t fast_sample_vecs(int64_t n) {
@@ -177,6 +178,7 @@ struct SrcF32 {                 // |x| of an fp32 score array
   using Chunk = NoChunk;
   static constexpr int kAhead = kChunkIters;
   __device__ __forceinline__ Chunk chunk_begin(int64_t) { return Chunk{}; }
+  __device__ __forceinline__ void chunk_hyper(int64_t) {}
   template <bool FULL>
   __device__ __forceinline__ void fetch(const Chunk&, int64_t i, int64_t n, Raw& r) {
     r = ldraw_f32<FULL>(x, i, n, vec);
@@ -758,8 +760,11 @@ __global__ __launch_bounds__(kBlock) void k_sample(Src src, int64_t n, int64_t n
 // aux[0] descends to the upper end (smaller rank = larger key), aux[1] to the
 // lower end.  Also zeroes both histogram sets.
 static __global__ void k_bracket_ranks(SelState* aux, uint32_t* hist, int nhist, uint32_t k,
-                                       double n, double ns) {
+                                       double n, double ns, uint32_t* seg_cnt, uint32_t* hi_part,
+                                       uint32_t* nf_part) {
   for (int i = threadIdx.x; i < nhist; i += blockDim.x) hist[i] = 0u;
+  for (int i = threadIdx.x; i <= kSegWaves; i += blockDim.x) seg_cnt[i] = 0u;
+  for (int i = threadIdx.x; i < kSweepParts; i += blockDim.x) { hi_part[i] = 0u; nf_part[i] = 0u; }
   if (threadIdx.x != 0) return;
   const double frac = (double)k / n;
   const double r = frac * ns;
@@ -772,26 +777,78 @@ static __global__ void k_bracket_ranks(SelState* aux, uint32_t* hist, int nhist,
   aux[1] = lo;
 }
 
-// The one sweep over the data.  A persistent grid of kSegWaves waves; each
-// wave owns a private candidate segment, so no atomics are needed and the
-// candidates of a chunk stay in ascending index order.
+// The one sweep over the data: a one-shot grid, one 1024-element chunk per
+// wave (a capped grid that strides over the chunks reads 15 % slower).  The
+// keys inside the bracket are first gathered, in index order, in the wave's
+// LDS buffer; at the end of the chunk the wave reserves room for all of them
+// with ONE atomic add on the counter of the candidate segment its chunk
+// hashes to (kSegWaves counters, so neighbouring waves hit different
+// addresses) and copies them there.  A chunk's candidates therefore stay
+// contiguous and index-ordered in the list; the order of the chunks inside a
+// segment is arbitrary and nothing downstream depends on it.
+constexpr int kWaveCandCap = 256;          // candidates one chunk can hold before the sweep gives up
+
+// LDS of one wave of the sweep.
+struct SweepLds {
+  uint32_t idx[kWaveCandCap];              // the chunk's candidates, index order
+  uint32_t key[kWaveCandCap];
+  uint32_t planes[kPlaneWordsPerChunk];    // the chunk's 32 plane words ("key above the bracket")
+};
+
+// The flags of a slab live as four wave ballots (element e of every lane), i.e.
+// on the scalar unit: counts are popcounts, "any" is a scalar test, and the
+// index-ordered position of a flagged element is the number of mask bits
+// below its lane over the four ballots plus the lane's own earlier elements.
+struct Ballot4 {
+  uint64_t m[4];
+  __device__ __forceinline__ uint64_t any() const { return m[0] | m[1] | m[2] | m[3]; }
+  __device__ __forceinline__ uint32_t count() const {
+    return (uint32_t)(__popcll(m[0]) + __popcll(m[1]) + __popcll(m[2]) + __popcll(m[3]));
+  }
+  __device__ __forceinline__ uint32_t below_lane() const {
+    return lanes_below(m[0]) + lanes_below(m[1]) + lanes_below(m[2]) + lanes_below(m[3]);
+  }
+  __device__ __forceinline__ bool mine(int e) const { return (m[e] >> lane_id()) & 1ull; }
+};
+
+// Appends the flagged elements of one slab in index order: put(pos, e).
+template <class F>
+__device__ __forceinline__ void ballot_append(const Ballot4& f, uint32_t& count, F&& put) {
+  if (f.any() == 0) return;                      // scalar branch
+  uint32_t pos = count + f.below_lane();
+#pragma unroll
+  for (int e = 0; e < 4; ++e)
+    if (f.mine(e)) { put(pos, e); ++pos; }
+  count += f.count();
+}
+
+// The slab's four "above" ballots are eight of the chunk's 32 plane words
+// (words 8 it + 2 e + h): one lane parks them in the wave's LDS planes, from
+// where the chunk's 128 bytes are stored in one piece.
+__device__ __forceinline__ void plane_put(const Ballot4& a, int it, uint32_t* lds_planes) {
+  if (lane_id() == 0) {
+    uint64_t* w = reinterpret_cast<uint64_t*>(lds_planes) + it * 4;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) w[e] = a.m[e];
+  }
+}
+
+// One chunk of the sweep.  chi / tot_nf / mycnt are wave totals (scalar).
 template <class Src, bool FULL, bool PM>
 __device__ __forceinline__ void bracket_chunk(Src& src, const typename Src::Chunk& ck, int64_t n,
                                               int64_t c, uint32_t T_LO,
                                               uint32_t T_HI, uint32_t& chi, uint32_t& tot_nf,
-                                              uint32_t& mycnt, uint32_t seg_cap,
-                                              uint32_t* __restrict__ my_idx,
-                                              uint32_t* __restrict__ my_key,
+                                              uint32_t& mycnt, SweepLds& lds,
                                               uint32_t* __restrict__ pbits) {
   // The loads of kAhead slabs (256 elements each) are issued together, then
   // their keys are formed slab by slab: expensive key sources (Adam-normalised
-  // scores) look fewer slabs ahead to stay within the register budget of four
-  // workgroups per CU.  The ragged path (last chunk, unaligned views) goes one
-  // slab at a time through a rolled loop: it only has to be small.
-  uint32_t pword = 0u;
+  // scores) look fewer slabs ahead to stay within their register budget.  The
+  // ragged path (last chunk, unaligned views) goes one slab at a time through
+  // a rolled loop: it only has to be small.
   constexpr int kAhead = FULL ? Src::kAhead : 1;
   static_assert(kChunkIters % kAhead == 0, "look-ahead divides the slabs of a chunk");
   constexpr int kGroupUnroll = kAhead == kChunkIters ? kChunkIters : 1;
+  src.chunk_hyper(c);        // measured: looking the tensor up behind the first loads instead is slower
 #pragma unroll kGroupUnroll
   for (int g0 = 0; g0 < kChunkIters; g0 += kAhead) {
     typename Src::Raw raw[kAhead];
@@ -806,81 +863,86 @@ __device__ __forceinline__ void bracket_chunk(Src& src, const typename Src::Chun
       const int64_t i = c * kChunk + it * (kWave * kVec) + lane_id() * kVec;
       uint32_t key[4] = {0u, 0u, 0u, 0u};
       if (FULL || i < n) src.template keys<FULL>(ck, i, n, raw[u], key);
-      bool cand[4];
-      uint32_t mine = 0, above[4];
+      Ballot4 above, cand;
+      uint64_t nf = 0;
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        const bool valid = FULL || i + e < n;
-        above[e] = (valid && key[e] >= T_HI);
-        chi += above[e];
-        tot_nf += (valid && key[e] >= 0x7F800000u);
-        cand[e] = valid && key[e] >= T_LO && key[e] < T_HI;
-        mine += cand[e];
+        const uint64_t valid = FULL ? ~0ull : ballot64(i + e < n);
+        above.m[e] = ballot64(key[e] >= T_HI) & valid;
+        cand.m[e] = ballot64(key[e] >= T_LO) & valid & ~above.m[e];
+        nf |= ballot64(key[e] >= 0x7F800000u) & valid;
       }
-      if (PM) {
-        // provisional mask as bit planes: everything above the bracket is
-        // certainly selected; the few keys inside it are settled after the
-        // candidate descent.  One 128-byte store per chunk.
-        plane_collect(above, it, pword);
-      }
-      if (ballot64(mine != 0)) {
-        const uint32_t incl = wave_incl_scan(mine);
-        uint32_t pos = mycnt + incl - mine;
+      chi += above.count();
+      if (nf) {                                  // rare: count them properly
 #pragma unroll
         for (int e = 0; e < 4; ++e)
-          if (cand[e]) {
-            if (pos < seg_cap) { my_idx[pos] = (uint32_t)(i + e); my_key[pos] = key[e]; }
-            ++pos;
-          }
-        mycnt += __shfl(incl, kWave - 1, kWave);
+          tot_nf += (uint32_t)__popcll(ballot64(key[e] >= 0x7F800000u && (FULL || i + e < n)));
       }
+      ballot_append(cand, mycnt, [&](uint32_t pos, int e) {
+        if (pos < (uint32_t)kWaveCandCap) { lds.idx[pos] = (uint32_t)(i + e); lds.key[pos] = key[e]; }
+      });
+      // provisional mask as bit planes: everything above the bracket is
+      // certainly selected; the few keys inside it are settled after the
+      // candidate descent.  One 128-byte store per chunk.
+      if (PM) plane_put(above, it, lds.planes);
     }
   }
-  if (PM && lane_id() < 32) pbits[c * 32 + lane_id()] = pword;
+  if (PM) {
+    __builtin_amdgcn_wave_barrier();
+    if (lane_id() < kPlaneWordsPerChunk) pbits[c * kPlaneWordsPerChunk + lane_id()] = lds.planes[lane_id()];
+  }
 }
 
 template <class Src, bool PM>
-__global__ __launch_bounds__(kBlock, 4) void k_bracket_sweep(
+__global__ __launch_bounds__(kBlock) void k_bracket_sweep(
     Src src, int64_t n, SelState* __restrict__ st, const SelState* __restrict__ aux,
     uint32_t* __restrict__ tile_gt, uint32_t* __restrict__ tile_eq, uint32_t* __restrict__ seg_idx,
     uint32_t* __restrict__ seg_key, uint32_t* __restrict__ seg_cnt, uint32_t seg_cap,
-    uint32_t* __restrict__ pbits) {
+    uint32_t* __restrict__ pbits, uint32_t* __restrict__ hi_part, uint32_t* __restrict__ nf_part) {
   __shared__ uint32_t s_hi[kChunksPerBlock], s_nf[kChunksPerBlock];
+  __shared__ SweepLds s_lds[kChunksPerBlock];
   // keys equal to the upper sample key stay candidates; a skipped end means
   // the bracket is open on that side
   const uint32_t T_HI = aux[0].skip ? 0x80000000u : aux[0].thresh_bits + 1u;
   const uint32_t T_LO = aux[1].skip ? 0u : aux[1].thresh_bits;
   if (blockIdx.x == 0 && threadIdx.x == 0) { st->t_lo = T_LO; st->t_hi = T_HI; }
   const int64_t n_chunks = cdiv64(n, kChunk);
-  const int64_t gw = (int64_t)blockIdx.x * kChunksPerBlock + wave_id();
-  const int64_t W = (int64_t)gridDim.x * kChunksPerBlock;
-  uint32_t mycnt = 0, tot_hi = 0, tot_nf = 0;
-  uint32_t* my_idx = seg_idx + gw * seg_cap;
-  uint32_t* my_key = seg_key + gw * seg_cap;
-  for (int64_t c = gw; c < n_chunks; c += W) {
-    uint32_t chi = 0;
+  const int64_t c = (int64_t)blockIdx.x * kChunksPerBlock + wave_id();
+  uint32_t chi = 0, tot_nf = 0;
+  if (c < n_chunks) {
+    uint32_t mycnt = 0;
+    SweepLds& lds = s_lds[wave_id()];
+    uint32_t* const my_idx = lds.idx;
+    uint32_t* const my_key = lds.key;
     const typename Src::Chunk ck = src.chunk_begin(c);
     if (src.vec && (c + 1) * kChunk <= n)
-      bracket_chunk<Src, true, PM>(src, ck, n, c, T_LO, T_HI, chi, tot_nf, mycnt, seg_cap, my_idx, my_key, pbits);
+      bracket_chunk<Src, true, PM>(src, ck, n, c, T_LO, T_HI, chi, tot_nf, mycnt, lds, pbits);
     else
-      bracket_chunk<Src, false, PM>(src, ck, n, c, T_LO, T_HI, chi, tot_nf, mycnt, seg_cap, my_idx, my_key, pbits);
-    chi = wave_sum(chi);
-    tot_hi += chi;
-    if (lane_id() == 0) { tile_gt[c] = chi; tile_eq[c] = 0u; }
+      bracket_chunk<Src, false, PM>(src, ck, n, c, T_LO, T_HI, chi, tot_nf, mycnt, lds, pbits);
+    if (lane_id() == 0) { tile_gt[c] = chi; tile_eq[c] = 0u; }     // chi / tot_nf are wave totals
+    if (mycnt) {                                        // wave-uniform
+      const uint32_t seg = (uint32_t)c & (uint32_t)(kSegWaves - 1);
+      uint32_t base = 0;
+      if (lane_id() == 0) base = atomicAdd(&seg_cnt[seg], mycnt);   // a segment over its capacity is seen by the check
+      base = __shfl(base, 0, kWave);
+      if (mycnt > (uint32_t)kWaveCandCap) {
+        if (lane_id() == 0) atomicOr(&st->overflow, 1u);
+      } else {
+        __builtin_amdgcn_wave_barrier();                // the wave's LDS stores above are read below
+        uint32_t* const g_idx = seg_idx + (int64_t)seg * seg_cap;
+        uint32_t* const g_key = seg_key + (int64_t)seg * seg_cap;
+        for (uint32_t j = lane_id(); j < mycnt; j += kWave)
+          if (base + j < seg_cap) { g_idx[base + j] = my_idx[j]; g_key[base + j] = my_key[j]; }
+      }
+    }
   }
-  tot_nf = wave_sum(tot_nf);
-  if (lane_id() == 0) {
-    seg_cnt[gw] = mycnt < seg_cap ? mycnt : seg_cap;
-    s_hi[wave_id()] = tot_hi;
-    s_nf[wave_id()] = tot_nf;
-    if (mycnt > seg_cap) atomicOr(&st->overflow, 1u);
-  }
+  if (lane_id() == 0) { s_hi[wave_id()] = chi; s_nf[wave_id()] = tot_nf; }
   __syncthreads();
   if (threadIdx.x == 0) {
     const uint32_t h = s_hi[0] + s_hi[1] + s_hi[2] + s_hi[3];
     const uint32_t f = s_nf[0] + s_nf[1] + s_nf[2] + s_nf[3];
-    if (h) atomicAdd(&st->n_hi, h);
-    if (f) atomicAdd(&st->nonfinite, f);
+    if (h) atomicAdd(&hi_part[blockIdx.x & (kSweepParts - 1)], h);
+    if (f) atomicAdd(&nf_part[blockIdx.x & (kSweepParts - 1)], f);
   }
 }
 
@@ -890,14 +952,17 @@ static __global__ __launch_bounds__(kBlock) void k_bracket_check(SelState* __res
                                                                  SelState* __restrict__ aux,
                                                                  uint32_t* __restrict__ seg_cnt,
                                                                  uint32_t* __restrict__ hist, int nhist,
-                                                                 int n_waves) {
+                                                                 uint32_t seg_cap,
+                                                                 const uint32_t* __restrict__ hi_part,
+                                                                 const uint32_t* __restrict__ nf_part) {
   __shared__ uint32_t s_w4[kChunksPerBlock];
-  constexpr int PER = kSegWaves / kBlock;   // 16
-  uint32_t v[PER], mine = 0;
+  constexpr int PER = kSegWaves / kBlock;   // 32
+  uint32_t v[PER], mine = 0, over = 0;
 #pragma unroll
   for (int j = 0; j < PER; ++j) {
-    const int wv = threadIdx.x * PER + j;
-    v[j] = wv < n_waves ? seg_cnt[wv] : 0u;   // waves the sweep did not launch own nothing
+    const uint32_t cnt = seg_cnt[threadIdx.x * PER + j];
+    over |= cnt > seg_cap;                    // the sweep reserved more than the segment holds
+    v[j] = cnt < seg_cap ? cnt : seg_cap;
     mine += v[j];
   }
   uint32_t total;
@@ -905,15 +970,28 @@ static __global__ __launch_bounds__(kBlock) void k_bracket_check(SelState* __res
 #pragma unroll
   for (int j = 0; j < PER; ++j) { seg_cnt[threadIdx.x * PER + j] = run; run += v[j]; }
   for (int i = threadIdx.x; i < nhist; i += kBlock) hist[i] = 0u;
+  static_assert(kSweepParts == kBlock, "one partial counter per thread");
+  uint32_t dummy;
+  __syncthreads();
+  block_excl_scan(hi_part[threadIdx.x], s_w4, dummy);
+  const uint32_t n_hi = dummy;
+  __syncthreads();
+  block_excl_scan(nf_part[threadIdx.x], s_w4, dummy);
+  const uint32_t n_nf = dummy;
+  __syncthreads();
+  block_excl_scan(over, s_w4, dummy);
+  const bool any_over = dummy != 0;
   if (threadIdx.x == 0) {
     seg_cnt[kSegWaves] = total;
-    const uint32_t k = st->k, n_hi = st->n_hi;
-    const bool ok = !st->overflow && n_hi < k && k <= n_hi + total;
+    const uint32_t k = st->k;
+    const bool ok = !st->overflow && !any_over && n_hi < k && k <= n_hi + total;
+    st->n_hi = n_hi;
     st->cand_count = total;
     st->bracket_ok = ok ? 1u : 0u;
     st->skip = ok ? 1u : 0u;          // the radix passes run only when the bracket failed
     st->path = ok ? 1u : 0u;
-    if (!ok) { st->nonfinite = 0u; st->status = 0u; }   // recounted by the radix passes
+    st->nonfinite = ok ? n_nf : 0u;   // recounted by the radix passes otherwise
+    if (!ok) st->status = 0u;
     SelState z = {};
     z.k = ok ? k - n_hi : 0u;
     z.skip = ok ? 0u : 1u;
@@ -1119,32 +1197,6 @@ static __global__ __launch_bounds__(kBlock) void k_mask_to_planes(const uint8_t*
   }
 }
 
-// Persistent grid of the bracket sweep = exactly what the device holds at
-// once for THIS instantiation (a partial second round would idle most of the
-// chip).
-template <class Src, bool PM>
-static inline int sweep_grid() {
-  constexpr int kMaxDev = 64;
-  static std::atomic<int> cache[kMaxDev];     // per device; 0 = not asked yet
-  int dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDev) dev = -1;
-  int blocks = dev >= 0 ? cache[dev].load(std::memory_order_relaxed) : 0;
-  if (blocks == 0) {
-    int per_cu = 0;
-    hipDeviceProp_t prop;
-    if (dev >= 0 && hipGetDeviceProperties(&prop, dev) == hipSuccess &&
-        hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, k_bracket_sweep<Src, PM>, kBlock, 0) ==
-            hipSuccess && per_cu > 0) {
-      blocks = per_cu * prop.multiProcessorCount;
-    } else {
-      blocks = 1024;
-    }
-    if (blocks > kSegWaves / kChunksPerBlock) blocks = kSegWaves / kChunksPerBlock;
-    if (dev >= 0) cache[dev].store(blocks, std::memory_order_relaxed);
-  }
-  return blocks;
-}
-
 // planes (optional): the sweep also records there, as bit planes, which keys
 // lie above the bracket, so a caller that only wants the mask can finish from
 // those bits and the candidates (finish_mask / finish_planes) instead of
@@ -1163,24 +1215,26 @@ static inline void run_select(Src src, int64_t n, int64_t k, int tie_all, bool f
     const int64_t ns = n_sv * 4;
     hipLaunchKernelGGL((k_sample<Src>), dim3(stream_grid(n_sv, kBlock)), dim3(kBlock), 0, s, src, n,
                        n_sv, win, w.sample);
+    // the sweep's two totals go through 256 partial counters (blk_gt / blk_eq are free until the
+    // tile scan, which runs after the check has read them)
     hipLaunchKernelGGL(k_bracket_ranks, dim3(1), dim3(kBlock), 0, s, w.aux, w.hist, kHistStride * 2,
-                       (uint32_t)k, (double)n, (double)ns);
+                       (uint32_t)k, (double)n, (double)ns, w.seg_cnt, w.blk_gt, w.blk_eq);
     SrcU32 ssrc{w.sample};
     for (int level = 0; level < 3; ++level)
       launch_level<SrcU32, 2, true>(ssrc, ns, (const uint32_t*)nullptr, level, w.aux, w, s, kRawKeyBlocks);
-    const int sweep_blocks = want_mask ? sweep_grid<Src, true>() : sweep_grid<Src, false>();
+    const unsigned sweep_blocks = (unsigned)cdiv64(n_tiles, kChunksPerBlock);
     ProfPair* pp = prof_begin(SGA_PROF_SELECT_SWEEP, s);
     if (want_mask)
       hipLaunchKernelGGL((k_bracket_sweep<Src, true>), dim3(sweep_blocks), dim3(kBlock), 0, s,
                          src, n, w.st, w.aux, w.tile_gt, w.tile_eq, w.seg_idx, w.seg_key, w.seg_cnt,
-                         (uint32_t)w.seg_cap, planes);
+                         (uint32_t)w.seg_cap, planes, w.blk_gt, w.blk_eq);
     else
       hipLaunchKernelGGL((k_bracket_sweep<Src, false>), dim3(sweep_blocks), dim3(kBlock), 0, s,
                          src, n, w.st, w.aux, w.tile_gt, w.tile_eq, w.seg_idx, w.seg_key, w.seg_cnt,
-                         (uint32_t)w.seg_cap, (uint32_t*)nullptr);
+                         (uint32_t)w.seg_cap, (uint32_t*)nullptr, w.blk_gt, w.blk_eq);
     prof_end(pp, s);
     hipLaunchKernelGGL(k_bracket_check, dim3(1), dim3(kBlock), 0, s, w.st, w.aux, w.seg_cnt, w.hist,
-                       kHistStride * 2, sweep_blocks * kChunksPerBlock);
+                       kHistStride * 2, (uint32_t)w.seg_cap, w.blk_gt, w.blk_eq);
     hipLaunchKernelGGL(k_cand_compact, dim3(256), dim3(kBlock), 0, s, w.aux, w.seg_cnt, w.seg_idx,
                        w.seg_key, (uint32_t)w.seg_cap, w.cand_idx, w.cand_key);
     SrcU32 csrc{w.cand_key};
