@@ -64,23 +64,40 @@ __device__ __forceinline__ uint32_t score_key(float q, float p, float m, float v
   return abs_key(score_value<SCORE>(q, p, m, v, h));
 }
 
-// Segment cursor: segments tile [0, n) in ascending order.
+// Segment cursor: segments tile [0, n) in ascending order.  `dir` (optional)
+// is a directory over blocks of 2^kSegDirLog coordinates: dir[b] = segment
+// that holds coordinate b << kSegDirLog, from where a seek walks forward the
+// few tensors that start inside the block instead of bisecting the table.
+constexpr int kSegDirLog = 16;
+constexpr int kSegDirEntries = 1 << (31 - kSegDirLog);     // covers n < 2^31
 struct SegCursor {
   const sga_segment* segs;
+  const int32_t* dir;
   int n_segs;
   int64_t lo, hi;
   int at;                               // index of the cached segment (uniform seeks only)
   Hyper h;
-  __host__ __device__ __forceinline__ void init(const sga_segment* s, int ns) {
-    segs = s; n_segs = ns; lo = 1; hi = 0; at = 0;
+  __host__ __device__ __forceinline__ void init(const sga_segment* s, int ns,
+                                                const int32_t* d = nullptr) {
+    segs = s; dir = d; n_segs = ns; lo = 1; hi = 0; at = 0;
   }
-  __device__ __forceinline__ void seek(int64_t i) {
-    if (i >= lo && i < hi) return;
+  // last segment with start <= i
+  __device__ __forceinline__ int find(int64_t i) const {
+    if (dir) {
+      int a = dir[i >> kSegDirLog];
+      while (a + 1 < n_segs && segs[a + 1].start <= i) ++a;
+      return a;
+    }
     int a = 0, b = n_segs - 1;
-    while (a < b) {                      // last segment with start <= i
+    while (a < b) {
       const int mid = (a + b + 1) >> 1;
       if (segs[mid].start <= i) a = mid; else b = mid - 1;
     }
+    return a;
+  }
+  __device__ __forceinline__ void seek(int64_t i) {
+    if (i >= lo && i < hi) return;
+    const int a = find(i);
     lo = segs[a].start;
     hi = lo + segs[a].n;
     h = hyper_of(segs[a]);
@@ -98,10 +115,17 @@ struct SegCursor {
   }
   __device__ __forceinline__ void seek_uniform(int64_t i) {
     if (i >= lo && i < hi) return;
-    int a = 0, b = n_segs - 1;
-    while (a < b) {
-      const int mid = (a + b + 1) >> 1;
-      if (uniform_i64(segs[mid].start) <= i) a = mid; else b = mid - 1;
+    int a;
+    if (dir) {
+      a = uniform_i32(dir[i >> kSegDirLog]);
+      while (a + 1 < n_segs && uniform_i64(segs[a + 1].start) <= i) ++a;
+    } else {
+      a = 0;
+      int b = n_segs - 1;
+      while (a < b) {
+        const int mid = (a + b + 1) >> 1;
+        if (uniform_i64(segs[mid].start) <= i) a = mid; else b = mid - 1;
+      }
     }
     take_uniform(a);
   }
@@ -113,6 +137,27 @@ struct SegCursor {
     take_uniform(a);
   }
 };
+
+// Builds the directory of a segment table: dir[b] = last segment with start <= b << kSegDirLog.
+static __global__ __launch_bounds__(kBlock) void k_seg_dir(const sga_segment* __restrict__ segs,
+                                                           int n_segs, int64_t n,
+                                                           int32_t* __restrict__ dir) {
+  const int64_t nb = (n + (1ll << kSegDirLog) - 1) >> kSegDirLog;
+  for (int64_t b = (int64_t)blockIdx.x * kBlock + threadIdx.x; b < nb; b += (int64_t)gridDim.x * kBlock) {
+    const int64_t i = b << kSegDirLog;
+    int lo = 0, hi = n_segs - 1;
+    while (lo < hi) {
+      const int mid = (lo + hi + 1) >> 1;
+      if (segs[mid].start <= i) lo = mid; else hi = mid - 1;
+    }
+    dir[b] = lo;
+  }
+}
+static inline void launch_seg_dir(const sga_segment* segs, int n_segs, int64_t n, int32_t* dir,
+                                  hipStream_t s) {
+  const int64_t nb = (n + (1ll << kSegDirLog) - 1) >> kSegDirLog;
+  hipLaunchKernelGGL(k_seg_dir, dim3(stream_grid(nb, kBlock, 128)), dim3(kBlock), 0, s, segs, n_segs, n, dir);
+}
 
 // Keys of one slab of a chunk-structured sweep: lane l holds the quad at
 // i = s0 + 4 l of the 256-element slab [s0, s0 + 256).  Hyper-parameters

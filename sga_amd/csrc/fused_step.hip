@@ -314,15 +314,15 @@ __global__ __launch_bounds__(kBlock, (PLANES || SCORE == SGA_SCORE_ABS_G || SCOR
 void k_fused_final(
     FinalArgs a, const sga_segment* __restrict__ segs, int n_segs,
     const SelState* __restrict__ st, const uint32_t* __restrict__ tile_sel,
-    const uint32_t* __restrict__ tile_eq, int when) {
+    const uint32_t* __restrict__ tile_eq, int when, const int32_t* __restrict__ seg_dir) {
   if (when != 0 && (st->bracket_ok != 0) != (when == 1)) return;
   a.T = st->thresh_bits;
   a.need = st->need;
   const int64_t n_chunks = cdiv64(a.n, kChunk);
   const int64_t wstride = (int64_t)gridDim.x * kChunksPerBlock;
   SegCursor sc, lc;              // sc: wave-uniform (scalar unit); lc: per lane, key forming only
-  sc.init(segs, n_segs);
-  lc.init(segs, n_segs);
+  sc.init(segs, n_segs, seg_dir);
+  lc.init(segs, n_segs, seg_dir);
   const bool can_full = a.vec && (a.mask_out == nullptr || a.mvec);
   for (int64_t c = (int64_t)blockIdx.x * kChunksPerBlock + wave_id(); c < n_chunks;
        c += wstride) {
@@ -356,7 +356,9 @@ static int run_fused(const void* g, float* resid, float* p, float* m, float* v, 
   const bool vec = aligned4(g, BF16G ? 2 : 4) && aligned4(resid, 4) && aligned4(p, 4) &&
                    aligned4(m, 4) && aligned4(v, 4);
   SrcFused<BF16G, SCORE> src{g, resid, p, m, v, vec, {}, pack_extra};
-  src.sc.init(segs, n_segs);
+  static_assert(kSelDirEntries == kSegDirEntries, "the workspace holds one directory");
+  launch_seg_dir(segs, n_segs, n, w.seg_dir, s);
+  src.sc.init(segs, n_segs, w.seg_dir);
   // Adam-normalised scores with the one-sweep select armed: the sweep leaves the selection as bit
   // planes (settled by the candidates) and the final sweep reads one bit per coordinate instead of
   // evaluating the score chain a second time; if the bracket fails on the device, the key-forming
@@ -380,14 +382,14 @@ static int run_fused(const void* g, float* resid, float* p, float* m, float* v, 
   const dim3 one_shot(stream_grid(n_tiles, kChunksPerBlock, 1 << 20));
   if (planes) {
     hipLaunchKernelGGL((k_fused_final<BF16G, BF16V, SGA_SCORE_ABS_G, true>), one_shot, dim3(kBlock), 0, s,
-                       fa, segs, n_segs, w.st, w.tile_gt, w.tile_eq, 1);
+                       fa, segs, n_segs, w.st, w.tile_gt, w.tile_eq, 1, w.seg_dir);
     // the rare other outcome: a small grid that strides over the chunks (returns at once otherwise)
     hipLaunchKernelGGL((k_fused_final<BF16G, BF16V, SCORE, false>),
                        dim3(stream_grid(n_tiles, kChunksPerBlock, 2048)), dim3(kBlock), 0, s, fa,
-                       segs, n_segs, w.st, w.tile_gt, w.tile_eq, 2);
+                       segs, n_segs, w.st, w.tile_gt, w.tile_eq, 2, w.seg_dir);
   } else {
     hipLaunchKernelGGL((k_fused_final<BF16G, BF16V, SCORE, false>), one_shot, dim3(kBlock), 0, s, fa,
-                       segs, n_segs, w.st, w.tile_gt, w.tile_eq, 0);
+                       segs, n_segs, w.st, w.tile_gt, w.tile_eq, 0, w.seg_dir);
   }
   prof_end(pp, s);
   if (result) hipLaunchKernelGGL(k_sel_result, dim3(1), dim3(1), 0, s, w.st, result);

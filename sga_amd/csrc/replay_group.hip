@@ -54,84 +54,138 @@ __device__ __forceinline__ void load_gd(const void* g, int64_t i, int64_t n, flo
 }
 
 // ------------------------------------------------------------------ pass 1
-// Two launches per step, each with its config count as a template argument
-// so the per-config loads are unrolled and all in flight together: one over
-// the configs at a cycle boundary (q = gd + res), one over the others
-// (q = gd * sel).  Both write their configs' slots of the same partials table.
+// One launch per step: the gradient is read once for all configurations.
+// The configs at a cycle boundary with a live residual (q = gd + res) load
+// their residual quads -- their number NB is a template argument so those
+// loads are unrolled and in flight together; every other config is a masked
+// sum of gd^2 (q = gd * sel, from the mask's bit planes on the scalar unit;
+// no mask = every coordinate, which also serves the boundary configs whose
+// residual is known to be zero).  Squares are fp32 like the reference's
+// (q * q).sum(); a lane adds the four squares of its quad in fp32 and widens
+// once per quad into its double accumulator (the reference sums whole chunks
+// in fp32), then the usual fixed-order fold.
 struct P1Alias {
   int src[kMaxCfg];           // partials slot that holds config c's sums
 };
 
 struct P1List {
-  const void* ptr[kMaxCfg];   // res (boundary list) or sel (masked list)
-  int slot[kMaxCfg];          // config index of each entry
+  const float* res[kMaxCfg];       // boundary list: residual arrays
+  int res_slot[kMaxCfg];
+  const uint32_t* sel[kMaxCfg];    // masked list: bit planes, or null for "every coordinate"
+  int sel_slot[kMaxCfg];
+  int n_sel;
 };
 
-template <bool BF16G, bool BOUNDARY, int NC>
+template <bool BF16G, int NB>
 __global__ __launch_bounds__(kBlock) void k_replay_pass1(const void* __restrict__ g, int64_t n,
                                                          float coef_dense, P1List lst,
                                                          double* __restrict__ partials, bool vec,
                                                          int64_t pack_extra) {
-  __shared__ double s_w[kChunksPerBlock][NC];
-  double acc[NC];
+  constexpr int NBA = NB > 0 ? NB : 1;
+  __shared__ double s_w[kChunksPerBlock][2 * kMaxCfg];
+  double accb[NBA], accm[kMaxCfg];
 #pragma unroll
-  for (int c = 0; c < NC; ++c) acc[c] = 0.0;
+  for (int c = 0; c < NBA; ++c) accb[c] = 0.0;
+#pragma unroll
+  for (int c = 0; c < kMaxCfg; ++c) accm[c] = 0.0;
+  const int n_sel = lst.n_sel;
   const float is_one = coef_dense == 1.0f ? 1.0f : 0.0f;
-  const int64_t stride = (int64_t)gridDim.x * kBlock * kVec;
-  for (int64_t base = (int64_t)blockIdx.x * kBlock * kVec; base < n; base += stride) {
-    const int64_t i = base + (int64_t)threadIdx.x * kVec;
-    const bool full = vec && base + kBlock * kVec <= n;
-    if (!full && i >= n) continue;
-    float gd[4];
-    if (full) load_gd<BF16G, true>(g, i, n, is_one, coef_dense, gd, true);
-    else load_gd<BF16G, false>(g, i, n, is_one, coef_dense, gd, vec);
-    if (BOUNDARY) {
-      float rr[NC][4];
+  // chunk-structured: a wave owns 1024-element chunks and has the gradient quads of a chunk's four
+  // slabs in flight together (8 bytes per lane and load: one load at a time is bound by latency)
+  const int64_t n_chunks = cdiv64(n, kChunk);
+  const int64_t wstride = (int64_t)gridDim.x * kChunksPerBlock;
+  for (int64_t ch = (int64_t)blockIdx.x * kChunksPerBlock + wave_id(); ch < n_chunks; ch += wstride) {
+    const bool full = vec && (ch + 1) * kChunk <= n;
+    float gq[kChunkIters][4];
 #pragma unroll
-      for (int c = 0; c < NC; ++c) {
-        const float* rp = reinterpret_cast<const float*>(lst.ptr[c]) +
-                          (full ? pack_shift<true>(i, pack_extra) : pack_shift<false>(i, pack_extra));
-        if (full) ld_f32<true>(rp, i, n, rr[c], true);
-        else load4_f32(rp, i, n, rr[c], vec);
-      }
+    for (int it = 0; it < kChunkIters; ++it) {
+      const int64_t i = ch * kChunk + it * (kWave * kVec) + lane_id() * kVec;
+      gq[it][0] = gq[it][1] = gq[it][2] = gq[it][3] = 0.0f;
+      if (full) load_gd<BF16G, true>(g, i, n, is_one, coef_dense, gq[it], true);
+      else if (i < n) load_gd<BF16G, false>(g, i, n, is_one, coef_dense, gq[it], vec);
+    }
 #pragma unroll
-      for (int c = 0; c < NC; ++c)
+    for (int it = 0; it < kChunkIters; ++it) {
+      const int64_t i = ch * kChunk + it * (kWave * kVec) + lane_id() * kVec;
+      const float* gd = gq[it];
+      if (NB > 0) {
+        float rr[NBA][4];
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const float q = gd[e] + rr[c][e];
-          if (full || i + e < n) acc[c] += (double)(q * q);
+        for (int c = 0; c < NB; ++c) {
+          const float* rp = lst.res[c] + pack_shift<true>(ch * kChunk, pack_extra);
+          rr[c][0] = rr[c][1] = rr[c][2] = rr[c][3] = 0.0f;
+          if (full) ld_f32<true>(rp, i, n, rr[c], true);
+          else if (i < n) load4_f32(rp, i, n, rr[c], vec);
         }
-    } else {
-      // q = gd * {0, 1}: q*q is gd*gd or 0, squared once for all configs
-      float gd2[4];
 #pragma unroll
-      for (int e = 0; e < 4; ++e) gd2[e] = (full || i + e < n) ? gd[e] * gd[e] : 0.0f;
-      bool sl[NC][4];
+        for (int c = 0; c < NB; ++c) {
+          float part = 0.0f;
 #pragma unroll
-      for (int c = 0; c < NC; ++c) {
-        const uint32_t* sp = reinterpret_cast<const uint32_t*>(lst.ptr[c]);
-        if (!sp) {                       // no mask: every coordinate counts (q = gd)
-          sl[c][0] = sl[c][1] = sl[c][2] = sl[c][3] = true;
+          for (int e = 0; e < 4; ++e) {
+            const float q = gd[e] + rr[c][e];
+            part += (full || i + e < n) ? q * q : 0.0f;
+          }
+          accb[c] += (double)part;
+        }
+      }
+    }
+    // q = gd * {0, 1}: q * q is gd * gd or 0, squared once for all configs.  Config by config the
+    // chunk's 32 plane words come in as ONE batch of scalar loads (a load per slab would leave the
+    // wave waiting on the scalar cache 4 x n_sel times per chunk) and serve directly as lane masks;
+    // the lane's 16 squares are added in fp32, in a fixed order, and widened once.
+    float gd2[kChunkIters][4];
+#pragma unroll
+    for (int it = 0; it < kChunkIters; ++it) {
+      const int64_t i = ch * kChunk + it * (kWave * kVec) + lane_id() * kVec;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) gd2[it][e] = (full || i + e < n) ? gq[it][e] * gq[it][e] : 0.0f;
+    }
+#pragma unroll
+    for (int c = 0; c < kMaxCfg; ++c) {
+      if (c < n_sel) {                            // uniform
+        const uint32_t* sp = lst.sel[c];
+        float part = 0.0f;
+        if (!sp) {                                // no mask: every coordinate counts (q = gd)
+#pragma unroll
+          for (int it = 0; it < kChunkIters; ++it)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) part += gd2[it][e];
         } else {
-          plane_wave_flags4(sp, i, sl[c]);     // bits past n are zero
+          const uint64_t* w = reinterpret_cast<const uint64_t*>(sp) + uniform_i64(ch) * (kChunkIters * 4);
+          uint64_t mk[kChunkIters * 4];
+#pragma unroll
+          for (int j = 0; j < kChunkIters * 4; ++j) mk[j] = w[j];     // bits past n are zero
+#pragma unroll
+          for (int it = 0; it < kChunkIters; ++it)
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+              part += __builtin_amdgcn_inverse_ballot_w64(mk[it * 4 + e]) ? gd2[it][e] : 0.0f;
         }
+        accm[c] += (double)part;
       }
-#pragma unroll
-      for (int c = 0; c < NC; ++c)
-#pragma unroll
-        for (int e = 0; e < 4; ++e) acc[c] += (double)(sl[c][e] ? gd2[e] : 0.0f);
     }
   }
 #pragma unroll
-  for (int c = 0; c < NC; ++c) {
-    const double t = wave_sum(acc[c]);
+  for (int c = 0; c < NB; ++c) {
+    const double t = wave_sum(accb[c]);
     if (lane_id() == 0) s_w[wave_id()][c] = t;
   }
+#pragma unroll
+  for (int c = 0; c < kMaxCfg; ++c) {
+    if (c < n_sel) {
+      const double t = wave_sum(accm[c]);
+      if (lane_id() == 0) s_w[wave_id()][kMaxCfg + c] = t;
+    }
+  }
   __syncthreads();
-  if (threadIdx.x < NC) {
-    const int c = threadIdx.x;
-    partials[(int64_t)blockIdx.x * kMaxCfg + lst.slot[c]] =
-        s_w[0][c] + s_w[1][c] + s_w[2][c] + s_w[3][c];
+  const int t = threadIdx.x;
+  if (t < NB)
+    partials[(int64_t)blockIdx.x * kMaxCfg + lst.res_slot[t]] =
+        s_w[0][t] + s_w[1][t] + s_w[2][t] + s_w[3][t];
+  if (t >= kMaxCfg && t < kMaxCfg + n_sel) {
+    const int c = t - kMaxCfg;
+    partials[(int64_t)blockIdx.x * kMaxCfg + lst.sel_slot[c]] =
+        s_w[0][t] + s_w[1][t] + s_w[2][t] + s_w[3][t];
   }
 }
 
@@ -553,26 +607,19 @@ using namespace sga;
 
 static_assert(sizeof(RSeg) == sizeof(sga_replay_segment), "replay segment layout");
 
-template <bool BOUNDARY, bool BF16G, int NC>
-static void launch_pass1_n(unsigned nb, hipStream_t s, const void* g, int64_t n, float coef_dense,
-                           const P1List& lst, double* partials, bool vec, int64_t pack_extra) {
-  hipLaunchKernelGGL((k_replay_pass1<BF16G, BOUNDARY, NC>), dim3(nb), dim3(kBlock), 0, s, g, n,
-                     coef_dense, lst, partials, vec, pack_extra);
-}
-
-template <bool BOUNDARY>
-static void launch_pass1(bool bg, int count, unsigned nb, hipStream_t s, const void* g, int64_t n,
+template <bool BF16G>
+static void launch_pass1(int n_b, unsigned nb, hipStream_t s, const void* g, int64_t n,
                          float coef_dense, const P1List& lst, double* partials, bool vec,
                          int64_t pack_extra) {
-#define SGA_P1(NC)                                                                             \
-  case NC:                                                                                     \
-    if (bg) launch_pass1_n<BOUNDARY, true, NC>(nb, s, g, n, coef_dense, lst, partials, vec, pack_extra); \
-    else launch_pass1_n<BOUNDARY, false, NC>(nb, s, g, n, coef_dense, lst, partials, vec, pack_extra);   \
+#define SGA_P1(NB)                                                                              \
+  case NB:                                                                                      \
+    hipLaunchKernelGGL((k_replay_pass1<BF16G, NB>), dim3(nb), dim3(kBlock), 0, s, g, n,         \
+                       coef_dense, lst, partials, vec, pack_extra);                             \
     break;
-  switch (count) {
-    SGA_P1(1) SGA_P1(2) SGA_P1(3) SGA_P1(4) SGA_P1(5) SGA_P1(6) SGA_P1(7) SGA_P1(8)
+  switch (n_b) {
+    SGA_P1(0) SGA_P1(1) SGA_P1(2) SGA_P1(3) SGA_P1(4) SGA_P1(5) SGA_P1(6) SGA_P1(7) SGA_P1(8)
     SGA_P1(9) SGA_P1(10) SGA_P1(11) SGA_P1(12) SGA_P1(13) SGA_P1(14) SGA_P1(15) SGA_P1(16)
-    default: break;                       // no config of this kind at this step
+    default: break;
   }
 #undef SGA_P1
 }
@@ -590,27 +637,28 @@ extern "C" int sga_replay_pass1(const void* g, int g_dtype, int64_t n, float coe
   }
   const bool bg = g_dtype == SGA_BF16;
   const bool vec = aligned4(g, bg ? 2 : 4) && group_aligned(grp);
-  const unsigned nb = stream_grid(n, (int64_t)kBlock * kVec, kReplayBlocks);
+  const unsigned nb = stream_grid(cdiv64(n, kChunk), kChunksPerBlock, kReplayBlocks);
   hipStream_t s = (hipStream_t)stream;
-  P1List lb = {}, lm = {};
+  P1List lst = {};
   P1Alias al;
   int n_b = 0, n_m = 0, plain = -1;
   for (int c = 0; c < G; ++c) {
     al.src[c] = c;
     if (grp.c[c].boundary && grp.c[c].res_zero) {
       // q = gd + 0: one unmasked sum of squares serves every such config
-      if (plain < 0) { plain = c; lm.ptr[n_m] = nullptr; lm.slot[n_m++] = c; }
+      if (plain < 0) { plain = c; lst.sel[n_m] = nullptr; lst.sel_slot[n_m++] = c; }
       al.src[c] = plain;
     } else if (grp.c[c].boundary) {
-      lb.ptr[n_b] = grp.c[c].res; lb.slot[n_b++] = c;
+      lst.res[n_b] = grp.c[c].res; lst.res_slot[n_b++] = c;
     } else {
-      lm.ptr[n_m] = grp.c[c].sel; lm.slot[n_m++] = c;
+      lst.sel[n_m] = grp.c[c].sel; lst.sel_slot[n_m++] = c;
     }
   }
+  lst.n_sel = n_m;
   for (int c = G; c < kMaxCfg; ++c) al.src[c] = 0;
   ProfPair* pp = prof_begin(SGA_PROF_REPLAY_PASS1, s);
-  launch_pass1<true>(bg, n_b, nb, s, g, n, coef_dense, lb, partials, vec, grp.pack_extra);
-  launch_pass1<false>(bg, n_m, nb, s, g, n, coef_dense, lm, partials, vec, 0);
+  if (bg) launch_pass1<true>(n_b, nb, s, g, n, coef_dense, lst, partials, vec, grp.pack_extra);
+  else launch_pass1<false>(n_b, nb, s, g, n, coef_dense, lst, partials, vec, grp.pack_extra);
   prof_end(pp, s);
   hipLaunchKernelGGL(k_replay_coef, dim3(1), dim3(kBlock), 0, s, partials, (int)nb, G, clip, qn2, coef_d, coef_f, al);
   return check_launch("sga_replay_pass1");
@@ -647,7 +695,12 @@ static int run_reselect(const void* g, const float* res, const float* w, const f
                    aligned4(m, 4) && aligned4(v, 4);
   SrcReplay<BF16G, SCORE> src{g, res, w, m, v, coef_f, coef_dense, adams, vec, {},
                               packed ? kPackExtra : 0, res_zero};
-  src.sc.init(segs, n_segs);
+  if (SrcReplay<BF16G, SCORE>::kHyper) {          // the other scores never look a tensor up
+    launch_seg_dir(segs, n_segs, n, ws.seg_dir, s);
+    src.sc.init(segs, n_segs, ws.seg_dir);
+  } else {
+    src.sc.init(segs, n_segs);
+  }
   run_select(src, n, k, 0, true, ws, s, sel_out);
   finish_planes(src, n, 0, ws, sel_out, s);
   if (result) hipLaunchKernelGGL(k_sel_result, dim3(1), dim3(1), 0, s, ws.st, result);

@@ -55,6 +55,7 @@ struct SelWorkspace {
   uint32_t* tile_eq;   // n_tiles -> tie-count prefix
   uint32_t* blk_gt;    // kMaxTileBlocks
   uint32_t* blk_eq;    // kMaxTileBlocks
+  int32_t* seg_dir;    // kSelDirEntries: tensor directory of segment-keyed sources (adam_math.hpp)
   int64_t n_tiles_cap;
   // sampled-bracket path (null / 0 when the workspace has no room for it)
   uint32_t* sample;    // sample_cap keys
@@ -92,8 +93,9 @@ static inline int64_t fast_seg_cap(int64_t n) {
 // the same carve from (ws, ws_bytes) alone.
 constexpr int kHistEntries = 2 * kBinsBig + kBinsSmall;      // 8320
 constexpr int kHistStride = kHistEntries + 64;               // per-state stride
+constexpr int kSelDirEntries = 1 << 15;                        // n < 2^31 in blocks of 2^16
 constexpr size_t kSelFixedBytes =
-    512 + (size_t)kHistStride * 2 * 4 + (size_t)kMaxTileBlocks * 4 * 2;
+    512 + (size_t)kHistStride * 2 * 4 + (size_t)kMaxTileBlocks * 4 * 2 + (size_t)kSelDirEntries * 4;
 
 static inline size_t fast_bytes_for_tiles(int64_t nt) {
   const int64_t n = nt * kChunk;
@@ -132,6 +134,8 @@ static inline bool sel_ws_carve(void* ws, size_t bytes, int64_t n_tiles_needed,
   p += (size_t)kMaxTileBlocks * 4;
   out->blk_eq = reinterpret_cast<uint32_t*>(p);
   p += (size_t)kMaxTileBlocks * 4;
+  out->seg_dir = reinterpret_cast<int32_t*>(p);
+  p += (size_t)kSelDirEntries * 4;
   out->tile_gt = reinterpret_cast<uint32_t*>(p);
   p += (size_t)nt * 4;
   out->tile_eq = reinterpret_cast<uint32_t*>(p);

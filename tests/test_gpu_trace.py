@@ -119,7 +119,10 @@ def test_replay_window_end_to_end(dev, tmp_path, clip, g_dtype):
             assert abs(res["dense"][c.optimizer]["den_at"][h] - den[h]) <= 1e-5 * den[h]
             # the reference's own band for ||w_s - w_d|| (test_replay_cycle.py:318-319)
             assert abs(r["dist_at"][h] - o["dist"][h]) <= 1e-3 * max(1.0, o["dist"][h]), (ci, h)
-            assert abs(r["dist_at"][h] - o["dist"][h]) <= 2e-3 * o["dist"][h] + 1e-9, (ci, h)
+            # tighter, with a floor relative to the dense movement: at T = 1 the oracle's own clip
+            # coefficient undoes the recorded one exactly (distance 0.0), the device's differs in
+            # its last bits (order of the norm's sum) and leaves a few ulps of w
+            assert abs(r["dist_at"][h] - o["dist"][h]) <= 2e-3 * o["dist"][h] + 1e-6 * den[h], (ci, h)
             assert r["distortion"][h] == r["dist_at"][h] / res["dense"][c.optimizer]["den_at"][h]
         if c.T == 1:
             assert r["dist_at"][9] <= 1e-3 * den[9]          # T = 1 is the dense trajectory
