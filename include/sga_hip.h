@@ -337,14 +337,21 @@ int sga_opt_step_inplace(const float* q, float* m, float* v, float* w,
  * zeroed; sparse AdamW commit on p/m/v (engine order: engine.py:416-604,
  * pack kernels.py:166-187, commit adamw.py:637-724).
  * g_dtype / values_dtype: SGA_F32 | SGA_BF16.  mask_out may be NULL.
- * idx_out / values_out need room for k entries.  segs is a DEVICE array. */
+ * idx_out / values_out need room for k entries.  segs is a DEVICE array.
+ * flags: SGA_GC_ADAMS commits (and, for update / coi, scores) with the AdamS
+ * tail (adams.py:87-213, 507-654: v rebuilt from the pre-commit m, no bias
+ * corrections; bc1 / bc2 of the segments are ignored); SGA_GC_FOLD divides the
+ * new residual by `interval` (residual mean before a boundary, adamw.py:199-204;
+ * true division like adamw_torch.py:88-91).  Any other flag is refused: the
+ * dual-lr split belongs to full steps (adamw.py:570-580). */
 size_t sga_fused_workspace_bytes(int64_t n);
 int sga_fused_sparse_step(const void* g, int g_dtype, float* resid, float* p,
                           float* m, float* v, int64_t n, int64_t k,
                           const sga_segment* segs, int n_segs, int score_id,
                           int32_t* idx_out, void* values_out, int values_dtype,
                           uint8_t* mask_out, float factor, float coeff,
-                          int fast, sga_select_result* result, void* ws,
+                          int fast, int flags, float interval,
+                          sga_select_result* result, void* ws,
                           size_t ws_bytes, void* stream);
 
 /* Packed-state variant of the fused step for callers that let the library
@@ -364,7 +371,8 @@ int sga_fused_sparse_step_packed(const void* g, int g_dtype, float* state,
                                  int n_segs, int score_id, int32_t* idx_out,
                                  void* values_out, int values_dtype,
                                  uint8_t* mask_out, float factor, float coeff,
-                                 int fast, sga_select_result* result, void* ws,
+                                 int fast, int flags, float interval,
+                                 sga_select_result* result, void* ws,
                                  size_t ws_bytes, void* stream);
 int sga_state_repack(float* resid, float* p, float* m, float* v, float* state,
                      int64_t n, int unpack, void* stream);

@@ -22,7 +22,8 @@ from . import select as SEL
 
 def fused_sparse_step(g, resid, p, m, v, segments, step, ratio_percent=None,
                       k=None, score="abs_g", values_dtype=torch.float32,
-                      factor=1.0, coeff=1.0):
+                      factor=1.0, coeff=1.0, optimizer="adamw", fold=False,
+                      interval=1.0):
     """One step over a flat bucket.
 
     g        : flat gradient (bf16 or fp32), read only
@@ -30,6 +31,10 @@ def fused_sparse_step(g, resid, p, m, v, segments, step, ratio_percent=None,
     p, m, v  : flat fp32 state, updated in place
     segments : list of dicts {"start","n","lr","b1","b2","eps","wd"}
     score    : "abs_g" (= |g+r|), "update", "coi", "abs_m"
+    optimizer: "adamw" | "adams" -- AdamS scores through the replay-side
+               routing v := m*m, bc := 1 (replay.py:486-505) and commits with
+               ``adams_grad_correct`` (adams_torch.py:34-85)
+    fold     : divide the new residual by ``interval`` (adamw_torch.py:88-91)
     Returns (idx int32[k], values[k], mask bool[N], thresh).
     """
     n = resid.numel()
@@ -43,9 +48,10 @@ def fused_sparse_step(g, resid, p, m, v, segments, step, ratio_percent=None,
             a, b = s["start"], s["start"] + s["n"]
             bc1 = 1.0 - s["b1"] ** step
             bc2 = 1.0 - s["b2"] ** step
-            sc[a:b] = S.get_formula(score)(
-                p[a:b], m[a:b], v[a:b], buf[a:b], s["b1"], s["b2"], s["eps"],
-                s["wd"], bc1, bc2).abs()
+            sc[a:b] = S.score_formula(
+                score, p[a:b], m[a:b], v[a:b], buf[a:b], s["b1"], s["b2"],
+                s["eps"], s["wd"], bc1, bc2, optimizer,
+                update_includes_wd=True).abs()
     if k is None:
         k = SEL.k_for(n, ratio_percent)
     mask, thresh = SEL.select_topk_flat(sc, k)
@@ -54,7 +60,21 @@ def fused_sparse_step(g, resid, p, m, v, segments, step, ratio_percent=None,
     K.pack_selected(buf, idx, values, factor)
     for s in segments:
         a, b = s["start"], s["start"] + s["n"]
-        A.adamw_grad_correct_compact(
-            p[a:b], buf[a:b], m[a:b], v[a:b], idx, values, a, s["lr"],
-            s["b1"], s["b2"], s["eps"], s["wd"], step, coeff=coeff)
+        if optimizer == "adamw":
+            A.adamw_grad_correct_compact(
+                p[a:b], buf[a:b], m[a:b], v[a:b], idx, values, a, s["lr"],
+                s["b1"], s["b2"], s["eps"], s["wd"], step, coeff=coeff,
+                fold=fold, interval=interval)
+        else:
+            # the compact path's torch fallback (adams.py:507-654): scatter
+            # the record's values into the pack-cleared buffer, masked commit
+            seg_mask = mask[a:b].to(torch.uint8)
+            lo = int(torch.searchsorted(idx, a))
+            hi = int(torch.searchsorted(idx, b))
+            if hi > lo:
+                buf[a:b][idx[lo:hi].long() - a] = values[lo:hi].to(buf.dtype)
+            A.adams_grad_correct(
+                p[a:b], buf[a:b], m[a:b], v[a:b], s["lr"], s["b1"], s["b2"],
+                s["eps"], s["wd"], mask=seg_mask, coeff=coeff, clear=True,
+                fold=fold, interval=interval)
     return idx, values, mask, thresh

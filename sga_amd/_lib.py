@@ -88,10 +88,10 @@ SIGNATURES = {
     "sga_prof_read": (I32, [I32, P, P]),
     "sga_fused_workspace_bytes": (SZ, [I64]),
     "sga_fused_sparse_step": (I32, [P, I32, P, P, P, P, I64, I64, P, I32, I32, P, P,
-                                    I32, P, F, F, I32, P, P, SZ, P]),
+                                    I32, P, F, F, I32, I32, F, P, P, SZ, P]),
     "sga_packed_state_elems": (I64, [I64]),
     "sga_fused_sparse_step_packed": (I32, [P, I32, P, I64, I64, P, I32, I32, P, P,
-                                           I32, P, F, F, I32, P, P, SZ, P]),
+                                           I32, P, F, F, I32, I32, F, P, P, SZ, P]),
     "sga_state_repack": (I32, [P, P, P, P, P, I64, I32, P]),
 }
 

@@ -28,6 +28,7 @@ struct SrcFused {
   bool vec;
   SegCursor sc;        // per-thread cache of the current segment's hyper-parameters
   int64_t pack_extra;  // 0: separate arrays; else extra floats per kPackRun elements (packed state)
+  int adams;           // AdamS: the second moment is rebuilt from m (v := m*m), no bias corrections
   // Stepwise interface of the one-sweep select.
   struct Raw { RawG g; F4 r, p, m, v; };
   struct Chunk { int64_t sh; };
@@ -86,7 +87,11 @@ struct SrcFused {
     float q[4];
 #pragma unroll
     for (int e = 0; e < 4; ++e) q[e] = rr[e] + gg[e];
-    slab_score_keys<SCORE, FULL>(sc, 0, i, n, q, pp, mm, vv, key);
+    if (adams) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) vv[e] = mm[e] * mm[e];
+    }
+    slab_score_keys<SCORE, FULL>(sc, adams, i, n, q, pp, mm, vv, key);
   }
   template <bool FULL = false>
   __device__ __forceinline__ void load(int64_t i, int64_t n, uint32_t key[4]) {
@@ -113,7 +118,10 @@ struct SrcFused {
     for (int e = 0; e < 4; ++e) {
       if (FULL || i + e < n) {
         sc.seek(i + e);
-        key[e] = score_key<SCORE>(rr[e] + gg[e], pp[e], mm[e], vv[e], sc.h);
+        Hyper h = sc.h;
+        float ve = vv[e];
+        if (adams) { ve = mm[e] * mm[e]; h.bc1 = 1.0f; h.bc2 = 1.0f; }
+        key[e] = score_key<SCORE>(rr[e] + gg[e], pp[e], mm[e], ve, h);
       } else {
         key[e] = 0u;
       }
@@ -135,6 +143,8 @@ struct FinalArgs {
   float factor, coeff;
   uint32_t T, need;
   bool vec, mvec, scale, apply_coeff;
+  bool adams, fold;         // AdamS commit (adams.py:87-213); residual-mean fold of the new residual
+  float interval;           // fold divisor (true division, as adamw_torch.py does)
   int64_t pack_extra;
   const uint32_t* planes;   // the settled selection as bit planes (PLANES mode), else unused
 };
@@ -237,7 +247,10 @@ __device__ __forceinline__ void final_chunk(const FinalArgs& a, int64_t c, Chunk
         else {
           // only when the one-sweep select is off or failed: a per-lane cursor
           if (valid[e]) lc.seek(i + e);
-          key[e] = valid[e] ? score_key<SCORE>(q[e], pp[it][e], mm[it][e], vv[it][e], lc.h) : 0u;
+          Hyper hk = lc.h;
+          float ve = vv[it][e];
+          if (a.adams) { ve = mm[it][e] * mm[it][e]; hk.bc1 = 1.0f; hk.bc2 = 1.0f; }
+          key[e] = valid[e] ? score_key<SCORE>(q[e], pp[it][e], mm[it][e], ve, hk) : 0u;
         }
       }
       slab_select(key, valid, a.T, a.need, cur, sel, pos);
@@ -278,10 +291,13 @@ __device__ __forceinline__ void final_chunk(const FinalArgs& a, int64_t c, Chunk
       float pn[4], mn[4], vn[4];
       for (;;) {
         const bool whole = sc.lo <= s0 && sc.hi >= s1;
+        Hyper h = sc.h;
+        if (a.adams) { h.bc1 = 1.0f; h.bc2 = 1.0f; }
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-          const Commit cm = adamw_commit(pp[it][e], ge[e], mm[it][e], vv[it][e], sc.h);
-          const float pe = pp[it][e] - sc.h.lr * cm.upd;
+          const float ve = a.adams ? mm[it][e] * mm[it][e] : vv[it][e];
+          const Commit cm = adamw_commit(pp[it][e], ge[e], mm[it][e], ve, h);
+          const float pe = pp[it][e] - h.lr * cm.upd;
           if (whole || (i + e >= sc.lo && i + e < sc.hi)) { pn[e] = pe; mn[e] = cm.m_new; vn[e] = cm.v_new; }
         }
         const int64_t nxt = sc.hi;
@@ -294,6 +310,7 @@ __device__ __forceinline__ void final_chunk(const FinalArgs& a, int64_t c, Chunk
         if (!valid[e]) continue;
         pp[it][e] = pn[e]; mm[it][e] = mn[e]; vv[it][e] = vn[e];
         rr[it][e] = sel[e] ? 0.0f : q[e];
+        if (a.fold) rr[it][e] = __fdiv_rn(rr[it][e], a.interval);
       }
       st_f32<FULL>(R, i, n, rr[it], a.vec);
       st_f32<FULL>(M, i, n, mm[it], a.vec);
@@ -351,11 +368,12 @@ template <bool BF16G, bool BF16V, int SCORE>
 static int run_fused(const void* g, float* resid, float* p, float* m, float* v, int64_t n,
                      int64_t k, const sga_segment* segs, int n_segs, int32_t* idx_out,
                      void* values_out, uint8_t* mask_out, float factor, float coeff, int fast,
-                     sga_select_result* result, const SelWorkspace& w, hipStream_t s,
-                     int64_t pack_extra) {
+                     int flags, float interval, sga_select_result* result, const SelWorkspace& w,
+                     hipStream_t s, int64_t pack_extra) {
   const bool vec = aligned4(g, BF16G ? 2 : 4) && aligned4(resid, 4) && aligned4(p, 4) &&
                    aligned4(m, 4) && aligned4(v, 4);
-  SrcFused<BF16G, SCORE> src{g, resid, p, m, v, vec, {}, pack_extra};
+  const int adams = (flags & SGA_GC_ADAMS) ? 1 : 0;
+  SrcFused<BF16G, SCORE> src{g, resid, p, m, v, vec, {}, pack_extra, adams};
   static_assert(kSelDirEntries == kSegDirEntries, "the workspace holds one directory");
   launch_seg_dir(segs, n_segs, n, w.seg_dir, s);
   src.sc.init(segs, n_segs, w.seg_dir);
@@ -378,6 +396,7 @@ static int run_fused(const void* g, float* resid, float* p, float* m, float* v, 
   fa.vec = vec; fa.mvec = aligned4(mask_out, 1);
   fa.scale = factor != 1.0f; fa.apply_coeff = coeff != 1.0f;
   fa.pack_extra = pack_extra;
+  fa.adams = adams != 0; fa.fold = (flags & SGA_GC_FOLD) != 0; fa.interval = interval;
   fa.planes = w.pbits;
   const dim3 one_shot(stream_grid(n_tiles, kChunksPerBlock, 1 << 20));
   if (planes) {
@@ -406,8 +425,19 @@ static int fused_entry(const char* who, const void* g, int g_dtype, float* resid
                        float* m, float* v, int64_t pack_extra, int64_t n, int64_t k,
                        const sga_segment* segs, int n_segs, int score_id, int32_t* idx_out,
                        void* values_out, int values_dtype, uint8_t* mask_out, float factor,
-                       float coeff, int fast, sga_select_result* result, void* ws, size_t ws_bytes,
-                       void* stream) {
+                       float coeff, int fast, int flags, float interval, sga_select_result* result,
+                       void* ws, size_t ws_bytes, void* stream) {
+  if ((flags & ~(SGA_GC_ADAMS | SGA_GC_FOLD)) != 0) {
+    // the dual-lr split belongs to full steps (adamw.py:570-580); HAS_MASK / CLEAR / APPLY_COEFF
+    // are what this step does anyway (coeff != 1 applies the coefficient)
+    set_error("%s: flags may carry SGA_GC_ADAMS and SGA_GC_FOLD only (got %d); the boundary "
+              "dual-lr split requires a full step", who, flags);
+    return SGA_ERR_ARG;
+  }
+  if ((flags & SGA_GC_FOLD) && !(interval > 0.0f)) {
+    set_error("%s: SGA_GC_FOLD needs interval > 0 (got %g)", who, (double)interval);
+    return SGA_ERR_ARG;
+  }
   if (!g || !resid || !p || !m || !v || !segs || !idx_out || !values_out || n < 1 ||
       n >= (1ll << 31) || k < 1 || k > n || n_segs < 1 ||
       (g_dtype != SGA_F32 && g_dtype != SGA_BF16) ||
@@ -426,7 +456,8 @@ static int fused_entry(const char* who, const void* g, int g_dtype, float* resid
   const bool bg = g_dtype == SGA_BF16, bv = values_dtype == SGA_BF16;
 #define SGA_RUN(BG, BV, SC)                                                                   \
   return run_fused<BG, BV, SC>(g, resid, p, m, v, n, k, segs, n_segs, idx_out, values_out,   \
-                               mask_out, factor, coeff, fast, result, w, s, pack_extra)
+                               mask_out, factor, coeff, fast, flags, interval, result, w, s,   \
+                               pack_extra)
 #define SGA_RUN_SC(BG, BV)                    \
   switch (score_id) {                         \
     case 0: SGA_RUN(BG, BV, 0);               \
@@ -446,11 +477,12 @@ extern "C" int sga_fused_sparse_step(const void* g, int g_dtype, float* resid, f
                                      float* v, int64_t n, int64_t k, const sga_segment* segs,
                                      int n_segs, int score_id, int32_t* idx_out, void* values_out,
                                      int values_dtype, uint8_t* mask_out, float factor,
-                                     float coeff, int fast, sga_select_result* result, void* ws,
-                                     size_t ws_bytes, void* stream) {
+                                     float coeff, int fast, int flags, float interval,
+                                     sga_select_result* result, void* ws, size_t ws_bytes,
+                                     void* stream) {
   return fused_entry("sga_fused_sparse_step", g, g_dtype, resid, p, m, v, 0, n, k, segs, n_segs,
                      score_id, idx_out, values_out, values_dtype, mask_out, factor, coeff, fast,
-                     result, ws, ws_bytes, stream);
+                     flags, interval, result, ws, ws_bytes, stream);
 }
 
 extern "C" int64_t sga_packed_state_elems(int64_t n) {
@@ -461,8 +493,9 @@ extern "C" int sga_fused_sparse_step_packed(const void* g, int g_dtype, float* s
                                             int64_t k, const sga_segment* segs, int n_segs,
                                             int score_id, int32_t* idx_out, void* values_out,
                                             int values_dtype, uint8_t* mask_out, float factor,
-                                            float coeff, int fast, sga_select_result* result,
-                                            void* ws, size_t ws_bytes, void* stream) {
+                                            float coeff, int fast, int flags, float interval,
+                                            sga_select_result* result, void* ws, size_t ws_bytes,
+                                            void* stream) {
   if (state && (reinterpret_cast<uintptr_t>(state) & 15)) {
     set_error("sga_fused_sparse_step_packed: state must be 16-byte aligned");
     return SGA_ERR_ARG;
@@ -471,7 +504,7 @@ extern "C" int sga_fused_sparse_step_packed(const void* g, int g_dtype, float* s
                      state ? state + kPackRun : nullptr, state ? state + 2 * kPackRun : nullptr,
                      state ? state + 3 * kPackRun : nullptr, kPackExtra, n, k, segs, n_segs,
                      score_id, idx_out, values_out, values_dtype, mask_out, factor, coeff, fast,
-                     result, ws, ws_bytes, stream);
+                     flags, interval, result, ws, ws_bytes, stream);
 }
 
 // resid/p/m/v <-> packed state (dir 0: pack, 1: unpack); a null array is skipped.

@@ -67,11 +67,27 @@ class FusedSparseStep:
         self._seg_up.upload(self._seg_host)
         self._seg_step = step
 
+    @staticmethod
+    def _flags(optimizer, fold, interval, inactive_lr_scale):
+        if optimizer not in ("adamw", "adams"):
+            raise ValueError(f"unknown optimizer {optimizer!r} (adamw, adams)")
+        if inactive_lr_scale != 1.0:
+            raise ValueError("grad-correct boundary dual-lr (inactive_lr_scale="
+                             f"{inactive_lr_scale!r}) requires a full step (emit_score set) "
+                             "with a mask; the fused step is a sparse step")
+        if fold and not interval > 0.0:
+            raise ValueError(f"fold needs interval > 0 (got {interval!r})")
+        return (L.GC_ADAMS if optimizer == "adams" else 0) | (L.GC_FOLD if fold else 0)
+
     def step(self, g, resid, p, m, v, step, k=None, ratio_percent=None,
-             score="abs_g", factor=1.0, coeff=1.0, fast=True):
+             score="abs_g", factor=1.0, coeff=1.0, fast=True, optimizer="adamw", fold=False,
+             interval=1.0, inactive_lr_scale=1.0):
         """Run one fused step in place; returns (idx[:k], values[:k]) views.
         ``self.result`` holds the device-side select result (threshold bits,
-        counts); nothing is synchronised here."""
+        counts); nothing is synchronised here.  ``optimizer="adams"`` commits
+        (and scores) with the AdamS tail; ``fold`` divides the new residual by
+        ``interval`` (the residual mean taken before a boundary)."""
+        flags = self._flags(optimizer, fold, interval, inactive_lr_scale)
         n = self.n
         for t in (g, resid, p, m, v):
             L.require_dev(t)
@@ -88,14 +104,16 @@ class FusedSparseStep:
                L.ptr(m), L.ptr(v), n, k, L.ptr(self._seg_dev), len(self.segments),
                SCORE_MAP[score], L.ptr(self.idx), L.ptr(self.values),
                L.dtype_code(self.values), L.ptr(self.mask), L.f32(factor), L.f32(coeff),
-               1 if fast else 0, L.ptr(self.result), L.ptr(self.ws), self.ws_bytes,
-               L.stream())
+               1 if fast else 0, flags, L.f32(interval), L.ptr(self.result), L.ptr(self.ws),
+               self.ws_bytes, L.stream())
         return self.idx[:k], self.values[:k]
 
     def step_packed(self, g, state, step, k=None, ratio_percent=None, score="abs_g",
-                    factor=1.0, coeff=1.0, fast=True):
+                    factor=1.0, coeff=1.0, fast=True, optimizer="adamw", fold=False,
+                    interval=1.0, inactive_lr_scale=1.0):
         """Same step on a ``PackedState`` (resid/p/m/v interleaved in 64 KiB
-        records): same arithmetic and outputs, fewer DRAM bank conflicts."""
+        records): same arithmetic and outputs."""
+        flags = self._flags(optimizer, fold, interval, inactive_lr_scale)
         n = self.n
         L.require_dev(g, state.data)
         L.require_contig(g=g)
@@ -111,8 +129,8 @@ class FusedSparseStep:
         L.call("sga_fused_sparse_step_packed", L.ptr(g), L.dtype_code(g), L.ptr(state.data), n, k,
                L.ptr(self._seg_dev), len(self.segments), SCORE_MAP[score], L.ptr(self.idx),
                L.ptr(self.values), L.dtype_code(self.values), L.ptr(self.mask), L.f32(factor),
-               L.f32(coeff), 1 if fast else 0, L.ptr(self.result), L.ptr(self.ws), self.ws_bytes,
-               L.stream())
+               L.f32(coeff), 1 if fast else 0, flags, L.f32(interval), L.ptr(self.result),
+               L.ptr(self.ws), self.ws_bytes, L.stream())
         return self.idx[:k], self.values[:k]
 
     def read_result(self):

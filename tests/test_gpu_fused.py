@@ -27,7 +27,7 @@ def _segments(sizes, wd_every=2, vary=False):
 
 
 def _run(dev, sizes, steps, ratio, gdtype, vdtype, score="abs_g", seed0=0, vary=False,
-         expect_path=None):
+         expect_path=None, **knobs):
     from sga_amd.fused_step import FusedSparseStep
     segs, n = _segments(sizes, vary=vary)
     gen = torch.Generator().manual_seed(1234)
@@ -39,8 +39,8 @@ def _run(dev, sizes, steps, ratio, gdtype, vdtype, score="abs_g", seed0=0, vary=
     for step in range(1, steps + 1):
         g = student_t(n, seed0 + step - 1).to(gdtype)
         idx_ref, val_ref, mask_ref, th_ref = OF.fused_sparse_step(
-            g, r, p, m, v, segs, step, k=k, score=score, values_dtype=vdtype)
-        idx, vals = fs.step(g.to(dev), dr, dp, dm, dv, step, k=k, score=score)
+            g, r, p, m, v, segs, step, k=k, score=score, values_dtype=vdtype, **knobs)
+        idx, vals = fs.step(g.to(dev), dr, dp, dm, dv, step, k=k, score=score, **knobs)
         res = fs.read_result()
         assert res.status == 0 and res.nonfinite == 0 and res.n_selected == k
         assert expect_path is None or res.path == expect_path
@@ -89,6 +89,41 @@ def test_adam_scores_one_sweep_path_tensor_boundaries(dev, score):
     sizes = [300_000, 128, 37, 700_000, 3, 1024, 250_001, 130, 5, 60_000]
     _run(dev, sizes, 2, 1.0, torch.bfloat16, torch.bfloat16, score=score, vary=True,
          expect_path=1)
+
+
+@pytest.mark.parametrize("score", ["abs_g", "update", "coi"])
+@pytest.mark.parametrize("knobs", [dict(optimizer="adams"),
+                                   dict(optimizer="adamw", fold=True, interval=4.0),
+                                   dict(optimizer="adams", fold=True, interval=3.0, coeff=0.5)])
+def test_adams_and_fold_knobs(dev, score, knobs):
+    """The fused step under AdamS (v rebuilt from the pre-commit m, no bias
+    corrections: adams.py:87-213; the Adam-normalised scores through v := m*m,
+    bc := 1: replay.py:486-505), with the residual-mean fold of the new
+    residual (true division, adamw_torch.py:88-91; interval 3 is not a power
+    of two) and a clip coefficient, below and above the one-sweep select's
+    size, every output bit for bit over several steps."""
+    _run(dev, [200_000, 1024, 100_000], 3, 1.0, torch.bfloat16, torch.bfloat16, score=score,
+         **knobs)
+    _run(dev, [600_000, 130, 37, 500_000, 3, 1024, 100_001], 2, 1.0, torch.float32, torch.float32,
+         score=score, vary=True, expect_path=1, **knobs)
+
+
+def test_fused_step_refuses_dual_lr_and_unknown_flags(dev):
+    from sga_amd import _lib as L
+    from sga_amd.fused_step import FusedSparseStep
+    segs, n = _segments([4096])
+    fs = FusedSparseStep(n, segs, dev)
+    z = torch.zeros(n, device=dev)
+    with pytest.raises(ValueError, match="requires a full step"):
+        fs.step(z, z.clone(), z.clone(), z.clone(), z.clone(), 1, k=4, inactive_lr_scale=0.5)
+    with pytest.raises(ValueError, match="interval"):
+        fs.step(z, z.clone(), z.clone(), z.clone(), z.clone(), 1, k=4, fold=True, interval=0.0)
+    lib = L.load()
+    rc = lib.sga_fused_sparse_step(L.ptr(z), 0, L.ptr(z), L.ptr(z), L.ptr(z), L.ptr(z), n, 4,
+                                   L.ptr(fs._seg_dev), 1, 1, L.ptr(fs.idx), L.ptr(fs.values), 1,
+                                   None, 1.0, 1.0, 1, L.GC_LR_SPLIT, 1.0, None, L.ptr(fs.ws),
+                                   fs.ws_bytes, L.stream())
+    assert rc == -1 and b"requires a full step" in lib.sga_last_error()
 
 
 def test_tie_heavy_gradients(dev):
@@ -180,8 +215,9 @@ def test_randomized_configurations(dev, seed):
     """Seeded random draws of everything at once: tensor sizes (1 .. 700k
     elements, shuffled), per-tensor hyper-parameters (beta1 = 0 and eps = 1e-15
     included), score, gradient / value dtypes, ratio, and the magnitude of the
-    gradients, moments and residual (1e-12 .. 10, some all zero) -- three steps
-    each, every output bit for bit."""
+    gradients, moments and residual (1e-12 .. 10, some all zero), optimizer
+    (AdamW / AdamS), fold and clip coefficient -- three steps each, every
+    output bit for bit."""
     import random
     from sga_amd.fused_step import FusedSparseStep
     rng = random.Random(seed)
@@ -211,11 +247,13 @@ def test_randomized_configurations(dev, seed):
     dp, dm, dv, dr = (t.to(dev) for t in (p, m, v, r))
     fs = FusedSparseStep(n, segs, dev, values_dtype=vdtype, want_mask=True)
     k = SEL.k_for(n, rng.choice([0.1, 1.0, 10.0]))
+    knobs = dict(optimizer=rng.choice(["adamw", "adams"]), fold=rng.choice([False, True]),
+                 interval=rng.choice([2.0, 3.0, 16.0]), coeff=rng.choice([1.0, 0.37]))
     for step in range(1, 4):
         g = (student_t(n, seed * 10 + step) * (gscale / 1e-3)).to(gdtype)
         idx_ref, val_ref, mask_ref, th_ref = OF.fused_sparse_step(
-            g, r, p, m, v, segs, step, k=k, score=score, values_dtype=vdtype)
-        idx, vals = fs.step(g.to(dev), dr, dp, dm, dv, step, k=k, score=score)
+            g, r, p, m, v, segs, step, k=k, score=score, values_dtype=vdtype, **knobs)
+        idx, vals = fs.step(g.to(dev), dr, dp, dm, dv, step, k=k, score=score, **knobs)
         res = fs.read_result()
         assert res.status == 0 and res.thresh == th_ref, (step, res.thresh, th_ref)
         assert torch.equal(idx.cpu(), idx_ref) and torch.equal(fs.mask.cpu().bool(), mask_ref), step
