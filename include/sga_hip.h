@@ -30,6 +30,12 @@ extern "C" {
 #define SGA_SCORE_ABS_G 1
 #define SGA_SCORE_ABS_M 2
 #define SGA_SCORE_COI 3
+/* Two benchmark scores with NO counterpart in the reference's registry
+ * (scores.py:93-116), accepted by the fused step and the replay re-selection
+ * only: the residual-blind |g| (the recorded gradient alone ranks, while the
+ * residual keeps accumulating) and the literal |g + r| / sqrt(v + eps). */
+#define SGA_SCORE_ABS_G_BLIND 4
+#define SGA_SCORE_GR_OVER_SQRT_V 5
 
 /* grad-correct flags: constexprs of _grad_correct_kernel, adamw.py:88-106 */
 #define SGA_GC_HAS_MASK 1

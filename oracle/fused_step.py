@@ -30,7 +30,8 @@ def fused_sparse_step(g, resid, p, m, v, segments, step, ratio_percent=None,
     resid    : flat fp32 residual, updated in place (new residual)
     p, m, v  : flat fp32 state, updated in place
     segments : list of dicts {"start","n","lr","b1","b2","eps","wd"}
-    score    : "abs_g" (= |g+r|), "update", "coi", "abs_m"
+    score    : "abs_g" (= |g+r|), "update", "coi", "abs_m", or one of the two
+               build-side benchmark scores of ``scores.EXTRA_SCORES``
     optimizer: "adamw" | "adams" -- AdamS scores through the replay-side
                routing v := m*m, bc := 1 (replay.py:486-505) and commits with
                ``adams_grad_correct`` (adams_torch.py:34-85)
@@ -38,7 +39,8 @@ def fused_sparse_step(g, resid, p, m, v, segments, step, ratio_percent=None,
     Returns (idx int32[k], values[k], mask bool[N], thresh).
     """
     n = resid.numel()
-    resid.add_(g.float())                      # buf = r + g (one fp32 add)
+    gf = g.float()
+    resid.add_(gf)                             # buf = r + g (one fp32 add)
     buf = resid
     if score == "abs_g":
         sc = buf.abs()
@@ -48,10 +50,9 @@ def fused_sparse_step(g, resid, p, m, v, segments, step, ratio_percent=None,
             a, b = s["start"], s["start"] + s["n"]
             bc1 = 1.0 - s["b1"] ** step
             bc2 = 1.0 - s["b2"] ** step
-            sc[a:b] = S.score_formula(
-                score, p[a:b], m[a:b], v[a:b], buf[a:b], s["b1"], s["b2"],
-                s["eps"], s["wd"], bc1, bc2, optimizer,
-                update_includes_wd=True).abs()
+            sc[a:b] = S.step_score(
+                score, p[a:b], m[a:b], v[a:b], buf[a:b], gf[a:b], s["b1"],
+                s["b2"], s["eps"], s["wd"], bc1, bc2, optimizer)
     if k is None:
         k = SEL.k_for(n, ratio_percent)
     mask, thresh = SEL.select_topk_flat(sc, k)

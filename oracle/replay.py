@@ -142,11 +142,12 @@ def group_replay(entries, w0, m0, v0, sel0, configs, g_steps, metas, t0,
                 a, b = e["a"], e["a"] + e["n"]
                 bc1c, bc2c = bc_pair(c.optimizer, count, e["b1"], e["b2"])
                 q = (gd[a:b] + s["res"][a:b]) * coefs[ci]
-                sc = S.score_formula(c.score, s["w"][a:b], s["m"][a:b],
-                                     s["v"][a:b], q, e["b1"], e["b2"],
-                                     e["eps"], e["wd"], bc1c, bc2c,
-                                     c.optimizer, update_includes_wd=True)
-                score[a:b] = sc.abs().float()
+                # the residual-blind variant (build-side) ranks q without its residual term
+                blind = gd[a:b] * coefs[ci]
+                score[a:b] = S.step_score(c.score, s["w"][a:b], s["m"][a:b],
+                                          s["v"][a:b], q, blind, e["b1"],
+                                          e["b2"], e["eps"], e["wd"], bc1c,
+                                          bc2c, c.optimizer).float()
             newsel, _ = SEL.select_topk_flat(score, ks[c.ratio])
             if c.dual_lr != 1.0:
                 out_sel[ci] = s["sel"]

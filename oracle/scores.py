@@ -105,6 +105,24 @@ def score_formula(name, w, m, v, g, b1, b2, eps, wd, bc1, bc2, optimizer,
 
 
 def abs_gr_over_sqrt_v(g_plus_r, v, eps):
-    """Build-side literal ``|g+r| / sqrt(v + eps)``.  No reference
+    """Build-side literal ``|g+r| / sqrt(v + eps)`` as three separately rounded
+    fp32 ops (add, correctly rounded root, divide).  No reference
     implementation exists: PARITY UNPINNED (closed form only)."""
-    return g_plus_r.abs() / torch.sqrt(v + eps)
+    return g_plus_r.abs() / ieee.sqrt(v + eps)
+
+
+EXTRA_SCORES = ("abs_g_blind", "abs_gr_over_sqrt_v")
+
+
+def step_score(name, w, m, v, q, g_alone, b1, b2, eps, wd, bc1, bc2, optimizer):
+    """|score| as the fused step and the replay re-selection rank it: the
+    four registry names through ``score_formula`` (update with its wd term),
+    plus the two build-side benchmark scores -- ``abs_g_blind`` = |g_alone|
+    (the gradient term without the residual) and ``abs_gr_over_sqrt_v`` (AdamS:
+    v := m*m).  PARITY UNPINNED for the two extras (no reference counterpart)."""
+    if name == "abs_g_blind":
+        return g_alone.abs()
+    if name == "abs_gr_over_sqrt_v":
+        return abs_gr_over_sqrt_v(q, v if optimizer == "adamw" else m * m, eps)
+    return score_formula(name, w, m, v, q, b1, b2, eps, wd, bc1, bc2, optimizer,
+                         update_includes_wd=True).abs()

@@ -53,8 +53,10 @@ __device__ __forceinline__ float coi_u0(float m, float v, const Hyper& h) {
 // that ranks by them gets the same bits, the bits of the IEEE-754 evaluation.
 template <int SCORE>
 __device__ __forceinline__ float score_value(float q, float p, float m, float v, const Hyper& h) {
-  if (SCORE == SGA_SCORE_ABS_G) return fabsf(q);
+  if (SCORE == SGA_SCORE_ABS_G || SCORE == SGA_SCORE_ABS_G_BLIND) return fabsf(q);
   if (SCORE == SGA_SCORE_ABS_M) return fabsf(m);
+  // |g + r| / sqrt(v + eps): no counterpart in the reference's registry (a benchmark score)
+  if (SCORE == SGA_SCORE_GR_OVER_SQRT_V) return __fdiv_rn(fabsf(q), sqrt_rn(v + h.eps));
   const Commit c = adamw_commit(p, q, m, v, h);
   if (SCORE == SGA_SCORE_UPDATE) return c.upd;
   return fabsf(c.u - coi_u0(m, v, h));

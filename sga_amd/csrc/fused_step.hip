@@ -17,7 +17,9 @@ __device__ __forceinline__ void load_g(const void* g, int64_t i, int64_t n, floa
   else ld_f32<FULL>(reinterpret_cast<const float*>(g), i, n, out, vec);
 }
 
-// Key source for the select sweeps.
+// Key source for the select sweeps.  Which arrays a score reads:
+//   abs_g  g r          abs_m  m              update  g r p m v      coi  g r m v
+//   abs_g_blind  g      abs_gr_over_sqrt_v  g r v   (AdamS: m stands in for v = m*m)
 template <bool BF16G, int SCORE>
 struct SrcFused {
   const void* g;
@@ -32,88 +34,80 @@ struct SrcFused {
   // Stepwise interface of the one-sweep select.
   struct Raw { RawG g; F4 r, p, m, v; };
   struct Chunk { int64_t sh; };
-  static constexpr bool kHyper = SCORE == SGA_SCORE_UPDATE || SCORE == SGA_SCORE_COI;
-  // measured: the |g + r| sweep is bound by DRAM and loses ~5 % with more slabs in flight; the
-  // Adam-normalised scores are bound by arithmetic and gain from hiding the load latency
-  #ifndef SGA_AHEAD_ABSG
-#define SGA_AHEAD_ABSG 1
-#endif
-#ifndef SGA_AHEAD_HYPER
-#define SGA_AHEAD_HYPER 2
-#endif
-  static constexpr int kAhead = kHyper ? SGA_AHEAD_HYPER : SGA_AHEAD_ABSG;
+  // scores that need the tensor's hyper-parameters
+  static constexpr bool kHyper = SCORE == SGA_SCORE_UPDATE || SCORE == SGA_SCORE_COI ||
+                                 SCORE == SGA_SCORE_GR_OVER_SQRT_V;
+  static constexpr bool kNeedG = SCORE != SGA_SCORE_ABS_M;
+  static constexpr bool kNeedR = kNeedG && SCORE != SGA_SCORE_ABS_G_BLIND;
+  static constexpr bool kNeedP = SCORE == SGA_SCORE_UPDATE;
+  static constexpr bool kNeedV = kHyper;                       // v, or m in its place under AdamS
+  __device__ __forceinline__ bool need_m() const {
+    return SCORE == SGA_SCORE_UPDATE || SCORE == SGA_SCORE_COI || SCORE == SGA_SCORE_ABS_M ||
+           (kNeedV && adams);
+  }
+  // measured: look-ahead makes no difference beyond one slab for |g + r| and two for the chains
+  static constexpr int kAhead = kHyper ? 2 : 1;
   __device__ __forceinline__ Chunk chunk_begin(int64_t c) {
     const int64_t i0 = uniform_i64(c) * kChunk;
     return Chunk{(i0 >> kPackRunLog) * pack_extra};
   }
-  // The tensor of the chunk's first element: a search over the segment table, placed by the
-  // sweep behind the chunk's first loads so that their latencies overlap.
+  // The tensor of the chunk's first element (a walk from the segment directory).
   __device__ __forceinline__ void chunk_hyper(int64_t c) {
     if (kHyper) sc.seek_uniform(uniform_i64(c) * kChunk);
   }
   template <bool FULL>
   __device__ __forceinline__ void fetch(const Chunk& ck, int64_t i, int64_t n, Raw& w) {
-    fetch_g<BF16G, FULL>(g, i, n, vec, w.g);
-    w.r = ldraw_f32<FULL>(r + ck.sh, i, n, vec);
-    if (SCORE == SGA_SCORE_ABS_G) return;
-    w.m = ldraw_f32<FULL>(m + ck.sh, i, n, vec);
-    if (SCORE != SGA_SCORE_ABS_M) {
-      w.p = ldraw_f32<FULL>(p + ck.sh, i, n, vec);
-      w.v = ldraw_f32<FULL>(v + ck.sh, i, n, vec);
-    }
+    if (kNeedG) fetch_g<BF16G, FULL>(g, i, n, vec, w.g);
+    if (kNeedR) w.r = ldraw_f32<FULL>(r + ck.sh, i, n, vec);
+    if (need_m()) w.m = ldraw_f32<FULL>(m + ck.sh, i, n, vec);
+    if (kNeedP) w.p = ldraw_f32<FULL>(p + ck.sh, i, n, vec);
+    if (kNeedV && !adams) w.v = ldraw_f32<FULL>(v + ck.sh, i, n, vec);
   }
   template <bool FULL>
   __device__ __forceinline__ void keys(const Chunk& ck, int64_t i, int64_t n, const Raw& w,
                                        uint32_t key[4]) {
-    float gg[4], rr[4];
-    unpack_g<BF16G, FULL>(w.g, gg);
-    unpack_f32(w.r, rr);
-    if (SCORE == SGA_SCORE_ABS_G) {
+    float q[4] = {0, 0, 0, 0}, rr[4] = {0, 0, 0, 0};
+    float pp[4] = {0, 0, 0, 0}, mm[4] = {0, 0, 0, 0}, vv[4] = {0, 0, 0, 0};
+    if (kNeedG) unpack_g<BF16G, FULL>(w.g, q);
+    if (kNeedR) {
+      unpack_f32(w.r, rr);
 #pragma unroll
-      for (int e = 0; e < 4; ++e) key[e] = abs_key(rr[e] + gg[e]);
+      for (int e = 0; e < 4; ++e) q[e] = rr[e] + q[e];
+    }
+    if (need_m()) unpack_f32(w.m, mm);
+    if (!kHyper) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) key[e] = abs_key(SCORE == SGA_SCORE_ABS_M ? mm[e] : q[e]);
       return;
     }
-    float pp[4] = {0, 0, 0, 0}, mm[4], vv[4] = {0, 0, 0, 0};
-    unpack_f32(w.m, mm);
-    if (SCORE == SGA_SCORE_ABS_M) {
-#pragma unroll
-      for (int e = 0; e < 4; ++e) key[e] = abs_key(mm[e]);
-      return;
-    }
-    if (SCORE != SGA_SCORE_ABS_M) {
-      unpack_f32(w.p, pp);
-      unpack_f32(w.v, vv);
-    }
-    float q[4];
-#pragma unroll
-    for (int e = 0; e < 4; ++e) q[e] = rr[e] + gg[e];
+    if (kNeedP) unpack_f32(w.p, pp);
     if (adams) {
 #pragma unroll
       for (int e = 0; e < 4; ++e) vv[e] = mm[e] * mm[e];
+    } else {
+      unpack_f32(w.v, vv);
     }
     slab_score_keys<SCORE, FULL>(sc, adams, i, n, q, pp, mm, vv, key);
   }
   template <bool FULL = false>
   __device__ __forceinline__ void load(int64_t i, int64_t n, uint32_t key[4]) {
     const int64_t sh = pack_shift<FULL>(i, pack_extra);
-    const float* r = this->r + sh;
-    const float* p = this->p + sh;
-    const float* m = this->m + sh;
-    const float* v = this->v + sh;
-    float gg[4], rr[4];
-    load_g<BF16G, FULL>(g, i, n, gg, vec);
-    ld_f32<FULL>(r, i, n, rr, vec);
-    if (SCORE == SGA_SCORE_ABS_G) {
+    float q[4] = {0, 0, 0, 0}, rr[4] = {0, 0, 0, 0};
+    float pp[4] = {0, 0, 0, 0}, mm[4] = {0, 0, 0, 0}, vv[4] = {0, 0, 0, 0};
+    if (kNeedG) load_g<BF16G, FULL>(g, i, n, q, vec);
+    if (kNeedR) {
+      ld_f32<FULL>(r + sh, i, n, rr, vec);
 #pragma unroll
-      for (int e = 0; e < 4; ++e) key[e] = abs_key(rr[e] + gg[e]);
+      for (int e = 0; e < 4; ++e) q[e] = rr[e] + q[e];
+    }
+    if (need_m()) ld_f32<FULL>(m + sh, i, n, mm, vec);
+    if (!kHyper) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) key[e] = abs_key(SCORE == SGA_SCORE_ABS_M ? mm[e] : q[e]);
       return;
     }
-    float pp[4] = {0, 0, 0, 0}, mm[4], vv[4] = {0, 0, 0, 0};
-    ld_f32<FULL>(m, i, n, mm, vec);
-    if (SCORE != SGA_SCORE_ABS_M) {
-      ld_f32<FULL>(p, i, n, pp, vec);
-      ld_f32<FULL>(v, i, n, vv, vec);
-    }
+    if (kNeedP) ld_f32<FULL>(p + sh, i, n, pp, vec);
+    if (!adams) ld_f32<FULL>(v + sh, i, n, vv, vec);
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
       if (FULL || i + e < n) {
@@ -121,7 +115,7 @@ struct SrcFused {
         Hyper h = sc.h;
         float ve = vv[e];
         if (adams) { ve = mm[e] * mm[e]; h.bc1 = 1.0f; h.bc2 = 1.0f; }
-        key[e] = score_key<SCORE>(rr[e] + gg[e], pp[e], mm[e], ve, h);
+        key[e] = score_key<SCORE>(q[e], pp[e], mm[e], ve, h);
       } else {
         key[e] = 0u;
       }
@@ -243,6 +237,7 @@ __device__ __forceinline__ void final_chunk(const FinalArgs& a, int64_t c, Chunk
         valid[e] = FULL || i + e < n;
         q[e] = rr[it][e] + gg[it][e];
         if (SCORE == SGA_SCORE_ABS_G) key[e] = abs_key(q[e]);
+        else if (SCORE == SGA_SCORE_ABS_G_BLIND) key[e] = abs_key(gg[it][e]);
         else if (SCORE == SGA_SCORE_ABS_M) key[e] = abs_key(mm[it][e]);
         else {
           // only when the one-sweep select is off or failed: a per-lane cursor
@@ -327,7 +322,8 @@ __device__ __forceinline__ void final_chunk(const FinalArgs& a, int64_t c, Chunk
 // keys are formed again here).
 // (five waves per SIMD wherever the key is not an Adam-normalised chain formed in this kernel)
 template <bool BF16G, bool BF16V, int SCORE, bool PLANES>
-__global__ __launch_bounds__(kBlock, (PLANES || SCORE == SGA_SCORE_ABS_G || SCORE == SGA_SCORE_ABS_M) ? 5 : 1)
+__global__ __launch_bounds__(kBlock, (PLANES || SCORE == SGA_SCORE_ABS_G || SCORE == SGA_SCORE_ABS_M ||
+                                      SCORE == SGA_SCORE_ABS_G_BLIND) ? 5 : 1)
 void k_fused_final(
     FinalArgs a, const sga_segment* __restrict__ segs, int n_segs,
     const SelState* __restrict__ st, const uint32_t* __restrict__ tile_sel,
@@ -441,7 +437,8 @@ static int fused_entry(const char* who, const void* g, int g_dtype, float* resid
   if (!g || !resid || !p || !m || !v || !segs || !idx_out || !values_out || n < 1 ||
       n >= (1ll << 31) || k < 1 || k > n || n_segs < 1 ||
       (g_dtype != SGA_F32 && g_dtype != SGA_BF16) ||
-      (values_dtype != SGA_F32 && values_dtype != SGA_BF16) || score_id < 0 || score_id > 3) {
+      (values_dtype != SGA_F32 && values_dtype != SGA_BF16) || score_id < 0 ||
+      score_id > SGA_SCORE_GR_OVER_SQRT_V) {
     set_error("%s: bad argument (n=%lld k=%lld n_segs=%d score=%d; need 1 <= k <= n < 2^31)", who,
               (long long)n, (long long)k, n_segs, score_id);
     return SGA_ERR_ARG;
@@ -463,7 +460,9 @@ static int fused_entry(const char* who, const void* g, int g_dtype, float* resid
     case 0: SGA_RUN(BG, BV, 0);               \
     case 1: SGA_RUN(BG, BV, 1);               \
     case 2: SGA_RUN(BG, BV, 2);               \
-    default: SGA_RUN(BG, BV, 3);              \
+    case 3: SGA_RUN(BG, BV, 3);               \
+    case 4: SGA_RUN(BG, BV, 4);               \
+    default: SGA_RUN(BG, BV, 5);              \
   }
   if (bg && bv) { SGA_RUN_SC(true, true) }
   else if (bg) { SGA_RUN_SC(true, false) }

@@ -392,7 +392,10 @@ __global__ __launch_bounds__(kBlock) void k_dense_step(const void* __restrict__ 
 }
 
 // --------------------------------------------------- pass 2 score source
-// key = |registry score| of q = (gd + res) * coef against one config's state.
+// key = |score| of q = (gd + res) * coef against one config's state; the
+// residual-blind |g| takes q = gd * coef.  Arrays read: as for the fused step
+// (abs_g: g res; abs_m: m; update: g res w m v; coi: g res m v;
+// abs_g_blind: g; abs_gr_over_sqrt_v: g res v; AdamS: m in the place of v).
 template <bool BF16G, int SCORE>
 struct SrcReplay {
   const void* g;
@@ -410,7 +413,17 @@ struct SrcReplay {
   // Stepwise interface of the one-sweep select.
   struct Raw { RawG g; F4 r, w, m, v; };
   struct Chunk { int64_t sh; float coef; };
-  static constexpr bool kHyper = SCORE == SGA_SCORE_UPDATE || SCORE == SGA_SCORE_COI;
+  static constexpr bool kHyper = SCORE == SGA_SCORE_UPDATE || SCORE == SGA_SCORE_COI ||
+                                 SCORE == SGA_SCORE_GR_OVER_SQRT_V;
+  static constexpr bool kNeedG = SCORE != SGA_SCORE_ABS_M;
+  static constexpr bool kNeedR = kNeedG && SCORE != SGA_SCORE_ABS_G_BLIND;
+  static constexpr bool kNeedW = SCORE == SGA_SCORE_UPDATE;
+  static constexpr bool kNeedV = kHyper;
+  __device__ __forceinline__ bool need_r() const { return kNeedR && !res_zero; }
+  __device__ __forceinline__ bool need_m() const {
+    return SCORE == SGA_SCORE_UPDATE || SCORE == SGA_SCORE_COI || SCORE == SGA_SCORE_ABS_M ||
+           (kNeedV && adams);
+  }
   // measured: |q| mostly reads the bf16 gradient alone and is bound by latency, four slabs ahead
   // is 25 % faster than one; the Adam-normalised scores fit two slabs in the register budget
   static constexpr int kAhead = kHyper ? 2 : kChunkIters;
@@ -423,76 +436,65 @@ struct SrcReplay {
   }
   template <bool FULL>
   __device__ __forceinline__ void fetch(const Chunk& ck, int64_t i, int64_t n, Raw& t) {
-    fetch_g<BF16G, FULL>(g, i, n, vec, t.g);
-    if (!res_zero) t.r = ldraw_f32<FULL>(res + ck.sh, i, n, vec);
-    if (SCORE == SGA_SCORE_ABS_G) return;
-    t.m = ldraw_f32<FULL>(m + ck.sh, i, n, vec);
-    if (SCORE != SGA_SCORE_ABS_M) {
-      t.w = ldraw_f32<FULL>(w + ck.sh, i, n, vec);
-      if (!adams) t.v = ldraw_f32<FULL>(v + ck.sh, i, n, vec);
-    }
+    if (kNeedG) fetch_g<BF16G, FULL>(g, i, n, vec, t.g);
+    if (need_r()) t.r = ldraw_f32<FULL>(res + ck.sh, i, n, vec);
+    if (need_m()) t.m = ldraw_f32<FULL>(m + ck.sh, i, n, vec);
+    if (kNeedW) t.w = ldraw_f32<FULL>(w + ck.sh, i, n, vec);
+    if (kNeedV && !adams) t.v = ldraw_f32<FULL>(v + ck.sh, i, n, vec);
   }
-  template <bool FULL>
-  __device__ __forceinline__ void keys(const Chunk& ck, int64_t i, int64_t n, const Raw& t,
-                                       uint32_t key[4]) {
-    float gd[4], rr[4] = {0, 0, 0, 0};
-    unpack_g<BF16G, FULL>(t.g, gd);
+  // q of the four coordinates from the raw gradient quad and residual
+  __device__ __forceinline__ void form_q(float gd[4], const float rr[4], float coef, float q[4]) const {
     if (coef_dense != 1.0f) {
 #pragma unroll
       for (int e = 0; e < 4; ++e) gd[e] = __fdiv_rn(gd[e], coef_dense);
     }
-    if (!res_zero) unpack_f32(t.r, rr);
-    float q[4];
 #pragma unroll
-    for (int e = 0; e < 4; ++e) q[e] = (gd[e] + rr[e]) * ck.coef;
-    if (SCORE == SGA_SCORE_ABS_G) {
+    for (int e = 0; e < 4; ++e) q[e] = (gd[e] + rr[e]) * coef;
+  }
+  template <bool FULL>
+  __device__ __forceinline__ void keys(const Chunk& ck, int64_t i, int64_t n, const Raw& t,
+                                       uint32_t key[4]) {
+    float gd[4] = {0, 0, 0, 0}, rr[4] = {0, 0, 0, 0}, q[4] = {0, 0, 0, 0};
+    float ww[4] = {0, 0, 0, 0}, mm[4] = {0, 0, 0, 0}, vv[4] = {0, 0, 0, 0};
+    if (kNeedG) {
+      unpack_g<BF16G, FULL>(t.g, gd);
+      if (need_r()) unpack_f32(t.r, rr);
+      form_q(gd, rr, ck.coef, q);
+    }
+    if (need_m()) unpack_f32(t.m, mm);
+    if (!kHyper) {
 #pragma unroll
-      for (int e = 0; e < 4; ++e) key[e] = abs_key(q[e]);
+      for (int e = 0; e < 4; ++e) key[e] = abs_key(SCORE == SGA_SCORE_ABS_M ? mm[e] : q[e]);
       return;
     }
-    float ww[4] = {0, 0, 0, 0}, mm[4], vv[4] = {0, 0, 0, 0};
-    unpack_f32(t.m, mm);
-    if (SCORE == SGA_SCORE_ABS_M) {
-#pragma unroll
-      for (int e = 0; e < 4; ++e) key[e] = abs_key(mm[e]);
-      return;
-    }
-    if (SCORE != SGA_SCORE_ABS_M) {
-      unpack_f32(t.w, ww);
-      if (!adams) unpack_f32(t.v, vv);
-    }
+    if (kNeedW) unpack_f32(t.w, ww);
     if (adams) {
 #pragma unroll
       for (int e = 0; e < 4; ++e) vv[e] = mm[e] * mm[e];
+    } else {
+      unpack_f32(t.v, vv);
     }
     slab_score_keys<SCORE, FULL>(sc, adams, i, n, q, ww, mm, vv, key);
   }
   template <bool FULL = false>
   __device__ __forceinline__ void load(int64_t i, int64_t n, uint32_t key[4]) {
     const int64_t sh = pack_shift<FULL>(i, pack_extra);
-    const float* res = this->res + sh;
-    const float* w = this->w + sh;
-    const float* m = this->m + sh;
-    const float* v = this->v + sh;
-    float gd[4], rr[4];
-    load_gd<BF16G, FULL>(g, i, n, coef_dense == 1.0f ? 1.0f : 0.0f, coef_dense, gd, vec);
-    if (res_zero) rr[0] = rr[1] = rr[2] = rr[3] = 0.0f;
-    else ld_f32<FULL>(res, i, n, rr, vec);
-    const float coef = coef_f[0];
-    float q[4];
+    float gd[4] = {0, 0, 0, 0}, rr[4] = {0, 0, 0, 0}, q[4] = {0, 0, 0, 0};
+    float ww[4] = {0, 0, 0, 0}, mm[4] = {0, 0, 0, 0}, vv[4] = {0, 0, 0, 0};
+    if (kNeedG) {
+      if (BF16G) ld_bf16<FULL>(reinterpret_cast<const uint16_t*>(g), i, n, gd, vec);
+      else ld_f32<FULL>(reinterpret_cast<const float*>(g), i, n, gd, vec);
+      if (need_r()) ld_f32<FULL>(res + sh, i, n, rr, vec);
+      form_q(gd, rr, coef_f[0], q);
+    }
+    if (need_m()) ld_f32<FULL>(m + sh, i, n, mm, vec);
+    if (!kHyper) {
 #pragma unroll
-    for (int e = 0; e < 4; ++e) q[e] = (gd[e] + rr[e]) * coef;
-    if (SCORE == SGA_SCORE_ABS_G) {
-#pragma unroll
-      for (int e = 0; e < 4; ++e) key[e] = abs_key(q[e]);
+      for (int e = 0; e < 4; ++e) key[e] = abs_key(SCORE == SGA_SCORE_ABS_M ? mm[e] : q[e]);
       return;
     }
-    float ww[4] = {0, 0, 0, 0}, mm[4], vv[4] = {0, 0, 0, 0};
-    ld_f32<FULL>(m, i, n, mm, vec);
-    if (SCORE != SGA_SCORE_ABS_M) {
-      ld_f32<FULL>(w, i, n, ww, vec);
-      if (!adams) ld_f32<FULL>(v, i, n, vv, vec);
-    }
+    if (kNeedW) ld_f32<FULL>(w + sh, i, n, ww, vec);
+    if (!adams) ld_f32<FULL>(v + sh, i, n, vv, vec);
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
       if (FULL || i + e < n) {
@@ -714,7 +716,7 @@ extern "C" int sga_replay_reselect(const void* g, int g_dtype, const float* res,
                                    int res_zero, uint32_t* sel_out, sga_select_result* result, void* ws,
                                    size_t ws_bytes, void* stream) {
   if (!g || !res || !w || !m || !v || !segs || !coef_f || !sel_out || n < 1 || n >= (1ll << 31) ||
-      k < 1 || k > n || n_segs < 1 || score_id < 0 || score_id > 3 ||
+      k < 1 || k > n || n_segs < 1 || score_id < 0 || score_id > SGA_SCORE_GR_OVER_SQRT_V ||
       (g_dtype != SGA_F32 && g_dtype != SGA_BF16)) {
     set_error("sga_replay_reselect: bad argument (n=%lld k=%lld)", (long long)n, (long long)k);
     return SGA_ERR_ARG;
@@ -727,9 +729,11 @@ extern "C" int sga_replay_reselect(const void* g, int g_dtype, const float* res,
   hipStream_t s = (hipStream_t)stream;
 #define SGA_RS(BG, SC) return run_reselect<BG, SC>(g, res, w, m, v, n, k, segs, n_segs, coef_f, coef_dense, adams, packed, res_zero, sel_out, result, sw, s)
   if (g_dtype == SGA_BF16) {
-    switch (score_id) { case 0: SGA_RS(true, 0); case 1: SGA_RS(true, 1); case 2: SGA_RS(true, 2); default: SGA_RS(true, 3); }
+    switch (score_id) { case 0: SGA_RS(true, 0); case 1: SGA_RS(true, 1); case 2: SGA_RS(true, 2);
+                        case 3: SGA_RS(true, 3); case 4: SGA_RS(true, 4); default: SGA_RS(true, 5); }
   } else {
-    switch (score_id) { case 0: SGA_RS(false, 0); case 1: SGA_RS(false, 1); case 2: SGA_RS(false, 2); default: SGA_RS(false, 3); }
+    switch (score_id) { case 0: SGA_RS(false, 0); case 1: SGA_RS(false, 1); case 2: SGA_RS(false, 2);
+                        case 3: SGA_RS(false, 3); case 4: SGA_RS(false, 4); default: SGA_RS(false, 5); }
   }
 #undef SGA_RS
 }

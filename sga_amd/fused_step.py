@@ -6,7 +6,7 @@ import ctypes as C
 import torch
 
 from . import _lib as L
-from .scores import SCORE_MAP
+from .scores import STEP_SCORE_MAP as SCORE_MAP
 from .selection import read_result
 
 

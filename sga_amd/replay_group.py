@@ -11,7 +11,7 @@ import math
 import torch
 
 from . import _lib as L
-from .scores import SCORE_MAP
+from .scores import STEP_SCORE_MAP as SCORE_MAP
 from .selection import read_result
 
 MAX_CONFIGS = 16

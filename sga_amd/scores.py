@@ -9,6 +9,12 @@ import torch
 from . import _lib as L
 
 SCORE_MAP = {"update": 0, "abs_g": 1, "abs_m": 2, "coi": 3}   # adamw.py:75-80
+# Two benchmark scores OUTSIDE the reference's registry (not returned by
+# score_names / get_score_spec): the fused step and the replay group accept
+# them by these names.  abs_g_blind ranks by the recorded gradient alone while
+# the residual keeps accumulating; abs_gr_over_sqrt_v is |g + r| / sqrt(v + eps).
+EXTRA_SCORE_MAP = {"abs_g_blind": 4, "abs_gr_over_sqrt_v": 5}
+STEP_SCORE_MAP = dict(SCORE_MAP, **EXTRA_SCORE_MAP)
 
 
 @dataclass(frozen=True)

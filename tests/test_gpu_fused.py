@@ -108,6 +108,20 @@ def test_adams_and_fold_knobs(dev, score, knobs):
          score=score, vary=True, expect_path=1, **knobs)
 
 
+@pytest.mark.parametrize("opt", ["adamw", "adams"])
+@pytest.mark.parametrize("score", ["abs_g_blind", "abs_gr_over_sqrt_v"])
+def test_benchmark_scores_outside_the_registry(dev, score, opt):
+    """The two build-side benchmark scores (the residual-blind |g| and the
+    literal |g + r| / sqrt(v + eps)): NO reference implementation exists, so
+    their parity is UNPINNED -- the device is compared with the closed form
+    restated on the CPU (one fp32 add, a correctly rounded root, one divide),
+    bit for bit, through the same exact-k selection, pack and commit."""
+    _run(dev, [200_000, 1024, 100_000], 3, 1.0, torch.bfloat16, torch.bfloat16, score=score,
+         optimizer=opt)
+    _run(dev, [600_000, 130, 37, 500_000, 3, 1024, 100_001], 3, 10.0, torch.float32, torch.float32,
+         score=score, vary=True, expect_path=1, optimizer=opt)
+
+
 def test_fused_step_refuses_dual_lr_and_unknown_flags(dev):
     from sga_amd import _lib as L
     from sga_amd.fused_step import FusedSparseStep

@@ -134,9 +134,9 @@ def _run_group(dev, cfg_specs, clip, W=9, bf16=False, t0=10, sizes=(400_000, 300
     dcfg = [Config(*c) for c in cfg_specs]
     sel0 = []
     for c in ocfg:
-        sc = OS.score_formula(c.score, w0, m0, v0, grads[0].float(), 0.9, 0.95, 1e-8, 0.1,
-                              *OR.bc_pair(c.optimizer, t0 + 1, 0.9, 0.95), c.optimizer,
-                              update_includes_wd=True).abs()
+        g0 = grads[0].float()
+        sc = OS.step_score(c.score, w0, m0, v0, g0, g0, 0.9, 0.95, 1e-8, 0.1,
+                           *OR.bc_pair(c.optimizer, t0 + 1, 0.9, 0.95), c.optimizer)
         sel0.append(SEL.select_topk_flat(sc, SEL.replay_k(n, c.ratio))[0])
     grp = ReplayGroup(entries, w0.to(dev), m0.to(dev), v0.to(dev), [s.to(dev) for s in sel0],
                       dcfg, t0, W)
@@ -264,6 +264,20 @@ def test_group_adam_scores_one_sweep_long_cycle(dev, opt):
     grp, out, w0 = _run_group(dev, specs, clip=0.3, W=18, bf16=False, sizes=_RAGGED)
     assert grp.last_select().path == 1
     _assert_group_equal(grp, out, specs)
+
+
+def test_group_benchmark_scores_outside_the_registry(dev):
+    """Replay arms ranked by the two build-side scores (residual-blind |g| and
+    |g + r| / sqrt(v + eps)): no reference counterpart, parity UNPINNED; checked
+    bit for bit against the closed form in the oracle's group loop, with a live
+    residual, clipping, AdamS and above the one-sweep select's size."""
+    specs = [("abs_g_blind", 1.0, 2), ("abs_gr_over_sqrt_v", 1.0, 4), ("abs_g_blind", 10.0, 3, "adams"),
+             ("abs_gr_over_sqrt_v", 0.1, 2, "adams", True), ("abs_g", 1.0, 2)]
+    grp, out, w0 = _run_group(dev, specs, clip=0.3, W=7, bf16=True, sizes=_RAGGED)
+    assert grp.last_select().path == 1
+    _assert_group_equal(grp, out, specs)
+    # the blind arm really ignores the residual: it differs from the |g + r| arm of the same shape
+    assert not torch.equal(grp.state[0]["sel"], grp.state[4]["sel"])
 
 
 @pytest.mark.parametrize("seed", range(6))

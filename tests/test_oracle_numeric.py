@@ -556,3 +556,24 @@ def test_torch_sqrt_deviation_is_bounded(monkeypatch):
         assert moved[name] <= max(16, k // 1000), (name, moved[name], k)
     print(f"torch.sqrt vs correctly rounded sqrt at n=2^22: {lanes} score lanes differ in the "
           f"last bits; top-{k} sets differ by {moved} coordinates (symmetric difference)")
+
+
+def test_benchmark_score_closed_forms():
+    """The two build-side benchmark scores have no reference implementation
+    (parity unpinned); their oracle is pinned only by the closed form in
+    float64: |q| / sqrt(v + eps) within a few fp32 roundings, and the blind
+    score is |g| itself."""
+    g = torch.Generator().manual_seed(3)
+    q = torch.randn(50_000, generator=g) * 1e-3
+    v = torch.rand(50_000, generator=g) * 1e-8
+    m = torch.randn(50_000, generator=g) * 1e-4
+    for eps in (1e-8, 1e-12):
+        got = S.abs_gr_over_sqrt_v(q, v, eps)
+        ref = q.double().abs() / (v.double() + eps).sqrt()
+        assert got.dtype == torch.float32
+        assert torch.allclose(got.double(), ref, rtol=4e-7, atol=0.0)
+        ad = S.step_score("abs_gr_over_sqrt_v", None, m, v, q, q, .9, .95, eps, .1, 1., 1., "adams")
+        refa = q.double().abs() / ((m * m).double() + eps).sqrt()
+        assert torch.allclose(ad.double(), refa, rtol=4e-7, atol=0.0)
+    assert torch.equal(S.step_score("abs_g_blind", None, m, v, q + 1.0, q, .9, .95, 1e-8, .1, 1.,
+                                    1., "adamw"), q.abs())
