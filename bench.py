@@ -29,6 +29,10 @@ sys.path.insert(0, ROOT)
 HBM_PEAK = 8.0e12          # MI355X HBM3E, B/s
 ALG_BYTES_FINAL = 34.0     # final sweep: read g,r,p,m,v (18) + write r,p,m,v (16)
 PROF_FINAL, PROF_SWEEP, PROF_PASS3, PROF_PASS1 = 0, 1, 2, 3     # include/sga_hip_bench.h
+# score axis of the replay configuration: |g| (residual-blind, a build-side score with no reference
+# counterpart), |g + r| (the registry's abs_g on the accumulated buffer) and the Adam-normalised
+# `update`
+REPLAY_SCORES = ("abs_g_blind", "abs_g", "update")
 
 
 def sweep_bytes_per_elem(score, g_bytes=2.0):
@@ -99,7 +103,8 @@ def cpu_baseline(sample_n, steps, ratio, score="abs_g"):
 def replay_bench(G=8, W=32, seed=4):
     """Fused offline replay on the Qwen3-0.6B shapes: a window of W recorded
     bf16 gradient steps resident in HBM, G configs drawn with a fixed seed from
-    score x ratio x cycle length; per-config fp32 w/m/v/residual + byte mask."""
+    score {|g|, |g+r|, update} x ratio {0.1, 1, 10} % x cycle length {1, 4, 16};
+    per-config fp32 w/m/v/residual + mask bit planes."""
     import random
     import torch
     from sga_amd import _lib as L
@@ -111,7 +116,7 @@ def replay_bench(G=8, W=32, seed=4):
     entries = [{"a": s["start"], "n": s["n"], "b1": s["b1"], "b2": s["b2"], "eps": s["eps"],
                 "wd": s["wd"]} for s in segs]
     rnd = random.Random(seed)
-    axes = [(sc, r, t) for sc in ("abs_g", "update", "coi") for r in (0.1, 1.0, 10.0)
+    axes = [(sc, r, t) for sc in REPLAY_SCORES for r in (0.1, 1.0, 10.0)
             for t in (1, 4, 16)]
     picks = rnd.sample(axes, G)
     cfgs = [Config(*p) for p in picks]
@@ -157,7 +162,10 @@ def replay_bench(G=8, W=32, seed=4):
             alg_p3 += (24.0 + (0.0 if rz else 4.0) + (0.0 if (bnd and rz) else 4.0)
                        + (0.0 if bnd else 0.125)) * n
             if bnd and s > 0 and s + 1 < W:
-                per = (6.0 if c.score in ("abs_g", "abs_g_blind") else 18.0) - (4.0 if rz else 0.0)
+                if c.score == "abs_g_blind":
+                    per = 2.0                                # the gradient alone
+                else:
+                    per = (6.0 if c.score == "abs_g" else 18.0) - (4.0 if rz else 0.0)
                 alg_sw += (per + 0.125) * n                  # one score sweep + the new mask bits
                 n_resel += 1
     alg = alg_p1 + alg_p3 + alg_sw
@@ -203,7 +211,7 @@ def replay_cpu_baseline(G=8, W=8, seed=4, frac=24):
     entries = [{"a": s["start"], "n": s["n"], "b1": s["b1"], "b2": s["b2"], "eps": s["eps"],
                 "wd": s["wd"]} for s in segs]
     rnd = random.Random(seed)
-    axes = [(sc, r, t) for sc in ("abs_g", "update", "coi") for r in (0.1, 1.0, 10.0)
+    axes = [(sc, r, t) for sc in REPLAY_SCORES for r in (0.1, 1.0, 10.0)
             for t in (1, 4, 16)]
     cfgs = [OR.Config(*p) for p in rnd.sample(axes, G)]
     gen = torch.Generator().manual_seed(1)

@@ -15,6 +15,37 @@ from .trace_io import (ResidentWindow, ShardParams, TraceFile, WindowReader, dis
                        load_branch_state, lr_for_step, window_steps_for)
 
 
+# The reference's run-level switches of the fused replay (replay_fused.py:1137-1198): same names,
+# same allowed values, and the same contract that an unknown value raises instead of silently
+# leaving the switch a no-op.  Every "kill" arm routes the reference to a CPU / eager / mmap path
+# that does not exist here (no second code path by design), so asking for one is refused loudly.
+_REPLAY_SWITCHES = {
+    "REPLAY_FUSED_FRONT_SORT": (("auto", "cpu"), "auto"),
+    "REPLAY_FUSED_SELECT": (("auto", "cpu"), "auto"),
+    "REPLAY_FUSED_FRONT_RANK_BG": (("auto", "off"), "auto"),
+    "REPLAY_FUSED_KERNEL": (("auto", "off"), "auto"),
+    "REPLAY_FUSED_P1_READ": (("pread", "mmap"), "pread"),
+}
+
+
+def replay_switches(environ=None):
+    """Reads and validates the replay switches; returns {name: value}."""
+    import os
+    env = os.environ if environ is None else environ
+    out = {}
+    for name, (allowed, default) in _REPLAY_SWITCHES.items():
+        val = env.get(name, default)
+        if val not in allowed:
+            raise ValueError(f"{name}={val!r} is not one of the allowed values "
+                             f"({', '.join(repr(a) for a in allowed)})")
+        # the front ranking diagnostics are not built, so its background switch has nothing to do
+        if val != default and name != "REPLAY_FUSED_FRONT_RANK_BG":
+            raise RuntimeError(f"{name}={val} asks for the reference's {val} path; this build runs "
+                               "the HIP kernels only (no CPU / eager / mmap fallback)")
+        out[name] = val
+    return out
+
+
 def branch_scores(score, optimizer, sp, w0, m0, v0, g0, count, include_wd=True):
     """|registry score| at the branch point, evaluated in double and rounded
     once to fp32, flat over the shard (``replay_fused.py:1236-1265``)."""
@@ -53,6 +84,7 @@ def replay_window(trace_dir, t0, window, configs, horizons, device,
     distortions ``dist / den`` at every effective horizon, plus the resident
     ``ReplayGroup`` for inspection.
     """
+    replay_switches()
     catalog, names, _offs, N, state_files, g_files = discover_trace(trace_dir)
     if t0 not in state_files:
         raise ValueError(f"branch point {t0} has no step_{t0:06d}_state.pt in {trace_dir}")
@@ -111,4 +143,4 @@ def replay_window(trace_dir, t0, window, configs, horizons, device,
     return out
 
 
-__all__ = ["Config", "branch_scores", "replay_window"]
+__all__ = ["Config", "branch_scores", "replay_switches", "replay_window"]

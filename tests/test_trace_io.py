@@ -118,3 +118,23 @@ def test_reader_surfaces_errors(tmp_path):
     g_files[11] = os.path.join(d, "nope.pt")
     with pytest.raises(RuntimeError):
         list(T.WindowReader(g_files, [10, 11], sp, "cpu"))
+
+
+def test_replay_switches_validate_like_the_reference():
+    """Same names and allowed values as replay_fused.py:1137-1198; an unknown
+    value raises (a typo must not leave a switch a silent no-op); an arm that
+    needs the reference's CPU / eager / mmap path is refused."""
+    import pytest
+    from sga_amd.replay_run import replay_switches
+    assert replay_switches({}) == {"REPLAY_FUSED_FRONT_SORT": "auto", "REPLAY_FUSED_SELECT": "auto",
+                                   "REPLAY_FUSED_FRONT_RANK_BG": "auto",
+                                   "REPLAY_FUSED_KERNEL": "auto", "REPLAY_FUSED_P1_READ": "pread"}
+    assert replay_switches({"REPLAY_FUSED_FRONT_RANK_BG": "off"})["REPLAY_FUSED_FRONT_RANK_BG"] == "off"
+    for name, bad in (("REPLAY_FUSED_FRONT_SORT", "CPU"), ("REPLAY_FUSED_SELECT", "1"),
+                      ("REPLAY_FUSED_KERNEL", "on"), ("REPLAY_FUSED_P1_READ", "read")):
+        with pytest.raises(ValueError, match="is not one of the allowed values"):
+            replay_switches({name: bad})
+    for name, arm in (("REPLAY_FUSED_FRONT_SORT", "cpu"), ("REPLAY_FUSED_SELECT", "cpu"),
+                      ("REPLAY_FUSED_KERNEL", "off"), ("REPLAY_FUSED_P1_READ", "mmap")):
+        with pytest.raises(RuntimeError, match="HIP kernels only"):
+            replay_switches({name: arm})
