@@ -51,6 +51,16 @@ static inline unsigned stream_grid(int64_t n_items, int64_t items_per_block,
   return (unsigned)b;
 }
 
+// Workgroup ids are dealt round-robin over the 8 XCDs.  For a grid that walks
+// library-owned packed records this permutation of [0, nb) hands every XCD one
+// contiguous eighth of the range instead (measured: 2.4 % faster on the final
+// sweep's stream mix over 64 KiB records, 3 % slower on four flat arrays, so
+// only the packed layouts use it).  The tail beyond a multiple of 8 keeps its id.
+__device__ __forceinline__ unsigned xcd_contiguous_block(unsigned b, unsigned nb) {
+  const unsigned per = nb >> 3;
+  return b < (per << 3) ? (b & 7u) * per + (b >> 3) : b;
+}
+
 // True when p is aligned for 4-element vector access of `elem` bytes each.
 __host__ __device__ static inline bool aligned4(const void* p, int elem) {
   return p == nullptr || (reinterpret_cast<uintptr_t>(p) % (4 * (size_t)elem)) == 0;

@@ -337,7 +337,8 @@ void k_fused_final(
   sc.init(segs, n_segs, seg_dir);
   lc.init(segs, n_segs, seg_dir);
   const bool can_full = a.vec && (a.mask_out == nullptr || a.mvec);
-  for (int64_t c = (int64_t)blockIdx.x * kChunksPerBlock + wave_id(); c < n_chunks;
+  const unsigned blk = a.pack_extra != 0 ? xcd_contiguous_block(blockIdx.x, gridDim.x) : blockIdx.x;
+  for (int64_t c = (int64_t)blk * kChunksPerBlock + wave_id(); c < n_chunks;
        c += wstride) {
     ChunkCursor cur;
     cur.sel_run = tile_sel[c];

@@ -317,7 +317,8 @@ __global__ __launch_bounds__(kBlock) void k_replay_pass3(const void* __restrict_
   RSegCursor sc;
   sc.init(segs, n_segs);
   const int64_t stride = (int64_t)gridDim.x * kBlock * kVec;
-  for (int64_t base = (int64_t)blockIdx.x * kBlock * kVec; base < n; base += stride) {
+  const unsigned blk = grp.pack_extra != 0 ? xcd_contiguous_block(blockIdx.x, gridDim.x) : blockIdx.x;
+  for (int64_t base = (int64_t)blk * kBlock * kVec; base < n; base += stride) {
     const int64_t i = base + (int64_t)threadIdx.x * kVec;
     if (vec && base + kBlock * kVec <= n)
       pass3_vec<BF16G, true>(g, i, n, is_one, coef_dense, grp, coef_f, sc, true);
