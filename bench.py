@@ -516,6 +516,8 @@ def main():
     ap.add_argument("--layout", choices=("separate", "packed"), default="separate",
                     help="headline state layout: separate = the drop-in entry point on four flat "
                          "tensors; packed = the library-owned 64 KiB records")
+    ap.add_argument("--single-sweep", action="store_true",
+                    help="headline the single-sweep step (g / resid / p / m / v read once)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
     ap.add_argument("--cpu-sample", type=int, default=1 << 28)
     ap.add_argument("--calib", action="store_true",
@@ -602,7 +604,7 @@ def main():
 
     state = {"t": 0, "packed": None}
 
-    def time_leg(layout, score, ratio, warmup, steps):
+    def time_leg(layout, score, ratio, warmup, steps, single=False):
         """`warmup` untimed + exactly `steps` timed steps of one configuration."""
         k = k_for(n, ratio)
         if layout == "packed" and state["packed"] is None:
@@ -610,9 +612,10 @@ def main():
 
         def step_fn(t):
             if layout == "packed":
-                fs.step_packed(grads[t % 2], state["packed"], t + 1, k=k, score=score)
+                fs.step_packed(grads[t % 2], state["packed"], t + 1, k=k, score=score,
+                               single_sweep=single)
             else:
-                fs.step(grads[t % 2], r, p, m, v, t + 1, k=k, score=score)
+                fs.step(grads[t % 2], r, p, m, v, t + 1, k=k, score=score, single_sweep=single)
         for _ in range(warmup):
             step_fn(state["t"])
             state["t"] += 1
@@ -633,7 +636,7 @@ def main():
         sweep_bytes = n * sweep_bytes_per_elem(score)
         step_bytes = n * step_bytes_per_elem(score) + k * 6.0
         fin_avg, sw_avg = fin_ms / max(fin_n, 1), sw_ms / max(sw_n, 1)
-        return {"layout": layout, "score": score, "ratio_percent": ratio, "k": k, "steps": steps,
+        return {"layout": layout, "single_sweep": single, "score": score, "ratio_percent": ratio, "k": k, "steps": steps,
                 "seconds": dt, "ms_per_step": dt / steps * 1e3, "elem_per_s": n * steps / dt,
                 "alg_bytes_per_elem": step_bytes_per_elem(score),
                 "alg_bytes_per_step": step_bytes,
@@ -645,16 +648,18 @@ def main():
                 "select": {"thresh": res.thresh, "n_gt": res.n_gt, "n_eq": res.n_eq,
                            "path": res.path}}
 
-    head = time_leg(args.layout, args.score, args.ratio, args.warmup, args.steps)
+    head = time_leg(args.layout, args.score, args.ratio, args.warmup, args.steps, args.single_sweep)
     sweep = []
     if not args.no_sweep:
-        for layout in ("separate", "packed"):
-            for score in ("update", "abs_g"):
-                for ratio in (0.1, 1.0, 10.0):
-                    if (layout, score, ratio) == (args.layout, args.score, args.ratio):
-                        sweep.append(head)
-                    else:
-                        sweep.append(time_leg(layout, score, ratio, 1, 5))
+        for single in (False, True):
+            for layout in ("separate", "packed"):
+                for score in ("update", "abs_g"):
+                    for ratio in (0.1, 1.0, 10.0):
+                        if (layout, score, ratio, single) == (args.layout, args.score, args.ratio,
+                                                              args.single_sweep):
+                            sweep.append(head)
+                        else:
+                            sweep.append(time_leg(layout, score, ratio, 1, 5, single))
     if state["packed"] is not None:
         state["packed"].unpack(r, p, m, v)
         state["packed"] = None

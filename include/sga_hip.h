@@ -75,8 +75,9 @@ typedef struct sga_select_result {
   uint32_t n_eq;        /* count of |score| == thresh                      */
   uint32_t n_selected;  /* coordinates selected under the tie mode         */
   uint32_t nonfinite;   /* NaN/Inf lanes seen (selection is undefined > 0) */
-  uint32_t status;      /* 0 ok; 1 k out of range; 2 fast path fell back   */
-  uint32_t path;        /* 0 radix passes, 1 sampled bracket               */
+  uint32_t status;      /* 0 ok; 1 k out of range; 2 fast path fell back;
+                           3 single-sweep bracket missed (step invalid)    */
+  uint32_t path;        /* 0 radix passes, 1 sampled bracket, 2 single sweep */
 } sga_select_result;
 
 /* ---- scheme-agnostic masked ops (sga/kernels.py) ------------------------ */
@@ -359,6 +360,40 @@ int sga_fused_sparse_step(const void* g, int g_dtype, float* resid, float* p,
                           int fast, int flags, float interval,
                           sga_select_result* result, void* ws,
                           size_t ws_bytes, void* stream);
+
+/* Single-sweep variant of the fused step (no counterpart in the reference,
+ * whose engine runs score, select, pack and commit as separate passes,
+ * engine.py:416-604): g, resid, p, m, v are read ONCE.  The sampled bracket
+ * around the k-th key is known before the sweep and decides all but a few
+ * coordinates; those are committed in the sweep itself, the ones inside the
+ * bracket afterwards from their records, and the pack is written in index
+ * order from two bit planes.  Same arithmetic and outputs as
+ * sga_fused_sparse_step whenever result->status == 0.  status == 3: the
+ * bracket missed the k-th key after coordinates were committed on it -- the
+ * step is then invalid and cannot be repaired (margins: 12 sigma of the
+ * sample rank; `seed` moves the sample offsets so no fixed input can defeat
+ * them).  Shapes the sweep does not take are done by the two-sweep step
+ * behind the same call (n < 2^20, a bracket open below or too wide for the
+ * candidate buffers); a plateau of equal keys inside the bracket is seen in
+ * the sample BEFORE anything is committed and done by the radix passes.
+ * ws: sga_fused_workspace_bytes(n); ws2: 256-byte aligned,
+ * sga_fused_single_sweep_workspace_bytes(n, values_dtype) bytes (one staged
+ * pack value per coordinate, 128 B of bit planes per 1024, candidate records). */
+size_t sga_fused_single_sweep_workspace_bytes(int64_t n, int values_dtype);
+int sga_fused_sparse_step_single_sweep(
+    const void* g, int g_dtype, float* resid, float* p, float* m, float* v,
+    int64_t n, int64_t k, const sga_segment* segs, int n_segs, int score_id,
+    int32_t* idx_out, void* values_out, int values_dtype, uint8_t* mask_out,
+    float factor, float coeff, int flags, float interval, uint32_t seed,
+    sga_select_result* result, void* ws, size_t ws_bytes, void* ws2,
+    size_t ws2_bytes, void* stream);
+int sga_fused_sparse_step_single_sweep_packed(
+    const void* g, int g_dtype, float* state, int64_t n, int64_t k,
+    const sga_segment* segs, int n_segs, int score_id, int32_t* idx_out,
+    void* values_out, int values_dtype, uint8_t* mask_out, float factor,
+    float coeff, int flags, float interval, uint32_t seed,
+    sga_select_result* result, void* ws, size_t ws_bytes, void* ws2,
+    size_t ws2_bytes, void* stream);
 
 /* Packed-state variant of the fused step for callers that let the library
  * lay out the optimizer-side state (no counterpart in the reference, whose

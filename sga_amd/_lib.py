@@ -18,6 +18,7 @@ GC_HAS_MASK, GC_APPLY_COEFF, GC_CLEAR, GC_FOLD, GC_LR_SPLIT, GC_ADAMS = 1, 2, 4,
 RP_HAS_LAB, RP_ADAMS, RP_SPLIT = 1, 2, 4
 
 P, I64, I32, F, SZ = C.c_void_p, C.c_int64, C.c_int, C.c_float, C.c_size_t
+U32 = C.c_uint32
 
 
 class Segment(C.Structure):
@@ -93,6 +94,12 @@ SIGNATURES = {
     "sga_fused_sparse_step_packed": (I32, [P, I32, P, I64, I64, P, I32, I32, P, P,
                                            I32, P, F, F, I32, I32, F, P, P, SZ, P]),
     "sga_state_repack": (I32, [P, P, P, P, P, I64, I32, P]),
+    "sga_fused_single_sweep_workspace_bytes": (SZ, [I64, I32]),
+    "sga_fused_sparse_step_single_sweep": (I32, [P, I32, P, P, P, P, I64, I64, P, I32, I32, P, P,
+                                                 I32, P, F, F, I32, F, U32, P, P, SZ, P, SZ, P]),
+    "sga_fused_sparse_step_single_sweep_packed": (I32, [P, I32, P, I64, I64, P, I32, I32, P, P,
+                                                        I32, P, F, F, I32, F, U32, P, P, SZ, P,
+                                                        SZ, P]),
 }
 
 _lib = None

@@ -319,7 +319,8 @@ __device__ __forceinline__ void final_chunk(const FinalArgs& a, int64_t c, Chunk
 // Final sweep: select flags in index order, pack, residual, commit.
 // `when`: 0 run always; 1 only if the sampled bracket held (the planes are
 // settled); 2 only if it failed (the radix passes fixed the threshold and the
-// keys are formed again here).
+// keys are formed again here); 3 like 2, and only if the single-sweep step
+// stood back before it touched anything.
 // (five waves per SIMD wherever the key is not an Adam-normalised chain formed in this kernel)
 template <bool BF16G, bool BF16V, int SCORE, bool PLANES>
 __global__ __launch_bounds__(kBlock, (PLANES || SCORE == SGA_SCORE_ABS_G || SCORE == SGA_SCORE_ABS_M ||
@@ -328,7 +329,8 @@ void k_fused_final(
     FinalArgs a, const sga_segment* __restrict__ segs, int n_segs,
     const SelState* __restrict__ st, const uint32_t* __restrict__ tile_sel,
     const uint32_t* __restrict__ tile_eq, int when, const int32_t* __restrict__ seg_dir) {
-  if (when != 0 && (st->bracket_ok != 0) != (when == 1)) return;
+  if (when == 3) { if (st->bracket_ok != 0 || st->spec != 0) return; }
+  else if (when != 0 && (st->bracket_ok != 0) != (when == 1)) return;
   a.T = st->thresh_bits;
   a.need = st->need;
   const int64_t n_chunks = cdiv64(a.n, kChunk);
@@ -412,6 +414,715 @@ static int run_fused(const void* g, float* resid, float* p, float* m, float* v, 
   return check_launch("sga_fused_sparse_step");
 }
 
+
+// ====================================================== single-sweep step
+// The step above reads the score inputs twice because the threshold is global.
+// The sampled bracket [T_LO, T_HI) is known BEFORE any sweep, though, and it
+// decides all but a few coordinates: a key at or above T_HI is selected, a key
+// below T_LO is not, whatever the exact threshold turns out to be.  The
+// single-sweep step therefore reads g, resid, p, m, v ONCE and commits every
+// coordinate on the spot.  A coordinate inside the bracket is committed on a
+// guess -- selected if its key is at or above the bracket's midpoint T_MID --
+// and recorded with its key and the four inputs of its commit.  The candidate
+// descent over the recorded keys then fixes the exact threshold; the guesses
+// that turn out wrong (keys between the midpoint and the threshold: a few per
+// cent of the records) are committed again from their records, and the pack
+// is written in index order from two bit planes: S (what the sweep took as
+// selected: it parked those pack values in a chunk-strided staging array) and
+// F (the exact selection: S patched by the settlement).
+//
+// Exactness: whenever the bracket holds the k-th key and the record lists have
+// room, every output is the two-sweep step's, bit for bit.  What cannot be
+// undone is a commit on a bracket that MISSED: the margins are 12 sigma of the
+// sample rank (6 sigma if the four neighbours of every sampled quad were
+// perfectly correlated), the offsets move with a caller-provided seed, and a
+// miss is reported as status 3 (the step is then invalid).  The kernel stands
+// back, before touching anything, when the sample says the bracket holds more
+// keys than the lists (plateaus of equal keys) or the bracket is open below:
+// the radix passes and the key-forming final sweep then do the step exactly.
+struct SpecArgs {
+  uint32_t* splane;       // S: keys at or above T_MID (128 B per chunk), as the sweep committed
+  uint32_t* fplane;       // F: starts as S, patched by the settlement into the exact selection
+  void* stage;            // pack values of the S coordinates, chunk c at [c * 1024, ...)
+  uint32_t* seg_idx;
+  uint32_t* seg_key;
+  F4* seg_rec;            // (q, p, m, v) of each recorded coordinate
+  uint32_t* seg_cnt;
+  uint32_t seg_cap;
+  uint32_t* tile_gt;
+  uint32_t* tile_eq;
+  uint32_t* hi_part;
+  uint32_t* nf_part;
+  uint32_t* ovf_idx;      // shared overflow list: chunks whose segment is full, and what a
+  uint32_t* ovf_key;      // chunk records beyond a wave's LDS buffer
+  F4* ovf_rec;
+  uint32_t* ovf_cnt;
+  uint32_t ovf_cap;
+  uint32_t chunks_per_seg; // consecutive chunks share a segment: the lists come out in address order
+  double n_over_ns;       // population / sample size
+  double est_limit;       // stand back when the sample predicts more bracket keys than this
+};
+
+constexpr int kSpecCandCap = 256;          // records a chunk gathers in LDS before it spills
+
+struct SpecLds {
+  uint32_t idx[kSpecCandCap];
+  uint32_t key[kSpecCandCap];
+  F4 rec[kSpecCandCap];
+  uint32_t splane[kPlaneWordsPerChunk];
+};
+
+// Midpoint of the bracket in key space: the guess for the coordinates inside it.
+__device__ __forceinline__ uint32_t spec_mid(uint32_t t_lo, uint32_t t_hi) {
+  return t_hi > 0x7FFFFFFFu ? t_hi : t_lo + ((t_hi - t_lo) >> 1);   // open above: guess "not selected"
+}
+
+// Pack value and commit gradient of a selected coordinate (the same chain as the final sweep).
+template <bool BF16V>
+__device__ __forceinline__ float spec_value(const FinalArgs& a, float q, uint16_t& hb, float& val) {
+  val = q;
+  if (a.scale) val = val * a.factor;
+  float ge;
+  if (BF16V) { hb = f32_to_bf16(val); ge = bf16_to_f32(hb); }
+  else { hb = 0; ge = val; }
+  if (a.apply_coeff) ge = ge * a.coeff;
+  return ge;
+}
+
+// One 256-element slab of the single sweep.  chi: keys at or above T_HI so far
+// in the chunk; s_run: S coordinates so far; mycnt: records so far.
+template <bool BF16G, bool BF16V, int SCORE, bool FULL>
+__device__ __forceinline__ void spec_slab(const FinalArgs& a, const SpecArgs& sa, SelState* st,
+                                          int64_t c, int it, uint32_t T_LO, uint32_t T_MID,
+                                          uint32_t T_HI, SegCursor& sc, uint32_t& chi,
+                                          uint32_t& s_run, uint32_t& tot_nf, uint32_t& mycnt,
+                                          SpecLds& lds, float* R, float* P, float* M, float* V) {
+  constexpr bool kHyper = SCORE == SGA_SCORE_UPDATE || SCORE == SGA_SCORE_COI ||
+                          SCORE == SGA_SCORE_GR_OVER_SQRT_V;
+  const int64_t n = a.n;
+  const int64_t i = c * kChunk + it * (kWave * kVec) + lane_id() * kVec;
+  float gg[4] = {0, 0, 0, 0}, rr[4] = {0, 0, 0, 0}, pp[4] = {0, 0, 0, 0}, mm[4] = {0, 0, 0, 0},
+        vv[4] = {0, 0, 0, 0};
+  if (FULL) {
+    H4 gh; F4 gf;
+    if (BF16G) gh = ldh4_nt(reinterpret_cast<const uint16_t*>(a.g) + i);
+    else gf = ld4_nt(reinterpret_cast<const float*>(a.g) + i);
+    const F4 r4 = ld4_nt(R + i), p4 = ld4_nt(P + i), m4 = ld4_nt(M + i), v4 = ld4_nt(V + i);
+    __builtin_amdgcn_sched_barrier(0);
+    if (BF16G) { gg[0] = bf16_to_f32(gh.x); gg[1] = bf16_to_f32(gh.y); gg[2] = bf16_to_f32(gh.z); gg[3] = bf16_to_f32(gh.w); }
+    else { gg[0] = gf.x; gg[1] = gf.y; gg[2] = gf.z; gg[3] = gf.w; }
+    unpack_f32(r4, rr); unpack_f32(p4, pp); unpack_f32(m4, mm); unpack_f32(v4, vv);
+  } else if (i < n) {
+    load_g<BF16G, false>(a.g, i, n, gg, a.vec);
+    load4_f32(R, i, n, rr, a.vec);
+    load4_f32(P, i, n, pp, a.vec);
+    load4_f32(M, i, n, mm, a.vec);
+    load4_f32(V, i, n, vv, a.vec);
+  }
+  float q[4];
+  uint32_t key[4] = {0u, 0u, 0u, 0u};
+#pragma unroll
+  for (int e = 0; e < 4; ++e) q[e] = rr[e] + gg[e];
+  if (!kHyper) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+      key[e] = abs_key(SCORE == SGA_SCORE_ABS_M ? mm[e] : SCORE == SGA_SCORE_ABS_G_BLIND ? gg[e] : q[e]);
+  } else if (FULL || uniform_i64(i) < n) {
+    float vk[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) vk[e] = a.adams ? mm[e] * mm[e] : vv[e];
+    slab_score_keys<SCORE, FULL>(sc, a.adams ? 1 : 0, i, n, q, pp, mm, vk, key);
+  }
+  Ballot4 above, cand, S;
+  uint64_t nf = 0;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const uint64_t valid = FULL ? ~0ull : ballot64(i + e < n);
+    above.m[e] = ballot64(key[e] >= T_HI) & valid;
+    cand.m[e] = ballot64(key[e] >= T_LO) & valid & ~above.m[e];
+    S.m[e] = ballot64(key[e] >= T_MID) & valid;
+    nf |= ballot64(key[e] >= 0x7F800000u) & valid;
+  }
+  chi += above.count();
+  if (nf) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+      tot_nf += (uint32_t)__popcll(ballot64(key[e] >= 0x7F800000u && (FULL || i + e < n)));
+  }
+  // records of the bracket's coordinates: the wave's LDS buffer, and past its end straight to
+  // the overflow list (a reservation per slab; nothing downstream needs a chunk's records in
+  // one piece)
+  if (cand.any()) {                                      // scalar branch
+    const uint32_t cnt = cand.count();
+    const uint32_t room = mycnt < (uint32_t)kSpecCandCap ? (uint32_t)kSpecCandCap - mycnt : 0u;
+    uint32_t obase = 0;
+    bool fits = true;
+    if (cnt > room) {
+      if (lane_id() == 0) obase = atomicAdd(sa.ovf_cnt, cnt - room);
+      obase = __shfl(obase, 0, kWave);
+      fits = obase + (cnt - room) <= sa.ovf_cap;         // a list over its capacity is seen by the check
+    }
+    uint32_t pos = cand.below_lane();                    // position among the slab's records
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      if (!cand.mine(e)) continue;
+      const F4 rec{q[e], pp[e], mm[e], vv[e]};
+      if (pos < room) {
+        lds.idx[mycnt + pos] = (uint32_t)(i + e); lds.key[mycnt + pos] = key[e]; lds.rec[mycnt + pos] = rec;
+      } else if (fits) {
+        const uint32_t o = obase + (pos - room);
+        sa.ovf_idx[o] = (uint32_t)(i + e); sa.ovf_key[o] = key[e]; sa.ovf_rec[o] = rec;
+      }
+      ++pos;
+    }
+    mycnt += cnt < room ? cnt : room;
+  }
+  plane_put(S, it, lds.splane);
+  const uint32_t s_before = s_run;
+  s_run += S.count();
+  if (!FULL && i >= n) return;
+  bool sel[4], valid[4];
+  float ge[4];
+  uint32_t spos = s_before + S.below_lane();
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    valid[e] = FULL || i + e < n;
+    sel[e] = S.mine(e);
+    ge[e] = 0.0f;
+    if (!sel[e]) continue;
+    uint16_t hb; float val;
+    ge[e] = spec_value<BF16V>(a, q[e], hb, val);
+    if (BF16V) reinterpret_cast<uint16_t*>(sa.stage)[c * kChunk + spos] = hb;
+    else reinterpret_cast<float*>(sa.stage)[c * kChunk + spos] = val;
+    ++spos;
+  }
+  const int64_t s0 = uniform_i64(c) * kChunk + it * (kWave * kVec);
+  int64_t s1 = s0 + kWave * kVec;
+  if (!FULL && s1 > n) s1 = n;
+  if (s0 < sc.lo || s0 >= sc.hi) sc.seek_uniform(s0);
+  float pn[4], mn[4], vn[4];
+  for (;;) {
+    const bool whole = sc.lo <= s0 && sc.hi >= s1;
+    Hyper h = sc.h;
+    if (a.adams) { h.bc1 = 1.0f; h.bc2 = 1.0f; }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const float ve = a.adams ? mm[e] * mm[e] : vv[e];
+      const Commit cm = adamw_commit(pp[e], ge[e], mm[e], ve, h);
+      const float pe = pp[e] - h.lr * cm.upd;
+      if (whole || (i + e >= sc.lo && i + e < sc.hi)) { pn[e] = pe; mn[e] = cm.m_new; vn[e] = cm.v_new; }
+    }
+    const int64_t nxt = sc.hi;
+    if (whole || nxt >= s1) break;
+    sc.advance_uniform(nxt);
+    if (sc.hi <= nxt) break;              // the table does not tile [0, n): stop
+  }
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    if (!valid[e]) continue;
+    pp[e] = pn[e]; mm[e] = mn[e]; vv[e] = vn[e];
+    rr[e] = sel[e] ? 0.0f : q[e];
+    if (a.fold) rr[e] = __fdiv_rn(rr[e], a.interval);
+  }
+  st_f32<FULL>(R, i, n, rr, a.vec);
+  st_f32<FULL>(M, i, n, mm, a.vec);
+  st_f32<FULL>(V, i, n, vv, a.vec);
+  st_f32<FULL>(P, i, n, pp, a.vec);
+}
+
+template <bool BF16G, bool BF16V, int SCORE>
+__global__ __launch_bounds__(kBlock) void k_fused_spec(
+    FinalArgs a, SpecArgs sa, const sga_segment* __restrict__ segs, int n_segs,
+    SelState* __restrict__ st, const SelState* __restrict__ aux,
+    const int32_t* __restrict__ seg_dir) {
+  __shared__ uint32_t s_hi[kChunksPerBlock], s_nf[kChunksPerBlock];
+  __shared__ SpecLds s_lds[kChunksPerBlock];
+  // the sample's own count of keys inside the bracket predicts the records
+  const SelState hi = aux[0], lo = aux[1];
+  if (lo.skip) return;                                   // open below: nothing bounds the records
+  const double in_bracket = (double)(lo.k - lo.need + lo.n_eq) - (hi.skip ? 0.0 : (double)(hi.k - hi.need));
+  if (in_bracket * sa.n_over_ns > sa.est_limit) return;  // plateau inside the bracket: stand back
+  const uint32_t T_HI = hi.skip ? 0x80000000u : hi.thresh_bits + 1u;
+  const uint32_t T_LO = lo.thresh_bits;
+  const uint32_t T_MID = spec_mid(T_LO, T_HI);
+  if (blockIdx.x == 0 && threadIdx.x == 0) { st->t_lo = T_LO; st->t_hi = T_HI; st->spec = 1u; }
+  const int64_t n_chunks = cdiv64(a.n, kChunk);
+  const unsigned blk = a.pack_extra != 0 ? xcd_contiguous_block(blockIdx.x, gridDim.x) : blockIdx.x;
+  const int64_t c = (int64_t)blk * kChunksPerBlock + wave_id();
+  uint32_t chi = 0, tot_nf = 0;
+  if (c < n_chunks) {
+    uint32_t mycnt = 0, s_run = 0;
+    SpecLds& lds = s_lds[wave_id()];
+    SegCursor sc;
+    sc.init(segs, n_segs, seg_dir);
+    const int64_t sh = pack_shift<true>(c << 10, a.pack_extra);
+    float* const R = a.r + sh;
+    float* const P = a.p + sh;
+    float* const M = a.m + sh;
+    float* const V = a.v + sh;
+    sc.seek_uniform(uniform_i64(c) * kChunk);
+#define SGA_SPEC_SLAB(FULLP, IT) \
+    spec_slab<BF16G, BF16V, SCORE, FULLP>(a, sa, st, c, IT, T_LO, T_MID, T_HI, sc, chi, s_run, tot_nf, mycnt, lds, R, P, M, V)
+    if (a.vec && (c + 1) * kChunk <= a.n) {
+      SGA_SPEC_SLAB(true, 0); SGA_SPEC_SLAB(true, 1); SGA_SPEC_SLAB(true, 2); SGA_SPEC_SLAB(true, 3);
+    } else {
+      SGA_SPEC_SLAB(false, 0); SGA_SPEC_SLAB(false, 1); SGA_SPEC_SLAB(false, 2); SGA_SPEC_SLAB(false, 3);
+    }
+#undef SGA_SPEC_SLAB
+    __builtin_amdgcn_wave_barrier();
+    if (lane_id() < kPlaneWordsPerChunk) {
+      sa.splane[c * kPlaneWordsPerChunk + lane_id()] = lds.splane[lane_id()];
+      sa.fplane[c * kPlaneWordsPerChunk + lane_id()] = lds.splane[lane_id()];
+    }
+    if (lane_id() == 0) { sa.tile_gt[c] = chi; sa.tile_eq[c] = 0u; }
+    if (mycnt) {                                        // wave-uniform
+      // The chunk's LDS records go, in one piece, to the segment of its range of chunks; when
+      // that is full (the reservation is taken back: every later one then sees the true count),
+      // to the shared overflow list.
+      uint32_t seg = (uint32_t)(c / sa.chunks_per_seg);
+      if (seg > (uint32_t)(kSegWaves - 1)) seg = kSegWaves - 1;
+      uint32_t base = 0;
+      if (lane_id() == 0) {
+        base = atomicAdd(&sa.seg_cnt[seg], mycnt);
+        if (base + mycnt > sa.seg_cap) { atomicSub(&sa.seg_cnt[seg], mycnt); base = 0xFFFFFFFFu; }
+      }
+      base = __shfl(base, 0, kWave);
+      uint32_t* g_idx = sa.seg_idx + (int64_t)seg * sa.seg_cap;
+      uint32_t* g_key = sa.seg_key + (int64_t)seg * sa.seg_cap;
+      F4* g_rec = sa.seg_rec + (int64_t)seg * sa.seg_cap;
+      bool room = true;
+      if (base == 0xFFFFFFFFu) {
+        if (lane_id() == 0) base = atomicAdd(sa.ovf_cnt, mycnt);
+        base = __shfl(base, 0, kWave);
+        room = base + mycnt <= sa.ovf_cap;
+        g_idx = sa.ovf_idx; g_key = sa.ovf_key; g_rec = sa.ovf_rec;
+      }
+      if (room)
+        for (uint32_t j = lane_id(); j < mycnt; j += kWave) {
+          g_idx[base + j] = lds.idx[j]; g_key[base + j] = lds.key[j]; g_rec[base + j] = lds.rec[j];
+        }
+    }
+  }
+  if (lane_id() == 0) { s_hi[wave_id()] = chi; s_nf[wave_id()] = tot_nf; }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    const uint32_t h = s_hi[0] + s_hi[1] + s_hi[2] + s_hi[3];
+    const uint32_t f = s_nf[0] + s_nf[1] + s_nf[2] + s_nf[3];
+    if (h) atomicAdd(&sa.hi_part[blockIdx.x & (kSweepParts - 1)], h);
+    if (f) atomicAdd(&sa.nf_part[blockIdx.x & (kSweepParts - 1)], f);
+  }
+}
+
+// Ties at the threshold are granted in index order.  After the tile scan
+// tile_eq[c] counts the ties before chunk c, so only the one chunk where the
+// quota runs out has to rank its ties: this pass gathers that chunk's ties
+// (at most 1024) so the settlement can rank them wherever their records lie.
+constexpr int kSpecTieCap = 1024;
+static __global__ __launch_bounds__(kBlock) void k_spec_ties(
+    const SelState* __restrict__ st, const uint32_t* __restrict__ cand_idx,
+    const uint32_t* __restrict__ cand_key, const uint32_t* __restrict__ tile_eq,
+    int64_t n_tiles, uint32_t* __restrict__ tie_cnt, uint32_t* __restrict__ tie_idx) {
+  if (!st->bracket_ok || !st->spec) return;
+  const uint32_t T = st->thresh_bits, nc = st->cand_count, n_eq = st->n_eq, need = st->need;
+  if (need >= n_eq) return;                              // every tie is taken
+  for (uint32_t j = blockIdx.x * kBlock + threadIdx.x; j < nc; j += gridDim.x * kBlock) {
+    if (cand_key[j] != T) continue;
+    const uint32_t idx = cand_idx[j], c = idx >> 10;
+    const uint32_t before = tile_eq[c];
+    const uint32_t upto = (int64_t)c + 1 < n_tiles ? tile_eq[c + 1] : n_eq;
+    if (before < need && upto > need) {
+      const uint32_t at = atomicAdd(tie_cnt, 1u);
+      if (at < (uint32_t)kSpecTieCap) tie_idx[at] = idx;
+    }
+  }
+}
+
+// Settlement: the exact selection of every recorded coordinate against the
+// sweep's guess; where they differ the F plane is patched.
+static __global__ __launch_bounds__(kBlock) void k_spec_settle(
+    const SelState* __restrict__ st, const uint32_t* __restrict__ cand_idx,
+    const uint32_t* __restrict__ cand_key, const uint32_t* __restrict__ tile_eq,
+    int64_t n_tiles, const uint32_t* __restrict__ tie_cnt, const uint32_t* __restrict__ tie_idx,
+    uint32_t* __restrict__ fplane) {
+  if (!st->bracket_ok || !st->spec) return;
+  const uint32_t T = st->thresh_bits, nc = st->cand_count, n_eq = st->n_eq, need = st->need;
+  const uint32_t T_MID = spec_mid(st->t_lo, st->t_hi);
+  for (uint32_t j = blockIdx.x * kBlock + threadIdx.x; j < nc; j += gridDim.x * kBlock) {
+    const uint32_t key = cand_key[j];
+    const uint32_t idx = cand_idx[j];
+    bool on = key >= T;
+    if (key == T && need < n_eq) {
+      const uint32_t c = idx >> 10;
+      const uint32_t before = tile_eq[c];
+      const uint32_t upto = (int64_t)c + 1 < n_tiles ? tile_eq[c + 1] : n_eq;
+      if (before >= need) {
+        on = false;
+      } else if (upto > need) {            // the quota ends inside this chunk
+        uint32_t rank = before;
+        const uint32_t nt = *tie_cnt < (uint32_t)kSpecTieCap ? *tie_cnt : (uint32_t)kSpecTieCap;
+        for (uint32_t t = 0; t < nt; ++t) rank += tie_idx[t] < idx;
+        on = rank < need;
+      }
+    }
+    if (on != (key >= T_MID)) {
+      const uint32_t lane = (idx >> 2) & 63u, e = idx & 3u;
+      uint32_t* w = &fplane[(idx >> 8) * 8 + 2 * e + (lane >> 5)];
+      if (on) atomicOr(w, 1u << (lane & 31));
+      else atomicAnd(w, ~(1u << (lane & 31)));
+    }
+  }
+}
+
+// Selected coordinates before element `idx` inside its 256-element slab of a
+// bit plane: the lanes below its lane over the four ballots, plus its lane's
+// earlier elements.
+__device__ __forceinline__ uint32_t slab_rank_before(const uint32_t* __restrict__ plane, uint32_t idx) {
+  const uint32_t lane0 = (idx >> 2) & 63u, e0 = idx & 3u;
+  const U4* wp = reinterpret_cast<const U4*>(plane + (int64_t)(idx >> 8) * 8);
+  const U4 x0 = wp[0], x1 = wp[1];
+  const uint32_t w[8] = {x0.x, x0.y, x0.z, x0.w, x1.x, x1.y, x1.z, x1.w};
+  const uint64_t below = lane0 ? (~0ull >> (64 - lane0)) : 0ull;
+  uint32_t rank = 0;
+#pragma unroll
+  for (uint32_t e = 0; e < 4; ++e) {
+    const uint64_t m = ((uint64_t)w[2 * e + 1] << 32) | (uint64_t)w[2 * e];
+    rank += (uint32_t)__popcll(m & below);
+    if (e < e0) rank += (uint32_t)((m >> lane0) & 1ull);
+  }
+  return rank;
+}
+
+// Pack entries of the coordinates the sweep took as selected and the exact
+// selection keeps (S & F), from the staging array.  One LANE per 256-element
+// slab (a wave per slab spends a whole wave's ballot arithmetic on the two or
+// three entries a slab holds at 1 %), one wave per workgroup: the lane reads
+// its slab's 8 + 8 plane words, takes its starts inside the chunk from its
+// three neighbours (a chunk is four consecutive lanes), then walks its set
+// bits in index order.  The 64 slabs of a wave fill ONE contiguous run of the
+// pack, so the entries go through LDS, a window of kPackWindow positions at a
+// time, and leave as whole coalesced lines (a lane writing its own few entries
+// straight to memory leaves every line half written when it is evicted: 4 ms
+// instead of 0.3 at 10 %).  Positions of coordinates the repair pass adds
+// (F without S) stay untouched: the window is pre-filled with a sentinel.
+// slab_pos[slab] = pack position of the slab's first selected coordinate.
+constexpr int kPackWindow = 1024;
+constexpr int kPackAhead = 8;             // staged values a lane requests before it walks its bits
+template <bool BF16V>
+__global__ __launch_bounds__(kWave) void k_spec_pack(
+    FinalArgs a, const SelState* __restrict__ st, const void* __restrict__ stage,
+    const uint32_t* __restrict__ splane, const uint32_t* __restrict__ fplane,
+    const uint32_t* __restrict__ tile_sel, uint32_t* __restrict__ slab_pos) {
+  __shared__ uint32_t l_idx[kPackWindow + 4];
+  __shared__ uint32_t l_val[kPackWindow + 4];
+  if (!st->bracket_ok || !st->spec) return;
+  const int64_t n_slabs = cdiv64(a.n, kChunk) * kChunkIters;
+  const int64_t slab = (int64_t)blockIdx.x * kWave + threadIdx.x;
+  const bool live = slab < n_slabs;
+  uint64_t S[4] = {0, 0, 0, 0}, F[4] = {0, 0, 0, 0};
+  uint32_t base = 0;
+  if (live) {
+    const U4* ws = reinterpret_cast<const U4*>(splane + slab * 8);
+    const U4* wf = reinterpret_cast<const U4*>(fplane + slab * 8);
+    const U4 x0 = ws[0], x1 = ws[1], y0 = wf[0], y1 = wf[1];
+    base = tile_sel[slab >> 2];
+    S[0] = ((uint64_t)x0.y << 32) | x0.x; S[1] = ((uint64_t)x0.w << 32) | x0.z;
+    S[2] = ((uint64_t)x1.y << 32) | x1.x; S[3] = ((uint64_t)x1.w << 32) | x1.z;
+    F[0] = ((uint64_t)y0.y << 32) | y0.x; F[1] = ((uint64_t)y0.w << 32) | y0.z;
+    F[2] = ((uint64_t)y1.y << 32) | y1.x; F[3] = ((uint64_t)y1.w << 32) | y1.z;
+  }
+  const uint32_t cntS = (uint32_t)(__popcll(S[0]) + __popcll(S[1]) + __popcll(S[2]) + __popcll(S[3]));
+  const uint32_t cntF = (uint32_t)(__popcll(F[0]) + __popcll(F[1]) + __popcll(F[2]) + __popcll(F[3]));
+  uint32_t ps = 0, pf = 0;
+#pragma unroll
+  for (int o = 1; o < kChunkIters; ++o) {
+    const uint32_t ts = __shfl_up(cntS, o, kWave), tf = __shfl_up(cntF, o, kWave);
+    if ((lane_id() & (kChunkIters - 1)) >= o) { ps += ts; pf += tf; }
+  }
+  const uint32_t f_start = base + pf;
+  if (live) slab_pos[slab] = f_start;
+  // the wave's run of the pack: [F0, F0 + len)
+  const uint32_t F0 = __shfl(f_start, 0, kWave);
+  uint32_t end = live ? f_start + cntF : 0u;
+#pragma unroll
+  for (int o = kWave / 2; o > 0; o >>= 1) { const uint32_t t = __shfl_xor(end, o, kWave); end = t > end ? t : end; }
+  const uint32_t len = end - F0;
+  const int64_t c = slab >> 2;
+  uint64_t U = S[0] | S[1] | S[2] | S[3];
+  // the lane's first staged values, all requested before the first is used (its run of the
+  // staging array is contiguous); a slab with more entries loads the rest as it goes
+  uint32_t ahead[kPackAhead];
+#pragma unroll
+  for (int t = 0; t < kPackAhead; ++t) {
+    ahead[t] = 0u;
+    if ((uint32_t)t < cntS) {
+      if (BF16V) ahead[t] = reinterpret_cast<const uint16_t*>(stage)[c * kChunk + ps + t];
+      else ahead[t] = reinterpret_cast<const uint32_t*>(stage)[c * kChunk + ps + t];
+    }
+  }
+  for (uint32_t w0 = 0; w0 < len; w0 += kPackWindow) {
+    const uint32_t wlen = len - w0 < (uint32_t)kPackWindow + 3u ? len - w0 : (uint32_t)kPackWindow + 3u;
+    for (uint32_t t = lane_id(); t < wlen; t += kWave) l_idx[t] = 0xFFFFFFFFu;
+    __syncthreads();
+    while (U) {
+      const int L = __ffsll((unsigned long long)U) - 1;
+      const uint64_t below = L ? (~0ull >> (64 - L)) : 0ull;
+      uint32_t fr = f_start + (uint32_t)(__popcll(F[0] & below) + __popcll(F[1] & below) +
+                                         __popcll(F[2] & below) + __popcll(F[3] & below));
+      if (fr - F0 >= w0 + (uint32_t)kPackWindow) break;     // belongs to a later window
+      U &= U - 1;
+      uint32_t sr = ps + (uint32_t)(__popcll(S[0] & below) + __popcll(S[1] & below) +
+                                    __popcll(S[2] & below) + __popcll(S[3] & below));
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const bool in_s = (S[e] >> L) & 1ull, in_f = (F[e] >> L) & 1ull;
+        if (in_s && in_f) {
+          const uint32_t t = fr - F0 - w0;
+          l_idx[t] = (uint32_t)(slab * (kWave * kVec) + L * kVec + e);
+          const uint32_t u = sr - ps;
+          uint32_t val;
+          if (u < (uint32_t)kPackAhead) {
+            val = ahead[0];
+#pragma unroll
+            for (int q = 1; q < kPackAhead; ++q) val = u == (uint32_t)q ? ahead[q] : val;
+          } else if (BF16V) {
+            val = reinterpret_cast<const uint16_t*>(stage)[c * kChunk + sr];
+          } else {
+            val = reinterpret_cast<const uint32_t*>(stage)[c * kChunk + sr];
+          }
+          l_val[t] = val;
+        }
+        sr += in_s;
+        fr += in_f;
+      }
+    }
+    __syncthreads();
+    for (uint32_t t = lane_id(); t < wlen; t += kWave) {
+      const uint32_t ix = l_idx[t];
+      const int64_t pos = (int64_t)F0 + w0 + t;
+      if (ix != 0xFFFFFFFFu && pos < a.k) {
+        a.idx_out[pos] = (int32_t)ix;
+        if (BF16V) reinterpret_cast<uint16_t*>(a.values_out)[pos] = (uint16_t)l_val[t];
+        else reinterpret_cast<uint32_t*>(a.values_out)[pos] = l_val[t];
+      }
+    }
+    __syncthreads();
+  }
+}
+
+// Repair: the recorded coordinates whose guess was wrong are committed again,
+// from their records, the way the exact selection says; the newly selected
+// ones also get their pack entry.
+template <bool BF16V>
+__global__ __launch_bounds__(kBlock) void k_spec_repair(
+    FinalArgs a, const sga_segment* __restrict__ segs, int n_segs,
+    const int32_t* __restrict__ seg_dir, const SelState* __restrict__ st,
+    const uint32_t* __restrict__ cand_idx, const uint32_t* __restrict__ cand_key,
+    const F4* __restrict__ cand_rec, const uint32_t* __restrict__ fplane,
+    const uint32_t* __restrict__ slab_pos) {
+  if (!st->bracket_ok || !st->spec) return;
+  const uint32_t nc = st->cand_count;
+  const uint32_t T_MID = spec_mid(st->t_lo, st->t_hi);
+  SegCursor lc;
+  lc.init(segs, n_segs, seg_dir);
+  for (uint32_t j = blockIdx.x * kBlock + threadIdx.x; j < nc; j += gridDim.x * kBlock) {
+    const uint32_t idx = cand_idx[j];
+    const uint32_t lane = (idx >> 2) & 63u, e = idx & 3u;
+    const bool on = (fplane[(idx >> 8) * 8 + 2 * e + (lane >> 5)] >> (lane & 31)) & 1u;
+    if (on == (cand_key[j] >= T_MID)) continue;          // the sweep's commit stands
+    const F4 rec = cand_rec[j];
+    lc.seek((int64_t)idx);
+    Hyper h = lc.h;
+    if (a.adams) { h.bc1 = 1.0f; h.bc2 = 1.0f; }
+    float ge = 0.0f, val = 0.0f;
+    uint16_t hb = 0;
+    if (on) ge = spec_value<BF16V>(a, rec.x, hb, val);
+    const float ve = a.adams ? rec.z * rec.z : rec.w;
+    const Commit cm = adamw_commit(rec.y, ge, rec.z, ve, h);
+    const float pe = rec.y - h.lr * cm.upd;
+    float rn = on ? 0.0f : rec.x;
+    if (a.fold) rn = __fdiv_rn(rn, a.interval);
+    const int64_t at = (int64_t)idx + pack_shift<false>((int64_t)idx, a.pack_extra);
+    a.r[at] = rn;
+    a.p[at] = pe;
+    a.m[at] = cm.m_new;
+    a.v[at] = cm.v_new;
+    if (on) {
+      const uint32_t pos = slab_pos[idx >> 8] + slab_rank_before(fplane, idx);
+      if ((int64_t)pos < a.k) {
+        a.idx_out[pos] = (int32_t)idx;
+        if (BF16V) reinterpret_cast<uint16_t*>(a.values_out)[pos] = hb;
+        else reinterpret_cast<float*>(a.values_out)[pos] = val;
+      }
+    }
+  }
+}
+
+// Overflow list -> tail of the dense candidate list (behind the segments' records).
+static __global__ __launch_bounds__(kBlock) void k_spec_ovf_compact(
+    const SelState* __restrict__ aux, const uint32_t* __restrict__ seg_off,
+    const uint32_t* __restrict__ ovf_idx, const uint32_t* __restrict__ ovf_key,
+    const F4* __restrict__ ovf_rec, uint32_t ovf_cap, uint32_t* __restrict__ cand_idx,
+    uint32_t* __restrict__ cand_key, F4* __restrict__ cand_rec, uint32_t* __restrict__ tie_cnt) {
+  if (blockIdx.x == 0 && threadIdx.x == 0) *tie_cnt = 0u;     // the tie list of this step starts empty
+  if (aux->skip) return;
+  const uint32_t off = seg_off[kSegWaves];
+  uint32_t cnt = seg_off[kSegWaves + 1];
+  if (cnt > ovf_cap) cnt = ovf_cap;
+  for (uint32_t j = blockIdx.x * kBlock + threadIdx.x; j < cnt; j += gridDim.x * kBlock) {
+    cand_idx[off + j] = ovf_idx[j];
+    cand_key[off + j] = ovf_key[j];
+    cand_rec[off + j] = ovf_rec[j];
+  }
+}
+
+// Extra workspace of the single-sweep step: [dplane: 128 B per chunk | records: 16 B per
+// candidate slot | staging: one pack value per coordinate, chunk-strided].
+struct SpecWorkspace {
+  uint32_t* dplane;
+  uint32_t* slab_pos;
+  F4* seg_rec;
+  F4* cand_rec;
+  uint32_t* ovf_idx;
+  uint32_t* ovf_key;
+  F4* ovf_rec;
+  int64_t ovf_cap;
+  uint32_t* tie_cnt;      // [0]: ties gathered; tie_idx follows
+  uint32_t* tie_idx;
+  void* stage;
+};
+static inline size_t spec_ws_bytes(int64_t n, int val_bytes) {
+  const int64_t nt = cdiv64(n, kChunk) + 8;
+  // records of the segments (16 B), dense records (16 B), overflow list (24 B, half the capacity)
+  size_t b = (size_t)nt * (128 + 16) + (size_t)kSegWaves * fast_seg_cap(nt * kChunk) * (16 * 2 + 12) +
+             (size_t)nt * kChunk * val_bytes + 4096 + 8192;
+  return (b + 255) & ~(size_t)255;
+}
+static inline bool spec_ws_carve(void* ws, size_t bytes, int64_t n, int val_bytes, int64_t seg_cap,
+                                 SpecWorkspace* out) {
+  if (!ws || (reinterpret_cast<uintptr_t>(ws) & 255) || bytes < spec_ws_bytes(n, val_bytes)) return false;
+  const int64_t nt = cdiv64(n, kChunk) + 8;
+  char* p = reinterpret_cast<char*>(ws);
+  out->dplane = reinterpret_cast<uint32_t*>(p);
+  p += (size_t)nt * 128;
+  out->slab_pos = reinterpret_cast<uint32_t*>(p);
+  p += (size_t)nt * 16;
+  p = reinterpret_cast<char*>((reinterpret_cast<uintptr_t>(p) + 255) & ~(uintptr_t)255);
+  out->seg_rec = reinterpret_cast<F4*>(p);
+  p += (size_t)kSegWaves * seg_cap * 16;
+  p = reinterpret_cast<char*>((reinterpret_cast<uintptr_t>(p) + 255) & ~(uintptr_t)255);
+  out->cand_rec = reinterpret_cast<F4*>(p);
+  p += (size_t)kSegWaves * seg_cap * 16;
+  p = reinterpret_cast<char*>((reinterpret_cast<uintptr_t>(p) + 255) & ~(uintptr_t)255);
+  out->ovf_cap = (int64_t)kSegWaves * seg_cap / 2;
+  out->ovf_rec = reinterpret_cast<F4*>(p);
+  p += (size_t)out->ovf_cap * 16;
+  out->ovf_idx = reinterpret_cast<uint32_t*>(p);
+  p += (size_t)out->ovf_cap * 4;
+  out->ovf_key = reinterpret_cast<uint32_t*>(p);
+  p += (size_t)out->ovf_cap * 4;
+  p = reinterpret_cast<char*>((reinterpret_cast<uintptr_t>(p) + 255) & ~(uintptr_t)255);
+  out->tie_cnt = reinterpret_cast<uint32_t*>(p);
+  out->tie_idx = out->tie_cnt + 64;
+  p += 256 + (size_t)kSpecTieCap * 4;
+  p = reinterpret_cast<char*>((reinterpret_cast<uintptr_t>(p) + 255) & ~(uintptr_t)255);
+  out->stage = p;
+  return true;
+}
+
+// Margin of the single-sweep bracket, in standard deviations of the sample rank.
+constexpr double kSpecSigmas = 12.0;
+
+template <bool BF16G, bool BF16V, int SCORE>
+static int run_fused_spec(const void* g, float* resid, float* p, float* m, float* v, int64_t n,
+                          int64_t k, const sga_segment* segs, int n_segs, int32_t* idx_out,
+                          void* values_out, uint8_t* mask_out, float factor, float coeff,
+                          int flags, float interval, uint32_t seed, sga_select_result* result,
+                          const SelWorkspace& w, const SpecWorkspace& x, hipStream_t s,
+                          int64_t pack_extra) {
+  const bool vec = aligned4(g, BF16G ? 2 : 4) && aligned4(resid, 4) && aligned4(p, 4) &&
+                   aligned4(m, 4) && aligned4(v, 4);
+  const int adams = (flags & SGA_GC_ADAMS) ? 1 : 0;
+  SrcFused<BF16G, SCORE> src{g, resid, p, m, v, vec, {}, pack_extra, adams};
+  launch_seg_dir(segs, n_segs, n, w.seg_dir, s);
+  src.sc.init(segs, n_segs, w.seg_dir);
+  const int64_t n_tiles = cdiv64(n, kChunk);
+  FinalArgs fa;
+  fa.g = g; fa.r = resid; fa.p = p; fa.m = m; fa.v = v; fa.n = n; fa.k = k;
+  fa.idx_out = idx_out; fa.values_out = values_out; fa.mask_out = mask_out;
+  fa.factor = factor; fa.coeff = coeff; fa.T = 0; fa.need = 0;
+  fa.vec = vec; fa.mvec = aligned4(mask_out, 1);
+  fa.scale = factor != 1.0f; fa.apply_coeff = coeff != 1.0f;
+  fa.pack_extra = pack_extra;
+  fa.adams = adams != 0; fa.fold = (flags & SGA_GC_FOLD) != 0; fa.interval = interval;
+  fa.planes = w.pbits;
+  // sample -> bracket with the wide margins
+  launch_begin((uint32_t)k, w, s);
+  int64_t n_sv = w.sample_cap / 4;
+  const int64_t n_vec = n / 4;
+  if (n_sv > n_vec) n_sv = n_vec;
+  const int64_t win = n_vec / n_sv;
+  const int64_t ns = n_sv * 4;
+  hipLaunchKernelGGL((k_sample<SrcFused<BF16G, SCORE>>), dim3(stream_grid(n_sv, kBlock)), dim3(kBlock), 0, s,
+                     src, n, n_sv, win, w.sample, seed);
+  hipLaunchKernelGGL(k_bracket_ranks, dim3(1), dim3(kBlock), 0, s, w.aux, w.hist, kHistStride * 2,
+                     (uint32_t)k, (double)n, (double)ns, w.seg_cnt, w.blk_gt, w.blk_eq, kSpecSigmas);
+  SrcU32 ssrc{w.sample};
+  for (int level = 0; level < 3; ++level)
+    launch_level<SrcU32, 2, true>(ssrc, ns, (const uint32_t*)nullptr, level, w.aux, w, s, kRawKeyBlocks);
+  // the sweep
+  SpecArgs sa;
+  sa.splane = w.pbits; sa.fplane = x.dplane; sa.stage = x.stage;
+  sa.seg_idx = w.seg_idx; sa.seg_key = w.seg_key; sa.seg_rec = x.seg_rec; sa.seg_cnt = w.seg_cnt;
+  sa.seg_cap = (uint32_t)w.seg_cap;
+  sa.tile_gt = w.tile_gt; sa.tile_eq = w.tile_eq; sa.hi_part = w.blk_gt; sa.nf_part = w.blk_eq;
+  sa.ovf_idx = x.ovf_idx; sa.ovf_key = x.ovf_key; sa.ovf_rec = x.ovf_rec;
+  sa.ovf_cnt = w.seg_cnt + kSegWaves + 1; sa.ovf_cap = (uint32_t)x.ovf_cap;
+  sa.chunks_per_seg = (uint32_t)cdiv64(n_tiles, kSegWaves);
+  sa.n_over_ns = (double)n / (double)ns;
+  sa.est_limit = 0.5 * (double)kSegWaves * (double)w.seg_cap;
+  const dim3 one_shot((unsigned)cdiv64(n_tiles, kChunksPerBlock));
+  ProfPair* pp = prof_begin(SGA_PROF_FUSED_FINAL, s);
+  hipLaunchKernelGGL((k_fused_spec<BF16G, BF16V, SCORE>), one_shot, dim3(kBlock), 0, s, fa, sa, segs,
+                     n_segs, w.st, w.aux, w.seg_dir);
+  prof_end(pp, s);
+  hipLaunchKernelGGL(k_bracket_check, dim3(1), dim3(kBlock), 0, s, w.st, w.aux, w.seg_cnt, w.hist,
+                     kHistStride * 2, (uint32_t)w.seg_cap, w.blk_gt, w.blk_eq, 1, (uint32_t)x.ovf_cap);
+  hipLaunchKernelGGL(k_cand_compact, dim3(512), dim3(kBlock), 0, s, w.aux, w.seg_cnt, w.seg_idx,
+                     w.seg_key, (uint32_t)w.seg_cap, w.cand_idx, w.cand_key, x.seg_rec, x.cand_rec);
+  hipLaunchKernelGGL(k_spec_ovf_compact, dim3(64), dim3(kBlock), 0, s, w.aux, w.seg_cnt, x.ovf_idx,
+                     x.ovf_key, x.ovf_rec, (uint32_t)x.ovf_cap, w.cand_idx, w.cand_key, x.cand_rec,
+                     x.tie_cnt);
+  SrcU32 csrc{w.cand_key};
+  const int64_t cmax = (int64_t)kSegWaves * w.seg_cap;
+  for (int level = 0; level < 3; ++level)
+    launch_level<SrcU32, 1, true>(csrc, cmax, &w.st->cand_count, level, w.aux, w, s, 3 * kRawKeyBlocks);
+  hipLaunchKernelGGL(k_cand_tiles, dim3(512), dim3(kBlock), 0, s, w.st, w.aux, w.cand_idx,
+                     w.cand_key, w.tile_gt, w.tile_eq);
+  // only when the sweep stood back: the radix passes over the untouched data
+  for (int level = 0; level < 3; ++level)
+    launch_level<SrcFused<BF16G, SCORE>, 1, true>(src, n, (const uint32_t*)nullptr, level, w.st, w, s);
+  launch_tile_count(src, n, 0, w, s);
+  launch_tile_scan(n_tiles, 0, w, s);
+  hipLaunchKernelGGL(k_spec_ties, dim3(512), dim3(kBlock), 0, s, w.st, w.cand_idx, w.cand_key,
+                     w.tile_eq, n_tiles, x.tie_cnt, x.tie_idx);
+  hipLaunchKernelGGL(k_spec_settle, dim3(512), dim3(kBlock), 0, s, w.st, w.cand_idx, w.cand_key,
+                     w.tile_eq, n_tiles, x.tie_cnt, x.tie_idx, x.dplane);
+  hipLaunchKernelGGL((k_spec_pack<BF16V>), dim3((unsigned)cdiv64(n_tiles * kChunkIters, kWave)),
+                     dim3(kWave), 0, s, fa, w.st, x.stage, w.pbits, x.dplane, w.tile_gt, x.slab_pos);
+  hipLaunchKernelGGL((k_spec_repair<BF16V>), dim3(1024), dim3(kBlock), 0, s, fa, segs, n_segs,
+                     w.seg_dir, w.st, w.cand_idx, w.cand_key, x.cand_rec, x.dplane, x.slab_pos);
+  if (mask_out)
+    hipLaunchKernelGGL(k_expand_mask, dim3(stream_grid(n_tiles, kChunksPerBlock, 1 << 22)), dim3(kBlock),
+                       0, s, w.st, x.dplane, n, mask_out, (reinterpret_cast<uintptr_t>(mask_out) & 15) == 0);
+  // the sweep stood back: the key-forming final sweep does the step (a small grid that strides
+  // over the chunks; it returns at once otherwise)
+  hipLaunchKernelGGL((k_fused_final<BF16G, BF16V, SCORE, false>),
+                     dim3(stream_grid(n_tiles, kChunksPerBlock, 2048)), dim3(kBlock), 0, s, fa,
+                     segs, n_segs, w.st, w.tile_gt, w.tile_eq, 3, w.seg_dir);
+  if (result) hipLaunchKernelGGL(k_sel_result, dim3(1), dim3(1), 0, s, w.st, result);
+  return check_launch("sga_fused_sparse_step_single_sweep");
+}
+
 }  // namespace sga
 
 using namespace sga;
@@ -423,7 +1134,8 @@ static int fused_entry(const char* who, const void* g, int g_dtype, float* resid
                        const sga_segment* segs, int n_segs, int score_id, int32_t* idx_out,
                        void* values_out, int values_dtype, uint8_t* mask_out, float factor,
                        float coeff, int fast, int flags, float interval, sga_select_result* result,
-                       void* ws, size_t ws_bytes, void* stream) {
+                       void* ws, size_t ws_bytes, void* stream, bool single = false,
+                       void* ws2 = nullptr, size_t ws2_bytes = 0, uint32_t seed = 0u) {
   if ((flags & ~(SGA_GC_ADAMS | SGA_GC_FOLD)) != 0) {
     // the dual-lr split belongs to full steps (adamw.py:570-580); HAS_MASK / CLEAR / APPLY_COEFF
     // are what this step does anyway (coeff != 1 applies the coefficient)
@@ -452,7 +1164,34 @@ static int fused_entry(const char* who, const void* g, int g_dtype, float* resid
   }
   hipStream_t s = (hipStream_t)stream;
   const bool bg = g_dtype == SGA_BF16, bv = values_dtype == SGA_BF16;
+  SpecWorkspace x = {};
+  if (single) {
+    if (!spec_ws_carve(ws2, ws2_bytes, n, bv ? 2 : 4, fast_seg_cap((cdiv64(n, kChunk) + 8) * kChunk), &x)) {
+      set_error("%s: second workspace missing, not 256-byte aligned or smaller than "
+                "sga_fused_single_sweep_workspace_bytes(n, values_dtype)=%zu", who,
+                spec_ws_bytes(n, bv ? 2 : 4));
+      return SGA_ERR_WORKSPACE;
+    }
+    // Shapes the single sweep does not take (the two-sweep step does them, same outputs): buckets
+    // too small for the sampled bracket, a bracket that would be open below, or one whose
+    // expected candidates do not fit the buffers.
+    bool take = n >= kFastMinN && w.sample != nullptr && w.pbits != nullptr &&
+                w.seg_cap == fast_seg_cap((cdiv64(n, kChunk) + 8) * kChunk);
+    if (take) {
+      int64_t n_sv = w.sample_cap / 4;
+      if (n_sv > n / 4) n_sv = n / 4;
+      const double ns = (double)n_sv * 4.0, frac = (double)k / (double)n, r = frac * ns;
+      const double d = kSpecSigmas * sqrt(r * (1.0 - frac) + 1.0) + 8.0;
+      if (r + d > ns) take = false;
+      if ((2.0 * d + 2.0) * ((double)n / ns) > 0.25 * (double)kSegWaves * (double)w.seg_cap) take = false;
+    }
+    if (!take) { single = false; fast = 1; }
+  }
 #define SGA_RUN(BG, BV, SC)                                                                   \
+  if (single)                                                                                 \
+    return run_fused_spec<BG, BV, SC>(g, resid, p, m, v, n, k, segs, n_segs, idx_out,        \
+                                      values_out, mask_out, factor, coeff, flags, interval,   \
+                                      seed, result, w, x, s, pack_extra);                     \
   return run_fused<BG, BV, SC>(g, resid, p, m, v, n, k, segs, n_segs, idx_out, values_out,   \
                                mask_out, factor, coeff, fast, flags, interval, result, w, s,   \
                                pack_extra)
@@ -483,6 +1222,39 @@ extern "C" int sga_fused_sparse_step(const void* g, int g_dtype, float* resid, f
   return fused_entry("sga_fused_sparse_step", g, g_dtype, resid, p, m, v, 0, n, k, segs, n_segs,
                      score_id, idx_out, values_out, values_dtype, mask_out, factor, coeff, fast,
                      flags, interval, result, ws, ws_bytes, stream);
+}
+
+extern "C" size_t sga_fused_single_sweep_workspace_bytes(int64_t n, int values_dtype) {
+  return spec_ws_bytes(n < 0 ? 0 : n, values_dtype == SGA_BF16 ? 2 : 4);
+}
+
+extern "C" int sga_fused_sparse_step_single_sweep(
+    const void* g, int g_dtype, float* resid, float* p, float* m, float* v, int64_t n, int64_t k,
+    const sga_segment* segs, int n_segs, int score_id, int32_t* idx_out, void* values_out,
+    int values_dtype, uint8_t* mask_out, float factor, float coeff, int flags, float interval,
+    uint32_t seed, sga_select_result* result, void* ws, size_t ws_bytes, void* ws2,
+    size_t ws2_bytes, void* stream) {
+  return fused_entry("sga_fused_sparse_step_single_sweep", g, g_dtype, resid, p, m, v, 0, n, k,
+                     segs, n_segs, score_id, idx_out, values_out, values_dtype, mask_out, factor,
+                     coeff, 1, flags, interval, result, ws, ws_bytes, stream, true, ws2, ws2_bytes,
+                     seed);
+}
+
+extern "C" int sga_fused_sparse_step_single_sweep_packed(
+    const void* g, int g_dtype, float* state, int64_t n, int64_t k, const sga_segment* segs,
+    int n_segs, int score_id, int32_t* idx_out, void* values_out, int values_dtype,
+    uint8_t* mask_out, float factor, float coeff, int flags, float interval, uint32_t seed,
+    sga_select_result* result, void* ws, size_t ws_bytes, void* ws2, size_t ws2_bytes,
+    void* stream) {
+  if (state && (reinterpret_cast<uintptr_t>(state) & 15)) {
+    set_error("sga_fused_sparse_step_single_sweep_packed: state must be 16-byte aligned");
+    return SGA_ERR_ARG;
+  }
+  return fused_entry("sga_fused_sparse_step_single_sweep_packed", g, g_dtype, state,
+                     state ? state + kPackRun : nullptr, state ? state + 2 * kPackRun : nullptr,
+                     state ? state + 3 * kPackRun : nullptr, kPackExtra, n, k, segs, n_segs,
+                     score_id, idx_out, values_out, values_dtype, mask_out, factor, coeff, 1,
+                     flags, interval, result, ws, ws_bytes, stream, true, ws2, ws2_bytes, seed);
 }
 
 extern "C" int64_t sga_packed_state_elems(int64_t n) {

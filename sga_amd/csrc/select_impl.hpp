@@ -43,7 +43,8 @@ struct SelState {
   uint32_t overflow;    // a candidate segment ran out of room
   uint32_t skip;        // 1: kernels driven by this state do nothing
   uint32_t done[3];     // per-level "workgroups finished" tickets (last one scans)
-  uint32_t pad_[8];
+  uint32_t spec;        // 1: the single-sweep step committed on the sampled bracket (no way back)
+  uint32_t pad_[7];
 };
 static_assert(sizeof(SelState) == 128, "SelState layout");
 
@@ -747,12 +748,13 @@ __device__ __forceinline__ uint32_t mix32(uint32_t x) {
 }
 
 // One 4-element vector per window of `win` vectors, at a hashed offset.
+// `seed` moves the offsets (0: the fixed pattern); the select is exact for any of them.
 template <class Src>
 __global__ __launch_bounds__(kBlock) void k_sample(Src src, int64_t n, int64_t n_sv, int64_t win,
-                                                   uint32_t* __restrict__ keys) {
+                                                   uint32_t* __restrict__ keys, uint32_t seed = 0u) {
   for (int64_t j = (int64_t)blockIdx.x * kBlock + threadIdx.x; j < n_sv;
        j += (int64_t)gridDim.x * kBlock) {
-    const int64_t vec = j * win + (int64_t)(mix32((uint32_t)j) % (uint32_t)win);
+    const int64_t vec = j * win + (int64_t)(mix32((uint32_t)j + seed * 0x9E3779B9u) % (uint32_t)win);
     uint32_t key[4];
     src.template load<false>(vec * 4, n, key);
     U4 o{key[0], key[1], key[2], key[3]};
@@ -765,14 +767,14 @@ __global__ __launch_bounds__(kBlock) void k_sample(Src src, int64_t n, int64_t n
 // lower end.  Also zeroes both histogram sets.
 static __global__ void k_bracket_ranks(SelState* aux, uint32_t* hist, int nhist, uint32_t k,
                                        double n, double ns, uint32_t* seg_cnt, uint32_t* hi_part,
-                                       uint32_t* nf_part) {
+                                       uint32_t* nf_part, double sigmas = 5.0) {
   for (int i = threadIdx.x; i < nhist; i += blockDim.x) hist[i] = 0u;
-  for (int i = threadIdx.x; i <= kSegWaves; i += blockDim.x) seg_cnt[i] = 0u;
+  for (int i = threadIdx.x; i <= kSegWaves + 1; i += blockDim.x) seg_cnt[i] = 0u;   // + overflow count
   for (int i = threadIdx.x; i < kSweepParts; i += blockDim.x) { hi_part[i] = 0u; nf_part[i] = 0u; }
   if (threadIdx.x != 0) return;
   const double frac = (double)k / n;
   const double r = frac * ns;
-  const double d = 5.0 * sqrt(r * (1.0 - frac) + 1.0) + 8.0;
+  const double d = sigmas * sqrt(r * (1.0 - frac) + 1.0) + 8.0;
   SelState hi = {}, lo = {};
   const double rh = floor(r - d), rl = ceil(r + d);
   if (rh < 1.0) hi.skip = 1; else hi.k = (uint32_t)rh;
@@ -958,7 +960,8 @@ static __global__ __launch_bounds__(kBlock) void k_bracket_check(SelState* __res
                                                                  uint32_t* __restrict__ hist, int nhist,
                                                                  uint32_t seg_cap,
                                                                  const uint32_t* __restrict__ hi_part,
-                                                                 const uint32_t* __restrict__ nf_part) {
+                                                                 const uint32_t* __restrict__ nf_part,
+                                                                 int spec = 0, uint32_t ovf_cap = 0u) {
   __shared__ uint32_t s_w4[kChunksPerBlock];
   constexpr int PER = kSegWaves / kBlock;   // 32
   uint32_t v[PER], mine = 0, over = 0;
@@ -986,16 +989,25 @@ static __global__ __launch_bounds__(kBlock) void k_bracket_check(SelState* __res
   block_excl_scan(over, s_w4, dummy);
   const bool any_over = dummy != 0;
   if (threadIdx.x == 0) {
-    seg_cnt[kSegWaves] = total;
+    seg_cnt[kSegWaves] = total;       // where the overflow list's records go in the dense list
+    bool ovf_over = false;
+    if (ovf_cap) {                    // single-sweep step: records of the shared overflow list
+      const uint32_t oc = seg_cnt[kSegWaves + 1];
+      ovf_over = oc > ovf_cap || (uint64_t)total + oc > (uint64_t)kSegWaves * seg_cap;
+      total += oc < ovf_cap ? oc : ovf_cap;
+    }
     const uint32_t k = st->k;
-    const bool ok = !st->overflow && !any_over && n_hi < k && k <= n_hi + total;
+    const bool ok = !st->overflow && !any_over && !ovf_over && n_hi < k && k <= n_hi + total;
     st->n_hi = n_hi;
     st->cand_count = total;
+    // A single-sweep step that went ahead has already committed on the bracket: a miss cannot
+    // be repaired by the radix passes, it is reported (status 3) and nothing further runs.
+    const bool lost = spec && st->spec && !ok;
     st->bracket_ok = ok ? 1u : 0u;
-    st->skip = ok ? 1u : 0u;          // the radix passes run only when the bracket failed
-    st->path = ok ? 1u : 0u;
+    st->skip = (ok || lost) ? 1u : 0u;   // the radix passes run only when the bracket failed
+    st->path = ok ? (spec ? 2u : 1u) : 0u;
     st->nonfinite = ok ? n_nf : 0u;   // recounted by the radix passes otherwise
-    if (!ok) st->status = 0u;
+    if (!ok) st->status = lost ? 3u : 0u;
     SelState z = {};
     z.k = ok ? k - n_hi : 0u;
     z.skip = ok ? 0u : 1u;
@@ -1007,7 +1019,8 @@ static __global__ __launch_bounds__(kBlock) void k_bracket_check(SelState* __res
 static __global__ __launch_bounds__(kBlock) void k_cand_compact(
     const SelState* __restrict__ aux, const uint32_t* __restrict__ seg_off,
     const uint32_t* __restrict__ seg_idx, const uint32_t* __restrict__ seg_key, uint32_t seg_cap,
-    uint32_t* __restrict__ cand_idx, uint32_t* __restrict__ cand_key) {
+    uint32_t* __restrict__ cand_idx, uint32_t* __restrict__ cand_key,
+    const F4* __restrict__ seg_rec = nullptr, F4* __restrict__ cand_rec = nullptr) {
   if (aux->skip) return;
   for (int w = blockIdx.x * kChunksPerBlock + wave_id(); w < kSegWaves;
        w += gridDim.x * kChunksPerBlock) {
@@ -1015,6 +1028,7 @@ static __global__ __launch_bounds__(kBlock) void k_cand_compact(
     for (uint32_t j = lane_id(); j < cnt; j += kWave) {
       cand_idx[off + j] = seg_idx[(int64_t)w * seg_cap + j];
       cand_key[off + j] = seg_key[(int64_t)w * seg_cap + j];
+      if (seg_rec) cand_rec[off + j] = seg_rec[(int64_t)w * seg_cap + j];
     }
   }
 }
@@ -1047,7 +1061,7 @@ static_assert(kChunk == 1024, "candidate -> chunk mapping uses idx >> 10");
 // Each lane expands 16 consecutive bytes: 4 lanes x 4 elements of one slab.
 static __global__ __launch_bounds__(kBlock) void k_expand_mask(
     const SelState* __restrict__ st, const uint32_t* __restrict__ pbits, int64_t n,
-    uint8_t* __restrict__ mask, bool mvec) {
+    uint8_t* __restrict__ mask, bool mvec, const uint32_t* __restrict__ pbits2 = nullptr) {
   if (st && !st->bracket_ok) return;
   const int64_t n_chunks = cdiv64(n, kChunk);
   const int64_t wstride = (int64_t)gridDim.x * kChunksPerBlock;
@@ -1055,7 +1069,13 @@ static __global__ __launch_bounds__(kBlock) void k_expand_mask(
   const int it = l >> 4, sl0 = (l & 15) * 4;        // slab, first slab-lane
   for (int64_t c = (int64_t)blockIdx.x * kChunksPerBlock + wave_id(); c < n_chunks; c += wstride) {
     const U4* pw = reinterpret_cast<const U4*>(pbits + c * 32 + it * 8);
-    const U4 lo = pw[0], hi = pw[1];
+    U4 lo = pw[0], hi = pw[1];
+    if (pbits2) {                                   // union of two planes
+      const U4* qw = reinterpret_cast<const U4*>(pbits2 + c * 32 + it * 8);
+      const U4 l2 = qw[0], h2 = qw[1];
+      lo = U4{lo.x | l2.x, lo.y | l2.y, lo.z | l2.z, lo.w | l2.w};
+      hi = U4{hi.x | h2.x, hi.y | h2.y, hi.z | h2.z, hi.w | h2.w};
+    }
     const uint32_t w[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
     uint32_t out[4];
 #pragma unroll

@@ -53,6 +53,15 @@ class FusedSparseStep:
         self._seg_up = L.TableUploader(C.sizeof(self._seg_host), device)
         self._seg_dev = self._seg_up.dev
         self._seg_step = None
+        self._ws2 = None          # second workspace of the single-sweep step, on first use
+        self._calls = 0
+
+    def _single_sweep_ws(self):
+        if self._ws2 is None:
+            nbytes = int(L.raw("sga_fused_single_sweep_workspace_bytes", self.n,
+                               L.dtype_code(self.values)))
+            self._ws2 = torch.empty(nbytes, dtype=torch.uint8, device=self.device)
+        return self._ws2
 
     def _upload_segments(self, step):
         if self._seg_step == step:
@@ -81,12 +90,20 @@ class FusedSparseStep:
 
     def step(self, g, resid, p, m, v, step, k=None, ratio_percent=None,
              score="abs_g", factor=1.0, coeff=1.0, fast=True, optimizer="adamw", fold=False,
-             interval=1.0, inactive_lr_scale=1.0):
+             interval=1.0, inactive_lr_scale=1.0, single_sweep=False, seed=None):
         """Run one fused step in place; returns (idx[:k], values[:k]) views.
         ``self.result`` holds the device-side select result (threshold bits,
         counts); nothing is synchronised here.  ``optimizer="adams"`` commits
         (and scores) with the AdamS tail; ``fold`` divides the new residual by
-        ``interval`` (the residual mean taken before a boundary)."""
+        ``interval`` (the residual mean taken before a boundary).
+
+        ``single_sweep``: read g / resid / p / m / v once instead of twice --
+        coordinates outside the sampled bracket are committed in the sweep
+        itself, the few inside it afterwards from their records.  Same outputs
+        bit for bit; ``result.status == 3`` reports the one thing that cannot
+        be repaired, a sampled bracket that missed the k-th key after the
+        commit (12 sigma margins; ``seed`` moves the sample offsets, default a
+        per-call counter)."""
         flags = self._flags(optimizer, fold, interval, inactive_lr_scale)
         n = self.n
         for t in (g, resid, p, m, v):
@@ -100,6 +117,17 @@ class FusedSparseStep:
         if score not in SCORE_MAP:
             raise ValueError(f"Unknown SGA score '{score}'. Registered: {sorted(SCORE_MAP)}")
         self._upload_segments(step)
+        if single_sweep:
+            ws2 = self._single_sweep_ws()
+            self._calls += 1
+            L.call("sga_fused_sparse_step_single_sweep", L.ptr(g), L.dtype_code(g), L.ptr(resid),
+                   L.ptr(p), L.ptr(m), L.ptr(v), n, k, L.ptr(self._seg_dev), len(self.segments),
+                   SCORE_MAP[score], L.ptr(self.idx), L.ptr(self.values),
+                   L.dtype_code(self.values), L.ptr(self.mask), L.f32(factor), L.f32(coeff),
+                   flags, L.f32(interval), (self._calls if seed is None else seed) & 0xFFFFFFFF,
+                   L.ptr(self.result), L.ptr(self.ws), self.ws_bytes, L.ptr(ws2), ws2.numel(),
+                   L.stream())
+            return self.idx[:k], self.values[:k]
         L.call("sga_fused_sparse_step", L.ptr(g), L.dtype_code(g), L.ptr(resid), L.ptr(p),
                L.ptr(m), L.ptr(v), n, k, L.ptr(self._seg_dev), len(self.segments),
                SCORE_MAP[score], L.ptr(self.idx), L.ptr(self.values),
@@ -110,7 +138,7 @@ class FusedSparseStep:
 
     def step_packed(self, g, state, step, k=None, ratio_percent=None, score="abs_g",
                     factor=1.0, coeff=1.0, fast=True, optimizer="adamw", fold=False,
-                    interval=1.0, inactive_lr_scale=1.0):
+                    interval=1.0, inactive_lr_scale=1.0, single_sweep=False, seed=None):
         """Same step on a ``PackedState`` (resid/p/m/v interleaved in 64 KiB
         records): same arithmetic and outputs."""
         flags = self._flags(optimizer, fold, interval, inactive_lr_scale)
@@ -126,6 +154,17 @@ class FusedSparseStep:
         if score not in SCORE_MAP:
             raise ValueError(f"Unknown SGA score '{score}'. Registered: {sorted(SCORE_MAP)}")
         self._upload_segments(step)
+        if single_sweep:
+            ws2 = self._single_sweep_ws()
+            self._calls += 1
+            L.call("sga_fused_sparse_step_single_sweep_packed", L.ptr(g), L.dtype_code(g),
+                   L.ptr(state.data), n, k, L.ptr(self._seg_dev), len(self.segments),
+                   SCORE_MAP[score], L.ptr(self.idx), L.ptr(self.values),
+                   L.dtype_code(self.values), L.ptr(self.mask), L.f32(factor), L.f32(coeff),
+                   flags, L.f32(interval), (self._calls if seed is None else seed) & 0xFFFFFFFF,
+                   L.ptr(self.result), L.ptr(self.ws), self.ws_bytes, L.ptr(ws2), ws2.numel(),
+                   L.stream())
+            return self.idx[:k], self.values[:k]
         L.call("sga_fused_sparse_step_packed", L.ptr(g), L.dtype_code(g), L.ptr(state.data), n, k,
                L.ptr(self._seg_dev), len(self.segments), SCORE_MAP[score], L.ptr(self.idx),
                L.ptr(self.values), L.dtype_code(self.values), L.ptr(self.mask), L.f32(factor),

@@ -1,0 +1,114 @@
+"""GPU parity of the single-sweep fused step (g / resid / p / m / v read once)
+against the CPU oracle, every output bit for bit, and its stand-back routes."""
+import pytest
+import torch
+
+from oracle import fused_step as OF
+from oracle import select as SEL
+from tests.test_gpu_fused import _segments
+from tests.util import same_bits, student_t
+
+pytestmark = pytest.mark.gpu
+
+
+def _run(dev, sizes, steps, ratio, gdtype, vdtype, score="abs_g", seed0=0, vary=False,
+         expect_path=2, packed=False, grads=None, **knobs):
+    from sga_amd.fused_step import FusedSparseStep, PackedState
+    segs, n = _segments(sizes, vary=vary)
+    gen = torch.Generator().manual_seed(1234)
+    p = torch.randn(n, generator=gen) * 0.02
+    m, v, r = torch.zeros(n), torch.zeros(n), torch.zeros(n)
+    dp, dm, dv, dr = (t.to(dev) for t in (p, m, v, r))
+    st = PackedState(n, dev).pack(dr, dp, dm, dv) if packed else None
+    fs = FusedSparseStep(n, segs, dev, values_dtype=vdtype, want_mask=True)
+    k = SEL.k_for(n, ratio)
+    for step in range(1, steps + 1):
+        g = (grads(n, seed0 + step - 1) if grads else student_t(n, seed0 + step - 1)).to(gdtype)
+        idx_ref, val_ref, mask_ref, th_ref = OF.fused_sparse_step(
+            g, r, p, m, v, segs, step, k=k, score=score, values_dtype=vdtype, **knobs)
+        if packed:
+            idx, vals = fs.step_packed(g.to(dev), st, step, k=k, score=score, single_sweep=True,
+                                       **knobs)
+            st.unpack(dr, dp, dm, dv)
+        else:
+            idx, vals = fs.step(g.to(dev), dr, dp, dm, dv, step, k=k, score=score,
+                                single_sweep=True, **knobs)
+        res = fs.read_result()
+        assert res.status == 0 and res.nonfinite == 0 and res.n_selected == k, vars(res)
+        assert expect_path is None or res.path == expect_path, vars(res)
+        assert res.thresh == th_ref, (step, res.thresh, th_ref)
+        assert torch.equal(idx.cpu(), idx_ref), step
+        assert torch.equal(fs.mask.cpu().bool(), mask_ref), step
+        it = torch.int16 if vdtype == torch.bfloat16 else torch.int32
+        assert torch.equal(vals.cpu().view(it), val_ref.view(it)), step
+        assert same_bits(dr, r) and same_bits(dm, m) and same_bits(dv, v), step
+        assert same_bits(dp, p), step
+    return n, k
+
+
+@pytest.mark.parametrize("score", ["abs_g", "update", "coi", "abs_m", "abs_g_blind",
+                                   "abs_gr_over_sqrt_v"])
+def test_scores_ragged_tensors(dev, score):
+    sizes = [300_000, 128, 37, 700_000, 3, 1024, 250_001, 130, 5, 60_000]
+    # |m| is all zeros at the first step: one plateau, which the sweep stands back from
+    _run(dev, sizes, 3, 1.0, torch.bfloat16, torch.bfloat16, score=score, vary=True,
+         expect_path=None if score == "abs_m" else 2)
+
+
+@pytest.mark.parametrize("ratio", [0.1, 10.0, 0.001])
+def test_ratios(dev, ratio):
+    _run(dev, [1_500_003], 3, ratio, torch.bfloat16, torch.bfloat16, score="update")
+
+
+def test_fp32_grads_fp32_values_packed(dev):
+    _run(dev, [1 << 21, 999, 300_001], 3, 1.0, torch.float32, torch.float32, packed=True)
+
+
+@pytest.mark.parametrize("knobs", [dict(optimizer="adams"),
+                                   dict(optimizer="adamw", fold=True, interval=3.0, coeff=0.5),
+                                   dict(factor=0.125)])
+def test_knobs(dev, knobs):
+    _run(dev, [600_000, 130, 37, 500_000, 3, 1024, 100_001], 2, 1.0, torch.float32,
+         torch.bfloat16, score="update", vary=True, **knobs)
+
+
+def test_small_bucket_takes_the_two_sweep_step(dev):
+    _run(dev, [200_000, 1024, 100_000], 2, 1.0, torch.bfloat16, torch.bfloat16, expect_path=None)
+
+
+def test_wide_ratio_fills_the_small_segments(dev):
+    """At 60 % a chunk holds ~50 bracket keys against 64 slots of its own
+    segment: the chunks that do not fit go to the shared overflow list."""
+    _run(dev, [1_200_000], 2, 60.0, torch.bfloat16, torch.bfloat16, expect_path=2)
+
+
+def test_ratio_beyond_the_buffers_takes_the_two_sweep_step(dev):
+    _run(dev, [1 << 24], 1, 45.0, torch.bfloat16, torch.bfloat16, expect_path=None)
+
+
+def test_chunk_with_more_bracket_keys_than_lds_slots(dev):
+    """600 neighbouring coordinates sit within a hair of the k-th magnitude
+    (distinct values): their chunk overflows the wave's 256-slot buffer, is
+    read again and recorded straight in the overflow list."""
+    def grads(n, seed):
+        g = student_t(n, seed)
+        kth = g.abs().kthvalue(n - SEL.k_for(n, 1.0) + 1).values.item()
+        run = torch.arange(600, dtype=torch.float32)
+        g[500_000:500_600] = kth * (1.0 + (run - 300.0) * 1e-7)
+        return g
+    _run(dev, [1_400_000], 2, 1.0, torch.float32, torch.float32, grads=grads)
+    _run(dev, [700_000, 700_000], 1, 1.0, torch.float32, torch.bfloat16, score="update",
+         grads=grads, expect_path=None)
+
+
+def test_plateau_inside_the_bracket_stands_back(dev):
+    """Half of the coordinates share one magnitude that straddles the k-th
+    key: the sample sees the plateau, the sweep stands back before touching
+    anything and the radix passes do the step exactly."""
+    def grads(n, seed):
+        g = student_t(n, seed)
+        gen = torch.Generator().manual_seed(seed + 99)
+        flat = torch.rand(n, generator=gen) < 0.5
+        g[flat] = 3e-3
+        return g
+    _run(dev, [1_300_000], 1, 30.0, torch.float32, torch.float32, expect_path=0, grads=grads)
