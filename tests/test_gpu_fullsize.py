@@ -199,6 +199,40 @@ def test_llama1b_set_update_score(dev, ratio):
     assert torch.equal(m, m0 * 0.9 + gq * (1.0 - 0.9))
 
 
+@pytest.mark.parametrize("ratio", [0.1, 1.0, 10.0])
+def test_llama1b_set_update_score_single_sweep(dev, ratio):
+    """The same configuration through the single-sweep step (g / resid / p /
+    m / v read once): the same properties against the torch rebuild of the
+    score, and every output -- idx, values, mask, residual, p, m, v, threshold
+    -- equal bit for bit to the two-sweep step run from the same state."""
+    from sga_amd.fused_step import FusedSparseStep, k_for
+    from sga_amd.shapes import llama32_1b, segments_for
+    segs, n = segments_for(llama32_1b())
+    step = 5
+    g = _student_t(n, 3, dev).to(torch.bfloat16)
+    gen = torch.Generator(device=dev).manual_seed(2)
+    p = torch.randn(n, generator=gen, device=dev) * 0.02
+    m = torch.randn(n, generator=gen, device=dev) * 1e-4
+    v = torch.rand(n, generator=gen, device=dev) * 1e-8
+    r = _student_t(n, 4, dev, scale=3e-4)
+    k = k_for(n, ratio)
+    fs = FusedSparseStep(n, segs, dev, values_dtype=torch.bfloat16, max_k=k, want_mask=True)
+    r2, p2, m2, v2 = r.clone(), p.clone(), m.clone(), v.clone()
+    idx, vals = fs.step(g, r2, p2, m2, v2, step, k=k, score="update")
+    ref = fs.read_result()
+    idx2, vals2, mask2 = idx.clone(), vals.clone(), fs.mask.clone()
+    assert ref.status == 0 and ref.path == 1
+    idx, vals = fs.step(g, r, p, m, v, step, k=k, score="update", single_sweep=True)
+    res = fs.read_result()
+    assert res.status == 0 and res.n_selected == k and res.path == 2 and res.nonfinite == 0
+    assert (res.thresh_bits, res.need, res.n_gt, res.n_eq) == (ref.thresh_bits, ref.need, ref.n_gt,
+                                                              ref.n_eq)
+    assert torch.equal(idx, idx2) and torch.equal(fs.mask, mask2)
+    assert torch.equal(vals.view(torch.int16), vals2.view(torch.int16))
+    for a, b in ((r, r2), (p, p2), (m, m2), (v, v2)):
+        assert torch.equal(a.view(torch.int32), b.view(torch.int32))
+
+
 def _select_ok(score, mask, k):
     """Exact-k, dominance and lowest-index ties of a mask against a score."""
     assert int(mask.sum()) == k

@@ -112,3 +112,47 @@ def test_plateau_inside_the_bracket_stands_back(dev):
         g[flat] = 3e-3
         return g
     _run(dev, [1_300_000], 1, 30.0, torch.float32, torch.float32, expect_path=0, grads=grads)
+
+
+def _mix32(x):
+    x &= 0xFFFFFFFF
+    x ^= x >> 16
+    x = (x * 0x7FEB352D) & 0xFFFFFFFF
+    x ^= x >> 15
+    x = (x * 0x846CA68B) & 0xFFFFFFFF
+    x ^= x >> 16
+    return x
+
+
+def test_a_bracket_that_missed_is_reported(dev):
+    """The one outcome the single sweep cannot repair: every quad the sample
+    reads (its offsets restated here for the given seed) holds a magnitude in
+    [1, 2), every other coordinate one in [3, 4).  The sample's bracket sits
+    near 2, practically the whole bucket lies above it, and the check after
+    the sweep reports status 3 instead of a selection.  With another seed the
+    sample sees the real population and the same data gives the exact step."""
+    from sga_amd.fused_step import FusedSparseStep
+    n, seed = 1 << 21, 12345
+    n_sv, win = 16384, (n // 4) // 16384
+    gen = torch.Generator().manual_seed(5)
+    g = 3.0 + torch.rand(n, generator=gen)
+    for j in range(n_sv):
+        vec = j * win + _mix32(j + seed * 0x9E3779B9) % win
+        g[4 * vec: 4 * vec + 4] = 1.0 + torch.rand(4, generator=gen)
+    segs = [dict(start=0, n=n, lr=1e-4, b1=0.9, b2=0.95, eps=1e-8, wd=0.0)]
+    k = SEL.k_for(n, 1.0)
+
+    def run(sd):
+        p = torch.zeros(n, device=dev)
+        m, v, r = torch.zeros(n, device=dev), torch.zeros(n, device=dev), torch.zeros(n, device=dev)
+        fs = FusedSparseStep(n, segs, dev, values_dtype=torch.float32, want_mask=True)
+        idx, vals = fs.step(g.to(dev), r, p, m, v, 1, k=k, single_sweep=True, seed=sd)
+        return fs.read_result(), idx.cpu(), fs.mask.cpu().bool()
+
+    res, _, _ = run(seed)
+    assert res.status == 3 and res.path == 0, vars(res)
+    res, idx, mask = run(seed + 1)
+    assert res.status == 0 and res.n_selected == k, vars(res)
+    ref_mask, th = SEL.select_topk_flat(g.abs(), k)
+    assert res.thresh == th and torch.equal(mask, ref_mask)
+    assert torch.equal(idx.long(), torch.nonzero(ref_mask).reshape(-1))
