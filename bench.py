@@ -6,12 +6,14 @@ One "step" = score -> exact top-k (lowest-index ties) -> index pack (int32 idx
 Llama-3.2-1B-shaped gradient set (1,235,814,400 elements, 146 tensors, bf16
 Student-t(3) gradients, fp32 p/m/v/residual) with every input resident in HBM.
 
-The headline is the drop-in entry point (resid / p / m / v as the caller's four
+The headline is the drop-in layout (resid / p / m / v as the caller's four
 flat tensors, as the reference's buffers are) with the Adam-normalised score
-(`update`) at 1 %.  The same JSON line carries the whole sweep of the
-benchmark configuration -- scores {update, abs_g} x ratios {0.1, 1, 10} % x
-state layouts {separate, packed (library-owned 64 KiB records)} -- with each
-leg's own algorithmic bytes, one row for the Qwen3-0.6B per-bucket mask-layout
+(`update`) at 1 %, through the single-sweep step (every array read once;
+--two-sweep headlines the step that reads the score inputs twice).  The same
+JSON line carries the whole sweep of the benchmark configuration -- step
+variants {two-sweep, single-sweep} x scores {update, abs_g} x ratios {0.1, 1,
+10} % x state layouts {separate, packed (library-owned 64 KiB records)} -- with
+each leg's own algorithmic bytes, one row for the Qwen3-0.6B per-bucket mask-layout
 configuration, one for the 1e9-element stress buffer, the fused replay leg and
 the CPU oracle timed on a bounded sample of the headline workload.  The
 dominant kernels are timed live with HIP events on their launch stream.
@@ -487,7 +489,7 @@ def stress_row(steps=3):
                            "path": res.path}}
 
 
-def load_traffic(layout, score, ratio):
+def load_traffic(layout, score, ratio, single):
     """HBM bytes per launch of the final sweep from the committed counter
     profile -- only when that profile was taken on this very configuration."""
     tpath = os.path.join(ROOT, "profiles", "fused_final_llama1b_traffic.json")
@@ -499,7 +501,8 @@ def load_traffic(layout, score, ratio):
         entries = [entries]
     for e in entries:
         c = e.get("config", {})
-        if (c.get("layout"), c.get("score"), c.get("ratio_percent")) == (layout, score, ratio):
+        if (c.get("layout"), c.get("score"), c.get("ratio_percent"),
+                bool(c.get("single_sweep", False))) == (layout, score, ratio, bool(single)):
             return e.get("hbm_bytes_per_launch"), "profiles/fused_final_llama1b_traffic.json"
     return None, None
 
@@ -516,8 +519,9 @@ def main():
     ap.add_argument("--layout", choices=("separate", "packed"), default="separate",
                     help="headline state layout: separate = the drop-in entry point on four flat "
                          "tensors; packed = the library-owned 64 KiB records")
-    ap.add_argument("--single-sweep", action="store_true",
-                    help="headline the single-sweep step (g / resid / p / m / v read once)")
+    ap.add_argument("--two-sweep", dest="single_sweep", action="store_false",
+                    help="headline the two-sweep step (select sweep + final sweep: the score "
+                         "inputs are read twice) instead of the single-sweep step")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
     ap.add_argument("--cpu-sample", type=int, default=1 << 28)
     ap.add_argument("--calib", action="store_true",
@@ -632,15 +636,23 @@ def main():
         L.raw("sga_prof_enable", 0)
         res = fs.read_result()
         assert res.status == 0 and res.n_selected == k, vars(res)
-        final_bytes = n * ALG_BYTES_FINAL + k * 6.0
-        sweep_bytes = n * sweep_bytes_per_elem(score)
+        # dominant kernel: k_fused_final reads g, r, p, m, v, writes r, p, m, v and the pack
+        # (4 + 2 B per selected coordinate); k_fused_spec (single sweep) the same state traffic
+        # and one staged 2 B value per coordinate it takes as selected
+        final_bytes = n * ALG_BYTES_FINAL + k * (2.0 if single else 6.0)
+        sweep_bytes = 0.0 if single else n * sweep_bytes_per_elem(score)
+        # two-read model of the step (the select needs the score inputs once, the commit again)
         step_bytes = n * step_bytes_per_elem(score) + k * 6.0
+        # bytes a step that reads every array once has to move
+        once_bytes = n * ALG_BYTES_FINAL + k * 6.0
         fin_avg, sw_avg = fin_ms / max(fin_n, 1), sw_ms / max(sw_n, 1)
         return {"layout": layout, "single_sweep": single, "score": score, "ratio_percent": ratio, "k": k, "steps": steps,
                 "seconds": dt, "ms_per_step": dt / steps * 1e3, "elem_per_s": n * steps / dt,
                 "alg_bytes_per_elem": step_bytes_per_elem(score),
                 "alg_bytes_per_step": step_bytes,
                 "step_frac": step_bytes * steps / dt / HBM_PEAK,
+                "read_once_bytes_per_step": once_bytes,
+                "read_once_frac": once_bytes * steps / dt / HBM_PEAK,
                 "final_avg_ms": fin_avg, "final_bytes": final_bytes,
                 "final_frac": final_bytes / (fin_avg * 1e-3) / HBM_PEAK if fin_avg > 0 else None,
                 "sweep_avg_ms": sw_avg, "sweep_bytes": sweep_bytes,
@@ -663,13 +675,17 @@ def main():
     if state["packed"] is not None:
         state["packed"].unpack(r, p, m, v)
         state["packed"] = None
-    traffic, traffic_src = load_traffic(args.layout, args.score, args.ratio)
+    traffic, traffic_src = load_traffic(args.layout, args.score, args.ratio, args.single_sweep)
     k = head["k"]
     value = n * args.steps / head["seconds"]
-    layout_txt = ("resid/p/m/v interleaved in 64 KiB records (sga_fused_sparse_step_packed)"
+    entry = "sga_fused_sparse_step" + ("_single_sweep" if args.single_sweep else "")
+    layout_txt = (f"resid/p/m/v interleaved in 64 KiB records ({entry}_packed)"
                   if args.layout == "packed" else
-                  "resid/p/m/v as the caller's four flat tensors (sga_fused_sparse_step, the "
-                  "drop-in entry point)")
+                  f"resid/p/m/v as the caller's four flat tensors ({entry}, the drop-in layout)")
+    sweeps_txt = ("single sweep: g / resid / p / m / v read once, coordinates inside the sampled "
+                  "bracket committed on a guess and repaired after the candidate descent"
+                  if args.single_sweep else
+                  "two sweeps: select sweep over the score inputs, then the final sweep")
     out = {
         "metric": "grad elems/s (score+top-k+resid AdamW)",
         "value": value, "unit": "elem/s", "n_gpus": 1, "steps": args.steps,
@@ -679,21 +695,32 @@ def main():
         "config": {"workload": "Llama-3.2-1B-shaped set, 1,235,814,400 elems / 146 tensors, "
                                "bf16 Student-t(3) grads, fp32 p/m/v/residual, score "
                                f"{args.score}, exact top-k {args.ratio}% (k={k}), index pack "
-                               "int32+bf16, residual-aware AdamW; state layout: " + layout_txt,
+                               "int32+bf16, residual-aware AdamW; " + sweeps_txt +
+                               "; state layout: " + layout_txt,
                    "ratio_percent": args.ratio, "score": args.score, "k": k,
+                   "single_sweep": bool(args.single_sweep),
                    "state_layout": args.layout, "grad_dtype": "bf16", "values_dtype": "bf16",
                    "state_dtype": "f32", "arithmetic": "f32"},
         "roofline": {"bound": "hbm", "achieved": head["final_bytes"] / (head["final_avg_ms"] * 1e-3) / 1e9,
                      "peak": HBM_PEAK / 1e9, "unit": "GB/s", "frac": head["final_frac"],
                      "traffic": traffic, "traffic_source": traffic_src,
-                     "kernel": "k_fused_final", "avg_ms": head["final_avg_ms"],
+                     "kernel": "k_fused_spec" if args.single_sweep else "k_fused_final",
+                     "avg_ms": head["final_avg_ms"],
                      "alg_bytes_per_launch": head["final_bytes"]},
+        # whole step against two byte models: the two-read model the roofline target is stated
+        # on (the score inputs once for the select, every array again for the commit: 52 B per
+        # element for the Adam-normalised score, 40 for |g + r|), and the bytes a step that reads
+        # every array once has to move (34 B per element + the pack)
         "step_roofline": {"alg_bytes_per_elem": head["alg_bytes_per_elem"],
                           "achieved_GBps": head["alg_bytes_per_step"] / (head["ms_per_step"] * 1e-3) / 1e9,
                           "frac": head["step_frac"],
-                          "select_sweep": {"kernel": "k_bracket_sweep", "avg_ms": head["sweep_avg_ms"],
-                                           "alg_bytes_per_launch": head["sweep_bytes"],
-                                           "frac": head["sweep_frac"]}},
+                          "model": "two-read (select reads the score inputs, commit reads all)",
+                          "read_once_bytes_per_elem": ALG_BYTES_FINAL,
+                          "read_once_frac": head["read_once_frac"],
+                          "select_sweep": (None if args.single_sweep else
+                                           {"kernel": "k_bracket_sweep", "avg_ms": head["sweep_avg_ms"],
+                                            "alg_bytes_per_launch": head["sweep_bytes"],
+                                            "frac": head["sweep_frac"]})},
         "select": head["select"],
         "sweep": sweep,
     }
