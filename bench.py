@@ -376,6 +376,69 @@ def trace_io_bench(W=4, tmp=None):
         shutil.rmtree(d, ignore_errors=True)
 
 
+def placement_probe(reps=5, trials=6, seed=1):
+    """The final sweep's mix of streams (bf16 g and fp32 r, p, m, v read; r, p, m, v written:
+    34 B per element, math-free stand-in k_calib_streams) over the Llama-3.2-1B element count
+    on differently placed arrays of ONE process: fresh tensors, one carved 25 GB block with the
+    arrays back to back and at random 4 KiB-granular offsets, fresh tensors with random spacers
+    between them.  Virtual addresses are printed; what differs between runs of the same virtual
+    layout is the physical backing."""
+    import random
+    import torch
+    from sga_amd import _lib as L
+    from sga_amd.shapes import llama32_1b, segments_for
+    dev = torch.device("cuda:0")
+    _, n = segments_for(llama32_1b())
+    rows = []
+
+    def timeit(tag, g, r, p, m, v):
+        a = [L.ptr(g), L.ptr(r), L.ptr(p), L.ptr(m), L.ptr(v), n, L.stream()]
+        L.call("sga_calib_streams", *a)
+        ev = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
+        torch.cuda.synchronize()
+        ev[0].record()
+        for _ in range(reps):
+            L.call("sga_calib_streams", *a)
+        ev[1].record()
+        torch.cuda.synchronize()
+        ms = ev[0].elapsed_time(ev[1]) / reps
+        rows.append({"placement": tag, "ms": ms, "GBps": 34.0 * n / ms / 1e6,
+                     "ptrs": [hex(t.data_ptr()) for t in (g, r, p, m, v)]})
+
+    def fresh():
+        return (torch.zeros(n, dtype=torch.bfloat16, device=dev),
+                *[torch.zeros(n, device=dev) for _ in range(4)])
+
+    for i in range(2):
+        t = fresh()
+        timeit(f"fresh tensors #{i}", *t)
+        del t
+        torch.cuda.empty_cache()
+    mb2 = 2 << 20
+    ab = (n * 4 + mb2 - 1) // mb2 * mb2
+    slab = torch.zeros(ab * 5 + (64 << 20) * 8, dtype=torch.uint8, device=dev)
+
+    def carve(offs):
+        return (slab[offs[0]: offs[0] + 2 * n].view(torch.bfloat16),
+                *[slab[o: o + 4 * n].view(torch.float32) for o in offs[1:]])
+    timeit("one block, arrays back to back", *carve([i * ab for i in range(5)]))
+    rnd = random.Random(seed)
+    for i in range(trials):
+        timeit(f"one block, random 4 KiB-granular offsets #{i}",
+               *carve([j * ab + rnd.randrange(0, 64 << 20, 4096) for j in range(5)]))
+    del slab
+    torch.cuda.empty_cache()
+    for i in range(trials):
+        keep, ts = [], []
+        for j in range(5):
+            keep.append(torch.empty(rnd.randrange(1 << 20, 3 << 30), dtype=torch.uint8, device=dev))
+            ts.append(torch.zeros(n, dtype=torch.bfloat16 if j == 0 else torch.float32, device=dev))
+        timeit(f"fresh tensors, random spacers #{i}", *ts)
+        del ts, keep
+        torch.cuda.empty_cache()
+    return {"kernel": "k_calib_streams", "n": n, "bytes_per_launch": 34.0 * n, "rows": rows}
+
+
 def qwen_mask_layout_row(steps=5, warmup=2):
     """Qwen3-0.6B-shaped set, bf16 Gaussian grads with per-tensor std
     log-uniform in [1e-5, 1e-2], per-bucket exact top-k at 1 % (the embedding,
@@ -537,6 +600,9 @@ def main():
                          "back through the pread reader and the dense pass) and print its JSON")
     ap.add_argument("--primitives", action="store_true",
                     help="time the drop-in primitives on their own and print their JSON")
+    ap.add_argument("--placement", action="store_true",
+                    help="run just the placement probe of the final sweep's stream mix (same "
+                         "kernel, differently placed arrays) and print its JSON")
     ap.add_argument("--only-replay", action="store_true",
                     help="run just the fused replay leg (for profiling) and print its JSON")
     args = ap.parse_args()
@@ -554,6 +620,10 @@ def main():
     if args.only_replay:
         torch.cuda.set_device(0)
         print(json.dumps(replay_bench()))
+        return
+    if args.placement:
+        torch.cuda.set_device(0)
+        print(json.dumps(placement_probe()))
         return
     if args.trace_io:
         torch.cuda.set_device(0)
