@@ -1060,10 +1060,9 @@ static int run_fused_spec(const void* g, float* resid, float* p, float* m, float
   int64_t n_sv = w.sample_cap / 4;
   const int64_t n_vec = n / 4;
   if (n_sv > n_vec) n_sv = n_vec;
-  const int64_t win = n_vec / n_sv;
   const int64_t ns = n_sv * 4;
   hipLaunchKernelGGL((k_sample<SrcFused<BF16G, SCORE>>), dim3(stream_grid(n_sv, kBlock)), dim3(kBlock), 0, s,
-                     src, n, n_sv, win, w.sample, seed);
+                     src, n, n_sv, n_vec, w.sample, seed);
   hipLaunchKernelGGL(k_bracket_ranks, dim3(1), dim3(kBlock), 0, s, w.aux, w.hist, kHistStride * 2,
                      (uint32_t)k, (double)n, (double)ns, w.seg_cnt, w.blk_gt, w.blk_eq, kSpecSigmas);
   SrcU32 ssrc{w.sample};

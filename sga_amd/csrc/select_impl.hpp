@@ -747,14 +747,18 @@ __device__ __forceinline__ uint32_t mix32(uint32_t x) {
   return x;
 }
 
-// One 4-element vector per window of `win` vectors, at a hashed offset.
-// `seed` moves the offsets (0: the fixed pattern); the select is exact for any of them.
+// One 4-element vector per window, at a hashed offset; the n_sv windows tile
+// ALL n_vec vectors (window j = [j n_vec / n_sv, (j + 1) n_vec / n_sv)): a tail
+// that no window covered would bias the sample whenever the last tensors score
+// differently from the rest.  `seed` moves the offsets (0: the fixed pattern);
+// the select is exact for any of them.
 template <class Src>
-__global__ __launch_bounds__(kBlock) void k_sample(Src src, int64_t n, int64_t n_sv, int64_t win,
+__global__ __launch_bounds__(kBlock) void k_sample(Src src, int64_t n, int64_t n_sv, int64_t n_vec,
                                                    uint32_t* __restrict__ keys, uint32_t seed = 0u) {
   for (int64_t j = (int64_t)blockIdx.x * kBlock + threadIdx.x; j < n_sv;
        j += (int64_t)gridDim.x * kBlock) {
-    const int64_t vec = j * win + (int64_t)(mix32((uint32_t)j + seed * 0x9E3779B9u) % (uint32_t)win);
+    const int64_t w0 = j * n_vec / n_sv, w1 = (j + 1) * n_vec / n_sv;
+    const int64_t vec = w0 + (int64_t)(mix32((uint32_t)j + seed * 0x9E3779B9u) % (uint32_t)(w1 - w0));
     uint32_t key[4];
     src.template load<false>(vec * 4, n, key);
     U4 o{key[0], key[1], key[2], key[3]};
@@ -1235,10 +1239,9 @@ static inline void run_select(Src src, int64_t n, int64_t k, int tie_all, bool f
     int64_t n_sv = w.sample_cap / 4;
     const int64_t n_vec = n / 4;
     if (n_sv > n_vec) n_sv = n_vec;
-    const int64_t win = n_vec / n_sv;
     const int64_t ns = n_sv * 4;
     hipLaunchKernelGGL((k_sample<Src>), dim3(stream_grid(n_sv, kBlock)), dim3(kBlock), 0, s, src, n,
-                       n_sv, win, w.sample);
+                       n_sv, n_vec, w.sample);
     // the sweep's two totals go through 256 partial counters (blk_gt / blk_eq are free until the
     // tile scan, which runs after the check has read them)
     hipLaunchKernelGGL(k_bracket_ranks, dim3(1), dim3(kBlock), 0, s, w.aux, w.hist, kHistStride * 2,

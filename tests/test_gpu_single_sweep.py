@@ -133,11 +133,12 @@ def test_a_bracket_that_missed_is_reported(dev):
     sample sees the real population and the same data gives the exact step."""
     from sga_amd.fused_step import FusedSparseStep
     n, seed = 1 << 21, 12345
-    n_sv, win = 16384, (n // 4) // 16384
+    n_sv, n_vec = 16384, n // 4
     gen = torch.Generator().manual_seed(5)
     g = 3.0 + torch.rand(n, generator=gen)
     for j in range(n_sv):
-        vec = j * win + _mix32(j + seed * 0x9E3779B9) % win
+        w0, w1 = j * n_vec // n_sv, (j + 1) * n_vec // n_sv
+        vec = w0 + _mix32(j + seed * 0x9E3779B9) % (w1 - w0)
         g[4 * vec: 4 * vec + 4] = 1.0 + torch.rand(4, generator=gen)
     segs = [dict(start=0, n=n, lr=1e-4, b1=0.9, b2=0.95, eps=1e-8, wd=0.0)]
     k = SEL.k_for(n, 1.0)
@@ -156,3 +157,49 @@ def test_a_bracket_that_missed_is_reported(dev):
     ref_mask, th = SEL.select_topk_flat(g.abs(), k)
     assert res.thresh == th and torch.equal(mask, ref_mask)
     assert torch.equal(idx.long(), torch.nonzero(ref_mask).reshape(-1))
+
+
+def test_randomized_single_sweep_equals_two_sweep(dev):
+    """Seeded random draws of tensor layouts, hyper-parameters, scores, dtypes,
+    ratios, knobs and magnitudes: the single-sweep step and the two-sweep step
+    run from the same state and must agree in every output bit (idx, values,
+    mask, residual, p, m, v, threshold, tie counts) over several steps."""
+    import random
+    from sga_amd.fused_step import FusedSparseStep
+    rnd = random.Random(2024)
+    for draw in range(24):
+        sizes = [rnd.choice([3, 37, 130, 1024, 4097, 60_000]) for _ in range(rnd.randrange(2, 7))]
+        sizes.insert(rnd.randrange(len(sizes) + 1), rnd.randrange(1_100_000, 2_500_000))
+        segs, n = _segments(sizes, vary=True)
+        score = rnd.choice(["abs_g", "update", "coi", "abs_g_blind", "abs_gr_over_sqrt_v"])
+        gdt = rnd.choice([torch.bfloat16, torch.float32])
+        vdt = rnd.choice([torch.bfloat16, torch.float32])
+        ratio = rnd.choice([0.05, 0.5, 1.0, 3.0, 12.0])
+        knobs = rnd.choice([{}, dict(optimizer="adams"), dict(fold=True, interval=3.0),
+                            dict(factor=0.5, coeff=0.25)])
+        scale = 10.0 ** rnd.uniform(-8, 0)
+        gen = torch.Generator().manual_seed(draw)
+        p0 = (torch.randn(n, generator=gen) * 0.02).to(dev)
+        state = [[p0.clone(), torch.zeros(n, device=dev), torch.zeros(n, device=dev),
+                  torch.zeros(n, device=dev)] for _ in range(2)]
+        fs = [FusedSparseStep(n, segs, dev, values_dtype=vdt, want_mask=True) for _ in range(2)]
+        k = SEL.k_for(n, ratio)
+        for step in range(1, 4):
+            g = (student_t(n, 100 * draw + step) * (scale / 1e-3)).to(gdt).to(dev)
+            outs = []
+            for which in range(2):
+                pp, mm, vv, rr = state[which]
+                idx, vals = fs[which].step(g, rr, pp, mm, vv, step, k=k, score=score,
+                                           single_sweep=bool(which), **knobs)
+                res = fs[which].read_result()
+                assert res.status == 0 and res.n_selected == k, (draw, step, which, vars(res))
+                outs.append((idx, vals, fs[which].mask, res))
+            what = (draw, step, score, ratio, knobs)
+            assert outs[1][3].path in (0, 1, 2), what
+            assert (outs[0][3].thresh_bits, outs[0][3].need, outs[0][3].n_eq) == \
+                   (outs[1][3].thresh_bits, outs[1][3].need, outs[1][3].n_eq), what
+            assert torch.equal(outs[0][0], outs[1][0]) and torch.equal(outs[0][2], outs[1][2]), what
+            it = torch.int16 if vdt == torch.bfloat16 else torch.int32
+            assert torch.equal(outs[0][1].view(it), outs[1][1].view(it)), what
+            for a, b in zip(state[0], state[1]):
+                assert torch.equal(a.view(torch.int32), b.view(torch.int32)), what
