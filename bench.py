@@ -534,7 +534,7 @@ def stress_row(steps=3):
         dt = (time.perf_counter() - t0) / steps
         assert int(mask.sum()) == k
         sel[str(ratio)] = {"k": k, "ms": dt * 1e3, "elem_per_s": n / dt,
-                           "frac": n * (4.0 + 0.125 + 1.0) / dt / HBM_PEAK}
+                           "frac": n * (4.0 + 1.0) / dt / HBM_PEAK}
         del mask
     del score
     segs = [dict(start=0, n=n, lr=1e-4, b1=0.9, b2=0.95, eps=1e-8, wd=0.1)]
@@ -553,7 +553,7 @@ def stress_row(steps=3):
     assert res.status == 0 and res.n_selected == k, vars(res)
     alg = n * step_bytes_per_elem("abs_g", 4.0) + k * 8.0
     return {"workload": "one contiguous 1.0e9-element fp32 buffer, Student-t(3) with 5 % duplicated "
-                        "magnitudes; select_topk_flat alone (mask out; bytes = 4 read + 1/8 bit planes "
+                        "magnitudes; select_topk_flat alone (mask out; bytes = 4 read "
                         "+ 1 mask) and the fused step at 1 % (fp32 grads, idx int32 + fp32 values)",
             "n": n, "select_only": sel,
             "fused_step": {"k": k, "ms_per_step": dt * 1e3, "elem_per_s": n / dt,

@@ -335,8 +335,9 @@ extern "C" int sga_select_topk(const float* score, int64_t n, int64_t k, int tie
   hipStream_t s = (hipStream_t)stream;
   SrcF32 src{score, aligned4(score, 4)};
   const int tie_all = tie_mode == SGA_TIE_ALL;
-  run_select(src, n, k, tie_all, true, w, s, w.pbits);
-  finish_mask(src, n, tie_all, w, mask_out, s);
+  // the select sweep writes the keys above the bracket straight into mask_out
+  run_select(src, n, k, tie_all, true, w, s, nullptr, mask_out);
+  finish_mask(src, n, tie_all, w, mask_out, s, true);
   if (result) hipLaunchKernelGGL(k_sel_result, dim3(1), dim3(1), 0, s, w.st, result);
   return check_launch("sga_select_topk");
 }

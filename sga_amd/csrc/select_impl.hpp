@@ -844,12 +844,17 @@ __device__ __forceinline__ void plane_put(const Ballot4& a, int it, uint32_t* ld
 }
 
 // One chunk of the sweep.  chi / tot_nf / mycnt are wave totals (scalar).
-template <class Src, bool FULL, bool PM>
+// PM: 0 counts only; 1 the provisional selection (keys above the bracket) also goes out as bit
+// planes; 2 as mask bytes, straight into the caller's mask (a mask-only select then needs no
+// expansion pass: the candidates are settled in the bytes).
+template <class Src, bool FULL, int PM>
 __device__ __forceinline__ void bracket_chunk(Src& src, const typename Src::Chunk& ck, int64_t n,
                                               int64_t c, uint32_t T_LO,
                                               uint32_t T_HI, uint32_t& chi, uint32_t& tot_nf,
                                               uint32_t& mycnt, SweepLds& lds,
-                                              uint32_t* __restrict__ pbits) {
+                                              uint32_t* __restrict__ pbits,
+                                              uint8_t* __restrict__ mask_bytes = nullptr,
+                                              bool mvec = false) {
   // The loads of kAhead slabs (256 elements each) are issued together, then
   // their keys are formed slab by slab: expensive key sources (Adam-normalised
   // scores) look fewer slabs ahead to stay within their register budget.  The
@@ -894,21 +899,27 @@ __device__ __forceinline__ void bracket_chunk(Src& src, const typename Src::Chun
       // provisional mask as bit planes: everything above the bracket is
       // certainly selected; the few keys inside it are settled after the
       // candidate descent.  One 128-byte store per chunk.
-      if (PM) plane_put(above, it, lds.planes);
+      if (PM == 1) plane_put(above, it, lds.planes);
+      if (PM == 2 && (FULL || i < n)) {
+        const uint32_t mk[4] = {above.mine(0), above.mine(1), above.mine(2), above.mine(3)};
+        if (FULL && mvec) st_u8<true>(mask_bytes, i, n, mk, true);
+        else store4_u8(mask_bytes, i, n, mk, mvec);
+      }
     }
   }
-  if (PM) {
+  if (PM == 1) {
     __builtin_amdgcn_wave_barrier();
     if (lane_id() < kPlaneWordsPerChunk) pbits[c * kPlaneWordsPerChunk + lane_id()] = lds.planes[lane_id()];
   }
 }
 
-template <class Src, bool PM>
+template <class Src, int PM>
 __global__ __launch_bounds__(kBlock) void k_bracket_sweep(
     Src src, int64_t n, SelState* __restrict__ st, const SelState* __restrict__ aux,
     uint32_t* __restrict__ tile_gt, uint32_t* __restrict__ tile_eq, uint32_t* __restrict__ seg_idx,
     uint32_t* __restrict__ seg_key, uint32_t* __restrict__ seg_cnt, uint32_t seg_cap,
-    uint32_t* __restrict__ pbits, uint32_t* __restrict__ hi_part, uint32_t* __restrict__ nf_part) {
+    uint32_t* __restrict__ pbits, uint32_t* __restrict__ hi_part, uint32_t* __restrict__ nf_part,
+    uint8_t* __restrict__ mask_bytes = nullptr, bool mvec = false) {
   __shared__ uint32_t s_hi[kChunksPerBlock], s_nf[kChunksPerBlock];
   __shared__ SweepLds s_lds[kChunksPerBlock];
   // keys equal to the upper sample key stay candidates; a skipped end means
@@ -926,9 +937,9 @@ __global__ __launch_bounds__(kBlock) void k_bracket_sweep(
     uint32_t* const my_key = lds.key;
     const typename Src::Chunk ck = src.chunk_begin(c);
     if (src.vec && (c + 1) * kChunk <= n)
-      bracket_chunk<Src, true, PM>(src, ck, n, c, T_LO, T_HI, chi, tot_nf, mycnt, lds, pbits);
+      bracket_chunk<Src, true, PM>(src, ck, n, c, T_LO, T_HI, chi, tot_nf, mycnt, lds, pbits, mask_bytes, mvec);
     else
-      bracket_chunk<Src, false, PM>(src, ck, n, c, T_LO, T_HI, chi, tot_nf, mycnt, lds, pbits);
+      bracket_chunk<Src, false, PM>(src, ck, n, c, T_LO, T_HI, chi, tot_nf, mycnt, lds, pbits, mask_bytes, mvec);
     if (lane_id() == 0) { tile_gt[c] = chi; tile_eq[c] = 0u; }     // chi / tot_nf are wave totals
     if (mycnt) {                                        // wave-uniform
       const uint32_t seg = (uint32_t)c & (uint32_t)(kSegWaves - 1);
@@ -1231,7 +1242,8 @@ static __global__ __launch_bounds__(kBlock) void k_mask_to_planes(const uint8_t*
 // re-reading the data.
 template <class Src>
 static inline void run_select(Src src, int64_t n, int64_t k, int tie_all, bool fast,
-                              const SelWorkspace& w, hipStream_t s, uint32_t* planes = nullptr) {
+                              const SelWorkspace& w, hipStream_t s, uint32_t* planes = nullptr,
+                              uint8_t* mask_bytes = nullptr) {
   const bool want_mask = planes != nullptr;
   const int64_t n_tiles = cdiv64(n, kChunk);
   launch_begin((uint32_t)k, w, s);
@@ -1251,12 +1263,17 @@ static inline void run_select(Src src, int64_t n, int64_t k, int tie_all, bool f
       launch_level<SrcU32, 2, true>(ssrc, ns, (const uint32_t*)nullptr, level, w.aux, w, s, kRawKeyBlocks);
     const unsigned sweep_blocks = (unsigned)cdiv64(n_tiles, kChunksPerBlock);
     ProfPair* pp = prof_begin(SGA_PROF_SELECT_SWEEP, s);
-    if (want_mask)
-      hipLaunchKernelGGL((k_bracket_sweep<Src, true>), dim3(sweep_blocks), dim3(kBlock), 0, s,
+    if (mask_bytes)
+      hipLaunchKernelGGL((k_bracket_sweep<Src, 2>), dim3(sweep_blocks), dim3(kBlock), 0, s,
+                         src, n, w.st, w.aux, w.tile_gt, w.tile_eq, w.seg_idx, w.seg_key, w.seg_cnt,
+                         (uint32_t)w.seg_cap, (uint32_t*)nullptr, w.blk_gt, w.blk_eq, mask_bytes,
+                         (reinterpret_cast<uintptr_t>(mask_bytes) & 3) == 0);
+    else if (want_mask)
+      hipLaunchKernelGGL((k_bracket_sweep<Src, 1>), dim3(sweep_blocks), dim3(kBlock), 0, s,
                          src, n, w.st, w.aux, w.tile_gt, w.tile_eq, w.seg_idx, w.seg_key, w.seg_cnt,
                          (uint32_t)w.seg_cap, planes, w.blk_gt, w.blk_eq);
     else
-      hipLaunchKernelGGL((k_bracket_sweep<Src, false>), dim3(sweep_blocks), dim3(kBlock), 0, s,
+      hipLaunchKernelGGL((k_bracket_sweep<Src, 0>), dim3(sweep_blocks), dim3(kBlock), 0, s,
                          src, n, w.st, w.aux, w.tile_gt, w.tile_eq, w.seg_idx, w.seg_key, w.seg_cnt,
                          (uint32_t)w.seg_cap, (uint32_t*)nullptr, w.blk_gt, w.blk_eq);
     prof_end(pp, s);
@@ -1296,13 +1313,16 @@ static inline void finish_planes(Src src, int64_t n, int tie_all, const SelWorks
 // Byte mask of the selection after run_select(..., w.pbits): the bit planes
 // and the candidates settle it when the bracket held, else the ordered full
 // pass writes it.
+// in_bytes: the sweep already wrote the provisional selection as mask bytes (run_select(...,
+// nullptr, mask)); only the candidates are left to settle.
 template <class Src>
 static inline void finish_mask(Src src, int64_t n, int tie_all, const SelWorkspace& w,
-                               uint8_t* mask, hipStream_t s) {
+                               uint8_t* mask, hipStream_t s, bool in_bytes = false) {
   const int64_t nc = cdiv64(n, kChunk);
   if (w.pbits && n >= kFastMinN && n < (1ll << 32)) {
-    hipLaunchKernelGGL(k_expand_mask, dim3(stream_grid(nc, kChunksPerBlock, 1 << 22)), dim3(kBlock),
-                       0, s, w.st, w.pbits, n, mask, (reinterpret_cast<uintptr_t>(mask) & 15) == 0);
+    if (!in_bytes)
+      hipLaunchKernelGGL(k_expand_mask, dim3(stream_grid(nc, kChunksPerBlock, 1 << 22)), dim3(kBlock),
+                         0, s, w.st, w.pbits, n, mask, (reinterpret_cast<uintptr_t>(mask) & 15) == 0);
     hipLaunchKernelGGL(k_cand_mask, dim3(256), dim3(kBlock), 0, s, w.st, w.cand_idx, w.cand_key,
                        w.tile_eq, nc, tie_all, mask);
   }
