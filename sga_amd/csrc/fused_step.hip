@@ -458,7 +458,6 @@ struct SpecArgs {
   F4* ovf_rec;
   uint32_t* ovf_cnt;
   uint32_t ovf_cap;
-  uint32_t chunks_per_seg; // consecutive chunks share a segment: the lists come out in address order
   double n_over_ns;       // population / sample size
   double est_limit;       // stand back when the sample predicts more bracket keys than this
 };
@@ -676,11 +675,12 @@ __global__ __launch_bounds__(kBlock) void k_fused_spec(
     }
     if (lane_id() == 0) { sa.tile_gt[c] = chi; sa.tile_eq[c] = 0u; }
     if (mycnt) {                                        // wave-uniform
-      // The chunk's LDS records go, in one piece, to the segment of its range of chunks; when
-      // that is full (the reservation is taken back: every later one then sees the true count),
-      // to the shared overflow list.
-      uint32_t seg = (uint32_t)(c / sa.chunks_per_seg);
-      if (seg > (uint32_t)(kSegWaves - 1)) seg = kSegWaves - 1;
+      // The chunk's LDS records go, in one piece, to the segment its chunk index hashes to
+      // (neighbouring waves, which run at the same time, hit different counters: with one
+      // segment per range of consecutive chunks the sweep was 0.25 ms slower); when that is full
+      // (the reservation is taken back: every later one then sees the true count), to the
+      // shared overflow list.
+      const uint32_t seg = (uint32_t)c & (uint32_t)(kSegWaves - 1);
       uint32_t base = 0;
       if (lane_id() == 0) {
         base = atomicAdd(&sa.seg_cnt[seg], mycnt);
@@ -1076,7 +1076,6 @@ static int run_fused_spec(const void* g, float* resid, float* p, float* m, float
   sa.tile_gt = w.tile_gt; sa.tile_eq = w.tile_eq; sa.hi_part = w.blk_gt; sa.nf_part = w.blk_eq;
   sa.ovf_idx = x.ovf_idx; sa.ovf_key = x.ovf_key; sa.ovf_rec = x.ovf_rec;
   sa.ovf_cnt = w.seg_cnt + kSegWaves + 1; sa.ovf_cap = (uint32_t)x.ovf_cap;
-  sa.chunks_per_seg = (uint32_t)cdiv64(n_tiles, kSegWaves);
   sa.n_over_ns = (double)n / (double)ns;
   sa.est_limit = 0.5 * (double)kSegWaves * (double)w.seg_cap;
   const dim3 one_shot((unsigned)cdiv64(n_tiles, kChunksPerBlock));
