@@ -77,7 +77,8 @@ typedef struct sga_select_result {
   uint32_t nonfinite;   /* NaN/Inf lanes seen (selection is undefined > 0) */
   uint32_t status;      /* 0 ok; 1 k out of range; 2 fast path fell back;
                            3 single-sweep bracket missed (step invalid)    */
-  uint32_t path;        /* 0 radix passes, 1 sampled bracket, 2 single sweep */
+  uint32_t path;        /* low byte: 0 radix passes, 1 sampled bracket, 2 single
+                           sweep; bit 8: an fp32 score array held a value < 0 */
 } sga_select_result;
 
 /* ---- scheme-agnostic masked ops (sga/kernels.py) ------------------------ */

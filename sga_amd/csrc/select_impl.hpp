@@ -44,7 +44,8 @@ struct SelState {
   uint32_t skip;        // 1: kernels driven by this state do nothing
   uint32_t done[3];     // per-level "workgroups finished" tickets (last one scans)
   uint32_t spec;        // 1: the single-sweep step committed on the sampled bracket (no way back)
-  uint32_t pad_[7];
+  uint32_t negative;    // 1: an fp32 score array held a value below zero (magnitudes were ranked)
+  uint32_t pad_[6];
 };
 static_assert(sizeof(SelState) == 128, "SelState layout");
 
@@ -179,6 +180,8 @@ struct NoChunk {};
 struct SrcF32 {                 // |x| of an fp32 score array
   const float* x;
   bool vec;
+  uint32_t neg;                 // this lane has seen a value below zero (callers that promise
+                                // non-negative scores are told, without a pass of their own)
   using Raw = F4;
   using Chunk = NoChunk;
   static constexpr int kAhead = kChunkIters;
@@ -191,15 +194,24 @@ struct SrcF32 {                 // |x| of an fp32 score array
   template <bool FULL>
   __device__ __forceinline__ void keys(const Chunk&, int64_t, int64_t, const Raw& r, uint32_t key[4]) {
     key[0] = abs_key(r.x); key[1] = abs_key(r.y); key[2] = abs_key(r.z); key[3] = abs_key(r.w);
+    neg |= (uint32_t)((r.x < 0.0f) | (r.y < 0.0f) | (r.z < 0.0f) | (r.w < 0.0f));
   }
   template <bool FULL = false>
   __device__ __forceinline__ void load(int64_t i, int64_t n, uint32_t key[4]) {
     float v[4];
     ld_f32<FULL>(x, i, n, v, vec);
 #pragma unroll
-    for (int e = 0; e < 4; ++e) key[e] = abs_key(v[e]);
+    for (int e = 0; e < 4; ++e) { key[e] = abs_key(v[e]); neg |= (uint32_t)(v[e] < 0.0f); }
   }
 };
+// What a key source knows about the sign of its inputs (only fp32 score arrays keep track).
+template <class Src>
+__device__ __forceinline__ uint32_t src_negative(const Src&) { return 0u; }
+__device__ __forceinline__ uint32_t src_negative(const SrcF32& s) { return s.neg; }
+template <class Src>
+__device__ __forceinline__ void note_negative(const Src& src, SelState* st) {
+  if (ballot64(src_negative(src) != 0u) != 0ull && lane_id() == 0) atomicOr(&st->negative, 1u);
+}
 
 struct SrcU32 {                 // raw keys (sample / candidate buffers)
   const uint32_t* x;
@@ -428,7 +440,7 @@ static __global__ void k_sel_begin(SelState* st, uint32_t* hist, int nhist, uint
 template <class Src>
 __global__ __launch_bounds__(kBlock) void k_tile_count(Src src, int64_t n,
                                                        int64_t tile_base,
-                                                       const SelState* __restrict__ st,
+                                                       SelState* __restrict__ st,
                                                        uint32_t* __restrict__ tile_gt,
                                                        uint32_t* __restrict__ tile_eq) {
   if (st->skip) return;
@@ -468,6 +480,7 @@ __global__ __launch_bounds__(kBlock) void k_tile_count(Src src, int64_t n,
       tile_eq[tile_base + c] = ce;
     }
   }
+  note_negative(src, st);
 }
 
 // Tile scan, kernel 1: per-workgroup totals of (gt, eq).
@@ -678,7 +691,7 @@ static __global__ void k_sel_result(const SelState* st, sga_select_result* out) 
   out->n_selected = st->n_selected;
   out->nonfinite = st->nonfinite;
   out->status = st->status;
-  out->path = st->path;
+  out->path = st->path | (st->negative ? 0x100u : 0u);
 }
 
 // -------------------------------------------------------------- host drivers
@@ -957,6 +970,7 @@ __global__ __launch_bounds__(kBlock) void k_bracket_sweep(
       }
     }
   }
+  note_negative(src, st);
   if (lane_id() == 0) { s_hi[wave_id()] = chi; s_nf[wave_id()] = tot_nf; }
   __syncthreads();
   if (threadIdx.x == 0) {

@@ -48,7 +48,7 @@ def select_topk_flat(t, k, check=True):
         if r.nonfinite:
             raise ValueError("select_topk_flat requires finite scores (NaN/Inf would "
                              "land in the top bins and silently pollute the topk)")
-        if bool((flat < 0).any().item()):
+        if r.negative:        # seen by the select's own sweep: no pass of its own, no second sync
             raise ValueError("select_topk_flat requires non-negative scores")
     if r.n_selected != k:
         raise RuntimeError(f"internal tie-break error: selected {r.n_selected} != {k}")

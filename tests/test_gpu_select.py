@@ -345,3 +345,28 @@ def test_adjacent_views_take_the_flat_path(dev):
         assert read_result(rc).path == 0 and torch.equal(torch.cat(mc).cpu().bool(), m_ref)
         th, masks = select_masks_histogram(views, k, mode="exact")
         assert th == t_ref and torch.equal(torch.cat(masks).cpu().bool(), flat.abs() >= t_ref)
+
+
+@pytest.mark.parametrize("n", [1000, 300_000, (1 << 20) + 4097, 3_000_001])
+def test_negative_score_is_rejected_by_the_select_itself(dev, n):
+    """``sga/replay.py:545-547`` rejects a score below zero.  The select's own
+    sweep reports it (no extra pass): one negative anywhere, first / last /
+    mid element, in an aligned or a scalar-path view, on the radix path (small
+    n) and the one-sweep path (n >= 2^20).  -0.0 is not negative there
+    (``(t < 0).any()``), and is not here."""
+    from sga_amd.replay import select_topk_flat
+    base = student_t(n, 11 + n).abs()
+    k = max(1, n // 100)
+    for pos in (0, n // 2 + 1, n - 1):
+        t = base.clone()
+        t[pos] = -1.0e-30
+        with pytest.raises(ValueError, match="non-negative"):
+            select_topk_flat(t.to(dev), k)
+        with pytest.raises(ValueError, match="non-negative"):
+            select_topk_flat(torch.cat([torch.zeros(1), t]).to(dev)[1:], k)
+        select_topk_flat(t.to(dev), k, check=False)      # the unchecked form ranks magnitudes
+    t = base.clone()
+    t[n // 3] = -0.0
+    m_ref, t_ref = SEL.select_topk_flat(t, k)
+    m_dev, t_dev = select_topk_flat(t.to(dev), k)
+    assert t_dev == t_ref and torch.equal(m_dev.cpu(), m_ref)
