@@ -806,8 +806,9 @@ __device__ __forceinline__ uint32_t slab_rank_before(const uint32_t* __restrict_
 // (F without S) stay untouched: the window is pre-filled with a sentinel.
 // slab_pos[slab] = pack position of the slab's first selected coordinate.
 constexpr int kPackWindow = 1024;
+constexpr int kPackDenseCut = 32;         // k above n / this: a lane per quarter slab
 constexpr int kPackAhead = 8;             // staged values a lane requests before it walks its bits
-template <bool BF16V>
+template <bool BF16V, int SUB>
 __global__ __launch_bounds__(kWave) void k_spec_pack(
     FinalArgs a, const SelState* __restrict__ st, const void* __restrict__ stage,
     const uint32_t* __restrict__ splane, const uint32_t* __restrict__ fplane,
@@ -816,7 +817,8 @@ __global__ __launch_bounds__(kWave) void k_spec_pack(
   __shared__ uint32_t l_val[kPackWindow + 4];
   if (!st->bracket_ok || !st->spec) return;
   const int64_t n_slabs = cdiv64(a.n, kChunk) * kChunkIters;
-  const int64_t slab = (int64_t)blockIdx.x * kWave + threadIdx.x;
+  const int64_t part = (int64_t)blockIdx.x * kWave + threadIdx.x;
+  const int64_t slab = part / SUB;
   const bool live = slab < n_slabs;
   uint64_t S[4] = {0, 0, 0, 0}, F[4] = {0, 0, 0, 0};
   uint32_t base = 0;
@@ -829,17 +831,27 @@ __global__ __launch_bounds__(kWave) void k_spec_pack(
     S[2] = ((uint64_t)x1.y << 32) | x1.x; S[3] = ((uint64_t)x1.w << 32) | x1.z;
     F[0] = ((uint64_t)y0.y << 32) | y0.x; F[1] = ((uint64_t)y0.w << 32) | y0.z;
     F[2] = ((uint64_t)y1.y << 32) | y1.x; F[3] = ((uint64_t)y1.w << 32) | y1.z;
+    if (SUB > 1) {                             // this lane's run of lane positions of the slab
+      constexpr int kBits = kWave / SUB;
+      const uint64_t own = (~0ull >> (64 - kBits)) << ((uint32_t)(part % SUB) * kBits);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) { S[e] &= own; F[e] &= own; }
+    }
   }
   const uint32_t cntS = (uint32_t)(__popcll(S[0]) + __popcll(S[1]) + __popcll(S[2]) + __popcll(S[3]));
   const uint32_t cntF = (uint32_t)(__popcll(F[0]) + __popcll(F[1]) + __popcll(F[2]) + __popcll(F[3]));
-  uint32_t ps = 0, pf = 0;
+  // counts of the chunk's earlier lanes (a chunk is kChunkIters * SUB consecutive lanes)
+  constexpr int kGroup = kChunkIters * SUB;
+  uint32_t ps = cntS, pf = cntF;
 #pragma unroll
-  for (int o = 1; o < kChunkIters; ++o) {
-    const uint32_t ts = __shfl_up(cntS, o, kWave), tf = __shfl_up(cntF, o, kWave);
-    if ((lane_id() & (kChunkIters - 1)) >= o) { ps += ts; pf += tf; }
+  for (int o = 1; o < kGroup; o <<= 1) {
+    const uint32_t ts = __shfl_up(ps, o, kWave), tf = __shfl_up(pf, o, kWave);
+    if ((lane_id() & (kGroup - 1)) >= o) { ps += ts; pf += tf; }
   }
+  ps -= cntS;
+  pf -= cntF;
   const uint32_t f_start = base + pf;
-  if (live) slab_pos[slab] = f_start;
+  if (live && part % SUB == 0) slab_pos[slab] = f_start;
   // the wave's run of the pack: [F0, F0 + len)
   const uint32_t F0 = __shfl(f_start, 0, kWave);
   uint32_t end = live ? f_start + cntF : 0u;
@@ -847,7 +859,10 @@ __global__ __launch_bounds__(kWave) void k_spec_pack(
   for (int o = kWave / 2; o > 0; o >>= 1) { const uint32_t t = __shfl_xor(end, o, kWave); end = t > end ? t : end; }
   const uint32_t len = end - F0;
   const int64_t c = slab >> 2;
-  uint64_t U = S[0] | S[1] | S[2] | S[3];
+  // every lane position that holds a coordinate of either plane is visited, in index order, so
+  // the positions in the staged run (S) and in the pack (F) are running counts
+  uint64_t U = S[0] | S[1] | S[2] | S[3] | F[0] | F[1] | F[2] | F[3];
+  uint32_t sr = 0, fr = f_start;
   // the lane's first staged values, all requested before the first is used (its run of the
   // staging array is contiguous); a slab with more entries loads the rest as it goes
   uint32_t ahead[kPackAhead];
@@ -865,29 +880,23 @@ __global__ __launch_bounds__(kWave) void k_spec_pack(
     __syncthreads();
     while (U) {
       const int L = __ffsll((unsigned long long)U) - 1;
-      const uint64_t below = L ? (~0ull >> (64 - L)) : 0ull;
-      uint32_t fr = f_start + (uint32_t)(__popcll(F[0] & below) + __popcll(F[1] & below) +
-                                         __popcll(F[2] & below) + __popcll(F[3] & below));
       if (fr - F0 >= w0 + (uint32_t)kPackWindow) break;     // belongs to a later window
       U &= U - 1;
-      uint32_t sr = ps + (uint32_t)(__popcll(S[0] & below) + __popcll(S[1] & below) +
-                                    __popcll(S[2] & below) + __popcll(S[3] & below));
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         const bool in_s = (S[e] >> L) & 1ull, in_f = (F[e] >> L) & 1ull;
         if (in_s && in_f) {
           const uint32_t t = fr - F0 - w0;
           l_idx[t] = (uint32_t)(slab * (kWave * kVec) + L * kVec + e);
-          const uint32_t u = sr - ps;
           uint32_t val;
-          if (u < (uint32_t)kPackAhead) {
+          if (sr < (uint32_t)kPackAhead) {
             val = ahead[0];
 #pragma unroll
-            for (int q = 1; q < kPackAhead; ++q) val = u == (uint32_t)q ? ahead[q] : val;
+            for (int q = 1; q < kPackAhead; ++q) val = sr == (uint32_t)q ? ahead[q] : val;
           } else if (BF16V) {
-            val = reinterpret_cast<const uint16_t*>(stage)[c * kChunk + sr];
+            val = reinterpret_cast<const uint16_t*>(stage)[c * kChunk + ps + sr];
           } else {
-            val = reinterpret_cast<const uint32_t*>(stage)[c * kChunk + sr];
+            val = reinterpret_cast<const uint32_t*>(stage)[c * kChunk + ps + sr];
           }
           l_val[t] = val;
         }
@@ -1105,8 +1114,14 @@ static int run_fused_spec(const void* g, float* resid, float* p, float* m, float
                      w.tile_eq, n_tiles, x.tie_cnt, x.tie_idx);
   hipLaunchKernelGGL(k_spec_settle, dim3(512), dim3(kBlock), 0, s, w.st, w.cand_idx, w.cand_key,
                      w.tile_eq, n_tiles, x.tie_cnt, x.tie_idx, x.dplane);
-  hipLaunchKernelGGL((k_spec_pack<BF16V>), dim3((unsigned)cdiv64(n_tiles * kChunkIters, kWave)),
-                     dim3(kWave), 0, s, fa, w.st, x.stage, w.pbits, x.dplane, w.tile_gt, x.slab_pos);
+  // a lane per slab, or per quarter of one where a slab holds more entries than a lane has
+  // staged values in flight
+  if (k > n / kPackDenseCut)
+    hipLaunchKernelGGL((k_spec_pack<BF16V, 4>), dim3((unsigned)cdiv64(n_tiles * kChunkIters * 4, kWave)),
+                       dim3(kWave), 0, s, fa, w.st, x.stage, w.pbits, x.dplane, w.tile_gt, x.slab_pos);
+  else
+    hipLaunchKernelGGL((k_spec_pack<BF16V, 1>), dim3((unsigned)cdiv64(n_tiles * kChunkIters, kWave)),
+                       dim3(kWave), 0, s, fa, w.st, x.stage, w.pbits, x.dplane, w.tile_gt, x.slab_pos);
   hipLaunchKernelGGL((k_spec_repair<BF16V>), dim3(1024), dim3(kBlock), 0, s, fa, segs, n_segs,
                      w.seg_dir, w.st, w.cand_idx, w.cand_key, x.cand_rec, x.dplane, x.slab_pos);
   if (mask_out)
