@@ -805,6 +805,25 @@ def main():
     }
     if calib:
         out["copy_calibration"] = calib
+    if args.layout == "separate":
+        # What the same five read and four write streams reach WITHOUT the math, on the very
+        # tensors the headline ran on (their contents are not needed any more): the ceiling this
+        # placement of four flat tensors gives a kernel of that stream mix.
+        sargs = [L.ptr(grads[0]), L.ptr(r), L.ptr(p), L.ptr(m), L.ptr(v), n, L.stream()]
+        ev = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
+        L.call("sga_calib_streams", *sargs)
+        ev[0].record()
+        for _ in range(5):
+            L.call("sga_calib_streams", *sargs)
+        ev[1].record()
+        torch.cuda.synchronize()
+        ms = ev[0].elapsed_time(ev[1]) / 5
+        out["roofline"]["stream_mix_copy"] = {
+            "kernel": "k_calib_streams (g bf16, r/p/m/v fp32 read; r/p/m/v written; no score, no "
+                      "select, no commit arithmetic), same tensors as the headline",
+            "avg_ms": ms, "GBps": n * ALG_BYTES_FINAL / ms / 1e6,
+            "frac_of_peak": n * ALG_BYTES_FINAL / (ms * 1e-3) / HBM_PEAK,
+            "dominant_kernel_vs_copy": ms / head["final_avg_ms"]}
     del p, m, v, r, grads, fs
     torch.cuda.empty_cache()
     if not args.no_rows:
