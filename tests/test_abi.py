@@ -104,3 +104,18 @@ def test_header_is_plain_c_and_struct_sizes_agree(tmp_path):
     assert got == [ctypes.sizeof(L.Segment), ctypes.sizeof(SelectResult),
                    ctypes.sizeof(ReplayCfg), ctypes.sizeof(ReplaySegment),
                    ctypes.sizeof(GcRecord), ctypes.sizeof(GccRecord)]
+
+
+def test_result_block_decoding():
+    """The eight words of ``sga_select_result``: the path is the low byte of
+    the last word, bit 8 says that an fp32 score array held a value below
+    zero (what ``sga/replay.py:545-547`` rejects)."""
+    import struct
+    import torch
+    from sga_amd.selection import read_result
+    th = struct.unpack("i", struct.pack("f", 0.75))[0]
+    r = read_result(torch.tensor([th, 3, 10, 5, 13, 0, 0, 1 | 0x100], dtype=torch.int32))
+    assert (r.thresh, r.need, r.n_gt, r.n_eq, r.n_selected) == (0.75, 3, 10, 5, 13)
+    assert r.path == 1 and r.negative and r.status == 0 and r.nonfinite == 0
+    r = read_result(torch.tensor([th, 3, 10, 5, 13, 2, 3, 2], dtype=torch.int32))
+    assert r.path == 2 and not r.negative and r.status == 3 and r.nonfinite == 2
