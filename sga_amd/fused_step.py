@@ -88,6 +88,34 @@ class FusedSparseStep:
             raise ValueError(f"fold needs interval > 0 (got {interval!r})")
         return (L.GC_ADAMS if optimizer == "adams" else 0) | (L.GC_FOLD if fold else 0)
 
+    def _run(self, name, g, state_args, step, k, ratio_percent, score, factor, coeff, fast,
+             optimizer, fold, interval, inactive_lr_scale, single_sweep, seed):
+        """Checks shared by the two state layouts, then one call of entry point
+        ``name`` (``state_args``: what that entry point takes between the
+        gradient and ``n``)."""
+        flags = self._flags(optimizer, fold, interval, inactive_lr_scale)
+        n = self.n
+        if k is None:
+            k = k_for(n, ratio_percent)
+        if not (1 <= k <= min(n, self.max_k)):
+            raise ValueError(f"k={k} out of range (n={n}, max_k={self.max_k})")
+        if score not in SCORE_MAP:
+            raise ValueError(f"Unknown SGA score '{score}'. Registered: {sorted(SCORE_MAP)}")
+        self._upload_segments(step)
+        head = [L.ptr(g), L.dtype_code(g), *state_args, n, k, L.ptr(self._seg_dev),
+                len(self.segments), SCORE_MAP[score], L.ptr(self.idx), L.ptr(self.values),
+                L.dtype_code(self.values), L.ptr(self.mask), L.f32(factor), L.f32(coeff)]
+        if single_sweep:
+            ws2 = self._single_sweep_ws()
+            self._calls += 1
+            L.call(name, *head, flags, L.f32(interval),
+                   (self._calls if seed is None else seed) & 0xFFFFFFFF, L.ptr(self.result),
+                   L.ptr(self.ws), self.ws_bytes, L.ptr(ws2), ws2.numel(), L.stream())
+        else:
+            L.call(name, *head, 1 if fast else 0, flags, L.f32(interval), L.ptr(self.result),
+                   L.ptr(self.ws), self.ws_bytes, L.stream())
+        return self.idx[:k], self.values[:k]
+
     def step(self, g, resid, p, m, v, step, k=None, ratio_percent=None,
              score="abs_g", factor=1.0, coeff=1.0, fast=True, optimizer="adamw", fold=False,
              interval=1.0, inactive_lr_scale=1.0, single_sweep=False, seed=None):
@@ -104,73 +132,29 @@ class FusedSparseStep:
         be repaired, a sampled bracket that missed the k-th key after the
         commit (12 sigma margins; ``seed`` moves the sample offsets, default a
         per-call counter)."""
-        flags = self._flags(optimizer, fold, interval, inactive_lr_scale)
-        n = self.n
         for t in (g, resid, p, m, v):
             L.require_dev(t)
             L.require_contig(t=t)
-            assert t.numel() == n
-        if k is None:
-            k = k_for(n, ratio_percent)
-        if not (1 <= k <= min(n, self.max_k)):
-            raise ValueError(f"k={k} out of range (n={n}, max_k={self.max_k})")
-        if score not in SCORE_MAP:
-            raise ValueError(f"Unknown SGA score '{score}'. Registered: {sorted(SCORE_MAP)}")
-        self._upload_segments(step)
-        if single_sweep:
-            ws2 = self._single_sweep_ws()
-            self._calls += 1
-            L.call("sga_fused_sparse_step_single_sweep", L.ptr(g), L.dtype_code(g), L.ptr(resid),
-                   L.ptr(p), L.ptr(m), L.ptr(v), n, k, L.ptr(self._seg_dev), len(self.segments),
-                   SCORE_MAP[score], L.ptr(self.idx), L.ptr(self.values),
-                   L.dtype_code(self.values), L.ptr(self.mask), L.f32(factor), L.f32(coeff),
-                   flags, L.f32(interval), (self._calls if seed is None else seed) & 0xFFFFFFFF,
-                   L.ptr(self.result), L.ptr(self.ws), self.ws_bytes, L.ptr(ws2), ws2.numel(),
-                   L.stream())
-            return self.idx[:k], self.values[:k]
-        L.call("sga_fused_sparse_step", L.ptr(g), L.dtype_code(g), L.ptr(resid), L.ptr(p),
-               L.ptr(m), L.ptr(v), n, k, L.ptr(self._seg_dev), len(self.segments),
-               SCORE_MAP[score], L.ptr(self.idx), L.ptr(self.values),
-               L.dtype_code(self.values), L.ptr(self.mask), L.f32(factor), L.f32(coeff),
-               1 if fast else 0, flags, L.f32(interval), L.ptr(self.result), L.ptr(self.ws),
-               self.ws_bytes, L.stream())
-        return self.idx[:k], self.values[:k]
+            assert t.numel() == self.n
+        return self._run("sga_fused_sparse_step" + ("_single_sweep" if single_sweep else ""), g,
+                         [L.ptr(resid), L.ptr(p), L.ptr(m), L.ptr(v)], step, k, ratio_percent,
+                         score, factor, coeff, fast, optimizer, fold, interval, inactive_lr_scale,
+                         single_sweep, seed)
 
     def step_packed(self, g, state, step, k=None, ratio_percent=None, score="abs_g",
                     factor=1.0, coeff=1.0, fast=True, optimizer="adamw", fold=False,
                     interval=1.0, inactive_lr_scale=1.0, single_sweep=False, seed=None):
         """Same step on a ``PackedState`` (resid/p/m/v interleaved in 64 KiB
         records): same arithmetic and outputs."""
-        flags = self._flags(optimizer, fold, interval, inactive_lr_scale)
-        n = self.n
         L.require_dev(g, state.data)
         L.require_contig(g=g)
-        if g.numel() != n or state.n != n:
+        if g.numel() != self.n or state.n != self.n:
             raise ValueError("gradient / packed state length does not match the bucket")
-        if k is None:
-            k = k_for(n, ratio_percent)
-        if not (1 <= k <= min(n, self.max_k)):
-            raise ValueError(f"k={k} out of range (n={n}, max_k={self.max_k})")
-        if score not in SCORE_MAP:
-            raise ValueError(f"Unknown SGA score '{score}'. Registered: {sorted(SCORE_MAP)}")
-        self._upload_segments(step)
-        if single_sweep:
-            ws2 = self._single_sweep_ws()
-            self._calls += 1
-            L.call("sga_fused_sparse_step_single_sweep_packed", L.ptr(g), L.dtype_code(g),
-                   L.ptr(state.data), n, k, L.ptr(self._seg_dev), len(self.segments),
-                   SCORE_MAP[score], L.ptr(self.idx), L.ptr(self.values),
-                   L.dtype_code(self.values), L.ptr(self.mask), L.f32(factor), L.f32(coeff),
-                   flags, L.f32(interval), (self._calls if seed is None else seed) & 0xFFFFFFFF,
-                   L.ptr(self.result), L.ptr(self.ws), self.ws_bytes, L.ptr(ws2), ws2.numel(),
-                   L.stream())
-            return self.idx[:k], self.values[:k]
-        L.call("sga_fused_sparse_step_packed", L.ptr(g), L.dtype_code(g), L.ptr(state.data), n, k,
-               L.ptr(self._seg_dev), len(self.segments), SCORE_MAP[score], L.ptr(self.idx),
-               L.ptr(self.values), L.dtype_code(self.values), L.ptr(self.mask), L.f32(factor),
-               L.f32(coeff), 1 if fast else 0, flags, L.f32(interval), L.ptr(self.result),
-               L.ptr(self.ws), self.ws_bytes, L.stream())
-        return self.idx[:k], self.values[:k]
+        name = ("sga_fused_sparse_step_single_sweep_packed" if single_sweep else
+                "sga_fused_sparse_step_packed")
+        return self._run(name, g, [L.ptr(state.data)], step, k, ratio_percent, score, factor,
+                         coeff, fast, optimizer, fold, interval, inactive_lr_scale, single_sweep,
+                         seed)
 
     def read_result(self):
         return read_result(self.result)
