@@ -233,6 +233,54 @@ def test_llama1b_set_update_score_single_sweep(dev, ratio):
         assert torch.equal(a.view(torch.int32), b.view(torch.int32))
 
 
+def test_llama1b_set_single_sweep_seeded_configs(dev):
+    """Seeded draws of score, ratio (0.01 - 25 %), gradient and value dtype and
+    the commit knobs on the full 1.24 B-element set, three steps each from a
+    shared start: the single-sweep step and the two-sweep step agree in every
+    output bit.  At this size the record lists, their overflow list and the
+    dense pack all carry millions of entries."""
+    import random
+    from sga_amd.fused_step import FusedSparseStep, k_for
+    from sga_amd.shapes import llama32_1b, segments_for
+    segs, n = segments_for(llama32_1b())
+    rnd = random.Random(7)
+    gen = torch.Generator(device=dev).manual_seed(0)
+    p0 = torch.randn(n, generator=gen, device=dev) * 0.02
+    grads = [_student_t(n, 10 + i, dev) for i in range(2)]
+    for cfg in range(5):
+        score = rnd.choice(["abs_g", "update", "coi", "abs_g_blind", "abs_gr_over_sqrt_v"])
+        ratio = rnd.choice([0.01, 0.1, 1.0, 3.2, 10.0, 25.0])
+        vdt = rnd.choice([torch.bfloat16, torch.float32])
+        gdt = rnd.choice([torch.bfloat16, torch.float32])
+        knobs = rnd.choice([{}, dict(optimizer="adams"), dict(fold=True, interval=3.0),
+                            dict(factor=0.5, coeff=0.25)])
+        what = (cfg, score, ratio, vdt, gdt, knobs)
+        k = k_for(n, ratio)
+        state = [[p0.clone()] + [torch.zeros(n, device=dev) for _ in range(3)] for _ in range(2)]
+        fs = [FusedSparseStep(n, segs, dev, values_dtype=vdt, max_k=k, want_mask=True)
+              for _ in range(2)]
+        for step in range(1, 4):
+            g = grads[step % 2].to(gdt)
+            outs = []
+            for which in range(2):
+                pp, mm, vv, rr = state[which]
+                idx, vals = fs[which].step(g, rr, pp, mm, vv, step, k=k, score=score,
+                                           single_sweep=bool(which), **knobs)
+                res = fs[which].read_result()
+                assert res.status == 0 and res.n_selected == k, (what, step, which, vars(res))
+                outs.append((idx, vals, fs[which].mask, res))
+            a, b = outs[0][3], outs[1][3]
+            assert (a.thresh_bits, a.need, a.n_eq) == (b.thresh_bits, b.need, b.n_eq), (what, step)
+            assert torch.equal(outs[0][0], outs[1][0]), (what, step)
+            assert torch.equal(outs[0][2], outs[1][2]), (what, step)
+            it = torch.int16 if vdt == torch.bfloat16 else torch.int32
+            assert torch.equal(outs[0][1].view(it), outs[1][1].view(it)), (what, step)
+            for x, y in zip(state[0], state[1]):
+                assert torch.equal(x.view(torch.int32), y.view(torch.int32)), (what, step)
+        del fs, state
+        torch.cuda.empty_cache()
+
+
 def _select_ok(score, mask, k):
     """Exact-k, dominance and lowest-index ties of a mask against a score."""
     assert int(mask.sum()) == k
