@@ -381,8 +381,9 @@ def placement_probe(reps=5, trials=6, seed=1):
     34 B per element, math-free stand-in k_calib_streams) over the Llama-3.2-1B element count
     on differently placed arrays of ONE process: fresh tensors, one carved 25 GB block with the
     arrays back to back and at random 4 KiB-granular offsets, fresh tensors with random spacers
-    between them.  Virtual addresses are printed; what differs between runs of the same virtual
-    layout is the physical backing."""
+    between them, the same five tensors freed and allocated again eight times, and five arrays
+    at equal spacings of 5 to 24 GiB inside one block.  Virtual addresses are printed; what
+    differs between runs of the same virtual layout is the physical backing."""
     import random
     import torch
     from sga_amd import _lib as L
@@ -436,6 +437,23 @@ def placement_probe(reps=5, trials=6, seed=1):
         timeit(f"fresh tensors, random spacers #{i}", *ts)
         del ts, keep
         torch.cuda.empty_cache()
+    # the same five tensors freed and allocated again: same virtual addresses, a new draw of
+    # physical pages every round
+    for i in range(8):
+        t = fresh()
+        timeit(f"fresh tensors again, round {i}", *t)
+        del t
+        torch.cuda.empty_cache()
+    # five arrays at equal spacing inside one untouched block
+    gib = 1 << 30
+    blk = torch.zeros(4 * 24 * gib + 4 * n + 4096, dtype=torch.uint8, device=dev)
+    for d in (5, 8, 12, 15, 16, 20, 24):
+        offs = [j * d * gib for j in range(5)]
+        timeit(f"one block, arrays every {d} GiB",
+               blk[offs[0]: offs[0] + 2 * n].view(torch.bfloat16),
+               *[blk[o: o + 4 * n].view(torch.float32) for o in offs[1:]])
+    del blk
+    torch.cuda.empty_cache()
     return {"kernel": "k_calib_streams", "n": n, "bytes_per_launch": 34.0 * n, "rows": rows}
 
 
@@ -824,6 +842,42 @@ def main():
             "avg_ms": ms, "GBps": n * ALG_BYTES_FINAL / ms / 1e6,
             "frac_of_peak": n * ALG_BYTES_FINAL / (ms * 1e-3) / HBM_PEAK,
             "dominant_kernel_vs_copy": ms / head["final_avg_ms"]}
+    if not args.no_sweep and args.layout == "separate":
+        # The same step after the device allocator has been churned.  Which physical pages an
+        # array gets decides the rate of this stream mix (the first allocations on a fresh
+        # machine are the slow kind, memory handed out after large blocks were freed is mostly
+        # the fast kind); this leg frees the five arrays, allocates and frees 3 x 100 GB, then
+        # allocates the five arrays again the same way and times the headline configuration on
+        # them.  An extra: `value` stays the first draw.
+        del p, m, v, r, grads
+        torch.cuda.empty_cache()
+        for _ in range(3):
+            blocks = [torch.empty(20 << 30, dtype=torch.uint8, device=dev) for _ in range(5)]
+            del blocks
+            torch.cuda.empty_cache()
+        gen = torch.Generator(device=dev).manual_seed(0)
+        p = torch.randn(n, generator=gen, device=dev) * 0.02
+        m = torch.zeros(n, device=dev)
+        v = torch.zeros(n, device=dev)
+        r = torch.zeros(n, device=dev)
+        grads = [student_t_dev(n, 10 + i, dev) for i in range(2)]
+        state["t"] = 0
+        leg = time_leg("separate", args.score, args.ratio, 2, 5, args.single_sweep)
+        sargs = [L.ptr(grads[0]), L.ptr(r), L.ptr(p), L.ptr(m), L.ptr(v), n, L.stream()]
+        ev = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
+        L.call("sga_calib_streams", *sargs)
+        ev[0].record()
+        for _ in range(5):
+            L.call("sga_calib_streams", *sargs)
+        ev[1].record()
+        torch.cuda.synchronize()
+        out["placement_redraw"] = {
+            "what": "the headline configuration on the five arrays freed and allocated again "
+                    "after 3 x 100 GB of device memory were allocated and freed",
+            "ms_per_step": leg["ms_per_step"], "elem_per_s": leg["elem_per_s"],
+            "dominant_kernel_ms": leg["final_avg_ms"], "dominant_kernel_frac": leg["final_frac"],
+            "step_frac": leg["step_frac"],
+            "stream_mix_copy_ms": ev[0].elapsed_time(ev[1]) / 5}
     del p, m, v, r, grads, fs
     torch.cuda.empty_cache()
     if not args.no_rows:
