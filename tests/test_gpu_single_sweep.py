@@ -76,6 +76,16 @@ def test_small_bucket_takes_the_two_sweep_step(dev):
     _run(dev, [200_000, 1024, 100_000], 2, 1.0, torch.bfloat16, torch.bfloat16, expect_path=None)
 
 
+@pytest.mark.parametrize("sizes,k_ratio", [([1 << 20], 1.0), ([(1 << 20) + 1], 1.0),
+                                           ([(1 << 20) - 3, 3, 1], 0.5), ([1 << 20], 1.0e-4)])
+def test_buckets_at_the_size_where_the_single_sweep_starts(dev, sizes, k_ratio):
+    """2^20 elements is the smallest bucket the sampled bracket takes: exactly
+    that size, one element more (a ragged last chunk), a boundary three
+    elements before the end, and k = 1."""
+    _run(dev, sizes, 2, k_ratio, torch.bfloat16, torch.float32, score="update", vary=len(sizes) > 1,
+         expect_path=None)
+
+
 def test_wide_ratio_fills_the_small_segments(dev):
     """At 60 % a chunk holds ~50 bracket keys against 64 slots of its own
     segment: the chunks that do not fit go to the shared overflow list."""
