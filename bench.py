@@ -9,14 +9,20 @@ Student-t(3) gradients, fp32 p/m/v/residual) with every input resident in HBM.
 The headline is the drop-in layout (resid / p / m / v as the caller's four
 flat tensors, as the reference's buffers are) with the Adam-normalised score
 (`update`) at 1 %, through the single-sweep step (every array read once;
---two-sweep headlines the step that reads the score inputs twice).  The same
-JSON line carries the whole sweep of the benchmark configuration -- step
-variants {two-sweep, single-sweep} x scores {update, abs_g} x ratios {0.1, 1,
-10} % x state layouts {separate, packed (library-owned 64 KiB records)} -- with
-each leg's own algorithmic bytes, one row for the Qwen3-0.6B per-bucket mask-layout
-configuration, one for the 1e9-element stress buffer, the fused replay leg and
-the CPU oracle timed on a bounded sample of the headline workload.  The
-dominant kernels are timed live with HIP events on their launch stream.
+--two-sweep headlines the step that reads the score inputs twice; its figures
+ride along as `two_sweep` either way).
+
+Output: the LAST stdout line is one compact JSON object (a few KB): the
+headline, `roofline` of the dominant kernel (timed live with HIP events on its
+launch stream), `step_roofline` (the whole step against the bytes it has to
+move), `two_sweep`, `packed_layout`, one-line summaries of the Qwen3-0.6B
+per-bucket row (`cfg2`) and the 1e9-element stress row (`cfg5`), `replay` and
+`cpu_baseline`.  Everything longer -- per-leg tables, the optional full sweep
+(--sweep: step variants x scores x ratios x layouts), per-kernel replay
+figures, the replay stress draw -- goes to a side file (--detail, default
+gpurun_out/bench_detail.json), never to the last line.  Every field called
+`frac` is a fraction of the 8 TB/s HBM peak of bytes the measured code has to
+move, so none can exceed 1.
 """
 import argparse
 import ctypes
@@ -52,8 +58,12 @@ def step_bytes_per_elem(score, g_bytes=2.0):
 
 def prof_read(L, tag):
     tot, cnt = ctypes.c_double(0), ctypes.c_int(0)
-    L.call("sga_prof_read", tag, ctypes.byref(tot), ctypes.byref(cnt))
+    L.bench_call("sga_prof_read", tag, ctypes.byref(tot), ctypes.byref(cnt))
     return tot.value, cnt.value
+
+
+def prof_enable(L, on):
+    L.bench_call("sga_prof_enable", int(on))
 
 
 def student_t_dev(n, seed, dev, scale=1e-3, nu=3, chunk=1 << 26):
@@ -102,85 +112,106 @@ def cpu_baseline(sample_n, steps, ratio, score="abs_g"):
                       f"{dt:.1f} s; host cpu_count={os.cpu_count()}"}
 
 
-def replay_bench(G=8, W=32, seed=4):
-    """Fused offline replay on the Qwen3-0.6B shapes: a window of W recorded
-    bf16 gradient steps resident in HBM, G configs drawn with a fixed seed from
-    score {|g|, |g+r|, update} x ratio {0.1, 1, 10} % x cycle length {1, 4, 16};
-    per-config fp32 w/m/v/residual + mask bit planes."""
+REPLAY_AXES = [(sc, r, t) for sc in REPLAY_SCORES for r in (0.1, 1.0, 10.0) for t in (1, 4, 16)]
+# A second, fixed draw that leans on the expensive arms: five Adam-normalised configs (`update`,
+# `coi`) at cycle lengths 4 and 16 -- re-selections that read w, m, v and evaluate the exact
+# score chain -- and none at T = 1.
+REPLAY_STRESS_DRAW = [("update", 1.0, 4), ("update", 0.1, 16), ("coi", 1.0, 4), ("update", 10.0, 4),
+                      ("abs_g", 1.0, 4), ("abs_g_blind", 1.0, 16), ("abs_g", 10.0, 16),
+                      ("coi", 0.1, 16)]
+
+
+def replay_draw(G=8, seed=4):
     import random
+    return random.Random(seed).sample(REPLAY_AXES, G)
+
+
+def replay_bytes(n, W, picks):
+    """Algorithmic bytes of one window for a list of (score, ratio, T) configs
+    (bf16 g read once per pass for the whole group)."""
+    alg_p1 = alg_p3 = alg_sw = 0.0
+    n_resel = 0
+    for s in range(W):
+        alg_p1 += 2.0 * n                                    # g in pass 1
+        alg_p3 += 2.0 * n                                    # g in pass 3
+        for score, _ratio, T in picks:
+            bnd = s % T == 0
+            rz = s == 0 or (s - 1) % T == 0                  # res is all zeros: no traffic for it
+            alg_p1 += ((0.0 if rz else 4.0) if bnd else 0.125) * n  # pass 1: res | sel (1 bit)
+            # pass 3: m, v, w read+write; res read unless zero, written unless it stays zero
+            alg_p3 += (24.0 + (0.0 if rz else 4.0) + (0.0 if (bnd and rz) else 4.0)
+                       + (0.0 if bnd else 0.125)) * n
+            if bnd and s > 0 and s + 1 < W:
+                if score == "abs_g_blind":
+                    per = 2.0                                # the gradient alone
+                else:
+                    per = (6.0 if score == "abs_g" else 18.0) - (4.0 if rz else 0.0)
+                alg_sw += (per + 0.125) * n                  # one score sweep + the new mask bits
+                n_resel += 1
+    return alg_p1, alg_p3, alg_sw, n_resel
+
+
+def replay_bench(draws=None, W=32):
+    """Fused offline replay on the Qwen3-0.6B shapes: a window of W recorded
+    bf16 gradient steps resident in HBM, G = 8 configs from score {|g|, |g+r|,
+    update} x ratio {0.1, 1, 10} % x cycle length {1, 4, 16}; per-config fp32
+    w/m/v/residual + mask bit planes.  ``draws``: list of (name, picks); the
+    window and the branch state are built once and every draw replays it."""
     import torch
     from sga_amd import _lib as L
     from sga_amd.replay import select_topk_flat
     from sga_amd.replay_group import Config, ReplayGroup
     from sga_amd.shapes import qwen3_06b, segments_for
     dev = torch.device("cuda:0")
+    if draws is None:
+        draws = [("seed 4", replay_draw())]
     segs, n = segments_for(qwen3_06b())
     entries = [{"a": s["start"], "n": s["n"], "b1": s["b1"], "b2": s["b2"], "eps": s["eps"],
                 "wd": s["wd"]} for s in segs]
-    rnd = random.Random(seed)
-    axes = [(sc, r, t) for sc in REPLAY_SCORES for r in (0.1, 1.0, 10.0)
-            for t in (1, 4, 16)]
-    picks = rnd.sample(axes, G)
-    cfgs = [Config(*p) for p in picks]
     gen = torch.Generator(device=dev).manual_seed(1)
     w0 = torch.randn(n, generator=gen, device=dev) * 0.02
     m0 = torch.randn(n, generator=gen, device=dev) * 1e-4
     v0 = torch.rand(n, generator=gen, device=dev) * 1e-8
     # slowly drifting per-tensor scale: one scale vector per step applied on the fly
-    window = []
-    for s in range(W):
-        g = student_t_dev(n, 500 + s, dev, scale=1e-3 * (1.0 + 0.02 * s))
-        window.append(g)
-    sel0 = []
+    window = [student_t_dev(n, 500 + s, dev, scale=1e-3 * (1.0 + 0.02 * s)) for s in range(W)]
     base = window[0].float().abs()
-    for c in cfgs:                       # branch selection on |g0| (cheap stand-in for the front block)
-        sel0.append(select_topk_flat(base, max(1, int(round(c.ratio / 100.0 * n))))[0])
-    del base
-    grp = ReplayGroup(entries, w0, m0, v0, sel0, cfgs, t0=100, window=W)
-    del sel0
     meta = {"clip_grad": 1.0, "grad_norm": float("nan"), "lr": 1e-4}
-    torch.cuda.synchronize()
-    L.raw("sga_prof_enable", 1)
-    t0 = time.perf_counter()
-    for s in range(W):
-        grp.step(window[s], meta)
-    torch.cuda.synchronize()
-    dt = time.perf_counter() - t0
-    p3_ms, p3_n = prof_read(L, PROF_PASS3)
-    p1_ms, p1_n = prof_read(L, PROF_PASS1)
-    sw_ms, sw_n = prof_read(L, PROF_SWEEP)
-    L.raw("sga_prof_enable", 0)
-    # algorithmic bytes of this calendar (bf16 g read once per pass for the group)
-    alg = alg_p1 = alg_p3 = alg_sw = 0.0
-    n_resel = 0
-    for s in range(W):
-        alg_p1 += 2.0 * n                                    # g in pass 1
-        alg_p3 += 2.0 * n                                    # g in pass 3
-        for c in cfgs:
-            bnd = s % c.T == 0
-            rz = s == 0 or (s - 1) % c.T == 0                # res is all zeros: no traffic for it
-            alg_p1 += ((0.0 if rz else 4.0) if bnd else 0.125) * n  # pass 1: res | sel (1 bit)
-            # pass 3: m, v, w read+write; res read unless zero, written unless it stays zero
-            alg_p3 += (24.0 + (0.0 if rz else 4.0) + (0.0 if (bnd and rz) else 4.0)
-                       + (0.0 if bnd else 0.125)) * n
-            if bnd and s > 0 and s + 1 < W:
-                if c.score == "abs_g_blind":
-                    per = 2.0                                # the gradient alone
-                else:
-                    per = (6.0 if c.score == "abs_g" else 18.0) - (4.0 if rz else 0.0)
-                alg_sw += (per + 0.125) * n                  # one score sweep + the new mask bits
-                n_resel += 1
-    alg = alg_p1 + alg_p3 + alg_sw
-    kernels = {}
-    for name, ms, cnt, b in (("k_replay_pass3", p3_ms, p3_n, alg_p3),
-                             ("k_replay_pass1 (launches of one step)", p1_ms, p1_n, alg_p1),
-                             ("k_bracket_sweep<SrcReplay>", sw_ms, sw_n, alg_sw)):
-        if cnt:
-            kernels[name] = {"launches": cnt, "total_ms": ms, "avg_ms": ms / cnt, "alg_bytes": b,
-                             "frac": b / (ms * 1e-3) / HBM_PEAK if ms > 0 else None}
-    return {"metric": "replay config-steps/s", "value": G * W / dt, "unit": "config-steps/s",
-            "ms_per_window": dt * 1e3, "G": G, "W": W, "n": n, "reselects": n_resel,
-            "configs": [list(p) for p in picks],
+    out = []
+    for name, picks in draws:
+        cfgs = [Config(*p) for p in picks]
+        G = len(cfgs)
+        # branch selection on |g0| (cheap stand-in for the front block)
+        sel0 = [select_topk_flat(base, max(1, int(round(c.ratio / 100.0 * n))))[0] for c in cfgs]
+        grp = ReplayGroup(entries, w0, m0, v0, sel0, cfgs, t0=100, window=W)
+        del sel0
+        torch.cuda.synchronize()
+        prof_enable(L, 1)
+        t0 = time.perf_counter()
+        for s in range(W):
+            grp.step(window[s], meta)
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        p3_ms, p3_n = prof_read(L, PROF_PASS3)
+        p1_ms, p1_n = prof_read(L, PROF_PASS1)
+        sw_ms, sw_n = prof_read(L, PROF_SWEEP)
+        prof_enable(L, 0)
+        del grp
+        torch.cuda.empty_cache()
+        alg_p1, alg_p3, alg_sw, n_resel = replay_bytes(n, W, picks)
+        alg = alg_p1 + alg_p3 + alg_sw
+        kernels = {}
+        for kname, ms, cnt, b in (("k_replay_pass3", p3_ms, p3_n, alg_p3),
+                                  ("k_replay_pass1 (launches of one step)", p1_ms, p1_n, alg_p1),
+                                  ("k_bracket_sweep<SrcReplay>", sw_ms, sw_n, alg_sw)):
+            if cnt:
+                kernels[kname] = {"launches": cnt, "total_ms": ms, "avg_ms": ms / cnt,
+                                  "alg_bytes": b,
+                                  "frac": b / (ms * 1e-3) / HBM_PEAK if ms > 0 else None}
+        timed = p3_ms + p1_ms + sw_ms
+        out.append({
+            "draw": name, "metric": "replay config-steps/s", "value": G * W / dt,
+            "unit": "config-steps/s", "ms_per_window": dt * 1e3, "G": G, "W": W, "n": n,
+            "reselects": n_resel, "configs": [list(p) for p in picks],
             "alg_bytes": alg, "achieved_GBps": alg / dt / 1e9, "frac": alg / dt / HBM_PEAK,
             "roofline": {"bound": "hbm", "kernel": "k_replay_pass3",
                          "achieved": alg_p3 / (p3_ms * 1e-3) / 1e9 if p3_ms > 0 else None,
@@ -188,8 +219,10 @@ def replay_bench(G=8, W=32, seed=4):
                          "frac": alg_p3 / (p3_ms * 1e-3) / HBM_PEAK if p3_ms > 0 else None,
                          "avg_ms": p3_ms / max(p3_n, 1), "traffic": None},
             "kernels": kernels,
+            "other_kernels_and_gaps_ms": dt * 1e3 - timed,
             "workload": "Qwen3-0.6B shapes (596,049,920 elems, 310 tensors), bf16 Student-t(3) "
-                        "window, per-config fp32 w/m/v/res + u8 mask resident, clip 1.0"}
+                        "window, per-config fp32 w/m/v/res + mask bit planes resident, clip 1.0"})
+    return out
 
 
 def replay_cpu_baseline(G=8, W=8, seed=4, frac=24):
@@ -212,10 +245,7 @@ def replay_cpu_baseline(G=8, W=8, seed=4, frac=24):
     segs, n = segments_for(shapes)
     entries = [{"a": s["start"], "n": s["n"], "b1": s["b1"], "b2": s["b2"], "eps": s["eps"],
                 "wd": s["wd"]} for s in segs]
-    rnd = random.Random(seed)
-    axes = [(sc, r, t) for sc in REPLAY_SCORES for r in (0.1, 1.0, 10.0)
-            for t in (1, 4, 16)]
-    cfgs = [OR.Config(*p) for p in rnd.sample(axes, G)]
+    cfgs = [OR.Config(*p) for p in replay_draw(G, seed)]
     gen = torch.Generator().manual_seed(1)
     w0 = torch.randn(n, generator=gen) * 0.02
     m0 = torch.randn(n, generator=gen) * 1e-4
@@ -374,87 +404,6 @@ def trace_io_bench(W=4, tmp=None):
                 "dense_step_resident_ms": dt_res / W * 1e3}
     finally:
         shutil.rmtree(d, ignore_errors=True)
-
-
-def placement_probe(reps=5, trials=6, seed=1):
-    """The final sweep's mix of streams (bf16 g and fp32 r, p, m, v read; r, p, m, v written:
-    34 B per element, math-free stand-in k_calib_streams) over the Llama-3.2-1B element count
-    on differently placed arrays of ONE process: fresh tensors, one carved 25 GB block with the
-    arrays back to back and at random 4 KiB-granular offsets, fresh tensors with random spacers
-    between them, the same five tensors freed and allocated again eight times, and five arrays
-    at equal spacings of 5 to 24 GiB inside one block.  Virtual addresses are printed; what
-    differs between runs of the same virtual layout is the physical backing."""
-    import random
-    import torch
-    from sga_amd import _lib as L
-    from sga_amd.shapes import llama32_1b, segments_for
-    dev = torch.device("cuda:0")
-    _, n = segments_for(llama32_1b())
-    rows = []
-
-    def timeit(tag, g, r, p, m, v):
-        a = [L.ptr(g), L.ptr(r), L.ptr(p), L.ptr(m), L.ptr(v), n, L.stream()]
-        L.call("sga_calib_streams", *a)
-        ev = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
-        torch.cuda.synchronize()
-        ev[0].record()
-        for _ in range(reps):
-            L.call("sga_calib_streams", *a)
-        ev[1].record()
-        torch.cuda.synchronize()
-        ms = ev[0].elapsed_time(ev[1]) / reps
-        rows.append({"placement": tag, "ms": ms, "GBps": 34.0 * n / ms / 1e6,
-                     "ptrs": [hex(t.data_ptr()) for t in (g, r, p, m, v)]})
-
-    def fresh():
-        return (torch.zeros(n, dtype=torch.bfloat16, device=dev),
-                *[torch.zeros(n, device=dev) for _ in range(4)])
-
-    for i in range(2):
-        t = fresh()
-        timeit(f"fresh tensors #{i}", *t)
-        del t
-        torch.cuda.empty_cache()
-    mb2 = 2 << 20
-    ab = (n * 4 + mb2 - 1) // mb2 * mb2
-    slab = torch.zeros(ab * 5 + (64 << 20) * 8, dtype=torch.uint8, device=dev)
-
-    def carve(offs):
-        return (slab[offs[0]: offs[0] + 2 * n].view(torch.bfloat16),
-                *[slab[o: o + 4 * n].view(torch.float32) for o in offs[1:]])
-    timeit("one block, arrays back to back", *carve([i * ab for i in range(5)]))
-    rnd = random.Random(seed)
-    for i in range(trials):
-        timeit(f"one block, random 4 KiB-granular offsets #{i}",
-               *carve([j * ab + rnd.randrange(0, 64 << 20, 4096) for j in range(5)]))
-    del slab
-    torch.cuda.empty_cache()
-    for i in range(trials):
-        keep, ts = [], []
-        for j in range(5):
-            keep.append(torch.empty(rnd.randrange(1 << 20, 3 << 30), dtype=torch.uint8, device=dev))
-            ts.append(torch.zeros(n, dtype=torch.bfloat16 if j == 0 else torch.float32, device=dev))
-        timeit(f"fresh tensors, random spacers #{i}", *ts)
-        del ts, keep
-        torch.cuda.empty_cache()
-    # the same five tensors freed and allocated again: same virtual addresses, a new draw of
-    # physical pages every round
-    for i in range(8):
-        t = fresh()
-        timeit(f"fresh tensors again, round {i}", *t)
-        del t
-        torch.cuda.empty_cache()
-    # five arrays at equal spacing inside one untouched block
-    gib = 1 << 30
-    blk = torch.zeros(4 * 24 * gib + 4 * n + 4096, dtype=torch.uint8, device=dev)
-    for d in (5, 8, 12, 15, 16, 20, 24):
-        offs = [j * d * gib for j in range(5)]
-        timeit(f"one block, arrays every {d} GiB",
-               blk[offs[0]: offs[0] + 2 * n].view(torch.bfloat16),
-               *[blk[o: o + 4 * n].view(torch.float32) for o in offs[1:]])
-    del blk
-    torch.cuda.empty_cache()
-    return {"kernel": "k_calib_streams", "n": n, "bytes_per_launch": 34.0 * n, "rows": rows}
 
 
 def qwen_mask_layout_row(steps=5, warmup=2, n_streams=3):
@@ -618,18 +567,19 @@ def main():
                     help="also launch one plain copy of 2^30 fp32 (k_calib_copy) and the math-free "
                          "stream stand-in so counter runs can be scaled against known traffic")
     ap.add_argument("--no-replay", action="store_true", help="skip the fused replay leg")
-    ap.add_argument("--no-sweep", action="store_true",
-                    help="time only the headline configuration of the fused step")
+    ap.add_argument("--sweep", action="store_true",
+                    help="also time the whole sweep {two-sweep, single-sweep} x {update, abs_g} x "
+                         "{0.1, 1, 10 %} x {separate, packed} (24 legs; written to the detail file)")
     ap.add_argument("--no-rows", action="store_true",
                     help="skip the Qwen3-0.6B mask-layout row and the 1e9 stress row")
+    ap.add_argument("--detail", default=os.path.join(ROOT, "gpurun_out", "bench_detail.json"),
+                    help="side file for everything longer than the compact last line "
+                         "('' = do not write one)")
     ap.add_argument("--trace-io", action="store_true",
                     help="run just the recorded-trace leg (writes a temporary trace, streams it "
                          "back through the pread reader and the dense pass) and print its JSON")
     ap.add_argument("--primitives", action="store_true",
                     help="time the drop-in primitives on their own and print their JSON")
-    ap.add_argument("--placement", action="store_true",
-                    help="run just the placement probe of the final sweep's stream mix (same "
-                         "kernel, differently placed arrays) and print its JSON")
     ap.add_argument("--only-replay", action="store_true",
                     help="run just the fused replay leg (for profiling) and print its JSON")
     args = ap.parse_args()
@@ -640,17 +590,14 @@ def main():
 
     import torch
     from sga_amd import _lib as L
+    L.load_bench()          # timing observer + calibration kernels: before libsga_hip.so binds
     from sga_amd.fused_step import FusedSparseStep, PackedState, k_for
     from sga_amd.shapes import llama32_1b, segments_for
 
     L.load()
     if args.only_replay:
         torch.cuda.set_device(0)
-        print(json.dumps(replay_bench()))
-        return
-    if args.placement:
-        torch.cuda.set_device(0)
-        print(json.dumps(placement_probe()))
+        print(json.dumps(replay_bench()[0]))
         return
     if args.trace_io:
         torch.cuda.set_device(0)
@@ -672,19 +619,22 @@ def main():
     fs = FusedSparseStep(n, segs, dev, values_dtype=torch.bfloat16,
                          max_k=k_for(n, 10.0) + 16)
 
+    def events_ms(fn, reps=5):
+        ev = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
+        fn()
+        ev[0].record()
+        for _ in range(reps):
+            fn()
+        ev[1].record()
+        torch.cuda.synchronize()
+        return ev[0].elapsed_time(ev[1]) / reps
+
     calib = None
     if args.calib:
         cn = 1 << 30
         src = torch.ones(cn, device=dev)
         dst = torch.empty(cn, device=dev)
-        ev = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
-        L.call("sga_calib_copy", L.ptr(dst), L.ptr(src), cn, L.stream())
-        ev[0].record()
-        for _ in range(5):
-            L.call("sga_calib_copy", L.ptr(dst), L.ptr(src), cn, L.stream())
-        ev[1].record()
-        torch.cuda.synchronize()
-        ms = ev[0].elapsed_time(ev[1]) / 5
+        ms = events_ms(lambda: L.bench_call("sga_calib_copy", L.ptr(dst), L.ptr(src), cn, L.stream()))
         calib = {"kernel": "k_calib_copy", "bytes": cn * 8, "avg_ms": ms,
                  "GBps": cn * 8 / ms / 1e6}
         del src, dst
@@ -692,83 +642,104 @@ def main():
         sg = torch.zeros(n, dtype=torch.bfloat16, device=dev)
         sc = [torch.zeros(n, device=dev) for _ in range(4)]
         sargs = [L.ptr(sg)] + [L.ptr(t) for t in sc] + [n, L.stream()]
-        L.call("sga_calib_streams", *sargs)
-        ev[0].record()
-        for _ in range(5):
-            L.call("sga_calib_streams", *sargs)
-        ev[1].record()
-        torch.cuda.synchronize()
-        ms = ev[0].elapsed_time(ev[1]) / 5
+        ms = events_ms(lambda: L.bench_call("sga_calib_streams", *sargs))
         calib["streams"] = {"kernel": "k_calib_streams", "bytes": n * 34, "avg_ms": ms,
                             "GBps": n * 34 / ms / 1e6}
         del sg, sc
 
     state = {"t": 0, "packed": None}
+    max_steps = max(args.steps, 5)
+    results = torch.zeros(max_steps, 8, dtype=torch.int32, device=dev)   # a result block per step
 
     def time_leg(layout, score, ratio, warmup, steps, single=False):
         """`warmup` untimed + exactly `steps` timed steps of one configuration."""
         k = k_for(n, ratio)
         if layout == "packed" and state["packed"] is None:
             state["packed"] = PackedState(n, dev).pack(r, p, m, v)
+        elif layout == "separate" and state["packed"] is not None:
+            state["packed"].unpack(r, p, m, v)
+            state["packed"] = None
 
-        def step_fn(t):
+        def step_fn(t, res=None):
             if layout == "packed":
                 fs.step_packed(grads[t % 2], state["packed"], t + 1, k=k, score=score,
-                               single_sweep=single)
+                               single_sweep=single, check=False, result=res)
             else:
-                fs.step(grads[t % 2], r, p, m, v, t + 1, k=k, score=score, single_sweep=single)
+                fs.step(grads[t % 2], r, p, m, v, t + 1, k=k, score=score, single_sweep=single,
+                        check=False, result=res)
         for _ in range(warmup):
             step_fn(state["t"])
             state["t"] += 1
         torch.cuda.synchronize()
-        L.raw("sga_prof_enable", 1)
+        prof_enable(L, 1)
         t0 = time.perf_counter()
-        for _ in range(steps):
-            step_fn(state["t"])
+        for i in range(steps):
+            step_fn(state["t"], results[i])
             state["t"] += 1
         torch.cuda.synchronize()
         dt = time.perf_counter() - t0
         fin_ms, fin_n = prof_read(L, PROF_FINAL)
         sw_ms, sw_n = prof_read(L, PROF_SWEEP)
-        L.raw("sga_prof_enable", 0)
-        res = fs.read_result()
-        assert res.status == 0 and res.n_selected == k, vars(res)
+        prof_enable(L, 0)
+        # every timed step must have ended as an exact top-k step (status word 0, k selected)
+        rows = results[:steps].cpu()
+        assert bool((rows[:, 6] == 0).all()) and bool((rows[:, 4] == k).all()), rows.tolist()
+        from sga_amd.selection import read_result
+        res = read_result(results[steps - 1])
         # dominant kernel: k_fused_final reads g, r, p, m, v, writes r, p, m, v and the pack
         # (4 + 2 B per selected coordinate); k_fused_spec (single sweep) the same state traffic
         # and one staged 2 B value per coordinate it takes as selected
         final_bytes = n * ALG_BYTES_FINAL + k * (2.0 if single else 6.0)
         sweep_bytes = 0.0 if single else n * sweep_bytes_per_elem(score)
-        # two-read model of the step (the select needs the score inputs once, the commit again)
-        step_bytes = n * step_bytes_per_elem(score) + k * 6.0
-        # bytes a step that reads every array once has to move
+        # bytes the step has to move: every array once (34 B per element + the pack) for the
+        # single sweep; the score inputs once more for the two-sweep step's select
         once_bytes = n * ALG_BYTES_FINAL + k * 6.0
+        two_read_bytes = n * step_bytes_per_elem(score) + k * 6.0
+        moved = once_bytes if single else two_read_bytes
         fin_avg, sw_avg = fin_ms / max(fin_n, 1), sw_ms / max(sw_n, 1)
-        return {"layout": layout, "single_sweep": single, "score": score, "ratio_percent": ratio, "k": k, "steps": steps,
-                "seconds": dt, "ms_per_step": dt / steps * 1e3, "elem_per_s": n * steps / dt,
-                "alg_bytes_per_elem": step_bytes_per_elem(score),
-                "alg_bytes_per_step": step_bytes,
-                "step_frac": step_bytes * steps / dt / HBM_PEAK,
-                "read_once_bytes_per_step": once_bytes,
-                "read_once_frac": once_bytes * steps / dt / HBM_PEAK,
+        return {"layout": layout, "single_sweep": single, "score": score, "ratio_percent": ratio,
+                "k": k, "steps": steps, "seconds": dt, "ms_per_step": dt / steps * 1e3,
+                "elem_per_s": n * steps / dt,
+                "moved_bytes_per_elem": moved / n, "moved_bytes_per_step": moved,
+                "step_frac": moved * steps / dt / HBM_PEAK,
+                # not a roofline fraction: the rate this step would need under the two-read
+                # byte model (52 B per element for `update`, 40 for |g + r|), relative to peak
+                "speedup_vs_two_read_model": two_read_bytes * steps / dt / HBM_PEAK,
                 "final_avg_ms": fin_avg, "final_bytes": final_bytes,
                 "final_frac": final_bytes / (fin_avg * 1e-3) / HBM_PEAK if fin_avg > 0 else None,
                 "sweep_avg_ms": sw_avg, "sweep_bytes": sweep_bytes,
                 "sweep_frac": sweep_bytes / (sw_avg * 1e-3) / HBM_PEAK if sw_avg > 0 else None,
+                "other_kernels_ms": dt / steps * 1e3 - fin_avg - sw_avg,
                 "select": {"thresh": res.thresh, "n_gt": res.n_gt, "n_eq": res.n_eq,
                            "path": res.path}}
 
     head = time_leg(args.layout, args.score, args.ratio, args.warmup, args.steps, args.single_sweep)
+    stream_mix = None
+    if args.layout == "separate":
+        # What the same five read and four write streams reach WITHOUT the math, on the very
+        # tensors the headline ran on: the ceiling this placement of four flat tensors gives a
+        # kernel of that stream mix.  (It scribbles over r / p / m / v: they are reset below.)
+        sargs = [L.ptr(grads[0]), L.ptr(r), L.ptr(p), L.ptr(m), L.ptr(v), n, L.stream()]
+        ms = events_ms(lambda: L.bench_call("sga_calib_streams", *sargs))
+        stream_mix = {"kernel": "k_calib_streams (same five read / four write streams, no math), "
+                                "same tensors as the headline",
+                      "avg_ms": ms, "frac": n * ALG_BYTES_FINAL / (ms * 1e-3) / HBM_PEAK}
+        gen = torch.Generator(device=dev).manual_seed(0)
+        p.copy_(torch.randn(n, generator=gen, device=dev) * 0.02)
+        m.zero_(); v.zero_(); r.zero_()
+        state["t"] = 0
+    # the other step variant and the other layout of the headline configuration
+    other = time_leg(args.layout, args.score, args.ratio, 2, 5, not args.single_sweep)
+    two = other if args.single_sweep else head
+    packed_leg = time_leg("packed" if args.layout == "separate" else "separate", args.score,
+                          args.ratio, 2, 5, args.single_sweep)
     sweep = []
-    if not args.no_sweep:
+    if args.sweep:
         for single in (False, True):
             for layout in ("separate", "packed"):
                 for score in ("update", "abs_g"):
                     for ratio in (0.1, 1.0, 10.0):
-                        if (layout, score, ratio, single) == (args.layout, args.score, args.ratio,
-                                                              args.single_sweep):
-                            sweep.append(head)
-                        else:
-                            sweep.append(time_leg(layout, score, ratio, 1, 5, single))
+                        sweep.append(time_leg(layout, score, ratio, 1, 5, single))
     if state["packed"] is not None:
         state["packed"].unpack(r, p, m, v)
         state["packed"] = None
@@ -776,125 +747,100 @@ def main():
     k = head["k"]
     value = n * args.steps / head["seconds"]
     entry = "sga_fused_sparse_step" + ("_single_sweep" if args.single_sweep else "")
-    layout_txt = (f"resid/p/m/v interleaved in 64 KiB records ({entry}_packed)"
-                  if args.layout == "packed" else
-                  f"resid/p/m/v as the caller's four flat tensors ({entry}, the drop-in layout)")
-    sweeps_txt = ("single sweep: g / resid / p / m / v read once, coordinates inside the sampled "
-                  "bracket committed on a guess and repaired after the candidate descent"
-                  if args.single_sweep else
-                  "two sweeps: select sweep over the score inputs, then the final sweep")
     out = {
         "metric": "grad elems/s (score+top-k+resid AdamW)",
         "value": value, "unit": "elem/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": head["ms_per_step"],
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
-        "config": {"workload": "Llama-3.2-1B-shaped set, 1,235,814,400 elems / 146 tensors, "
-                               "bf16 Student-t(3) grads, fp32 p/m/v/residual, score "
-                               f"{args.score}, exact top-k {args.ratio}% (k={k}), index pack "
-                               "int32+bf16, residual-aware AdamW; " + sweeps_txt +
-                               "; state layout: " + layout_txt,
+        "config": {"workload": "Llama-3.2-1B-shaped set (BASELINE cfg 3), 1,235,814,400 elems / "
+                               "146 tensors, bf16 Student-t(3) grads, fp32 p/m/v/residual, score "
+                               f"{args.score}, exact top-k {args.ratio}%, index pack int32+bf16, "
+                               f"residual-aware AdamW; entry point {entry}"
+                               + ("_packed" if args.layout == "packed" else ""),
                    "ratio_percent": args.ratio, "score": args.score, "k": k,
-                   "single_sweep": bool(args.single_sweep),
-                   "state_layout": args.layout, "grad_dtype": "bf16", "values_dtype": "bf16",
-                   "state_dtype": "f32", "arithmetic": "f32"},
-        "roofline": {"bound": "hbm", "achieved": head["final_bytes"] / (head["final_avg_ms"] * 1e-3) / 1e9,
-                     "peak": HBM_PEAK / 1e9, "unit": "GB/s", "frac": head["final_frac"],
-                     "traffic": traffic, "traffic_source": traffic_src,
+                   "single_sweep": bool(args.single_sweep), "state_layout": args.layout},
+        "roofline": {"bound": "hbm",
                      "kernel": "k_fused_spec" if args.single_sweep else "k_fused_final",
                      "avg_ms": head["final_avg_ms"],
-                     "alg_bytes_per_launch": head["final_bytes"]},
-        # whole step against two byte models: the two-read model the roofline target is stated
-        # on (the score inputs once for the select, every array again for the commit: 52 B per
-        # element for the Adam-normalised score, 40 for |g + r|), and the bytes a step that reads
-        # every array once has to move (34 B per element + the pack)
-        "step_roofline": {"alg_bytes_per_elem": head["alg_bytes_per_elem"],
-                          "achieved_GBps": head["alg_bytes_per_step"] / (head["ms_per_step"] * 1e-3) / 1e9,
+                     "alg_bytes_per_launch": head["final_bytes"],
+                     "achieved": head["final_bytes"] / (head["final_avg_ms"] * 1e-3) / 1e9,
+                     "peak": HBM_PEAK / 1e9, "unit": "GB/s", "frac": head["final_frac"],
+                     "traffic": traffic,
+                     "stream_mix_copy_frac": stream_mix["frac"] if stream_mix else None},
+        # the whole step against the bytes this step variant has to move
+        "step_roofline": {"bytes_per_elem": head["moved_bytes_per_elem"],
                           "frac": head["step_frac"],
-                          "model": "two-read (select reads the score inputs, commit reads all)",
-                          "read_once_bytes_per_elem": ALG_BYTES_FINAL,
-                          "read_once_frac": head["read_once_frac"],
-                          "select_sweep": (None if args.single_sweep else
-                                           {"kernel": "k_bracket_sweep", "avg_ms": head["sweep_avg_ms"],
-                                            "alg_bytes_per_launch": head["sweep_bytes"],
-                                            "frac": head["sweep_frac"]})},
-        "select": head["select"],
-        "sweep": sweep,
+                          "other_kernels_ms": head["other_kernels_ms"]},
+        "two_sweep": {"ms_per_step": two["ms_per_step"], "elem_per_s": two["elem_per_s"],
+                      "bytes_per_elem": two["moved_bytes_per_elem"], "frac": two["step_frac"],
+                      "k_fused_final_ms": two["final_avg_ms"], "k_fused_final_frac": two["final_frac"],
+                      "k_bracket_sweep_ms": two["sweep_avg_ms"],
+                      "k_bracket_sweep_frac": two["sweep_frac"]},
+        ("packed_layout" if args.layout == "separate" else "separate_layout"): {
+            "ms_per_step": packed_leg["ms_per_step"], "elem_per_s": packed_leg["elem_per_s"],
+            "frac": packed_leg["step_frac"], "dominant_kernel_ms": packed_leg["final_avg_ms"],
+            "dominant_kernel_frac": packed_leg["final_frac"]},
     }
+    detail = {"headline_leg": head, "other_variant_leg": other, "other_layout_leg": packed_leg,
+              "select": head["select"], "traffic_source": traffic_src,
+              "stream_mix_copy": stream_mix}
+    if sweep:
+        detail["sweep"] = sweep
     if calib:
-        out["copy_calibration"] = calib
-    if args.layout == "separate":
-        # What the same five read and four write streams reach WITHOUT the math, on the very
-        # tensors the headline ran on (their contents are not needed any more): the ceiling this
-        # placement of four flat tensors gives a kernel of that stream mix.
-        sargs = [L.ptr(grads[0]), L.ptr(r), L.ptr(p), L.ptr(m), L.ptr(v), n, L.stream()]
-        ev = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
-        L.call("sga_calib_streams", *sargs)
-        ev[0].record()
-        for _ in range(5):
-            L.call("sga_calib_streams", *sargs)
-        ev[1].record()
-        torch.cuda.synchronize()
-        ms = ev[0].elapsed_time(ev[1]) / 5
-        out["roofline"]["stream_mix_copy"] = {
-            "kernel": "k_calib_streams (g bf16, r/p/m/v fp32 read; r/p/m/v written; no score, no "
-                      "select, no commit arithmetic), same tensors as the headline",
-            "avg_ms": ms, "GBps": n * ALG_BYTES_FINAL / ms / 1e6,
-            "frac_of_peak": n * ALG_BYTES_FINAL / (ms * 1e-3) / HBM_PEAK,
-            "dominant_kernel_vs_copy": ms / head["final_avg_ms"]}
-    if not args.no_sweep and args.layout == "separate":
-        # The same step after the device allocator has been churned.  Which physical pages an
-        # array gets decides the rate of this stream mix (the first allocations on a fresh
-        # machine are the slow kind, memory handed out after large blocks were freed is mostly
-        # the fast kind); this leg frees the five arrays, allocates and frees 3 x 100 GB, then
-        # allocates the five arrays again the same way and times the headline configuration on
-        # them.  An extra: `value` stays the first draw.
-        del p, m, v, r, grads
-        torch.cuda.empty_cache()
-        for _ in range(3):
-            blocks = [torch.empty(20 << 30, dtype=torch.uint8, device=dev) for _ in range(5)]
-            del blocks
-            torch.cuda.empty_cache()
-        gen = torch.Generator(device=dev).manual_seed(0)
-        p = torch.randn(n, generator=gen, device=dev) * 0.02
-        m = torch.zeros(n, device=dev)
-        v = torch.zeros(n, device=dev)
-        r = torch.zeros(n, device=dev)
-        grads = [student_t_dev(n, 10 + i, dev) for i in range(2)]
-        state["t"] = 0
-        leg = time_leg("separate", args.score, args.ratio, 2, 5, args.single_sweep)
-        sargs = [L.ptr(grads[0]), L.ptr(r), L.ptr(p), L.ptr(m), L.ptr(v), n, L.stream()]
-        ev = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
-        L.call("sga_calib_streams", *sargs)
-        ev[0].record()
-        for _ in range(5):
-            L.call("sga_calib_streams", *sargs)
-        ev[1].record()
-        torch.cuda.synchronize()
-        out["placement_redraw"] = {
-            "what": "the headline configuration on the five arrays freed and allocated again "
-                    "after 3 x 100 GB of device memory were allocated and freed",
-            "ms_per_step": leg["ms_per_step"], "elem_per_s": leg["elem_per_s"],
-            "dominant_kernel_ms": leg["final_avg_ms"], "dominant_kernel_frac": leg["final_frac"],
-            "step_frac": leg["step_frac"],
-            "stream_mix_copy_ms": ev[0].elapsed_time(ev[1]) / 5}
+        detail["copy_calibration"] = calib
     del p, m, v, r, grads, fs
     torch.cuda.empty_cache()
     if not args.no_rows:
-        out["qwen06b_mask_layout"] = qwen_mask_layout_row()
+        row = qwen_mask_layout_row()
+        detail["qwen06b_mask_layout"] = row
+        out["cfg2"] = {"what": "Qwen3-0.6B set, 8 buckets, abs_g 1 %, mask layout, two-sweep step",
+                       "ms_per_step": row["ms_per_step"], "elem_per_s": row["elem_per_s"],
+                       "bytes_per_elem": row["alg_bytes_per_step"] / row["n"],
+                       "frac": row["step_frac"]}
         torch.cuda.empty_cache()
-        out["stress_1e9"] = stress_row()
+        row = stress_row()
+        detail["stress_1e9"] = row
+        out["cfg5"] = {"what": "1e9 fp32, 5 % duplicated magnitudes: select_topk_flat alone "
+                               "(5 B/elem) at 0.01 % | 1 %, then the fused two-sweep step at 1 %",
+                       "select_ms": [row["select_only"]["0.01"]["ms"], row["select_only"]["1.0"]["ms"]],
+                       "select_frac": [row["select_only"]["0.01"]["frac"],
+                                       row["select_only"]["1.0"]["frac"]],
+                       "step_ms": row["fused_step"]["ms_per_step"],
+                       "step_frac": row["fused_step"]["step_frac"]}
         torch.cuda.empty_cache()
     if not args.no_replay:
-        out["replay"] = replay_bench()
+        draws = replay_bench([("seed 4", replay_draw()), ("stress", REPLAY_STRESS_DRAW)])
+        rp = draws[0]
+        detail["replay"] = rp
+        detail["replay_stress_draw"] = draws[1]
+        out["replay"] = {"value": rp["value"], "unit": rp["unit"],
+                         "ms_per_window": rp["ms_per_window"], "G": rp["G"], "W": rp["W"],
+                         "alg_bytes": rp["alg_bytes"], "frac": rp["frac"],
+                         "roofline": {"kernel": "k_replay_pass3", "avg_ms": rp["roofline"]["avg_ms"],
+                                      "frac": rp["roofline"]["frac"]},
+                         "stress_draw": {"value": draws[1]["value"], "frac": draws[1]["frac"]}}
         torch.cuda.empty_cache()
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(args.cpu_sample, 3, args.ratio, args.score)
         if "replay" in out:
-            out["replay"]["cpu_baseline"] = replay_cpu_baseline()
+            cb = replay_cpu_baseline()
+            detail["replay"]["cpu_baseline"] = cb
+            out["replay"]["cpu_baseline"] = {"value": cb["value"], "unit": cb["unit"],
+                                             "cores": cb["cores"], "kind": cb["kind"]}
     else:
         out["cpu_baseline"] = None
-    print(json.dumps(out))
+    if args.detail:
+        try:
+            os.makedirs(os.path.dirname(args.detail) or ".", exist_ok=True)
+            with open(args.detail, "w") as f:
+                json.dump(dict(out, detail=detail), f, indent=1)
+            out["detail_file"] = os.path.relpath(args.detail, ROOT)
+        except OSError as e:
+            out["detail_file"] = f"not written ({e.strerror})"
+    line = json.dumps(out, separators=(",", ":"))
+    assert len(line) < 6000, len(line)
+    print(line)
 
 
 if __name__ == "__main__":

@@ -1,9 +1,13 @@
-/* Benchmark-only entry points of libsga_hip.so.  They stand behind no
- * interface of wenqingqian/SGA and are NOT part of the drop-in boundary
- * (include/sga_hip.h): bench.py uses them to time the dominant kernels live
- * with HIP events on their launch stream and to calibrate the HBM traffic
- * counters.  Process-wide state behind a mutex; the hooks cost the product
- * path one relaxed atomic load per timed launch while disarmed.
+/* Entry points of libsga_hip_bench.so, the benchmark-only companion of
+ * libsga_hip.so.  They stand behind no interface of wenqingqian/SGA and are
+ * NOT part of the drop-in boundary (include/sga_hip.h; libsga_hip.so exports
+ * none of them): bench.py uses them to time the dominant kernels live with
+ * HIP events on their launch stream and to calibrate the HBM traffic
+ * counters.  libsga_hip.so holds two weak references (sga_bench_prof_begin /
+ * sga_bench_prof_end) that bind to this library when it was loaded first,
+ * into the global symbol scope (dlopen with RTLD_GLOBAL); without it they are
+ * null and a timed launch costs the product path one pointer test.
+ * Process-wide state behind a mutex.
  */
 #ifndef SGA_HIP_BENCH_H_
 #define SGA_HIP_BENCH_H_
@@ -24,6 +28,11 @@ extern "C" {
  * up to 4096 timed launches; enable(0) disarms.  read() waits for the recorded
  * events of one tag and returns their summed duration in ms and their number. */
 int sga_prof_enable(int on);
+/* the observer libsga_hip.so calls around a timed launch (not for callers) */
+void* sga_bench_prof_begin(int tag, void* stream);
+void sga_bench_prof_end(void* pair, void* stream);
+/* text of the last error of this library on the calling thread */
+const char* sga_bench_last_error(void);
 int sga_prof_read(int tag, double* total_ms, int* launches);
 
 /* dst[0..n) = src[0..n), fp32, n % 4 == 0: plain copy of known size used to

@@ -83,10 +83,6 @@ SIGNATURES = {
     "sga_planes_to_mask": (I32, [P, I64, P, P]),
     "sga_div_inplace": (I32, [P, I64, F, I32, P]),
     "sga_sq_dist": (I32, [P, I32, P, I64, P, P, P]),
-    "sga_calib_copy": (I32, [P, P, I64, P]),
-    "sga_calib_streams": (I32, [P, P, P, P, P, I64, P]),
-    "sga_prof_enable": (I32, [I32]),
-    "sga_prof_read": (I32, [I32, P, P]),
     "sga_fused_workspace_bytes": (SZ, [I64]),
     "sga_fused_sparse_step": (I32, [P, I32, P, P, P, P, I64, I64, P, I32, I32, P, P,
                                     I32, P, F, F, I32, I32, F, P, P, SZ, P]),
@@ -102,7 +98,48 @@ SIGNATURES = {
                                                         SZ, P]),
 }
 
+# include/sga_hip_bench.h: libsga_hip_bench.so, the benchmark-only companion
+BENCH_SIGNATURES = {
+    "sga_calib_copy": (I32, [P, P, I64, P]),
+    "sga_calib_streams": (I32, [P, P, P, P, P, I64, P]),
+    "sga_prof_enable": (I32, [I32]),
+    "sga_prof_read": (I32, [I32, P, P]),
+    "sga_bench_prof_begin": (P, [I32, P]),
+    "sga_bench_prof_end": (None, [P, P]),
+    "sga_bench_last_error": (C.c_char_p, []),
+}
+BENCH_LIB_PATH = os.path.join(_HERE, "libsga_hip_bench.so")
+
 _lib = None
+_bench = None
+
+
+def load_bench():
+    """Load the benchmark companion (timing observer + calibration kernels).
+    libsga_hip.so binds its two weak observer references when it is loaded,
+    so this has to come first and into the global symbol scope."""
+    global _bench
+    if _bench is not None:
+        return _bench
+    if _lib is not None:
+        raise RuntimeError("load_bench() must run before the first use of libsga_hip.so")
+    if not os.path.exists(BENCH_LIB_PATH):
+        raise RuntimeError(f"{BENCH_LIB_PATH} is missing (run `python -m sga_amd.build`)")
+    lib = C.CDLL(BENCH_LIB_PATH, mode=C.RTLD_GLOBAL)
+    for name, (res, args) in BENCH_SIGNATURES.items():
+        fn = getattr(lib, name)
+        fn.restype = res
+        fn.argtypes = args
+    _bench = lib
+    return lib
+
+
+def bench_call(name, *args):
+    lib = load_bench()
+    rc = getattr(lib, name)(*args)
+    if rc != 0:
+        raise RuntimeError(f"{name} failed ({rc}): "
+                           f"{lib.sga_bench_last_error().decode(errors='replace')}")
 
 
 def load():

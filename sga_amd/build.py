@@ -1,9 +1,11 @@
-"""Builds libsga_hip.so for gfx950 with hipcc (no torch dependency).
+"""Builds the HIP libraries for gfx950 with hipcc (no torch dependency).
 
-Usage: ``python -m sga_amd.build`` -- compiles every ``csrc/*.hip`` into
-``sga_amd/libsga_hip.so`` in-tree.  -ffp-contract=off keeps every fp32
-operation separately rounded (the kernels place FMAs explicitly where the
-arithmetic recipe has one).
+Usage: ``python -m sga_amd.build`` -- compiles every product source of
+``csrc/`` into ``sga_amd/libsga_hip.so`` (the C ABI of include/sga_hip.h and
+nothing else) and ``csrc/bench_hooks.hip`` into ``sga_amd/libsga_hip_bench.so``
+(timing observer + calibration kernels, loaded by bench.py only), both
+in-tree.  -ffp-contract=off keeps every fp32 operation separately rounded (the
+kernels place FMAs explicitly where the arithmetic recipe has one).
 """
 import os
 import subprocess
@@ -13,9 +15,10 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libsga_hip.so")
-SOURCES = ["runtime.hip", "scan.hip", "elementwise.hip", "adamw.hip",
-           "select.hip", "fused_step.hip", "replay.hip", "replay_group.hip",
-           "bench_hooks.hip"]
+BENCH_LIB = os.path.join(HERE, "libsga_hip_bench.so")
+SOURCES = ["fused_step.hip", "replay_group.hip", "select.hip", "elementwise.hip", "adamw.hip",
+           "replay.hip", "runtime.hip", "scan.hip"]
+BENCH_SOURCES = ["bench_hooks.hip"]
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
          "-ffp-contract=off", "-fno-fast-math",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
@@ -29,15 +32,30 @@ def _hipcc():
     raise RuntimeError("hipcc not found")
 
 
-def build(verbose=True, jobs=8, extra=()):
+def _stale(src, obj):
+    """True unless ``obj`` is newer than ``src`` and every header of csrc/ and include/."""
+    if not os.path.exists(obj):
+        return True
+    t = os.path.getmtime(obj)
+    deps = [src] + [os.path.join(d, f) for d in (CSRC, os.path.join(HERE, "..", "include"))
+                    for f in os.listdir(d) if f.endswith((".hpp", ".h"))]
+    return any(os.path.getmtime(d) > t for d in deps)
+
+
+def build(verbose=True, jobs=8, extra=(), incremental=False):
+    """Compile and link both libraries.  ``incremental`` (a convenience while
+    editing) skips sources whose object file is newer than the source and all
+    headers; the default compiles everything."""
     hipcc = _hipcc()
     objdir = os.path.join(HERE, "build")
     os.makedirs(objdir, exist_ok=True)
-    srcs = [s for s in SOURCES if os.path.exists(os.path.join(CSRC, s))]
 
     def one(src):
+        path = os.path.join(CSRC, src)
         obj = os.path.join(objdir, src.replace(".hip", ".o"))
-        cmd = [hipcc, *FLAGS, *extra, "-c", os.path.join(CSRC, src), "-o", obj]
+        if incremental and not extra and not _stale(path, obj):
+            return obj
+        cmd = [hipcc, *FLAGS, *extra, "-c", path, "-o", obj]
         r = subprocess.run(cmd, capture_output=True, text=True)
         if r.returncode != 0:
             raise RuntimeError(f"hipcc failed on {src}:\n{r.stdout}\n{r.stderr}")
@@ -50,15 +68,17 @@ def build(verbose=True, jobs=8, extra=()):
         return obj
 
     with ThreadPoolExecutor(max_workers=jobs) as ex:
-        objs = list(ex.map(one, srcs))
-    cmd = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", *objs, "-o", LIB]
-    r = subprocess.run(cmd, capture_output=True, text=True)
-    if r.returncode != 0:
-        raise RuntimeError(f"link failed:\n{r.stdout}\n{r.stderr}")
-    if verbose:
-        print(f"built {LIB} from {len(srcs)} sources")
+        objs = list(ex.map(one, SOURCES + BENCH_SOURCES))
+    for lib, group in ((LIB, objs[:len(SOURCES)]), (BENCH_LIB, objs[len(SOURCES):])):
+        cmd = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", *group, "-o", lib]
+        r = subprocess.run(cmd, capture_output=True, text=True)
+        if r.returncode != 0:
+            raise RuntimeError(f"link failed:\n{r.stdout}\n{r.stderr}")
+        if verbose:
+            print(f"built {lib} from {len(group)} sources")
     return LIB
 
 
 if __name__ == "__main__":
-    build(extra=tuple(a for a in sys.argv[1:] if a.startswith("-D")))
+    build(extra=tuple(a for a in sys.argv[1:] if a.startswith("-D")),
+          incremental="--incremental" in sys.argv[1:])

@@ -1,24 +1,49 @@
-// Benchmark-only hooks of libsga_hip.so (declared in include/sga_hip_bench.h,
-// not part of the drop-in boundary): live timing of the dominant kernels with
-// HIP events recorded on their launch stream, and two calibration kernels of
-// known HBM traffic.
+// libsga_hip_bench.so: benchmark-only companion of libsga_hip.so (declared in
+// include/sga_hip_bench.h, not part of the drop-in boundary).  It defines the
+// two timing-observer symbols that libsga_hip.so references weakly -- so it
+// has to be loaded, into the global symbol scope, BEFORE libsga_hip.so -- and
+// two calibration kernels of known HBM traffic.  It links against nothing of
+// the product library.
 #include <atomic>
 #include <mutex>
+#include <stdarg.h>
+#include <stdio.h>
 
+#define SGA_BENCH_LIBRARY 1
 #include "common.hpp"
 #include "../../include/sga_hip_bench.h"
 
-namespace sga {
+namespace {
 
+struct Pair { hipEvent_t a, b; int tag; int closed; };
 constexpr int kProfSlots = 4096;
-static std::atomic<int> g_prof_on{0};
-static std::mutex g_prof_mu;
-static ProfPair g_prof[kProfSlots];
-static int g_prof_made = 0, g_prof_used = 0;
+std::atomic<int> g_prof_on{0};
+std::mutex g_prof_mu;
+Pair g_prof[kProfSlots];
+int g_prof_made = 0, g_prof_used = 0;
+thread_local char g_err[256] = "";
 
-ProfPair* prof_begin(int tag, hipStream_t s) {
+void bench_error(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+}
+
+int bench_check(const char* what) {
+  const hipError_t e = hipGetLastError();
+  if (e == hipSuccess) return SGA_OK;
+  bench_error("%s: %s", what, hipGetErrorString(e));
+  return SGA_ERR_LAUNCH;
+}
+
+}  // namespace
+
+extern "C" const char* sga_bench_last_error(void) { return g_err; }
+
+extern "C" void* sga_bench_prof_begin(int tag, void* stream) {
   if (!g_prof_on.load(std::memory_order_relaxed)) return nullptr;
-  ProfPair* pp = nullptr;
+  Pair* pp = nullptr;
   {
     std::lock_guard<std::mutex> lock(g_prof_mu);
     if (!g_prof_on.load(std::memory_order_relaxed) || g_prof_used >= kProfSlots) return nullptr;
@@ -34,16 +59,19 @@ ProfPair* prof_begin(int tag, hipStream_t s) {
     pp->tag = tag;
     pp->closed = 0;
   }
-  (void)hipEventRecord(pp->a, s);
+  (void)hipEventRecord(pp->a, (hipStream_t)stream);
   return pp;
 }
 
-void prof_end(ProfPair* pp, hipStream_t s) {
+extern "C" void sga_bench_prof_end(void* pair, void* stream) {
+  Pair* pp = reinterpret_cast<Pair*>(pair);
   if (!pp) return;
-  (void)hipEventRecord(pp->b, s);
+  (void)hipEventRecord(pp->b, (hipStream_t)stream);
   std::lock_guard<std::mutex> lock(g_prof_mu);
   pp->closed = 1;
 }
+
+namespace sga {
 
 // Plain 128-bit copy of known size: the yardstick the HBM traffic counters
 // and the achievable streaming bandwidth are calibrated against.
@@ -97,7 +125,7 @@ extern "C" int sga_prof_enable(int on) {
 }
 
 extern "C" int sga_prof_read(int tag, double* total_ms, int* launches) {
-  if (!total_ms || !launches) { set_error("sga_prof_read: null output"); return SGA_ERR_ARG; }
+  if (!total_ms || !launches) { bench_error("sga_prof_read: null output"); return SGA_ERR_ARG; }
   std::lock_guard<std::mutex> lock(g_prof_mu);
   double tot = 0.0;
   int cnt = 0;
@@ -106,7 +134,7 @@ extern "C" int sga_prof_read(int tag, double* total_ms, int* launches) {
     float ms = 0.0f;
     if (hipEventSynchronize(g_prof[i].b) != hipSuccess ||
         hipEventElapsedTime(&ms, g_prof[i].a, g_prof[i].b) != hipSuccess) {
-      set_error("sga_prof_read: event %d not ready", i);
+      bench_error("sga_prof_read: event %d not ready", i);
       return SGA_ERR_LAUNCH;
     }
     tot += ms;
@@ -119,25 +147,25 @@ extern "C" int sga_prof_read(int tag, double* total_ms, int* launches) {
 
 extern "C" int sga_calib_copy(float* dst, const float* src, int64_t n, void* stream) {
   if (!dst || !src || n < 0 || (n & 3) || !aligned4(dst, 4) || !aligned4(src, 4)) {
-    set_error("sga_calib_copy: needs 16-byte aligned buffers and n %% 4 == 0");
+    bench_error("sga_calib_copy: needs 16-byte aligned buffers and n %% 4 == 0");
     return SGA_ERR_ARG;
   }
   if (n == 0) return SGA_OK;
   hipLaunchKernelGGL(k_calib_copy, dim3(stream_grid(n / 4, kBlock, 1 << 20)), dim3(kBlock), 0,
                      (hipStream_t)stream, dst, src, n / 4);
-  return check_launch("sga_calib_copy");
+  return bench_check("sga_calib_copy");
 }
 
 extern "C" int sga_calib_streams(const void* g_bf16, float* r, float* p, float* m, float* v,
                                  int64_t n, void* stream) {
   if (!g_bf16 || !r || !p || !m || !v || n < 0 || (n & 3) || !aligned4(g_bf16, 2) ||
       !aligned4(r, 4) || !aligned4(p, 4) || !aligned4(m, 4) || !aligned4(v, 4)) {
-    set_error("sga_calib_streams: needs aligned buffers and n a multiple of 4");
+    bench_error("sga_calib_streams: needs aligned buffers and n a multiple of 4");
     return SGA_ERR_ARG;
   }
   if (n == 0) return SGA_OK;
   hipLaunchKernelGGL(k_calib_streams, dim3((unsigned)cdiv64(n, (int64_t)kBlock * kVec)),
                      dim3(kBlock), 0, (hipStream_t)stream,
                      reinterpret_cast<const uint16_t*>(g_bf16), r, p, m, v, n);
-  return check_launch("sga_calib_streams");
+  return bench_check("sga_calib_streams");
 }

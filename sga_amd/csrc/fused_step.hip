@@ -283,7 +283,10 @@ __device__ __forceinline__ void final_chunk(const FinalArgs& a, int64_t c, Chunk
       int64_t s1 = s0 + kWave * kVec;
       if (!FULL && s1 > n) s1 = n;
       if (s0 < sc.lo || s0 >= sc.hi) sc.seek_uniform(s0);
-      float pn[4], mn[4], vn[4];
+      // a coordinate no tensor of the table covers keeps its p / m / v
+      float pn[4] = {pp[it][0], pp[it][1], pp[it][2], pp[it][3]};
+      float mn[4] = {mm[it][0], mm[it][1], mm[it][2], mm[it][3]};
+      float vn[4] = {vv[it][0], vv[it][1], vv[it][2], vv[it][3]};
       for (;;) {
         const bool whole = sc.lo <= s0 && sc.hi >= s1;
         Hyper h = sc.h;
@@ -448,6 +451,7 @@ struct SpecArgs {
   uint32_t* seg_key;
   F4* seg_rec;            // (q, p, m, v) of each recorded coordinate
   uint32_t* seg_cnt;
+  uint32_t* seg_fail;     // per segment: 0, or ~base of the first reservation that did not fit
   uint32_t seg_cap;
   uint32_t* tile_gt;
   uint32_t* tile_eq;
@@ -599,7 +603,9 @@ __device__ __forceinline__ void spec_slab(const FinalArgs& a, const SpecArgs& sa
   int64_t s1 = s0 + kWave * kVec;
   if (!FULL && s1 > n) s1 = n;
   if (s0 < sc.lo || s0 >= sc.hi) sc.seek_uniform(s0);
-  float pn[4], mn[4], vn[4];
+  // a coordinate no tensor of the table covers keeps its p / m / v
+  float pn[4] = {pp[0], pp[1], pp[2], pp[3]}, mn[4] = {mm[0], mm[1], mm[2], mm[3]},
+        vn[4] = {vv[0], vv[1], vv[2], vv[3]};
   for (;;) {
     const bool whole = sc.lo <= s0 && sc.hi >= s1;
     Hyper h = sc.h;
@@ -677,14 +683,21 @@ __global__ __launch_bounds__(kBlock) void k_fused_spec(
     if (mycnt) {                                        // wave-uniform
       // The chunk's LDS records go, in one piece, to the segment its chunk index hashes to
       // (neighbouring waves, which run at the same time, hit different counters: with one
-      // segment per range of consecutive chunks the sweep was 0.25 ms slower); when that is full
-      // (the reservation is taken back: every later one then sees the true count), to the
-      // shared overflow list.
+      // segment per range of consecutive chunks the sweep was 0.25 ms slower); when they do not
+      // fit there, to the shared overflow list.  A reservation is never taken back: the counter
+      // only grows, so once one reservation has failed every later one fails as well, and the
+      // records of the segment are exactly [0, base of the first failure) -- which the failing
+      // wave leaves in seg_fail (the smallest failing base wins) for the check to clamp the
+      // segment to.  (Taking the reservation back instead let a third wave slip into the gap
+      // between two failed ones and left unwritten slots inside the counted range.)
       const uint32_t seg = (uint32_t)c & (uint32_t)(kSegWaves - 1);
       uint32_t base = 0;
       if (lane_id() == 0) {
         base = atomicAdd(&sa.seg_cnt[seg], mycnt);
-        if (base + mycnt > sa.seg_cap) { atomicSub(&sa.seg_cnt[seg], mycnt); base = 0xFFFFFFFFu; }
+        if (base + mycnt > sa.seg_cap) {
+          if (base <= sa.seg_cap) atomicMax(&sa.seg_fail[seg], 0xFFFFFFFFu - base);
+          base = 0xFFFFFFFFu;
+        }
       }
       base = __shfl(base, 0, kWave);
       uint32_t* g_idx = sa.seg_idx + (int64_t)seg * sa.seg_cap;
@@ -997,13 +1010,14 @@ struct SpecWorkspace {
   int64_t ovf_cap;
   uint32_t* tie_cnt;      // [0]: ties gathered; tie_idx follows
   uint32_t* tie_idx;
+  uint32_t* seg_fail;     // kSegWaves words
   void* stage;
 };
 static inline size_t spec_ws_bytes(int64_t n, int val_bytes) {
   const int64_t nt = cdiv64(n, kChunk) + 8;
   // records of the segments (16 B), dense records (16 B), overflow list (24 B, half the capacity)
   size_t b = (size_t)nt * (128 + 16) + (size_t)kSegWaves * fast_seg_cap(nt * kChunk) * (16 * 2 + 12) +
-             (size_t)nt * kChunk * val_bytes + 4096 + 8192;
+             (size_t)nt * kChunk * val_bytes + 4096 + 8192 + (size_t)kSegWaves * 4;
   return (b + 255) & ~(size_t)255;
 }
 static inline bool spec_ws_carve(void* ws, size_t bytes, int64_t n, int val_bytes, int64_t seg_cap,
@@ -1034,6 +1048,8 @@ static inline bool spec_ws_carve(void* ws, size_t bytes, int64_t n, int val_byte
   out->tie_idx = out->tie_cnt + 64;
   p += 256 + (size_t)kSpecTieCap * 4;
   p = reinterpret_cast<char*>((reinterpret_cast<uintptr_t>(p) + 255) & ~(uintptr_t)255);
+  out->seg_fail = reinterpret_cast<uint32_t*>(p);
+  p += (size_t)kSegWaves * 4;
   out->stage = p;
   return true;
 }
@@ -1073,7 +1089,8 @@ static int run_fused_spec(const void* g, float* resid, float* p, float* m, float
   hipLaunchKernelGGL((k_sample<SrcFused<BF16G, SCORE>>), dim3(stream_grid(n_sv, kBlock)), dim3(kBlock), 0, s,
                      src, n, n_sv, n_vec, w.sample, seed);
   hipLaunchKernelGGL(k_bracket_ranks, dim3(1), dim3(kBlock), 0, s, w.aux, w.hist, kHistStride * 2,
-                     (uint32_t)k, (double)n, (double)ns, w.seg_cnt, w.blk_gt, w.blk_eq, kSpecSigmas);
+                     (uint32_t)k, (double)n, (double)ns, w.seg_cnt, w.blk_gt, w.blk_eq, kSpecSigmas,
+                     x.seg_fail);
   SrcU32 ssrc{w.sample};
   for (int level = 0; level < 3; ++level)
     launch_level<SrcU32, 2, true>(ssrc, ns, (const uint32_t*)nullptr, level, w.aux, w, s, kRawKeyBlocks);
@@ -1081,6 +1098,7 @@ static int run_fused_spec(const void* g, float* resid, float* p, float* m, float
   SpecArgs sa;
   sa.splane = w.pbits; sa.fplane = x.dplane; sa.stage = x.stage;
   sa.seg_idx = w.seg_idx; sa.seg_key = w.seg_key; sa.seg_rec = x.seg_rec; sa.seg_cnt = w.seg_cnt;
+  sa.seg_fail = x.seg_fail;
   sa.seg_cap = (uint32_t)w.seg_cap;
   sa.tile_gt = w.tile_gt; sa.tile_eq = w.tile_eq; sa.hi_part = w.blk_gt; sa.nf_part = w.blk_eq;
   sa.ovf_idx = x.ovf_idx; sa.ovf_key = x.ovf_key; sa.ovf_rec = x.ovf_rec;
@@ -1093,7 +1111,8 @@ static int run_fused_spec(const void* g, float* resid, float* p, float* m, float
                      n_segs, w.st, w.aux, w.seg_dir);
   prof_end(pp, s);
   hipLaunchKernelGGL(k_bracket_check, dim3(1), dim3(kBlock), 0, s, w.st, w.aux, w.seg_cnt, w.hist,
-                     kHistStride * 2, (uint32_t)w.seg_cap, w.blk_gt, w.blk_eq, 1, (uint32_t)x.ovf_cap);
+                     kHistStride * 2, (uint32_t)w.seg_cap, w.blk_gt, w.blk_eq, 1, (uint32_t)x.ovf_cap,
+                     x.seg_fail);
   hipLaunchKernelGGL(k_cand_compact, dim3(512), dim3(kBlock), 0, s, w.aux, w.seg_cnt, w.seg_idx,
                      w.seg_key, (uint32_t)w.seg_cap, w.cand_idx, w.cand_key, x.seg_rec, x.cand_rec);
   hipLaunchKernelGGL(k_spec_ovf_compact, dim3(64), dim3(kBlock), 0, s, w.aux, w.seg_cnt, x.ovf_idx,

@@ -784,8 +784,11 @@ __global__ __launch_bounds__(kBlock) void k_sample(Src src, int64_t n, int64_t n
 // lower end.  Also zeroes both histogram sets.
 static __global__ void k_bracket_ranks(SelState* aux, uint32_t* hist, int nhist, uint32_t k,
                                        double n, double ns, uint32_t* seg_cnt, uint32_t* hi_part,
-                                       uint32_t* nf_part, double sigmas = 5.0) {
+                                       uint32_t* nf_part, double sigmas = 5.0,
+                                       uint32_t* seg_fail = nullptr) {
   for (int i = threadIdx.x; i < nhist; i += blockDim.x) hist[i] = 0u;
+  if (seg_fail)
+    for (int i = threadIdx.x; i < kSegWaves; i += blockDim.x) seg_fail[i] = 0u;
   for (int i = threadIdx.x; i <= kSegWaves + 1; i += blockDim.x) seg_cnt[i] = 0u;   // + overflow count
   for (int i = threadIdx.x; i < kSweepParts; i += blockDim.x) { hi_part[i] = 0u; nf_part[i] = 0u; }
   if (threadIdx.x != 0) return;
@@ -990,13 +993,19 @@ static __global__ __launch_bounds__(kBlock) void k_bracket_check(SelState* __res
                                                                  uint32_t seg_cap,
                                                                  const uint32_t* __restrict__ hi_part,
                                                                  const uint32_t* __restrict__ nf_part,
-                                                                 int spec = 0, uint32_t ovf_cap = 0u) {
+                                                                 int spec = 0, uint32_t ovf_cap = 0u,
+                                                                 const uint32_t* __restrict__ seg_fail = nullptr) {
   __shared__ uint32_t s_w4[kChunksPerBlock];
   constexpr int PER = kSegWaves / kBlock;   // 32
   uint32_t v[PER], mine = 0, over = 0;
 #pragma unroll
   for (int j = 0; j < PER; ++j) {
-    const uint32_t cnt = seg_cnt[threadIdx.x * PER + j];
+    uint32_t cnt = seg_cnt[threadIdx.x * PER + j];
+    if (seg_fail && cnt > seg_cap) {
+      // single-sweep step: reservations are never taken back, the segment's records end where
+      // the first reservation that did not fit began (the later ones went to the overflow list)
+      cnt = 0xFFFFFFFFu - seg_fail[threadIdx.x * PER + j];
+    }
     over |= cnt > seg_cap;                    // the sweep reserved more than the segment holds
     v[j] = cnt < seg_cap ? cnt : seg_cap;
     mine += v[j];

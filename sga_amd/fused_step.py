@@ -10,6 +10,13 @@ from .scores import STEP_SCORE_MAP as SCORE_MAP
 from .selection import read_result
 
 
+class SingleSweepLost(RuntimeError):
+    """The single-sweep step committed on a sampled bracket that turned out not
+    to hold the k-th key (``result.status == 3``): resid / p / m / v of this
+    step are not the exact top-k step's and the pack was not written.  The
+    two-sweep step (``single_sweep=False``) has no such outcome."""
+
+
 def k_for(n_total, ratio_percent):
     """``sga/plugins/selection/topk.py:111-112``"""
     return max(1, int(round(n_total * ratio_percent / 100.0)))
@@ -89,7 +96,7 @@ class FusedSparseStep:
         return (L.GC_ADAMS if optimizer == "adams" else 0) | (L.GC_FOLD if fold else 0)
 
     def _run(self, name, g, state_args, step, k, ratio_percent, score, factor, coeff, fast,
-             optimizer, fold, interval, inactive_lr_scale, single_sweep, seed):
+             optimizer, fold, interval, inactive_lr_scale, single_sweep, seed, check, result):
         """Checks shared by the two state layouts, then one call of entry point
         ``name`` (``state_args``: what that entry point takes between the
         gradient and ``n``)."""
@@ -105,20 +112,34 @@ class FusedSparseStep:
         head = [L.ptr(g), L.dtype_code(g), *state_args, n, k, L.ptr(self._seg_dev),
                 len(self.segments), SCORE_MAP[score], L.ptr(self.idx), L.ptr(self.values),
                 L.dtype_code(self.values), L.ptr(self.mask), L.f32(factor), L.f32(coeff)]
+        if result is None:
+            result = self.result
+        elif (result.dtype != torch.int32 or result.numel() != 8 or not result.is_cuda
+              or not result.is_contiguous()):
+            raise ValueError("result: a contiguous int32[8] device tensor")
         if single_sweep:
             ws2 = self._single_sweep_ws()
             self._calls += 1
             L.call(name, *head, flags, L.f32(interval),
-                   (self._calls if seed is None else seed) & 0xFFFFFFFF, L.ptr(self.result),
+                   (self._calls if seed is None else seed) & 0xFFFFFFFF, L.ptr(result),
                    L.ptr(self.ws), self.ws_bytes, L.ptr(ws2), ws2.numel(), L.stream())
+            if check:
+                res = read_result(result)              # synchronises with the step
+                if res.status == 3:
+                    raise SingleSweepLost(
+                        f"single-sweep step {step}: the sampled bracket missed the k-th key "
+                        f"after the commit (k={k}, n={n}, seed={self._calls if seed is None else seed}); "
+                        "the state of this step is not the exact top-k step's -- restore it "
+                        "from the caller's copy, or use the two-sweep step")
         else:
-            L.call(name, *head, 1 if fast else 0, flags, L.f32(interval), L.ptr(self.result),
+            L.call(name, *head, 1 if fast else 0, flags, L.f32(interval), L.ptr(result),
                    L.ptr(self.ws), self.ws_bytes, L.stream())
         return self.idx[:k], self.values[:k]
 
     def step(self, g, resid, p, m, v, step, k=None, ratio_percent=None,
              score="abs_g", factor=1.0, coeff=1.0, fast=True, optimizer="adamw", fold=False,
-             interval=1.0, inactive_lr_scale=1.0, single_sweep=False, seed=None):
+             interval=1.0, inactive_lr_scale=1.0, single_sweep=False, seed=None, check=True,
+             result=None):
         """Run one fused step in place; returns (idx[:k], values[:k]) views.
         ``self.result`` holds the device-side select result (threshold bits,
         counts); nothing is synchronised here.  ``optimizer="adams"`` commits
@@ -131,7 +152,13 @@ class FusedSparseStep:
         bit for bit; ``result.status == 3`` reports the one thing that cannot
         be repaired, a sampled bracket that missed the k-th key after the
         commit (12 sigma margins; ``seed`` moves the sample offsets, default a
-        per-call counter)."""
+        per-call counter).  The reference has no such outcome, so this mode is
+        for callers that hold a restorable copy of the state (or accept
+        restarting from a checkpoint): with ``check`` (the default) the call
+        waits for the step and raises ``SingleSweepLost`` on status 3 instead
+        of handing back a pack that was not written; ``check=False`` leaves
+        the status to the caller (``result``: an int32[8] device tensor of the
+        caller's for this step's result block, default ``self.result``)."""
         for t in (g, resid, p, m, v):
             L.require_dev(t)
             L.require_contig(t=t)
@@ -139,11 +166,12 @@ class FusedSparseStep:
         return self._run("sga_fused_sparse_step" + ("_single_sweep" if single_sweep else ""), g,
                          [L.ptr(resid), L.ptr(p), L.ptr(m), L.ptr(v)], step, k, ratio_percent,
                          score, factor, coeff, fast, optimizer, fold, interval, inactive_lr_scale,
-                         single_sweep, seed)
+                         single_sweep, seed, check, result)
 
     def step_packed(self, g, state, step, k=None, ratio_percent=None, score="abs_g",
                     factor=1.0, coeff=1.0, fast=True, optimizer="adamw", fold=False,
-                    interval=1.0, inactive_lr_scale=1.0, single_sweep=False, seed=None):
+                    interval=1.0, inactive_lr_scale=1.0, single_sweep=False, seed=None,
+                    check=True, result=None):
         """Same step on a ``PackedState`` (resid/p/m/v interleaved in 64 KiB
         records): same arithmetic and outputs."""
         L.require_dev(g, state.data)
@@ -154,7 +182,7 @@ class FusedSparseStep:
                 "sga_fused_sparse_step_packed")
         return self._run(name, g, [L.ptr(state.data)], step, k, ratio_percent, score, factor,
                          coeff, fast, optimizer, fold, interval, inactive_lr_scale, single_sweep,
-                         seed)
+                         seed, check, result)
 
     def read_result(self):
         return read_result(self.result)

@@ -281,6 +281,112 @@ def test_llama1b_set_single_sweep_seeded_configs(dev):
         torch.cuda.empty_cache()
 
 
+def _both_steps_agree(dev, segs, n, grads, score, k, what, steps=2, p_seed=3):
+    """The single-sweep step against the two-sweep step from the same state
+    over `steps` steps: every output bit (idx, values, mask, residual, p, m,
+    v, threshold, tie counts), and the single sweep must have gone ahead
+    (path 2) and ended with status 0."""
+    from sga_amd.fused_step import FusedSparseStep
+    gen = torch.Generator(device=dev).manual_seed(p_seed)
+    p0 = torch.randn(n, generator=gen, device=dev) * 0.02
+    state = [[p0.clone()] + [torch.zeros(n, device=dev) for _ in range(3)] for _ in range(2)]
+    del p0
+    fs = [FusedSparseStep(n, segs, dev, values_dtype=torch.bfloat16, max_k=k, want_mask=True)
+          for _ in range(2)]
+    for step in range(1, steps + 1):
+        g = grads[(step - 1) % len(grads)]
+        outs = []
+        for which in range(2):
+            pp, mm, vv, rr = state[which]
+            idx, vals = fs[which].step(g, rr, pp, mm, vv, step, k=k, score=score,
+                                       single_sweep=bool(which), check=False)
+            res = fs[which].read_result()
+            assert res.status == 0 and res.n_selected == k, (what, step, which, vars(res))
+            outs.append((idx, vals, fs[which].mask, res))
+        a, b = outs[0][3], outs[1][3]
+        assert b.path == 2, (what, step, vars(b))
+        assert (a.thresh_bits, a.need, a.n_gt, a.n_eq) == (b.thresh_bits, b.need, b.n_gt, b.n_eq), (
+            what, step)
+        assert torch.equal(outs[0][0], outs[1][0]), (what, step)
+        assert torch.equal(outs[0][2], outs[1][2]), (what, step)
+        assert torch.equal(outs[0][1].view(torch.int16), outs[1][1].view(torch.int16)), (what, step)
+        for x, y in zip(state[0], state[1]):
+            assert torch.equal(x.view(torch.int32), y.view(torch.int32)), (what, step)
+    del fs, state
+    torch.cuda.empty_cache()
+
+
+def _qwen_log_uniform_grads(dev, segs, n, seed):
+    """bf16 Gaussian gradients with a per-tensor std log-uniform in [1e-5, 1e-2]."""
+    gen = torch.Generator(device=dev).manual_seed(seed)
+    cpu_gen = torch.Generator().manual_seed(seed)
+    g = torch.empty(n, dtype=torch.bfloat16, device=dev)
+    for s in segs:
+        std = 10 ** (-5 + 3 * float(torch.rand(1, generator=cpu_gen)))
+        g[s["start"]:s["start"] + s["n"]] = (torch.randn(s["n"], generator=gen, device=dev)
+                                             * std).to(torch.bfloat16)
+    return g
+
+
+@pytest.mark.parametrize("score", ["abs_g", "update"])
+def test_qwen06b_log_uniform_scales_single_sweep_one_bucket(dev, score):
+    """The single-sweep step on per-tensor scales three decades apart (config
+    2's gradient distribution), the whole 596 M-element set as ONE bucket: the
+    sampled bracket has to hold although a few tensors own the whole top 1 %."""
+    from sga_amd.fused_step import k_for
+    from sga_amd.shapes import qwen3_06b, segments_for
+    segs, n = segments_for(qwen3_06b())
+    grads = [_qwen_log_uniform_grads(dev, segs, n, 5 + i) for i in range(2)]
+    _both_steps_agree(dev, segs, n, grads, score, k_for(n, 1.0), ("one bucket", score))
+
+
+def test_qwen06b_log_uniform_scales_single_sweep_per_bucket(dev):
+    """The same distribution stepped as config 2 words it: the embedding and
+    seven buckets of four layers, each with its own top 1 %."""
+    from sga_amd.fused_step import k_for
+    from sga_amd.shapes import qwen3_06b, segments_for
+    segs, n = segments_for(qwen3_06b())
+    grads = [_qwen_log_uniform_grads(dev, segs, n, 5 + i) for i in range(2)]
+    cuts = [0, segs[1]["start"]] + [segs[1 + 11 * j]["start"] for j in range(4, 28, 4)] + [n]
+    for b, (lo, hi) in enumerate(zip(cuts[:-1], cuts[1:])):
+        bsegs = [dict(s, start=s["start"] - lo) for s in segs if lo <= s["start"] < hi]
+        _both_steps_agree(dev, bsegs, hi - lo, [g[lo:hi] for g in grads], "update",
+                          k_for(hi - lo, 1.0), ("bucket", b))
+
+
+@pytest.mark.parametrize("score", ["abs_g", "update"])
+def test_single_sweep_when_the_last_tensors_have_no_gradient(dev, score):
+    """Absent parameters: the last fifth of the set (whole tensors) has an
+    all-zero gradient, so the tail of the bucket scores unlike the rest."""
+    from sga_amd.fused_step import k_for
+    from sga_amd.shapes import qwen3_06b, segments_for
+    segs, n = segments_for(qwen3_06b())
+    cut = next(s["start"] for s in segs if s["start"] >= n - n // 5)
+    grads = []
+    for i in range(2):
+        g = _student_t(n, 20 + i, dev).to(torch.bfloat16)
+        g[cut:] = 0
+        grads.append(g)
+    _both_steps_agree(dev, segs, n, grads, score, k_for(n, 1.0), ("absent tail", score))
+
+
+@pytest.mark.parametrize("ratio", [1.0, 0.3])
+def test_single_sweep_when_the_last_percent_scores_100x(dev, ratio):
+    """The last 1 % of the coordinates carries gradients 100 times larger than
+    the rest: a sample that under-covered the end of the bucket would put the
+    bracket in the wrong place (k = 1 %: the k-th key lies right where the two
+    populations meet; k = 0.3 %: entirely inside the tail)."""
+    from sga_amd.fused_step import k_for
+    from sga_amd.shapes import qwen3_06b, segments_for
+    segs, n = segments_for(qwen3_06b())
+    grads = []
+    for i in range(2):
+        g = _student_t(n, 30 + i, dev)
+        g[n - n // 100:] *= 100.0
+        grads.append(g.to(torch.bfloat16))
+    _both_steps_agree(dev, segs, n, grads, "update", k_for(n, ratio), ("hot tail", ratio))
+
+
 def _select_ok(score, mask, k):
     """Exact-k, dominance and lowest-index ties of a mask against a score."""
     assert int(mask.sum()) == k

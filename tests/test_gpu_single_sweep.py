@@ -153,20 +153,77 @@ def test_a_bracket_that_missed_is_reported(dev):
     segs = [dict(start=0, n=n, lr=1e-4, b1=0.9, b2=0.95, eps=1e-8, wd=0.0)]
     k = SEL.k_for(n, 1.0)
 
-    def run(sd):
+    def run(sd, check=False):
         p = torch.zeros(n, device=dev)
         m, v, r = torch.zeros(n, device=dev), torch.zeros(n, device=dev), torch.zeros(n, device=dev)
         fs = FusedSparseStep(n, segs, dev, values_dtype=torch.float32, want_mask=True)
-        idx, vals = fs.step(g.to(dev), r, p, m, v, 1, k=k, single_sweep=True, seed=sd)
+        idx, vals = fs.step(g.to(dev), r, p, m, v, 1, k=k, single_sweep=True, seed=sd,
+                            check=check)
         return fs.read_result(), idx.cpu(), fs.mask.cpu().bool()
 
     res, _, _ = run(seed)
     assert res.status == 3 and res.path == 0, vars(res)
-    res, idx, mask = run(seed + 1)
+    # the wrapper's default waits for the step and refuses to hand back a pack that was not written
+    from sga_amd.fused_step import SingleSweepLost
+    with pytest.raises(SingleSweepLost, match="missed the k-th key"):
+        run(seed, check=True)
+    res, idx, mask = run(seed + 1, check=True)
     assert res.status == 0 and res.n_selected == k, vars(res)
     ref_mask, th = SEL.select_topk_flat(g.abs(), k)
     assert res.thresh == th and torch.equal(mask, ref_mask)
     assert torch.equal(idx.long(), torch.nonzero(ref_mask).reshape(-1))
+
+
+@pytest.mark.parametrize("packed", [False, True])
+def test_many_chunks_race_for_full_segments(dev, packed):
+    """Record segments that fill up while several chunks reserve room in them
+    at once.  1280 of the 65536 chunks hold magnitudes in [1, 2), the rest
+    ~1e-6, and k sits in the middle of the large ones: about a quarter of the
+    large values fall inside the sampled bracket, ~250 records per hot chunk.
+    The hot chunks are the ones whose index is below 160 modulo 8192, i.e. the
+    eight chunks c, c + 8192, ... of 160 segments of 256 slots each: one
+    chunk's records fit a segment, the other seven find it full and go to the
+    overflow list, and chunks over 256 records spill slab by slab.  Every
+    output equals the two-sweep step's, bit for bit, on both state layouts."""
+    from sga_amd.fused_step import FusedSparseStep, PackedState
+    n = 1 << 26
+    gen = torch.Generator().manual_seed(11)
+    g = torch.rand(n, generator=gen) * 1e-6
+    chunk = torch.arange(n // 1024)
+    hot = ((chunk & 8191) < 160).repeat_interleave(1024)
+    n_hot = int(hot.sum())
+    g[hot] = 1.0 + torch.rand(n_hot, generator=gen)
+    g *= torch.where(torch.rand(n, generator=gen) < 0.5, -1.0, 1.0)
+    k = n_hot // 2
+    segs = [dict(start=0, n=n, lr=1e-3, b1=0.9, b2=0.95, eps=1e-8, wd=0.1)]
+    gd = g.to(dev)
+    p0 = (torch.randn(n, generator=gen) * 0.02).to(dev)
+    outs = []
+    for single in (False, True):
+        r, m, v = (torch.zeros(n, device=dev) for _ in range(3))
+        p = p0.clone()
+        fs = FusedSparseStep(n, segs, dev, values_dtype=torch.float32, max_k=k, want_mask=True)
+        st = PackedState(n, dev).pack(r, p, m, v) if packed else None
+        for step in (1, 2):
+            if packed:
+                idx, vals = fs.step_packed(gd, st, step, k=k, single_sweep=single)
+            else:
+                idx, vals = fs.step(gd, r, p, m, v, step, k=k, single_sweep=single)
+            res = fs.read_result()
+            assert res.status == 0 and res.n_selected == k, (single, step, vars(res))
+            assert not single or res.path == 2, (step, vars(res))
+        if packed:
+            st.unpack(r, p, m, v)
+        outs.append((res, idx.clone(), vals.clone(), fs.mask.clone(), r, p, m, v))
+        del fs, st
+    a, b = outs
+    assert (a[0].thresh_bits, a[0].need, a[0].n_gt, a[0].n_eq) == (
+        b[0].thresh_bits, b[0].need, b[0].n_gt, b[0].n_eq)
+    assert a[0].thresh > 1.0          # the k-th key lies among the hot chunks
+    assert torch.equal(a[1], b[1]) and torch.equal(a[3], b[3])
+    for x, y in zip(a[2:], b[2:]):
+        assert torch.equal(x.view(torch.int32) if x.dtype == torch.float32 else x,
+                           y.view(torch.int32) if y.dtype == torch.float32 else y)
 
 
 def test_randomized_single_sweep_equals_two_sweep(dev):
