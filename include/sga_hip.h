@@ -483,6 +483,30 @@ int sga_replay_reselect(const void* g, int g_dtype, const float* res,
                         sga_select_result* result, void* ws, size_t ws_bytes,
                         void* stream);
 
+/* pass 2 under the `balanced-histogram` selection semantics
+ * (replay_fused.py:405-489, 1805-1809; _histogram.py:115-123, 203-216): the
+ * same on-the-fly score, selected like the online engine's approximate tier --
+ * histogram of the top 16 bits of |score| over the stride-8 subsample of every
+ * tensor's own grid (element j of tensor t is sampled when j = seg_phase[t]
+ * (mod 8), seg_phase[t] = (-p_off) mod 8; NULL = all zero), crossing bin
+ * b = searchsorted(cumsum(hist), rank), selection = top 16 bits >= b (the
+ * whole crossing bin; the count is approximate by construction), written as
+ * bit planes into sel_out.  rank is the caller's
+ * max(1, round(n_sampled * (n_total - k + 1) / n_total)) (host integers, as
+ * the reference computes it).  result: thresh_bits = the bin's lower edge,
+ * n_selected = coordinates selected, path 3.  hist: device scratch of
+ * sga_balanced_hist_words() uint32. */
+int64_t sga_balanced_hist_words(void);
+int sga_replay_reselect_balanced(const void* g, int g_dtype, const float* res,
+                                 const float* w, const float* m, const float* v,
+                                 int64_t n, int64_t rank, const sga_segment* segs,
+                                 int n_segs, const int32_t* seg_phase,
+                                 int score_id, const float* coef_f,
+                                 float coef_dense, int adams, int packed,
+                                 int res_zero, uint32_t* sel_out,
+                                 sga_select_result* result, uint32_t* hist,
+                                 void* ws, size_t ws_bytes, void* stream);
+
 /* pass 3 (replay_fused.py:1836-1889): commit + residual for all G
  * configurations in one sweep (the gradient is read once).  coef_f: device
  * float[G] from pass 1.  segs: DEVICE array.  cfgs: HOST array. */

@@ -77,7 +77,7 @@ class Config:
 
 def group_replay(entries, w0, m0, v0, sel0, configs, g_steps, metas, t0,
                  horizons=(), snapshots=None, norm_chunk=None, coef_hook=None,
-                 trace=None):
+                 trace=None, selection_semantics="topk"):
     """Fused-replay group loop on one shard (replay_fused.py:1536-1914).
 
     entries : list of dicts {"a": flat offset, "n": numel, "b1","b2","eps",
@@ -89,6 +89,8 @@ def group_replay(entries, w0, m0, v0, sel0, configs, g_steps, metas, t0,
     coef_hook(si, ci, coef) -> coef lets a test substitute the clip
     coefficient (e.g. the device's bits) so everything downstream is compared
     on identical inputs; trace (a list) receives (si, ci, qn2, coef).
+    selection_semantics: what a boundary re-selects with ("topk" |
+    "balanced-histogram", replay_fused.py:1340-1344, 1805-1812).
     Returns per-config dict with final w, m, v, res, sel and the per-horizon
     distances ``||w - snapshot||``.
     """
@@ -148,7 +150,14 @@ def group_replay(entries, w0, m0, v0, sel0, configs, g_steps, metas, t0,
                                           s["v"][a:b], q, blind, e["b1"],
                                           e["b2"], e["eps"], e["wd"], bc1c,
                                           bc2c, c.optimizer).float()
-            newsel, _ = SEL.select_topk_flat(score, ks[c.ratio])
+            if selection_semantics == "balanced-histogram":
+                newsel, _ = SEL.shard_select_balanced(score, ks[c.ratio],
+                                                      entries)
+            elif selection_semantics == "topk":
+                newsel, _ = SEL.select_topk_flat(score, ks[c.ratio])
+            else:
+                raise ValueError(f"unknown selection semantics "
+                                 f"{selection_semantics!r}")
             if c.dual_lr != 1.0:
                 out_sel[ci] = s["sel"]
             s["sel"] = newsel

@@ -75,6 +75,9 @@ SIGNATURES = {
     "sga_replay_pass1": (I32, [P, I32, I64, F, C.c_double, P, I32, P, P, P, P, P]),
     "sga_replay_reselect": (I32, [P, I32, P, P, P, P, I64, I64, P, I32, I32, P, F, I32, I32, I32,
                                   P, P, P, SZ, P]),
+    "sga_balanced_hist_words": (I64, []),
+    "sga_replay_reselect_balanced": (I32, [P, I32, P, P, P, P, I64, I64, P, I32, P, I32, P, F, I32,
+                                           I32, I32, P, P, P, P, SZ, P]),
     "sga_replay_pass3": (I32, [P, I32, I64, F, P, I32, P, P, I32, P]),
     "sga_branch_score_f64": (I32, [I32, P, P, P, P, P, I64] + [C.c_double] * 6 + [I32, I32, P]),
     "sga_dense_replay_step": (I32, [P, I32, P, P, P, P, I64, P, I32, I32, C.c_double, P, P, P]),

@@ -739,6 +739,235 @@ extern "C" int sga_replay_reselect(const void* g, int g_dtype, const float* res,
 #undef SGA_RS
 }
 
+// ------------------------------------------- balanced-histogram re-selection
+// The online engine's approximate tier at a replay boundary (replay_fused.py:405-489,
+// _histogram.py:115-123, 203-216): histogram of the keys' top 16 bits over a stride-8
+// subsample taken on every tensor's own grid (element j of a tensor is sampled when
+// j = phase (mod 8), phase = (-p_off) mod 8), crossing bin b = first bin whose running
+// count reaches the rank r, selection = every coordinate whose top 16 bits are >= b.
+// Two sweeps form the score on the fly; it is never materialised.
+namespace sga {
+
+constexpr int kBalBins = 32768;            // (31-bit key) >> 16
+constexpr int kBalShift = 16;
+constexpr int kBalStride = 8;
+constexpr int kBalWide = 1024;             // 16 waves share one 128 KiB LDS table
+constexpr int kBalState = 64;              // words behind the bins: [0] b, [1] selected, [2] non-finite
+
+// Walks one chunk through a key source's stepwise interface (loads of kAhead slabs in flight
+// before the first key is formed) and hands every slab's keys to f(it, i, key).
+template <class Src, bool FULL, class F>
+__device__ __forceinline__ void chunk_keys(Src& src, int64_t n, int64_t c, F&& f) {
+  constexpr int kAhead = FULL ? Src::kAhead : 1;
+  src.chunk_hyper(c);
+  const typename Src::Chunk ck = src.chunk_begin(c);
+#pragma unroll 1
+  for (int g0 = 0; g0 < kChunkIters; g0 += kAhead) {
+    typename Src::Raw raw[kAhead];
+#pragma unroll
+    for (int u = 0; u < kAhead; ++u) {
+      const int64_t i = c * kChunk + (g0 + u) * (kWave * kVec) + lane_id() * kVec;
+      if (FULL || i < n) src.template fetch<FULL>(ck, i, n, raw[u]);
+    }
+#pragma unroll
+    for (int u = 0; u < kAhead; ++u) {
+      const int64_t i = c * kChunk + (g0 + u) * (kWave * kVec) + lane_id() * kVec;
+      uint32_t key[4] = {0u, 0u, 0u, 0u};
+      if (FULL || i < n) src.template keys<FULL>(ck, i, n, raw[u], key);
+      f(g0 + u, i, key);
+    }
+  }
+}
+
+static __global__ __launch_bounds__(kBlock) void k_bal_zero(uint32_t* __restrict__ hist) {
+  for (int i = blockIdx.x * kBlock + threadIdx.x; i < kBalBins + kBalState; i += gridDim.x * kBlock)
+    hist[i] = 0u;
+}
+
+template <class Src>
+__global__ __launch_bounds__(kBalWide) void k_bal_hist(Src src, int64_t n,
+                                                       const sga_segment* __restrict__ segs,
+                                                       int n_segs, const int32_t* __restrict__ seg_dir,
+                                                       const int32_t* __restrict__ seg_phase,
+                                                       uint32_t* __restrict__ hist) {
+  extern __shared__ uint32_t s_bal[];
+  for (int b = threadIdx.x; b < kBalBins; b += kBalWide) s_bal[b] = 0u;
+  __syncthreads();
+  SegCursor pc;                              // per lane: which tensor a coordinate lies in
+  pc.init(segs, n_segs, seg_dir);
+  int64_t lo = 1, hi = 0;
+  int ph = 0;
+  const int64_t n_chunks = cdiv64(n, kChunk);
+  const int64_t wstride = (int64_t)gridDim.x * (kBalWide / kWave);
+  for (int64_t c = (int64_t)blockIdx.x * (kBalWide / kWave) + wave_id(); c < n_chunks; c += wstride) {
+    auto slab = [&](int, int64_t i, const uint32_t key[4]) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int64_t idx = i + e;
+        const bool valid = idx < n;
+        if (valid && (idx < lo || idx >= hi)) {
+          const int a = pc.find(idx);
+          lo = segs[a].start;
+          hi = lo + segs[a].n;
+          ph = seg_phase ? seg_phase[a] : 0;
+        }
+        const bool sampled = valid && idx >= lo && idx < hi &&
+                             (((idx - lo - (int64_t)ph) & (kBalStride - 1)) == 0);
+        lds_hist_add(s_bal, key[e] >> kBalShift, sampled);
+      }
+    };
+    if (src.vec && (c + 1) * kChunk <= n) chunk_keys<Src, true>(src, n, c, slab);
+    else chunk_keys<Src, false>(src, n, c, slab);
+  }
+  __syncthreads();
+  for (int b = threadIdx.x; b < kBalBins; b += kBalWide) {
+    const uint32_t cnt = s_bal[b];
+    if (cnt) atomicAdd(&hist[b], cnt);
+  }
+}
+
+// b = number of bins whose inclusive running count stays below the rank
+// (torch.searchsorted(cumsum(hist), r), left): one workgroup, 32 bins per lane.
+static __global__ __launch_bounds__(kBalWide) void k_bal_bin(uint32_t* __restrict__ hist, uint64_t rank) {
+  __shared__ uint64_t s_sum[kBalWide];
+  __shared__ uint32_t s_below[kBalWide];
+  constexpr int PER = kBalBins / kBalWide;
+  uint32_t loc[PER];
+  uint64_t mine = 0;
+#pragma unroll
+  for (int j = 0; j < PER; ++j) { loc[j] = hist[threadIdx.x * PER + j]; mine += loc[j]; }
+  s_sum[threadIdx.x] = mine;
+  __syncthreads();
+  for (int o = 1; o < kBalWide; o <<= 1) {                 // inclusive scan over the lanes
+    const uint64_t add = (int)threadIdx.x >= o ? s_sum[threadIdx.x - o] : 0ull;
+    __syncthreads();
+    s_sum[threadIdx.x] += add;
+    __syncthreads();
+  }
+  uint64_t run = s_sum[threadIdx.x] - mine;
+  uint32_t below = 0;
+#pragma unroll
+  for (int j = 0; j < PER; ++j) { run += loc[j]; below += run < rank; }
+  s_below[threadIdx.x] = below;
+  __syncthreads();
+  for (int o = kBalWide / 2; o > 0; o >>= 1) {
+    if ((int)threadIdx.x < o) s_below[threadIdx.x] += s_below[threadIdx.x + o];
+    __syncthreads();
+  }
+  // a rank beyond the sample's size: every bin stays below it, and searchsorted on the
+  // reference's table of 32769 bins (the last one is never hit by a 31-bit key) returns 32769
+  if (threadIdx.x == 0) hist[kBalBins] = s_below[0] < (uint32_t)kBalBins ? s_below[0] : kBalBins + 1u;
+}
+
+template <class Src>
+__global__ __launch_bounds__(kBlock) void k_bal_planes(Src src, int64_t n, uint32_t* __restrict__ hist,
+                                                       uint32_t* __restrict__ planes) {
+  __shared__ uint32_t s_planes[kChunksPerBlock][kPlaneWordsPerChunk];
+  const uint32_t b = hist[kBalBins];
+  const int64_t n_chunks = cdiv64(n, kChunk);
+  const int64_t c = (int64_t)blockIdx.x * kChunksPerBlock + wave_id();
+  if (c >= n_chunks) return;
+  uint32_t n_sel = 0, n_nf = 0;
+  uint32_t* const lp = s_planes[wave_id()];
+  auto slab = [&](int it, int64_t i, const uint32_t key[4]) {
+    Ballot4 on;
+    uint64_t nf = 0;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const uint64_t valid = ballot64(i + e < n);
+      on.m[e] = ballot64((key[e] >> kBalShift) >= b) & valid;
+      nf |= ballot64(key[e] >= 0x7F800000u) & valid;
+    }
+    n_sel += on.count();
+    if (nf) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) n_nf += (uint32_t)__popcll(ballot64(key[e] >= 0x7F800000u && i + e < n));
+    }
+    plane_put(on, it, lp);
+  };
+  if (src.vec && (c + 1) * kChunk <= n) chunk_keys<Src, true>(src, n, c, slab);
+  else chunk_keys<Src, false>(src, n, c, slab);
+  __builtin_amdgcn_wave_barrier();
+  if (lane_id() < kPlaneWordsPerChunk) planes[c * kPlaneWordsPerChunk + lane_id()] = lp[lane_id()];
+  if (lane_id() == 0) {
+    if (n_sel) atomicAdd(&hist[kBalBins + 1], n_sel);
+    if (n_nf) atomicAdd(&hist[kBalBins + 2], n_nf);
+  }
+}
+
+static __global__ void k_bal_result(const uint32_t* __restrict__ hist, sga_select_result* __restrict__ out) {
+  const uint32_t b = hist[kBalBins];
+  out->thresh_bits = (b << kBalShift) & 0x7FFFFFFFu;      // the bin's lower edge (_bin_edge_float)
+  out->need = 0u;
+  out->n_gt = hist[kBalBins + 1];
+  out->n_eq = 0u;
+  out->n_selected = hist[kBalBins + 1];
+  out->nonfinite = hist[kBalBins + 2];
+  out->status = 0u;
+  out->path = 3u;
+}
+
+template <bool BF16G, int SCORE>
+static int run_reselect_balanced(const void* g, const float* res, const float* w, const float* m,
+                                 const float* v, int64_t n, uint64_t rank, const sga_segment* segs,
+                                 int n_segs, const int32_t* seg_phase, const float* coef_f,
+                                 float coef_dense, int adams, int packed, int res_zero,
+                                 uint32_t* sel_out, sga_select_result* result, uint32_t* hist,
+                                 const SelWorkspace& ws, hipStream_t s) {
+  const bool vec = aligned4(g, BF16G ? 2 : 4) && aligned4(res, 4) && aligned4(w, 4) &&
+                   aligned4(m, 4) && aligned4(v, 4);
+  SrcReplay<BF16G, SCORE> src{g, res, w, m, v, coef_f, coef_dense, adams, vec, {},
+                              packed ? kPackExtra : 0, res_zero};
+  launch_seg_dir(segs, n_segs, n, ws.seg_dir, s);
+  src.sc.init(segs, n_segs, ws.seg_dir);
+  const int64_t n_chunks = cdiv64(n, kChunk);
+  hipLaunchKernelGGL(k_bal_zero, dim3(32), dim3(kBlock), 0, s, hist);
+  hipLaunchKernelGGL((k_bal_hist<SrcReplay<BF16G, SCORE>>),
+                     dim3(stream_grid(n_chunks, kBalWide / kWave, 256)), dim3(kBalWide),
+                     (size_t)kBalBins * 4, s, src, n, segs, n_segs, ws.seg_dir, seg_phase, hist);
+  hipLaunchKernelGGL(k_bal_bin, dim3(1), dim3(kBalWide), 0, s, hist, rank);
+  hipLaunchKernelGGL((k_bal_planes<SrcReplay<BF16G, SCORE>>), dim3((unsigned)cdiv64(n_chunks, kChunksPerBlock)),
+                     dim3(kBlock), 0, s, src, n, hist, sel_out);
+  if (result) hipLaunchKernelGGL(k_bal_result, dim3(1), dim3(1), 0, s, hist, result);
+  return check_launch("sga_replay_reselect_balanced");
+}
+
+}  // namespace sga
+
+extern "C" int64_t sga_balanced_hist_words(void) { return kBalBins + kBalState; }
+
+extern "C" int sga_replay_reselect_balanced(const void* g, int g_dtype, const float* res,
+                                            const float* w, const float* m, const float* v,
+                                            int64_t n, int64_t rank, const sga_segment* segs,
+                                            int n_segs, const int32_t* seg_phase, int score_id,
+                                            const float* coef_f, float coef_dense, int adams,
+                                            int packed, int res_zero, uint32_t* sel_out,
+                                            sga_select_result* result, uint32_t* hist, void* ws,
+                                            size_t ws_bytes, void* stream) {
+  if (!g || !res || !w || !m || !v || !segs || !coef_f || !sel_out || !hist || n < 1 ||
+      n >= (1ll << 31) || rank < 1 || n_segs < 1 || score_id < 0 ||
+      score_id > SGA_SCORE_GR_OVER_SQRT_V || (g_dtype != SGA_F32 && g_dtype != SGA_BF16)) {
+    set_error("sga_replay_reselect_balanced: bad argument (n=%lld rank=%lld)", (long long)n,
+              (long long)rank);
+    return SGA_ERR_ARG;
+  }
+  SelWorkspace sw;
+  if (!sel_ws_carve(ws, ws_bytes, cdiv64(n, kChunk), &sw)) {
+    set_error("sga_replay_reselect_balanced: workspace too small (sga_select_workspace_bytes(n))");
+    return SGA_ERR_WORKSPACE;
+  }
+  hipStream_t s = (hipStream_t)stream;
+#define SGA_RB(BG, SC) return run_reselect_balanced<BG, SC>(g, res, w, m, v, n, (uint64_t)rank, segs, n_segs, seg_phase, coef_f, coef_dense, adams, packed, res_zero, sel_out, result, hist, sw, s)
+  if (g_dtype == SGA_BF16) {
+    switch (score_id) { case 0: SGA_RB(true, 0); case 1: SGA_RB(true, 1); case 2: SGA_RB(true, 2);
+                        case 3: SGA_RB(true, 3); case 4: SGA_RB(true, 4); default: SGA_RB(true, 5); }
+  } else {
+    switch (score_id) { case 0: SGA_RB(false, 0); case 1: SGA_RB(false, 1); case 2: SGA_RB(false, 2);
+                        case 3: SGA_RB(false, 3); case 4: SGA_RB(false, 4); default: SGA_RB(false, 5); }
+  }
+#undef SGA_RB
+}
+
 extern "C" int sga_dense_replay_step(const void* g, int g_dtype, float* w, float* m, float* v,
                                      float* lab, int64_t n, const sga_replay_segment* segs,
                                      int n_segs, int adams, double coef_dense, double* partials,

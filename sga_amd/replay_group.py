@@ -15,6 +15,10 @@ from .scores import STEP_SCORE_MAP as SCORE_MAP
 from .selection import read_result
 
 MAX_CONFIGS = 16
+# what a boundary re-selects with (replay_fused.py:1340-1344): the exact top-k with the tie
+# layer filled in index order, or the online engine's balanced-histogram tier
+SELECTION_SEMANTICS = ("topk", "balanced-histogram")
+_BAL_STRIDE = 8
 
 
 class ReplayCfg(C.Structure):
@@ -106,9 +110,14 @@ class ReplayGroup:
     was given the snapshots.
     """
 
-    def __init__(self, entries, w0, m0, v0, sel0, configs, t0, window):
+    def __init__(self, entries, w0, m0, v0, sel0, configs, t0, window,
+                 selection_semantics="topk"):
         if not (1 <= len(configs) <= MAX_CONFIGS):
             raise ValueError(f"1..{MAX_CONFIGS} configs per group")
+        if selection_semantics not in SELECTION_SEMANTICS:
+            raise ValueError(f"unknown selection semantics {selection_semantics!r} "
+                             f"(expected one of {SELECTION_SEMANTICS})")
+        self.semantics = selection_semantics
         L.require_dev(w0, m0, v0, *sel0)
         self.N = w0.numel()
         off = 0
@@ -132,6 +141,14 @@ class ReplayGroup:
         self.ws_bytes = int(L.raw("sga_select_workspace_bytes", self.N))
         self.ws = torch.empty(self.ws_bytes, dtype=torch.uint8, device=dev)
         self.sel_result = torch.zeros(8, dtype=torch.int32, device=dev)
+        if selection_semantics == "balanced-histogram":
+            # every tensor is subsampled on its own param-relative stride-8 grid
+            phases = [(-int(e.get("p_off", 0))) % _BAL_STRIDE for e in entries]
+            self._n_sampled = sum(len(range(ph, e["n"], _BAL_STRIDE))
+                                  for ph, e in zip(phases, entries))
+            self._seg_phase = torch.tensor(phases, dtype=torch.int32, device=dev)
+            self._bal_hist = torch.zeros(int(L.raw("sga_balanced_hist_words")),
+                                         dtype=torch.int32, device=dev)
         self._cfg_host = (ReplayCfg * G)()
         self._rseg_host = (ReplaySegment * len(entries))()
         self._rseg_up = L.TableUploader(C.sizeof(self._rseg_host), dev)
@@ -204,14 +221,21 @@ class ReplayGroup:
             if not (bnd[ci] and si > 0 and si + 1 < self.W):
                 continue
             s = self.state[ci]
-            L.call("sga_replay_reselect", L.ptr(g), gd, C.c_void_p(s.base("res")),
-                   C.c_void_p(s.base("w")), C.c_void_p(s.base("m")), C.c_void_p(s.base("v")), N,
-                   self.ks[c.ratio],
-                   L.ptr(self._seg_dev), len(self.entries), SCORE_MAP[c.score],
-                   C.c_void_p(self.coef_f.data_ptr() + 4 * ci), L.f32(coef_dense),
-                   int(c.optimizer == "adams"), 1, int(self.res_zero[ci]), L.ptr(s.spare),
-                   L.ptr(self.sel_result),
-                   L.ptr(self.ws), self.ws_bytes, st)
+            state_ptrs = [C.c_void_p(s.base(x)) for x in ("res", "w", "m", "v")]
+            tail = [C.c_void_p(self.coef_f.data_ptr() + 4 * ci), L.f32(coef_dense),
+                    int(c.optimizer == "adams"), 1, int(self.res_zero[ci]), L.ptr(s.spare),
+                    L.ptr(self.sel_result)]
+            if self.semantics == "balanced-histogram":
+                k = self.ks[c.ratio]
+                rank = max(1, round(self._n_sampled * (N - k + 1) / N))   # _histogram.py:122
+                L.call("sga_replay_reselect_balanced", L.ptr(g), gd, *state_ptrs, N, rank,
+                       L.ptr(self._seg_dev), len(self.entries), L.ptr(self._seg_phase),
+                       SCORE_MAP[c.score], *tail, L.ptr(self._bal_hist), L.ptr(self.ws),
+                       self.ws_bytes, st)
+            else:
+                L.call("sga_replay_reselect", L.ptr(g), gd, *state_ptrs, N, self.ks[c.ratio],
+                       L.ptr(self._seg_dev), len(self.entries), SCORE_MAP[c.score], *tail,
+                       L.ptr(self.ws), self.ws_bytes, st)
             if c.dual_lr != 1.0:
                 out_sel[ci] = s.sel
             s.sel, s.spare = s.spare, s.sel

@@ -9,7 +9,7 @@ from . import _lib as L
 from .replay import _bc_pair, select_topk_flat
 from .replay_dense import dense_replay_dev
 from .replay_fused import shard_select_balanced
-from .replay_group import Config, ReplayGroup
+from .replay_group import SELECTION_SEMANTICS, Config, ReplayGroup
 from .scores import SCORE_MAP
 from .trace_io import (ResidentWindow, ShardParams, TraceFile, WindowReader, discover_trace,
                        load_branch_state, lr_for_step, window_steps_for)
@@ -77,7 +77,9 @@ def _branch_grad(state_path, sp, device):
 def replay_window(trace_dir, t0, window, configs, horizons, device,
                   selection_semantics="topk", depth=2):
     """Replays ``configs`` (``replay_group.Config``) over the recorded window
-    that starts at branch point ``t0``.
+    that starts at branch point ``t0``.  ``selection_semantics`` applies to
+    BOTH select sites, the branch-point select and every boundary
+    re-selection of the streaming pass (``replay_fused.py:1340-1344``).
 
     Returns a dict with the dense reference (``den_at``, ``label_total``,
     ``recon_steps``), and per config the distances ``||w_s(H) - w_d(H)||`` and
@@ -85,6 +87,9 @@ def replay_window(trace_dir, t0, window, configs, horizons, device,
     ``ReplayGroup`` for inspection.
     """
     replay_switches()
+    if selection_semantics not in SELECTION_SEMANTICS:
+        raise ValueError(f"unknown selection semantics {selection_semantics!r} "
+                         f"(expected one of {SELECTION_SEMANTICS})")
     catalog, names, _offs, N, state_files, g_files = discover_trace(trace_dir)
     if t0 not in state_files:
         raise ValueError(f"branch point {t0} has no step_{t0:06d}_state.pt in {trace_dir}")
@@ -127,7 +132,8 @@ def replay_window(trace_dir, t0, window, configs, horizons, device,
     results = [None] * len(configs)
     for opt, idxs in by_opt.items():
         group = ReplayGroup(sp.entries, w0, m0, v0, [sel0[i] for i in idxs],
-                            [configs[i] for i in idxs], t0, W)
+                            [configs[i] for i in idxs], t0, W,
+                            selection_semantics=selection_semantics)
         for _gstep, gmeta, g in window:
             meta = {"clip_grad": gmeta.get("clip_grad", 0.0),
                     "grad_norm": gmeta.get("grad_norm", float("nan")),

@@ -124,9 +124,13 @@ def _fixture(n_sizes, W, seed=2026, bf16=False, vary=False):
     return n, w0, m0, v0, grads, entries
 
 
-def _run_group(dev, cfg_specs, clip, W=9, bf16=False, t0=10, sizes=(400_000, 300_000, 170_000)):
+def _run_group(dev, cfg_specs, clip, W=9, bf16=False, t0=10, sizes=(400_000, 300_000, 170_000),
+               semantics="topk", p_offs=None):
     from sga_amd.replay_group import Config, ReplayGroup
     n, w0, m0, v0, grads, entries = _fixture(list(sizes), W, bf16=bf16)
+    if p_offs is not None:
+        for e, po in zip(entries, p_offs):
+            e["p_off"] = po
     lr = 5e-5
     norms = [float(g.float().norm()) * 1.3 for g in grads]
     metas = [{"clip_grad": clip, "grad_norm": norms[i], "lr": lr} for i in range(W)]
@@ -137,9 +141,12 @@ def _run_group(dev, cfg_specs, clip, W=9, bf16=False, t0=10, sizes=(400_000, 300
         g0 = grads[0].float()
         sc = OS.step_score(c.score, w0, m0, v0, g0, g0, 0.9, 0.95, 1e-8, 0.1,
                            *OR.bc_pair(c.optimizer, t0 + 1, 0.9, 0.95), c.optimizer)
-        sel0.append(SEL.select_topk_flat(sc, SEL.replay_k(n, c.ratio))[0])
+        if semantics == "topk":
+            sel0.append(SEL.select_topk_flat(sc, SEL.replay_k(n, c.ratio))[0])
+        else:
+            sel0.append(SEL.shard_select_balanced(sc, SEL.replay_k(n, c.ratio), entries)[0])
     grp = ReplayGroup(entries, w0.to(dev), m0.to(dev), v0.to(dev), [s.to(dev) for s in sel0],
-                      dcfg, t0, W)
+                      dcfg, t0, W, selection_semantics=semantics)
     dev_coefs, dev_qn2 = {}, {}
     for si in range(W):
         grp.step(grads[si].to(dev), metas[si])
@@ -148,7 +155,8 @@ def _run_group(dev, cfg_specs, clip, W=9, bf16=False, t0=10, sizes=(400_000, 300
             dev_coefs[(si, ci)], dev_qn2[(si, ci)] = cf[ci], q2[ci]
     trace = []
     out = OR.group_replay(entries, w0, m0, v0, sel0, ocfg, grads, metas, t0,
-                          coef_hook=lambda si, ci, c: dev_coefs[(si, ci)], trace=trace)
+                          coef_hook=lambda si, ci, c: dev_coefs[(si, ci)], trace=trace,
+                          selection_semantics=semantics)
     for si, ci, qn2, coef in trace:             # clip norms: 1e-6 reordering band
         assert abs(dev_qn2[(si, ci)] - qn2) <= 1e-6 * max(qn2, 1e-30), (si, ci)
         assert abs(dev_coefs[(si, ci)] - coef) <= 1e-6 * coef, (si, ci)
@@ -264,6 +272,63 @@ def test_group_adam_scores_one_sweep_long_cycle(dev, opt):
     grp, out, w0 = _run_group(dev, specs, clip=0.3, W=18, bf16=False, sizes=_RAGGED)
     assert grp.last_select().path == 1
     _assert_group_equal(grp, out, specs)
+
+
+@pytest.mark.parametrize("sizes,p_offs", [((400_000, 300_000, 170_000), None),
+                                          (tuple(_RAGGED), [3, 0, 13, 8005, 1, 0, 6, 2, 7])])
+def test_group_step_balanced_histogram_semantics(dev, sizes, p_offs):
+    """The group step under the `balanced-histogram` selection semantics
+    (replay_fused.py:1340-1344, 1805-1809): every boundary re-selects with the
+    online engine's approximate tier -- stride-8 subsample on each tensor's
+    own grid (non-zero param-relative phases in the ragged case), integer
+    crossing bin, the whole bin selected -- on scores formed on the fly.  All
+    registry scores, AdamS, fold and dual-lr arms, a live residual, clipping;
+    masks and state bit for bit against the oracle's loop under the same
+    semantics, and the masks differ from the exact top-k's."""
+    specs = [("abs_g", 1.0, 2), ("update", 10.0, 4), ("coi", 1.0, 3, "adams"),
+             ("abs_m", 1.0, 2), ("update", 0.1, 2, "adamw", True, 0.25),
+             ("abs_g_blind", 1.0, 4), ("abs_g", 10.0, 3, "adams", True)]
+    grp, out, w0 = _run_group(dev, specs, clip=0.3, W=9, bf16=True, sizes=sizes,
+                              semantics="balanced-histogram", p_offs=p_offs)
+    _assert_group_equal(grp, out, specs)
+    res = grp.last_select()
+    assert res.path == 3 and res.status == 0 and res.nonfinite == 0
+    assert res.thresh_bits & 0xFFFF == 0                       # a bin's lower edge
+    n = sum(sizes)
+    for ci, c in enumerate(specs):
+        cnt = int(out[ci]["sel"].sum())
+        assert abs(cnt - SEL.replay_k(n, c[1])) < 0.005 * n + 64, (ci, cnt)
+    assert int(out[0]["sel"].sum()) != SEL.replay_k(n, 1.0)     # approximate by construction
+
+
+def test_shard_select_balanced_twin_with_param_phases(dev):
+    """`sga_amd.replay_fused.shard_select_balanced` (one histogram call per
+    entry, param-relative phase) against the oracle's twin on the geometry
+    fixture of tests/test_selection_semantics_switch.py:176-186 with shard
+    slices that start inside their parameters (p_off != 0)."""
+    from sga_amd.replay_fused import shard_select_balanced
+    sizes, p_offs = [40001, 7, 65536, 100009], [3, 13, 0, 8005]
+    gen = torch.Generator().manual_seed(7)
+    score = torch.rand(sum(sizes), generator=gen) ** 4
+    ent, off = [], 0
+    for sz, po in zip(sizes, p_offs):
+        ent.append({"a": off, "n": sz, "p_off": po})
+        off += sz
+    score[ent[2]["a"]:ent[2]["a"] + sizes[2]] = 0.25
+    n = score.numel()
+    for k in (1, n // 100, 3 * n // 10, n - 1, n):
+        ref_mask, ref_th = SEL.shard_select_balanced(score, k, ent)
+        mask, th = shard_select_balanced(score.to(dev), k, None, ent)
+        assert th == ref_th and torch.equal(mask.cpu(), ref_mask), k
+    # whole views (no p_off key) are phase 0
+    plain = [{"a": e["a"], "n": e["n"]} for e in ent]
+    ref_mask, ref_th = SEL.shard_select_balanced(score, n // 100, plain)
+    mask, th = shard_select_balanced(score.to(dev), n // 100, None, plain)
+    assert th == ref_th and torch.equal(mask.cpu(), ref_mask)
+    bad = score.clone()
+    bad[5] = float("inf")
+    with pytest.raises(ValueError, match="finite"):
+        shard_select_balanced(bad.to(dev), 10, None, ent)
 
 
 def test_group_benchmark_scores_outside_the_registry(dev):

@@ -91,15 +91,21 @@ def test_dense_pass_matches_oracle(dev, tmp_path, g_dtype, opt):
             assert a["grad_norm"] == mt["grad_norm"]
 
 
-@pytest.mark.parametrize("clip,g_dtype", [(0.0, torch.bfloat16), (0.3, None)])
-def test_replay_window_end_to_end(dev, tmp_path, clip, g_dtype):
+@pytest.mark.parametrize("clip,g_dtype,semantics", [(0.0, torch.bfloat16, "topk"),
+                                                    (0.3, None, "topk"),
+                                                    (0.0, torch.bfloat16, "balanced-histogram")])
+def test_replay_window_end_to_end(dev, tmp_path, clip, g_dtype, semantics):
+    """One selection semantics at BOTH select sites (the branch-point select
+    and every boundary re-selection, replay_fused.py:1340-1344), against the
+    oracle's loop under the same semantics."""
     from sga_amd.replay_run import Config, replay_window
     d = str(tmp_path)
     W, t0 = 9, 10
     make_trace(d, steps=W, g_dtype=g_dtype, clip=clip, absent=(2, 3))
     specs = [("abs_g", 1.0, 1), ("abs_g", 10.0, 4), ("abs_m", 1.0, 3),
              ("abs_g", 1.0, 4, "adams", True), ("abs_g", 5.0, 4, "adamw", False, 0.25)]
-    res = replay_window(d, t0, W, [Config(*s) for s in specs], (1, 4, 9, 99), dev)
+    res = replay_window(d, t0, W, [Config(*s) for s in specs], (1, 4, 9, 99), dev,
+                        selection_semantics=semantics)
     assert res["window_steps"] == list(range(t0, t0 + W)) and res["horizons"] == [1, 4, 9]
     entries, n, w0, m0, v0, g0, gs, metas, meta = _oracle_inputs(d, t0, W)
     ocfg = [OR.Config(*s) for s in specs]
@@ -107,11 +113,15 @@ def test_replay_window_end_to_end(dev, tmp_path, clip, g_dtype):
              for o in ("adamw", "adams")}
     for ci, c in enumerate(ocfg):
         sc = OT.branch_scores(c.score, c.optimizer, entries, w0, m0, v0, g0, meta["step"] + 1)
-        sel0, _ = SEL.select_topk_flat(sc, SEL.replay_k(n, c.ratio))
+        if semantics == "topk":
+            sel0, _ = SEL.select_topk_flat(sc, SEL.replay_k(n, c.ratio))
+        else:
+            sel0, _ = SEL.shard_select_balanced(sc, SEL.replay_k(n, c.ratio), entries)
         ometas = [{"clip_grad": m["clip_grad"], "grad_norm": m["grad_norm"],
                    "lr": m["lr"]} for m in metas]
         o = OR.group_replay(entries, w0, m0, v0, [sel0], [c], gs, ometas, t0,
-                            horizons=(1, 4, 9), snapshots=dense[c.optimizer][4])[0]
+                            horizons=(1, 4, 9), snapshots=dense[c.optimizer][4],
+                            selection_semantics=semantics)[0]
         r = res["configs"][ci]
         s = r["group"].state[r["slot"]]
         den = dense[c.optimizer][2]

@@ -235,41 +235,86 @@ def test_coef_dense():
     assert R.coef_dense_for(0.3, 2.0) == 0.3 / (2.0 + 1e-6)
 
 
+def _spec_balanced(score, k, sizes):
+    """Balanced-histogram select from its wording (_histogram.py:115-123,
+    203-216; replay_fused.py:405-489 with p_off = 0): the sample is every
+    eighth element of each tensor counted from the tensor's own start, r the
+    rounded rank of the k-th largest inside the sample, the crossing bin the
+    r-th smallest sampled top-16 pattern, and every coordinate whose top 16
+    bits reach that bin is selected."""
+    top = score.float().abs().view(torch.int32) >> 16
+    sample, off = [], 0
+    for sz in sizes:
+        sample += top[off:off + sz][::8].tolist()
+        off += sz
+    sample.sort()
+    n = score.numel()
+    r = max(1, round(len(sample) * (n - k + 1) / n))
+    return top >= sample[r - 1]
+
+
 def _spec_cycle(w0, m0, v0, grads, norms, lr, clip, t0, k, T, b1, b2, eps, wd,
-                fold=False):
-    """From-spec float64-free double loop (shape of
-    tests/test_replay_cycle.py:141-223), abs_g score, adamw."""
-    def adam(w, m, v, q, count):
-        m = b1 * m + (1 - b1) * q
-        v = b2 * v + (1 - b2) * q * q
-        upd = (m / (1 - b1 ** count)) / (torch.sqrt(v / (1 - b2 ** count)) + eps)
-        return w * (1 - lr * wd) - lr * upd, m, v
+                fold=False, optimizer="adamw", dual_lr=1.0, semantics="topk", sizes=None):
+    """From-spec loop (shape of tests/test_replay_cycle.py:141-223), abs_g
+    score, written out of place from the formulas: AdamW, or AdamS (the second
+    moment rebuilt from the PRE-commit m, no bias corrections: replay.py:708-729);
+    at a boundary with dual_lr != 1 the whole displacement wd*w + upd is applied
+    at lr on the coordinates of the OUTGOING mask and at lr*dual_lr elsewhere
+    (replay_fused.py:1817-1824, 1866-1877; replay.py:674-684)."""
+    def select(score):
+        if semantics == "topk":
+            return SEL.select_topk_flat(score, k)[0]
+        return _spec_balanced(score, k, sizes)
+
+    def commit(w, m, v, q, count, lr_vec):
+        if optimizer == "adams":
+            v = b2 * (m * m) + (1 - b2) * q * q
+            m = b1 * m + (1 - b1) * q
+            upd = m / (torch.sqrt(v) + eps)
+        else:
+            m = b1 * m + (1 - b1) * q
+            v = b2 * v + (1 - b2) * q * q
+            upd = (m / (1 - b1 ** count)) / (torch.sqrt(v / (1 - b2 ** count)) + eps)
+        return w - lr_vec * (wd * w + upd), m, v
     ws, ms, vs = w0.clone(), m0.clone(), v0.clone()
     res = torch.zeros_like(w0)
-    sel = SEL.select_topk_flat(grads[0].abs(), k)[0]
+    sel = select(grads[0].abs())
     for si, gl in enumerate(grads):
         count = t0 + si + 1
         cd = min(1.0, clip / (norms[si] + 1e-6)) if clip > 0 else 1.0
         g = gl / cd
+        lr_vec = lr
         if si % T == 0:
             if fold and si > 0:
                 res = res / T
             qp = g + res
             coef = min(1.0, clip / (float(qp.norm()) + 1e-6)) if clip > 0 else 1.0
             q = qp * coef
+            outgoing = sel
             if si > 0 and si + 1 < len(grads):
-                sel = SEL.select_topk_flat(q.abs(), k)[0]
+                sel = select(q.abs())
+            if dual_lr != 1.0:
+                lr_vec = torch.where(outgoing, torch.tensor(lr), torch.tensor(lr * dual_lr))
             res = torch.zeros_like(res)
         else:
             coef = min(1.0, clip / (float((g * sel).norm()) + 1e-6)) if clip > 0 else 1.0
             q = g * sel * coef
             res = res + g * (~sel)
-        ws, ms, vs = adam(ws, ms, vs, q, count)
+        ws, ms, vs = commit(ws, ms, vs, q, count, lr_vec)
     return ws, sel, res
 
 
-@pytest.mark.parametrize("T,fold", [(1, False), (4, False), (4, True), (3, False)])
-def test_group_replay_vs_spec(T, fold):
+@pytest.mark.parametrize("T,fold,optimizer,dual_lr,semantics", [
+    (1, False, "adamw", 1.0, "topk"), (4, False, "adamw", 1.0, "topk"),
+    (4, True, "adamw", 1.0, "topk"), (3, False, "adamw", 1.0, "topk"),
+    (4, False, "adams", 1.0, "topk"), (3, True, "adams", 2.0, "topk"),
+    (4, False, "adamw", 0.25, "topk"), (2, False, "adamw", 0.0, "topk"),
+    (4, False, "adamw", 1.0, "balanced-histogram"),
+    (3, True, "adams", 0.25, "balanced-histogram")])
+def test_group_replay_vs_spec(T, fold, optimizer, dual_lr, semantics):
+    """The oracle's group loop against the from-spec loop on every arm of the
+    replay axis product: cycle length, fold, AdamS, the boundary dual-lr split
+    against the outgoing mask, and both selection semantics."""
     n, W, t0 = 5000, 9, 10
     b1, b2, eps, wd, lr, clip = 0.9, 0.95, 1e-8, 0.1, 5e-5, 0.3
     gen = torch.Generator().manual_seed(2026)
@@ -279,19 +324,31 @@ def test_group_replay_vs_spec(T, fold):
     grads = [torch.randn(n, generator=gen) * 1e-2 for _ in range(W)]
     norms = [float(g.norm()) for g in grads]
     k = SEL.replay_k(n, 10.0)
-    entries = [{"a": 0, "n": 3000, "b1": b1, "b2": b2, "eps": eps, "wd": wd},
-               {"a": 3000, "n": 2000, "b1": b1, "b2": b2, "eps": eps, "wd": wd}]
-    cfg = R.Config("abs_g", 10.0, T, fold=fold)
-    sel0 = SEL.select_topk_flat(grads[0].abs(), k)[0]
+    sizes = [3001, 1999]                    # the second tensor starts off the stride-8 grid
+    entries = [{"a": 0, "n": sizes[0], "b1": b1, "b2": b2, "eps": eps, "wd": wd},
+               {"a": sizes[0], "n": sizes[1], "b1": b1, "b2": b2, "eps": eps, "wd": wd}]
+    cfg = R.Config("abs_g", 10.0, T, optimizer=optimizer, fold=fold, dual_lr=dual_lr)
+    if semantics == "topk":
+        sel0 = SEL.select_topk_flat(grads[0].abs(), k)[0]
+    else:
+        sel0 = _spec_balanced(grads[0].abs(), k, sizes)
+        assert torch.equal(sel0, SEL.shard_select_balanced(grads[0].abs(), k, entries)[0])
+        assert abs(int(sel0.sum()) - k) < 0.02 * n and int(sel0.sum()) != k
     metas = [{"clip_grad": clip, "grad_norm": norms[i], "lr": lr} for i in range(W)]
-    out = R.group_replay(entries, w0, m0, v0, [sel0], [cfg], grads, metas, t0)[0]
+    out = R.group_replay(entries, w0, m0, v0, [sel0], [cfg], grads, metas, t0,
+                         selection_semantics=semantics)[0]
     ws, sel, res = _spec_cycle(w0, m0, v0, grads, norms, lr, clip, t0, k, T, b1, b2,
-                               eps, wd, fold)
+                               eps, wd, fold, optimizer, dual_lr, semantics, sizes)
     assert torch.equal(out["sel"], sel)
     torch.testing.assert_close(out["w"], ws, rtol=1e-5, atol=1e-7)
     torch.testing.assert_close(out["res"], res, rtol=1e-5, atol=1e-9)
     if T == 1:   # every step a boundary: residual never survives a step
         assert float(out["res"].abs().max()) == 0.0
+    if dual_lr == 0.0:
+        # scale 0 freezes the coordinates outside the outgoing mask at every boundary
+        # (tests/test_plugins_unit.py:992-1069): with T = 2 the one step that moves them is
+        # the masked step, where q = 0 there and only m's decay and weight decay act
+        assert not torch.equal(out["w"], w0)
 
 
 def test_fused_step_end_state_invariant():

@@ -142,6 +142,35 @@ def test_balanced_closed_form_and_edges():
     assert t2 == th and torch.equal(m2.to(torch.uint8), torch.cat(masks))
 
 
+def test_shard_select_balanced_param_relative_phase():
+    """The replay twin on shard slices that start inside a parameter
+    (``p_off`` != 0, replay_fused.py:420-432): the sample keeps the
+    parameter's own stride-8 grid, i.e. local element j is sampled when
+    ``(p_off + j) % 8 == 0``.  Brute force from that wording, on the geometry
+    fixture of tests/test_selection_semantics_switch.py:176-186 (sizes 40001,
+    7, 65536, 100009, a constant middle view)."""
+    sizes, p_offs = [40001, 7, 65536, 100009], [3, 13, 0, 8 * 1000 + 5]
+    gen = torch.Generator().manual_seed(7)
+    score = torch.rand(sum(sizes), generator=gen) ** 4
+    ent, off = [], 0
+    for sz, po in zip(sizes, p_offs):
+        ent.append({"a": off, "n": sz, "p_off": po})
+        off += sz
+    score[ent[2]["a"]:ent[2]["a"] + sizes[2]] = 0.25           # one constant view
+    n = score.numel()
+    top = SEL.abs_bit_top(score)
+    for k in (1, n // 100, 3 * n // 10, n - 1):
+        sample = []
+        for e in ent:
+            sample += [int(top[e["a"] + j]) for j in range(e["n"]) if (e["p_off"] + j) % 8 == 0]
+        sample.sort()
+        r = max(1, round(len(sample) * (n - k + 1) / n))
+        mask, th = SEL.shard_select_balanced(score, k, ent)
+        assert torch.equal(mask, top >= sample[r - 1]), k
+        bits = torch.tensor(th, dtype=torch.float32).view(torch.int32).item()
+        assert bits == sample[r - 1] << 16
+
+
 @pytest.mark.parametrize("kat", KATS["k_for"])
 def test_k_formulas(kat):
     assert SEL.k_for(kat["n"], kat["ratio"]) == kat["k"]
