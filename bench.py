@@ -406,14 +406,14 @@ def trace_io_bench(W=4, tmp=None):
         shutil.rmtree(d, ignore_errors=True)
 
 
-def qwen_mask_layout_row(steps=5, warmup=2, n_streams=3):
+def qwen_mask_layout_row(steps=5, warmup=2):
     """Qwen3-0.6B-shaped set, bf16 Gaussian grads with per-tensor std
     log-uniform in [1e-5, 1e-2], per-bucket exact top-k at 1 % (the embedding,
     then seven buckets of four layers), mask backend layout: the step's outputs
     are the uint8 mask and the ordered payload (what `torch_pipelined_mask`
     hands to the all-reduce), fp32 values."""
     import torch
-    from sga_amd.fused_step import FusedSparseStep, k_for
+    from sga_amd.fused_step import FusedSparseStep, fused_step_multi, k_for
     from sga_amd.shapes import qwen3_06b, segments_for
     dev = torch.device("cuda:0")
     segs, n = segments_for(qwen3_06b())
@@ -437,16 +437,16 @@ def qwen_mask_layout_row(steps=5, warmup=2, n_streams=3):
         buckets.append((lo, hi, k, FusedSparseStep(hi - lo, bsegs, dev, values_dtype=torch.float32,
                                                    max_k=k, want_mask=True)))
 
-    # Buckets are independent (disjoint slices, a workspace each): as in a trainer, where a bucket
-    # is stepped when its gradients are ready, they go out round-robin on a few streams (default
-    # priority), so the short kernels around one bucket's select run under another's sweeps.
-    streams = [torch.cuda.Stream(device=dev) for _ in range(n_streams)]
+    # The eight buckets go out as ONE call: the short dependent kernels around a select run once
+    # for all of them (the kernels take the bucket from the grid's second dimension), only the
+    # sweeps are launched per bucket.
+    steppers = [b[3] for b in buckets]
+    ks = [b[2] for b in buckets]
+    views = [[t[lo:hi] for lo, hi, _k, _fs in buckets] for t in (r, p, m, v)]
 
     def one(t):
         g = grads[t % 2]
-        for b, (lo, hi, k, fs) in enumerate(buckets):
-            with torch.cuda.stream(streams[b % n_streams]):
-                fs.step(g[lo:hi], r[lo:hi], p[lo:hi], m[lo:hi], v[lo:hi], t + 1, k=k)
+        fused_step_multi(steppers, [g[lo:hi] for lo, hi, _k, _fs in buckets], *views, t + 1, ks=ks)
 
     torch.cuda.synchronize()
     for t in range(warmup):
@@ -465,9 +465,9 @@ def qwen_mask_layout_row(steps=5, warmup=2, n_streams=3):
     return {"workload": "Qwen3-0.6B-shaped set (596,049,920 elems, 310 tensors), bf16 Gaussian grads "
                         "with per-tensor std log-uniform in [1e-5, 1e-2], per-bucket exact top-k 1 % "
                         f"over {len(buckets)} buckets, score abs_g, mask layout (u8 mask + ordered "
-                        f"fp32 payload), four flat state tensors, buckets round-robin on {n_streams} "
-                        "streams",
-            "n": n, "buckets": len(buckets), "streams": n_streams, "k_total": ktot,
+                        "fp32 payload), four flat state tensors, all buckets in one "
+                        "sga_fused_sparse_step_multi call",
+            "n": n, "buckets": len(buckets), "k_total": ktot,
             "ms_per_step": dt * 1e3,
             "elem_per_s": n / dt, "alg_bytes_per_step": alg,
             "step_frac": alg / dt / HBM_PEAK}

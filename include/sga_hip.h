@@ -362,6 +362,40 @@ int sga_fused_sparse_step(const void* g, int g_dtype, float* resid, float* p,
                           sga_select_result* result, void* ws,
                           size_t ws_bytes, void* stream);
 
+/* The same step for several buckets in one call -- the per-bucket online path,
+ * where every bucket of the optimizer selects its own top-k (engine.py:822-890;
+ * bucket layout torch_pipelined_mask.py:91-138, torch_pipelined_index.py:490-520).
+ * The buckets share dtypes, score and knobs; each has its own tensors, k,
+ * segment table, outputs, result block and workspace
+ * (sga_fused_workspace_bytes(n) bytes, 16-byte aligned, distinct per bucket).
+ * Outputs are bucket by bucket what sga_fused_sparse_step gives.  The chain of
+ * short dependent kernels around a select (sample, descents, check, candidate
+ * settlement, chunk scan) runs ONCE for up to 8 buckets (the kernels take the
+ * bucket from the grid's second dimension), only the data sweeps are launched
+ * per bucket.  `buckets` is a HOST array, read before the call returns. */
+typedef struct sga_fused_bucket {
+  const void* g;
+  float* resid;
+  float* p;
+  float* m;
+  float* v;
+  int64_t n;
+  int64_t k;
+  const sga_segment* segs;   /* DEVICE array */
+  int n_segs;
+  int pad_;
+  int32_t* idx_out;
+  void* values_out;
+  uint8_t* mask_out;         /* may be NULL */
+  sga_select_result* result; /* may be NULL */
+  void* ws;
+  size_t ws_bytes;
+} sga_fused_bucket;
+int sga_fused_sparse_step_multi(const sga_fused_bucket* buckets, int n_buckets,
+                                int g_dtype, int score_id, int values_dtype,
+                                float factor, float coeff, int fast, int flags,
+                                float interval, void* stream);
+
 /* Single-sweep variant of the fused step (no counterpart in the reference,
  * whose engine runs score, select, pack and commit as separate passes,
  * engine.py:416-604): g, resid, p, m, v are read ONCE.  The sampled bracket
@@ -482,6 +516,36 @@ int sga_replay_reselect(const void* g, int g_dtype, const float* res,
                         uint32_t* sel_out,
                         sga_select_result* result, void* ws, size_t ws_bytes,
                         void* stream);
+
+/* The boundary re-selections of ONE recorded step in one call
+ * (replay_fused.py:1752-1825 re-selects up to every configuration of the group
+ * at a step): each job is what sga_replay_reselect takes for one
+ * configuration, with a workspace of its own (distinct per job).  Jobs that
+ * rank by the same score run their short select kernels as one batch (up to 8
+ * per batch; the kernels take the job from the grid's second dimension), only
+ * the score sweeps are launched per job.  Same outputs, job by job, as
+ * sga_replay_reselect.  `jobs` is a HOST array, read before the call returns. */
+typedef struct sga_reselect_job {
+  const float* res;
+  const float* w;
+  const float* m;
+  const float* v;
+  int64_t k;
+  int score_id;
+  int adams;
+  int res_zero;
+  int pad_;
+  const float* coef_f;       /* device pointer to this configuration's coef */
+  uint32_t* sel_out;         /* bit planes, sga_plane_words(n) words        */
+  sga_select_result* result; /* may be NULL                                 */
+  void* ws;
+  size_t ws_bytes;
+} sga_reselect_job;
+int sga_replay_reselect_multi(const void* g, int g_dtype, int64_t n,
+                              const sga_segment* segs, int n_segs,
+                              float coef_dense, int packed,
+                              const sga_reselect_job* jobs, int n_jobs,
+                              void* stream);
 
 /* pass 2 under the `balanced-histogram` selection semantics
  * (replay_fused.py:405-489, 1805-1809; _histogram.py:115-123, 203-216): the

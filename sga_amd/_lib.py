@@ -29,6 +29,24 @@ class Segment(C.Structure):
                 ("bc1", C.c_float), ("bc2", C.c_float), ("pad_", C.c_float)]
 
 
+class FusedBucket(C.Structure):
+    """struct sga_fused_bucket"""
+    _fields_ = [("g", C.c_void_p), ("resid", C.c_void_p), ("p", C.c_void_p), ("m", C.c_void_p),
+                ("v", C.c_void_p), ("n", C.c_int64), ("k", C.c_int64), ("segs", C.c_void_p),
+                ("n_segs", C.c_int), ("pad_", C.c_int), ("idx_out", C.c_void_p),
+                ("values_out", C.c_void_p), ("mask_out", C.c_void_p), ("result", C.c_void_p),
+                ("ws", C.c_void_p), ("ws_bytes", C.c_size_t)]
+
+
+class ReselectJob(C.Structure):
+    """struct sga_reselect_job"""
+    _fields_ = [("res", C.c_void_p), ("w", C.c_void_p), ("m", C.c_void_p), ("v", C.c_void_p),
+                ("k", C.c_int64), ("score_id", C.c_int), ("adams", C.c_int),
+                ("res_zero", C.c_int), ("pad_", C.c_int), ("coef_f", C.c_void_p),
+                ("sel_out", C.c_void_p), ("result", C.c_void_p), ("ws", C.c_void_p),
+                ("ws_bytes", C.c_size_t)]
+
+
 # name -> (restype, argtypes); must list every symbol of include/sga_hip.h
 SIGNATURES = {
     "sga_version": (I32, []),
@@ -75,6 +93,7 @@ SIGNATURES = {
     "sga_replay_pass1": (I32, [P, I32, I64, F, C.c_double, P, I32, P, P, P, P, P]),
     "sga_replay_reselect": (I32, [P, I32, P, P, P, P, I64, I64, P, I32, I32, P, F, I32, I32, I32,
                                   P, P, P, SZ, P]),
+    "sga_replay_reselect_multi": (I32, [P, I32, I64, P, I32, F, I32, P, I32, P]),
     "sga_balanced_hist_words": (I64, []),
     "sga_replay_reselect_balanced": (I32, [P, I32, P, P, P, P, I64, I64, P, I32, P, I32, P, F, I32,
                                            I32, I32, P, P, P, P, SZ, P]),
@@ -89,6 +108,7 @@ SIGNATURES = {
     "sga_fused_workspace_bytes": (SZ, [I64]),
     "sga_fused_sparse_step": (I32, [P, I32, P, P, P, P, I64, I64, P, I32, I32, P, P,
                                     I32, P, F, F, I32, I32, F, P, P, SZ, P]),
+    "sga_fused_sparse_step_multi": (I32, [P, I32, I32, I32, I32, F, F, I32, I32, F, P]),
     "sga_packed_state_elems": (I64, [I64]),
     "sga_fused_sparse_step_packed": (I32, [P, I32, P, I64, I64, P, I32, I32, P, P,
                                            I32, P, F, F, I32, I32, F, P, P, SZ, P]),

@@ -141,9 +141,8 @@ struct SegCursor {
 };
 
 // Builds the directory of a segment table: dir[b] = last segment with start <= b << kSegDirLog.
-static __global__ __launch_bounds__(kBlock) void k_seg_dir(const sga_segment* __restrict__ segs,
-                                                           int n_segs, int64_t n,
-                                                           int32_t* __restrict__ dir) {
+__device__ __forceinline__ void seg_dir_body(const sga_segment* __restrict__ segs, int n_segs,
+                                             int64_t n, int32_t* __restrict__ dir) {
   const int64_t nb = (n + (1ll << kSegDirLog) - 1) >> kSegDirLog;
   for (int64_t b = (int64_t)blockIdx.x * kBlock + threadIdx.x; b < nb; b += (int64_t)gridDim.x * kBlock) {
     const int64_t i = b << kSegDirLog;
@@ -154,6 +153,19 @@ static __global__ __launch_bounds__(kBlock) void k_seg_dir(const sga_segment* __
     }
     dir[b] = lo;
   }
+}
+static __global__ __launch_bounds__(kBlock) void k_seg_dir(const sga_segment* __restrict__ segs,
+                                                           int n_segs, int64_t n,
+                                                           int32_t* __restrict__ dir) {
+  seg_dir_body(segs, n_segs, n, dir);
+}
+// The directories of up to 8 tables in one launch (blockIdx.y = table).
+struct SegDirJobs {
+  struct { const sga_segment* segs; int32_t* dir; int64_t n; int n_segs; } j[8];
+};
+static __global__ __launch_bounds__(kBlock) void k_seg_dir_batch(SegDirJobs jobs) {
+  const auto& J = jobs.j[blockIdx.y];
+  seg_dir_body(J.segs, J.n_segs, J.n, J.dir);
 }
 static inline void launch_seg_dir(const sga_segment* segs, int n_segs, int64_t n, int32_t* dir,
                                   hipStream_t s) {

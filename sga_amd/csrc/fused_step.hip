@@ -366,55 +366,90 @@ void k_fused_final(
   }
 }
 
+// One bucket of a (possibly batched) fused step.
+struct FusedJob {
+  const void* g;
+  float* resid;
+  float* p;
+  float* m;
+  float* v;
+  int64_t n, k;
+  const sga_segment* segs;
+  int n_segs;
+  int32_t* idx_out;
+  void* values_out;
+  uint8_t* mask_out;
+  sga_select_result* result;
+  SelWorkspace w;
+};
+
+// The two-sweep step for up to kMaxJobs buckets that share dtypes, score and knobs: the short
+// kernels of the buckets' selects run as one batched chain, the sweeps are launched per bucket.
 template <bool BF16G, bool BF16V, int SCORE>
-static int run_fused(const void* g, float* resid, float* p, float* m, float* v, int64_t n,
-                     int64_t k, const sga_segment* segs, int n_segs, int32_t* idx_out,
-                     void* values_out, uint8_t* mask_out, float factor, float coeff, int fast,
-                     int flags, float interval, sga_select_result* result, const SelWorkspace& w,
-                     hipStream_t s, int64_t pack_extra) {
-  const bool vec = aligned4(g, BF16G ? 2 : 4) && aligned4(resid, 4) && aligned4(p, 4) &&
-                   aligned4(m, 4) && aligned4(v, 4);
+static int run_fused(const FusedJob* fj, int count, float factor, float coeff, int fast, int flags,
+                     float interval, hipStream_t s, int64_t pack_extra, const char* who) {
+  using Src = SrcFused<BF16G, SCORE>;
   const int adams = (flags & SGA_GC_ADAMS) ? 1 : 0;
-  SrcFused<BF16G, SCORE> src{g, resid, p, m, v, vec, {}, pack_extra, adams};
   static_assert(kSelDirEntries == kSegDirEntries, "the workspace holds one directory");
-  launch_seg_dir(segs, n_segs, n, w.seg_dir, s);
-  src.sc.init(segs, n_segs, w.seg_dir);
+  SrcPack<Src> srcs = {};
+  SegDirJobs dj = {};
+  SelBatch B;
+  bool vec[kMaxJobs];
+  int64_t max_dir = 0;
   // Adam-normalised scores with the one-sweep select armed: the sweep leaves the selection as bit
   // planes (settled by the candidates) and the final sweep reads one bit per coordinate instead of
   // evaluating the score chain a second time; if the bracket fails on the device, the key-forming
   // final sweep runs instead.  For |g + r| and |m| the key is one instruction and re-forming it is
   // cheaper than writing and reading the planes (measured: 0.3 ms per step at 1.2e9 elements).
-  const bool planes = SrcFused<BF16G, SCORE>::kHyper && fast != 0 && n >= kFastMinN && w.pbits != nullptr;
-  run_select(src, n, k, 0, fast != 0, w, s, planes ? w.pbits : nullptr);
-  const int64_t n_tiles = cdiv64(n, kChunk);
-  if (planes)
-    hipLaunchKernelGGL(k_cand_bits, dim3(256), dim3(kBlock), 0, s, w.st, w.cand_idx, w.cand_key,
-                       w.tile_eq, n_tiles, 0, w.pbits);
-  ProfPair* pp = prof_begin(SGA_PROF_FUSED_FINAL, s);
-  FinalArgs fa;
-  fa.g = g; fa.r = resid; fa.p = p; fa.m = m; fa.v = v; fa.n = n; fa.k = k;
-  fa.idx_out = idx_out; fa.values_out = values_out; fa.mask_out = mask_out;
-  fa.factor = factor; fa.coeff = coeff; fa.T = 0; fa.need = 0;
-  fa.vec = vec; fa.mvec = aligned4(mask_out, 1);
-  fa.scale = factor != 1.0f; fa.apply_coeff = coeff != 1.0f;
-  fa.pack_extra = pack_extra;
-  fa.adams = adams != 0; fa.fold = (flags & SGA_GC_FOLD) != 0; fa.interval = interval;
-  fa.planes = w.pbits;
-  const dim3 one_shot(stream_grid(n_tiles, kChunksPerBlock, 1 << 20));
-  if (planes) {
-    hipLaunchKernelGGL((k_fused_final<BF16G, BF16V, SGA_SCORE_ABS_G, true>), one_shot, dim3(kBlock), 0, s,
-                       fa, segs, n_segs, w.st, w.tile_gt, w.tile_eq, 1, w.seg_dir);
-    // the rare other outcome: a small grid that strides over the chunks (returns at once otherwise)
-    hipLaunchKernelGGL((k_fused_final<BF16G, BF16V, SCORE, false>),
-                       dim3(stream_grid(n_tiles, kChunksPerBlock, 2048)), dim3(kBlock), 0, s, fa,
-                       segs, n_segs, w.st, w.tile_gt, w.tile_eq, 2, w.seg_dir);
-  } else {
-    hipLaunchKernelGGL((k_fused_final<BF16G, BF16V, SCORE, false>), one_shot, dim3(kBlock), 0, s, fa,
-                       segs, n_segs, w.st, w.tile_gt, w.tile_eq, 0, w.seg_dir);
+  bool use_fast = fast != 0;
+  for (int b = 0; b < count; ++b) use_fast = use_fast && SelBatch::fast_ok(fj[b].w, fj[b].n);
+  const bool planes = Src::kHyper && use_fast;
+  for (int b = 0; b < count; ++b) {
+    const FusedJob& f = fj[b];
+    vec[b] = aligned4(f.g, BF16G ? 2 : 4) && aligned4(f.resid, 4) && aligned4(f.p, 4) &&
+             aligned4(f.m, 4) && aligned4(f.v, 4);
+    srcs.s[b] = Src{f.g, f.resid, f.p, f.m, f.v, vec[b], {}, pack_extra, adams};
+    srcs.s[b].sc.init(f.segs, f.n_segs, f.w.seg_dir);
+    dj.j[b].segs = f.segs; dj.j[b].dir = f.w.seg_dir; dj.j[b].n = f.n; dj.j[b].n_segs = f.n_segs;
+    const int64_t nb = (f.n + (1ll << kSegDirLog) - 1) >> kSegDirLog;
+    if (nb > max_dir) max_dir = nb;
+    ChainJob& J = B.add(f.w, f.n, f.k, 0);
+    J.planes = planes ? f.w.pbits : nullptr;
+    J.result = f.result;
   }
-  prof_end(pp, s);
-  if (result) hipLaunchKernelGGL(k_sel_result, dim3(1), dim3(1), 0, s, w.st, result);
-  return check_launch("sga_fused_sparse_step");
+  hipLaunchKernelGGL(k_seg_dir_batch, B.grid(stream_grid(max_dir, kBlock, 128)), dim3(kBlock), 0, s, dj);
+  run_select_batch(srcs, B, use_fast, planes ? 1 : 0, s);
+  if (planes) hipLaunchKernelGGL(k_cand_bits, B.grid(256), dim3(kBlock), 0, s, B.jobs);
+  for (int b = 0; b < count; ++b) {
+    const FusedJob& f = fj[b];
+    const SelWorkspace& w = f.w;
+    const int64_t n_tiles = cdiv64(f.n, kChunk);
+    ProfPair* pp = prof_begin(SGA_PROF_FUSED_FINAL, s);
+    FinalArgs fa;
+    fa.g = f.g; fa.r = f.resid; fa.p = f.p; fa.m = f.m; fa.v = f.v; fa.n = f.n; fa.k = f.k;
+    fa.idx_out = f.idx_out; fa.values_out = f.values_out; fa.mask_out = f.mask_out;
+    fa.factor = factor; fa.coeff = coeff; fa.T = 0; fa.need = 0;
+    fa.vec = vec[b]; fa.mvec = aligned4(f.mask_out, 1);
+    fa.scale = factor != 1.0f; fa.apply_coeff = coeff != 1.0f;
+    fa.pack_extra = pack_extra;
+    fa.adams = adams != 0; fa.fold = (flags & SGA_GC_FOLD) != 0; fa.interval = interval;
+    fa.planes = w.pbits;
+    const dim3 one_shot(stream_grid(n_tiles, kChunksPerBlock, 1 << 20));
+    if (planes) {
+      hipLaunchKernelGGL((k_fused_final<BF16G, BF16V, SGA_SCORE_ABS_G, true>), one_shot, dim3(kBlock), 0, s,
+                         fa, f.segs, f.n_segs, w.st, w.tile_gt, w.tile_eq, 1, w.seg_dir);
+      // the rare other outcome: a small grid that strides over the chunks (returns at once otherwise)
+      hipLaunchKernelGGL((k_fused_final<BF16G, BF16V, SCORE, false>),
+                         dim3(stream_grid(n_tiles, kChunksPerBlock, 2048)), dim3(kBlock), 0, s, fa,
+                         f.segs, f.n_segs, w.st, w.tile_gt, w.tile_eq, 2, w.seg_dir);
+    } else {
+      hipLaunchKernelGGL((k_fused_final<BF16G, BF16V, SCORE, false>), one_shot, dim3(kBlock), 0, s, fa,
+                         f.segs, f.n_segs, w.st, w.tile_gt, w.tile_eq, 0, w.seg_dir);
+    }
+    prof_end(pp, s);
+  }
+  launch_result(B, s);
+  return check_launch(who);
 }
 
 
@@ -1080,20 +1115,18 @@ static int run_fused_spec(const void* g, float* resid, float* p, float* m, float
   fa.pack_extra = pack_extra;
   fa.adams = adams != 0; fa.fold = (flags & SGA_GC_FOLD) != 0; fa.interval = interval;
   fa.planes = w.pbits;
-  // sample -> bracket with the wide margins
-  launch_begin((uint32_t)k, w, s);
-  int64_t n_sv = w.sample_cap / 4;
-  const int64_t n_vec = n / 4;
-  if (n_sv > n_vec) n_sv = n_vec;
-  const int64_t ns = n_sv * 4;
-  hipLaunchKernelGGL((k_sample<SrcFused<BF16G, SCORE>>), dim3(stream_grid(n_sv, kBlock)), dim3(kBlock), 0, s,
-                     src, n, n_sv, n_vec, w.sample, seed);
-  hipLaunchKernelGGL(k_bracket_ranks, dim3(1), dim3(kBlock), 0, s, w.aux, w.hist, kHistStride * 2,
-                     (uint32_t)k, (double)n, (double)ns, w.seg_cnt, w.blk_gt, w.blk_eq, kSpecSigmas,
-                     x.seg_fail);
-  SrcU32 ssrc{w.sample};
-  for (int level = 0; level < 3; ++level)
-    launch_level<SrcU32, 2, true>(ssrc, ns, (const uint32_t*)nullptr, level, w.aux, w, s, kRawKeyBlocks);
+  // sample -> bracket with the wide margins (the chain kernels as a batch of one)
+  SrcPack<SrcFused<BF16G, SCORE>> srcs = {};
+  srcs.s[0] = src;
+  SelBatch B;
+  ChainJob& J = B.add(w, n, k, 0);
+  J.seed = seed; J.spec = 1; J.ovf_cap = (uint32_t)x.ovf_cap; J.seg_fail = x.seg_fail;
+  J.seg_rec = x.seg_rec; J.cand_rec = x.cand_rec; J.result = result;
+  const int64_t ns = J.n_sv * 4;
+  hipLaunchKernelGGL(k_chain_begin, B.grid(1), dim3(kBlock), 0, s, B.jobs, 1, kSpecSigmas);
+  hipLaunchKernelGGL((k_sample<SrcFused<BF16G, SCORE>>), B.grid(stream_grid(B.max_nsv, kBlock)),
+                     dim3(kBlock), 0, s, srcs, B.jobs);
+  for (int level = 0; level < 3; ++level) launch_level_raw<false>(B, level, s, kRawKeyBlocks);
   // the sweep
   SpecArgs sa;
   sa.splane = w.pbits; sa.fplane = x.dplane; sa.stage = x.stage;
@@ -1110,25 +1143,18 @@ static int run_fused_spec(const void* g, float* resid, float* p, float* m, float
   hipLaunchKernelGGL((k_fused_spec<BF16G, BF16V, SCORE>), one_shot, dim3(kBlock), 0, s, fa, sa, segs,
                      n_segs, w.st, w.aux, w.seg_dir);
   prof_end(pp, s);
-  hipLaunchKernelGGL(k_bracket_check, dim3(1), dim3(kBlock), 0, s, w.st, w.aux, w.seg_cnt, w.hist,
-                     kHistStride * 2, (uint32_t)w.seg_cap, w.blk_gt, w.blk_eq, 1, (uint32_t)x.ovf_cap,
-                     x.seg_fail);
-  hipLaunchKernelGGL(k_cand_compact, dim3(512), dim3(kBlock), 0, s, w.aux, w.seg_cnt, w.seg_idx,
-                     w.seg_key, (uint32_t)w.seg_cap, w.cand_idx, w.cand_key, x.seg_rec, x.cand_rec);
+  hipLaunchKernelGGL(k_bracket_check, B.grid(1), dim3(kBlock), 0, s, B.jobs);
+  hipLaunchKernelGGL(k_cand_compact, B.grid(512), dim3(kBlock), 0, s, B.jobs);
   hipLaunchKernelGGL(k_spec_ovf_compact, dim3(64), dim3(kBlock), 0, s, w.aux, w.seg_cnt, x.ovf_idx,
                      x.ovf_key, x.ovf_rec, (uint32_t)x.ovf_cap, w.cand_idx, w.cand_key, x.cand_rec,
                      x.tie_cnt);
-  SrcU32 csrc{w.cand_key};
-  const int64_t cmax = (int64_t)kSegWaves * w.seg_cap;
-  for (int level = 0; level < 3; ++level)
-    launch_level<SrcU32, 1, true>(csrc, cmax, &w.st->cand_count, level, w.aux, w, s, 3 * kRawKeyBlocks);
-  hipLaunchKernelGGL(k_cand_tiles, dim3(512), dim3(kBlock), 0, s, w.st, w.aux, w.cand_idx,
-                     w.cand_key, w.tile_gt, w.tile_eq);
+  for (int level = 0; level < 3; ++level) launch_level_raw<true>(B, level, s, 3 * kRawKeyBlocks);
+  hipLaunchKernelGGL(k_cand_tiles, B.grid(512), dim3(kBlock), 0, s, B.jobs);
   // only when the sweep stood back: the radix passes over the untouched data
   for (int level = 0; level < 3; ++level)
-    launch_level<SrcFused<BF16G, SCORE>, 1, true>(src, n, (const uint32_t*)nullptr, level, w.st, w, s);
-  launch_tile_count(src, n, 0, w, s);
-  launch_tile_scan(n_tiles, 0, w, s);
+    launch_level_data<SrcFused<BF16G, SCORE>, true>(srcs, B, level, s);
+  launch_tile_count(srcs, B, 0, s);
+  launch_tile_scan(B, s);
   hipLaunchKernelGGL(k_spec_ties, dim3(512), dim3(kBlock), 0, s, w.st, w.cand_idx, w.cand_key,
                      w.tile_eq, n_tiles, x.tie_cnt, x.tie_idx);
   hipLaunchKernelGGL(k_spec_settle, dim3(512), dim3(kBlock), 0, s, w.st, w.cand_idx, w.cand_key,
@@ -1151,7 +1177,7 @@ static int run_fused_spec(const void* g, float* resid, float* p, float* m, float
   hipLaunchKernelGGL((k_fused_final<BF16G, BF16V, SCORE, false>),
                      dim3(stream_grid(n_tiles, kChunksPerBlock, 2048)), dim3(kBlock), 0, s, fa,
                      segs, n_segs, w.st, w.tile_gt, w.tile_eq, 3, w.seg_dir);
-  if (result) hipLaunchKernelGGL(k_sel_result, dim3(1), dim3(1), 0, s, w.st, result);
+  launch_result(B, s);
   return check_launch("sga_fused_sparse_step_single_sweep");
 }
 
@@ -1219,14 +1245,13 @@ static int fused_entry(const char* who, const void* g, int g_dtype, float* resid
     }
     if (!take) { single = false; fast = 1; }
   }
+  const FusedJob job{g, resid, p, m, v, n, k, segs, n_segs, idx_out, values_out, mask_out, result, w};
 #define SGA_RUN(BG, BV, SC)                                                                   \
   if (single)                                                                                 \
     return run_fused_spec<BG, BV, SC>(g, resid, p, m, v, n, k, segs, n_segs, idx_out,        \
                                       values_out, mask_out, factor, coeff, flags, interval,   \
                                       seed, result, w, x, s, pack_extra);                     \
-  return run_fused<BG, BV, SC>(g, resid, p, m, v, n, k, segs, n_segs, idx_out, values_out,   \
-                               mask_out, factor, coeff, fast, flags, interval, result, w, s,   \
-                               pack_extra)
+  return run_fused<BG, BV, SC>(&job, 1, factor, coeff, fast, flags, interval, s, pack_extra, who)
 #define SGA_RUN_SC(BG, BV)                    \
   switch (score_id) {                         \
     case 0: SGA_RUN(BG, BV, 0);               \
@@ -1254,6 +1279,78 @@ extern "C" int sga_fused_sparse_step(const void* g, int g_dtype, float* resid, f
   return fused_entry("sga_fused_sparse_step", g, g_dtype, resid, p, m, v, 0, n, k, segs, n_segs,
                      score_id, idx_out, values_out, values_dtype, mask_out, factor, coeff, fast,
                      flags, interval, result, ws, ws_bytes, stream);
+}
+
+extern "C" int sga_fused_sparse_step_multi(const sga_fused_bucket* buckets, int n_buckets,
+                                           int g_dtype, int score_id, int values_dtype,
+                                           float factor, float coeff, int fast, int flags,
+                                           float interval, void* stream) {
+  const char* who = "sga_fused_sparse_step_multi";
+  if ((flags & ~(SGA_GC_ADAMS | SGA_GC_FOLD)) != 0) {
+    set_error("%s: flags may carry SGA_GC_ADAMS and SGA_GC_FOLD only (got %d)", who, flags);
+    return SGA_ERR_ARG;
+  }
+  if ((flags & SGA_GC_FOLD) && !(interval > 0.0f)) {
+    set_error("%s: SGA_GC_FOLD needs interval > 0 (got %g)", who, (double)interval);
+    return SGA_ERR_ARG;
+  }
+  if (!buckets || n_buckets < 1 || (g_dtype != SGA_F32 && g_dtype != SGA_BF16) ||
+      (values_dtype != SGA_F32 && values_dtype != SGA_BF16) || score_id < 0 ||
+      score_id > SGA_SCORE_GR_OVER_SQRT_V) {
+    set_error("%s: bad argument (n_buckets=%d score=%d)", who, n_buckets, score_id);
+    return SGA_ERR_ARG;
+  }
+  hipStream_t s = (hipStream_t)stream;
+  const bool bg = g_dtype == SGA_BF16, bv = values_dtype == SGA_BF16;
+  // buckets that take the sampled-bracket path and buckets too small for it go through the
+  // chain in separate batches of up to kMaxJobs
+  for (int pass = 0; pass < 2; ++pass) {
+    FusedJob jobs[kMaxJobs];
+    int cnt = 0;
+    for (int b = 0; b <= n_buckets; ++b) {
+      if (b < n_buckets) {
+        const sga_fused_bucket& u = buckets[b];
+        if (!u.g || !u.resid || !u.p || !u.m || !u.v || !u.segs || !u.idx_out || !u.values_out ||
+            u.n < 1 || u.n >= (1ll << 31) || u.k < 1 || u.k > u.n || u.n_segs < 1) {
+          set_error("%s: bucket %d: bad argument (n=%lld k=%lld n_segs=%d; need 1 <= k <= n < 2^31)",
+                    who, b, (long long)u.n, (long long)u.k, u.n_segs);
+          return SGA_ERR_ARG;
+        }
+        SelWorkspace w;
+        if (!sel_ws_carve(u.ws, u.ws_bytes, cdiv64(u.n, kChunk), &w)) {
+          set_error("%s: bucket %d: workspace missing, misaligned or smaller than "
+                    "sga_fused_workspace_bytes(n)=%zu", who, b, sel_ws_bytes(u.n));
+          return SGA_ERR_WORKSPACE;
+        }
+        const bool is_fast = fast != 0 && SelBatch::fast_ok(w, u.n);
+        if (is_fast != (pass == 0)) continue;
+        jobs[cnt++] = FusedJob{u.g, u.resid, u.p, u.m, u.v, u.n, u.k, u.segs, u.n_segs, u.idx_out,
+                               u.values_out, u.mask_out, u.result, w};
+      }
+      if (cnt == kMaxJobs || (b == n_buckets && cnt > 0)) {
+        int rc;
+#define SGA_RUNM(BG, BV, SC) rc = run_fused<BG, BV, SC>(jobs, cnt, factor, coeff, pass == 0, flags, interval, s, 0, who); break
+#define SGA_RUNM_SC(BG, BV)                    \
+        switch (score_id) {                    \
+          case 0: SGA_RUNM(BG, BV, 0);         \
+          case 1: SGA_RUNM(BG, BV, 1);         \
+          case 2: SGA_RUNM(BG, BV, 2);         \
+          case 3: SGA_RUNM(BG, BV, 3);         \
+          case 4: SGA_RUNM(BG, BV, 4);         \
+          default: SGA_RUNM(BG, BV, 5);        \
+        }
+        if (bg && bv) { SGA_RUNM_SC(true, true) }
+        else if (bg) { SGA_RUNM_SC(true, false) }
+        else if (bv) { SGA_RUNM_SC(false, true) }
+        else { SGA_RUNM_SC(false, false) }
+#undef SGA_RUNM_SC
+#undef SGA_RUNM
+        if (rc != SGA_OK) return rc;
+        cnt = 0;
+      }
+    }
+  }
+  return SGA_OK;
 }
 
 extern "C" size_t sga_fused_single_sweep_workspace_bytes(int64_t n, int values_dtype) {

@@ -688,26 +688,120 @@ extern "C" int sga_replay_pass3(const void* g, int g_dtype, int64_t n, float coe
   return check_launch("sga_replay_pass3");
 }
 
+// One boundary configuration of a (possibly batched) re-selection.
+struct ReselJob {
+  const float* res;
+  const float* w;
+  const float* m;
+  const float* v;
+  int64_t k;
+  const float* coef_f;
+  int adams, res_zero;
+  uint32_t* sel_out;
+  sga_select_result* result;
+  SelWorkspace ws;
+};
+
+// Exact top-k re-selection of up to kMaxJobs configurations that rank by the same score over
+// the same recorded gradient: their short select kernels run as one batched chain.
 template <bool BF16G, int SCORE>
-static int run_reselect(const void* g, const float* res, const float* w, const float* m,
-                        const float* v, int64_t n, int64_t k, const sga_segment* segs, int n_segs,
-                        const float* coef_f, float coef_dense, int adams, int packed, int res_zero,
-                        uint32_t* sel_out, sga_select_result* result, const SelWorkspace& ws,
-                        hipStream_t s) {
-  const bool vec = aligned4(g, BF16G ? 2 : 4) && aligned4(res, 4) && aligned4(w, 4) &&
-                   aligned4(m, 4) && aligned4(v, 4);
-  SrcReplay<BF16G, SCORE> src{g, res, w, m, v, coef_f, coef_dense, adams, vec, {},
-                              packed ? kPackExtra : 0, res_zero};
-  if (SrcReplay<BF16G, SCORE>::kHyper) {          // the other scores never look a tensor up
-    launch_seg_dir(segs, n_segs, n, ws.seg_dir, s);
-    src.sc.init(segs, n_segs, ws.seg_dir);
-  } else {
-    src.sc.init(segs, n_segs);
+static int run_reselect(const void* g, int64_t n, const sga_segment* segs, int n_segs,
+                        float coef_dense, int packed, const ReselJob* rj, int count, hipStream_t s,
+                        const char* who) {
+  using Src = SrcReplay<BF16G, SCORE>;
+  static_assert(kMaxJobs <= 8, "one directory launch per batch");
+  SrcPack<Src> srcs = {};
+  SegDirJobs dj = {};
+  SelBatch B;
+  bool fast = true;
+  for (int b = 0; b < count; ++b) {
+    const ReselJob& r = rj[b];
+    const bool vec = aligned4(g, BF16G ? 2 : 4) && aligned4(r.res, 4) && aligned4(r.w, 4) &&
+                     aligned4(r.m, 4) && aligned4(r.v, 4);
+    srcs.s[b] = Src{g, r.res, r.w, r.m, r.v, r.coef_f, coef_dense, r.adams, vec, {},
+                    packed ? kPackExtra : 0, r.res_zero};
+    // only the Adam-normalised scores ever look a tensor up
+    srcs.s[b].sc.init(segs, n_segs, Src::kHyper ? r.ws.seg_dir : nullptr);
+    dj.j[b].segs = segs; dj.j[b].dir = r.ws.seg_dir; dj.j[b].n = n; dj.j[b].n_segs = n_segs;
+    ChainJob& J = B.add(r.ws, n, r.k, 0);
+    J.planes = r.sel_out;
+    J.result = r.result;
+    fast = fast && SelBatch::fast_ok(r.ws, n);
   }
-  run_select(src, n, k, 0, true, ws, s, sel_out);
-  finish_planes(src, n, 0, ws, sel_out, s);
-  if (result) hipLaunchKernelGGL(k_sel_result, dim3(1), dim3(1), 0, s, ws.st, result);
-  return check_launch("sga_replay_reselect");
+  if (Src::kHyper) {
+    const int64_t nb = (n + (1ll << kSegDirLog) - 1) >> kSegDirLog;
+    hipLaunchKernelGGL(k_seg_dir_batch, B.grid(stream_grid(nb, kBlock, 128)), dim3(kBlock), 0, s, dj);
+  }
+  run_select_batch(srcs, B, fast, 1, s);
+  finish_planes_batch(srcs, B, fast, s);
+  launch_result(B, s);
+  return check_launch(who);
+}
+
+template <bool BF16G>
+static int run_reselect_score(int score_id, const void* g, int64_t n, const sga_segment* segs,
+                              int n_segs, float coef_dense, int packed, const ReselJob* rj,
+                              int count, hipStream_t s, const char* who) {
+#define SGA_RS(SC) return run_reselect<BF16G, SC>(g, n, segs, n_segs, coef_dense, packed, rj, count, s, who)
+  switch (score_id) { case 0: SGA_RS(0); case 1: SGA_RS(1); case 2: SGA_RS(2);
+                      case 3: SGA_RS(3); case 4: SGA_RS(4); default: SGA_RS(5); }
+#undef SGA_RS
+}
+
+extern "C" int sga_replay_reselect_multi(const void* g, int g_dtype, int64_t n,
+                                         const sga_segment* segs, int n_segs, float coef_dense,
+                                         int packed, const sga_reselect_job* jobs, int n_jobs,
+                                         void* stream) {
+  const char* who = "sga_replay_reselect_multi";
+  if (!g || !segs || !jobs || n < 1 || n >= (1ll << 31) || n_segs < 1 || n_jobs < 1 ||
+      (g_dtype != SGA_F32 && g_dtype != SGA_BF16)) {
+    set_error("%s: bad argument (n=%lld n_jobs=%d)", who, (long long)n, n_jobs);
+    return SGA_ERR_ARG;
+  }
+  hipStream_t s = (hipStream_t)stream;
+  // configurations that rank by the same score share a batch (the key source is a template
+  // argument of the sweeps); a workspace too small for the sampled bracket gets its own
+  bool done[64] = {};
+  if (n_jobs > 64) { set_error("%s: at most 64 jobs per call", who); return SGA_ERR_ARG; }
+  for (int a = 0; a < n_jobs; ++a) {
+    const sga_reselect_job& u = jobs[a];
+    if (!u.res || !u.w || !u.m || !u.v || !u.coef_f || !u.sel_out || u.k < 1 || u.k > n ||
+        u.score_id < 0 || u.score_id > SGA_SCORE_GR_OVER_SQRT_V) {
+      set_error("%s: job %d: bad argument (k=%lld score=%d)", who, a, (long long)u.k, u.score_id);
+      return SGA_ERR_ARG;
+    }
+  }
+  for (int a = 0; a < n_jobs; ++a) {
+    if (done[a]) continue;
+    ReselJob rj[kMaxJobs];
+    int cnt = 0;
+    bool fast0 = false;
+    for (int b = a; b < n_jobs && cnt < kMaxJobs; ++b) {
+      if (done[b] || jobs[b].score_id != jobs[a].score_id) continue;
+      const sga_reselect_job& u = jobs[b];
+      SelWorkspace sw;
+      if (!sel_ws_carve(u.ws, u.ws_bytes, cdiv64(n, kChunk), &sw)) {
+        set_error("%s: job %d: workspace too small (sga_select_workspace_bytes(n))", who, b);
+        return SGA_ERR_WORKSPACE;
+      }
+      for (int c = 0; c < cnt; ++c)
+        if (rj[c].ws.st == sw.st) {
+          set_error("%s: jobs %d shares its workspace with an earlier job of the call", who, b);
+          return SGA_ERR_ARG;
+        }
+      const bool f = SelBatch::fast_ok(sw, n);
+      if (cnt == 0) fast0 = f;
+      else if (f != fast0) continue;
+      rj[cnt++] = ReselJob{u.res, u.w, u.m, u.v, u.k, u.coef_f, u.adams, u.res_zero, u.sel_out,
+                           u.result, sw};
+      done[b] = true;
+    }
+    const int rc = g_dtype == SGA_BF16
+        ? run_reselect_score<true>(jobs[a].score_id, g, n, segs, n_segs, coef_dense, packed, rj, cnt, s, who)
+        : run_reselect_score<false>(jobs[a].score_id, g, n, segs, n_segs, coef_dense, packed, rj, cnt, s, who);
+    if (rc != SGA_OK) return rc;
+  }
+  return SGA_OK;
 }
 
 extern "C" int sga_replay_reselect(const void* g, int g_dtype, const float* res, const float* w,
@@ -727,16 +821,11 @@ extern "C" int sga_replay_reselect(const void* g, int g_dtype, const float* res,
     set_error("sga_replay_reselect: workspace too small (sga_select_workspace_bytes(n))");
     return SGA_ERR_WORKSPACE;
   }
+  const ReselJob rj{res, w, m, v, k, coef_f, adams, res_zero, sel_out, result, sw};
   hipStream_t s = (hipStream_t)stream;
-#define SGA_RS(BG, SC) return run_reselect<BG, SC>(g, res, w, m, v, n, k, segs, n_segs, coef_f, coef_dense, adams, packed, res_zero, sel_out, result, sw, s)
-  if (g_dtype == SGA_BF16) {
-    switch (score_id) { case 0: SGA_RS(true, 0); case 1: SGA_RS(true, 1); case 2: SGA_RS(true, 2);
-                        case 3: SGA_RS(true, 3); case 4: SGA_RS(true, 4); default: SGA_RS(true, 5); }
-  } else {
-    switch (score_id) { case 0: SGA_RS(false, 0); case 1: SGA_RS(false, 1); case 2: SGA_RS(false, 2);
-                        case 3: SGA_RS(false, 3); case 4: SGA_RS(false, 4); default: SGA_RS(false, 5); }
-  }
-#undef SGA_RS
+  return g_dtype == SGA_BF16
+      ? run_reselect_score<true>(score_id, g, n, segs, n_segs, coef_dense, packed, &rj, 1, s, "sga_replay_reselect")
+      : run_reselect_score<false>(score_id, g, n, segs, n_segs, coef_dense, packed, &rj, 1, s, "sga_replay_reselect");
 }
 
 // ------------------------------------------- balanced-histogram re-selection

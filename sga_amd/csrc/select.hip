@@ -251,7 +251,9 @@ extern "C" int sga_sel_begin(int64_t k, void* ws, size_t ws_bytes, void* stream)
     set_error("sga_sel_begin: k=%lld out of range", (long long)k);
     return SGA_ERR_ARG;
   }
-  launch_begin((uint32_t)k, w, (hipStream_t)stream);
+  SelBatch B;
+  B.add(w, 1, k, 0);
+  hipLaunchKernelGGL(k_chain_begin, B.grid(1), dim3(kBlock), 0, (hipStream_t)stream, B.jobs, 0, 0.0);
   return check_launch("sga_sel_begin");
 }
 
@@ -264,8 +266,12 @@ extern "C" int sga_sel_hist(const float* score, int64_t n, int level, void* ws,
     set_error("sga_sel_hist: bad argument");
     return SGA_ERR_ARG;
   }
-  SrcF32 src{score, aligned4(score, 4)};
-  launch_level_hist(src, n, level, w, (hipStream_t)stream);
+  // histogram only: several views feed one level before its scan
+  SrcPack<SrcF32> srcs = {};
+  srcs.s[0] = SrcF32{score, aligned4(score, 4)};
+  SelBatch B;
+  B.add(w, n, 1, 0);
+  launch_level_data<SrcF32, false>(srcs, B, level, (hipStream_t)stream);
   return check_launch("sga_sel_hist");
 }
 
@@ -273,7 +279,9 @@ extern "C" int sga_sel_scan(int level, void* ws, size_t ws_bytes, void* stream) 
   SelWorkspace w;
   if (int rc = carve(ws, ws_bytes, 0, &w, "sga_sel_scan")) return rc;
   if (level < 0 || level > 2) { set_error("sga_sel_scan: bad level"); return SGA_ERR_ARG; }
-  launch_level_scan(level, w, (hipStream_t)stream);
+  SelBatch B;
+  B.add(w, 1, 1, 0);
+  launch_level_scan(level, B, (hipStream_t)stream);
   return check_launch("sga_sel_scan");
 }
 
@@ -283,8 +291,11 @@ extern "C" int sga_sel_count(const float* score, int64_t n, int64_t tile_base, v
   SelWorkspace w;
   if (int rc = carve(ws, ws_bytes, tile_base + cdiv64(n, kChunk), &w, "sga_sel_count")) return rc;
   if (!score || n < 0 || tile_base < 0) { set_error("sga_sel_count: bad argument"); return SGA_ERR_ARG; }
-  SrcF32 src{score, aligned4(score, 4)};
-  launch_tile_count(src, n, tile_base, w, (hipStream_t)stream);
+  SrcPack<SrcF32> srcs = {};
+  srcs.s[0] = SrcF32{score, aligned4(score, 4)};
+  SelBatch B;
+  B.add(w, n, 1, 0);
+  launch_tile_count(srcs, B, tile_base, (hipStream_t)stream);
   return check_launch("sga_sel_count");
 }
 
@@ -296,7 +307,9 @@ extern "C" int sga_sel_tile_scan(int64_t n_tiles, int tie_mode, void* ws, size_t
     set_error("sga_sel_tile_scan: n_tiles=%lld out of range", (long long)n_tiles);
     return SGA_ERR_ARG;
   }
-  launch_tile_scan(n_tiles, tie_mode == SGA_TIE_ALL, w, (hipStream_t)stream);
+  SelBatch B;
+  B.add(w, n_tiles * kChunk, 1, tie_mode == SGA_TIE_ALL);
+  launch_tile_scan(B, (hipStream_t)stream);
   return check_launch("sga_sel_tile_scan");
 }
 
@@ -306,11 +319,13 @@ extern "C" int sga_sel_mask(const float* score, int64_t n, int64_t tile_base, in
   SelWorkspace w;
   if (int rc = carve(ws, ws_bytes, tile_base + cdiv64(n, kChunk), &w, "sga_sel_mask")) return rc;
   if (!score || !mask_out || n < 0 || tile_base < 0) { set_error("sga_sel_mask: bad argument"); return SGA_ERR_ARG; }
-  SrcF32 src{score, aligned4(score, 4)};
-  const int64_t nc = cdiv64(n, kChunk);
-  hipLaunchKernelGGL((k_write_mask<SrcF32>), dim3(stream_grid(nc, kChunksPerBlock, 1 << 22)), dim3(kBlock), 0,
-                     (hipStream_t)stream, src, n, tile_base, tie_mode == SGA_TIE_ALL, w.st,
-                     w.tile_gt, w.tile_eq, mask_out, aligned4(mask_out, 1));
+  SrcPack<SrcF32> srcs = {};
+  srcs.s[0] = SrcF32{score, aligned4(score, 4)};
+  SelBatch B;
+  B.add(w, n, 1, tie_mode == SGA_TIE_ALL).mask = mask_out;
+  hipLaunchKernelGGL((k_write_mask<SrcF32>), B.grid(stream_grid(B.max_tiles, kChunksPerBlock, 1 << 22)),
+                     dim3(kBlock), 0, (hipStream_t)stream, srcs, B.jobs, tile_base, 0,
+                     (uint8_t*)nullptr);
   return check_launch("sga_sel_mask");
 }
 
@@ -318,7 +333,9 @@ extern "C" int sga_sel_result(sga_select_result* result, void* ws, size_t ws_byt
   SelWorkspace w;
   if (int rc = carve(ws, ws_bytes, 0, &w, "sga_sel_result")) return rc;
   if (!result) { set_error("sga_sel_result: null result"); return SGA_ERR_ARG; }
-  hipLaunchKernelGGL(k_sel_result, dim3(1), dim3(1), 0, (hipStream_t)stream, w.st, result);
+  SelBatch B;
+  B.add(w, 1, 1, 0).result = result;
+  launch_result(B, (hipStream_t)stream);
   return check_launch("sga_sel_result");
 }
 
@@ -333,12 +350,17 @@ extern "C" int sga_select_topk(const float* score, int64_t n, int64_t k, int tie
   SelWorkspace w;
   if (int rc = carve(ws, ws_bytes, cdiv64(n, kChunk), &w, "sga_select_topk")) return rc;
   hipStream_t s = (hipStream_t)stream;
-  SrcF32 src{score, aligned4(score, 4)};
-  const int tie_all = tie_mode == SGA_TIE_ALL;
+  SrcPack<SrcF32> srcs = {};
+  srcs.s[0] = SrcF32{score, aligned4(score, 4)};
+  SelBatch B;
+  ChainJob& J = B.add(w, n, k, tie_mode == SGA_TIE_ALL);
+  J.mask = mask_out;
+  J.result = result;
+  const bool fast = SelBatch::fast_ok(w, n);
   // the select sweep writes the keys above the bracket straight into mask_out
-  run_select(src, n, k, tie_all, true, w, s, nullptr, mask_out);
-  finish_mask(src, n, tie_all, w, mask_out, s, true);
-  if (result) hipLaunchKernelGGL(k_sel_result, dim3(1), dim3(1), 0, s, w.st, result);
+  run_select_batch(srcs, B, fast, 2, s);
+  finish_mask_batch(srcs, B, fast, s);
+  launch_result(B, s);
   return check_launch("sga_select_topk");
 }
 

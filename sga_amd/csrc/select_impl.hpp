@@ -88,6 +88,40 @@ static inline int64_t fast_seg_cap(int64_t n) {
   return c;
 }
 
+// Batched chain: every short kernel around a select takes up to kMaxJobs
+// independent select problems in one launch (blockIdx.y = job), so that a
+// caller with several buckets (or several re-selections of one replay step)
+// pays the chain of dependent launches once instead of once per problem.
+// The operands travel by value in the kernel arguments.
+constexpr int kMaxJobs = 8;
+struct ChainJob {
+  SelState* st;
+  SelState* aux;
+  uint32_t* hist;
+  uint32_t* tile_gt;
+  uint32_t* tile_eq;
+  uint32_t* blk_gt;
+  uint32_t* blk_eq;
+  uint32_t* sample;
+  uint32_t* seg_cnt;
+  uint32_t* seg_idx;
+  uint32_t* seg_key;
+  uint32_t* cand_idx;
+  uint32_t* cand_key;
+  uint32_t* seg_fail;          // single-sweep step: per-segment first failed reservation
+  const F4* seg_rec;           // single-sweep step: records beside the segments' keys
+  F4* cand_rec;
+  uint32_t* planes;            // where the settlement writes the selection (bit planes) ...
+  uint8_t* mask;               // ... or mask bytes
+  sga_select_result* result;
+  int64_t n, n_tiles, n_sv, n_vec;
+  uint32_t k, seg_cap, seed, ovf_cap;
+  int tie_all, spec;
+};
+struct ChainJobs { ChainJob j[kMaxJobs]; };
+template <class Src>
+struct SrcPack { Src s[kMaxJobs]; };
+
 // Workspace layout: [fixed: states | level histograms | tile-scan block sums]
 // [tile_gt[nt] | tile_eq[nt]] [fast-path buffers sized from nt: sample keys,
 // per-wave candidate segments, dense candidates, 128 B of bit planes per
@@ -330,10 +364,10 @@ __device__ __forceinline__ uint32_t* level_hist_of(uint32_t* hist_set) {
 // not take part.  MERGE: the last workgroup to finish also runs the level's
 // scan, so hist + scan is one launch.
 template <class Src, int LEVEL, int NS, bool MERGE>
-__global__ __launch_bounds__(kBlock) void k_level_hist(Src src, int64_t n,
-                                                       const uint32_t* __restrict__ n_dev,
-                                                       SelState* __restrict__ st,
-                                                       uint32_t* __restrict__ hist) {
+__device__ __forceinline__ void level_hist_body(Src& src, int64_t n,
+                                                const uint32_t* __restrict__ n_dev,
+                                                SelState* __restrict__ st,
+                                                uint32_t* __restrict__ hist) {
   constexpr int NB = LEVEL == 2 ? kBinsSmall : kBinsBig;
   __shared__ uint32_t s_h[NS][NB];
   __shared__ uint32_t s_suf[kBlock + 1];
@@ -412,38 +446,48 @@ __global__ __launch_bounds__(kBlock) void k_level_hist(Src src, int64_t n,
     if (on[q]) level_scan_body<LEVEL>(&st[q], level_hist_of<LEVEL>(hist + q * kHistStride), s_suf);
   if (threadIdx.x == 0) st[0].done[LEVEL] = 0u;
 }
+// over the data itself (a key source per job): the radix passes, state = st
+template <class Src, int LEVEL, bool MERGE>
+__global__ __launch_bounds__(kBlock) void k_level_hist(SrcPack<Src> srcs, ChainJobs jobs) {
+  const ChainJob& J = jobs.j[blockIdx.y];
+  Src src = srcs.s[blockIdx.y];
+  level_hist_body<Src, LEVEL, 1, MERGE>(src, J.n, nullptr, J.st, J.hist);
+}
+// over a raw key buffer of the job: the sample (both bracket ends descend together, states
+// aux[0], aux[1]) or the candidates (their count lives on the device; state aux[0])
+template <int LEVEL, bool CAND>
+__global__ __launch_bounds__(kBlock) void k_level_hist_raw(ChainJobs jobs) {
+  const ChainJob& J = jobs.j[blockIdx.y];
+  SrcU32 src{CAND ? J.cand_key : J.sample};
+  if (CAND)
+    level_hist_body<SrcU32, LEVEL, 1, true>(src, (int64_t)kSegWaves * J.seg_cap, &J.st->cand_count,
+                                            J.aux, J.hist);
+  else
+    level_hist_body<SrcU32, LEVEL, 2, true>(src, J.n_sv * 4, nullptr, J.aux, J.hist);
+}
 
 // Stand-alone scan (used when one level's histogram is built by several
 // launches, one per view).
 template <int LEVEL>
-__global__ __launch_bounds__(kBlock) void k_level_scan(SelState* __restrict__ st,
-                                                       uint32_t* __restrict__ hist) {
+__global__ __launch_bounds__(kBlock) void k_level_scan(ChainJobs jobs) {
   __shared__ uint32_t s_suf[kBlock + 1];
-  if (st->skip) return;
-  level_scan_body<LEVEL>(st, level_hist_of<LEVEL>(hist), s_suf);
-}
-
-// Zero the level histograms and reset a state for a new descent.  With
-// `from` given, the rank comes from the device (from->krem) and the descent
-// is skipped when from->skip == skip_when... see the callers.
-static __global__ void k_sel_begin(SelState* st, uint32_t* hist, int nhist, uint32_t k) {
-  for (int i = threadIdx.x; i < nhist; i += blockDim.x) hist[i] = 0u;
-  if (threadIdx.x == 0) {
-    SelState z = {};
-    z.k = k;
-    *st = z;
-  }
+  const ChainJob& J = jobs.j[blockIdx.y];
+  if (J.st->skip) return;
+  level_scan_body<LEVEL>(J.st, level_hist_of<LEVEL>(J.hist), s_suf);
 }
 
 // Per-chunk (1024 elements, one wave) counts of keys above / equal to the
 // threshold.
 template <class Src>
-__global__ __launch_bounds__(kBlock) void k_tile_count(Src src, int64_t n,
-                                                       int64_t tile_base,
-                                                       SelState* __restrict__ st,
-                                                       uint32_t* __restrict__ tile_gt,
-                                                       uint32_t* __restrict__ tile_eq) {
+__global__ __launch_bounds__(kBlock) void k_tile_count(SrcPack<Src> srcs, ChainJobs jobs,
+                                                       int64_t tile_base) {
+  const ChainJob& J = jobs.j[blockIdx.y];
+  SelState* __restrict__ st = J.st;
   if (st->skip) return;
+  Src src = srcs.s[blockIdx.y];
+  const int64_t n = J.n;
+  uint32_t* __restrict__ tile_gt = J.tile_gt;
+  uint32_t* __restrict__ tile_eq = J.tile_eq;
   const uint32_t T = st->thresh_bits;
   const int64_t n_chunks = cdiv64(n, kChunk);
   const int64_t wstride = (int64_t)gridDim.x * kChunksPerBlock;
@@ -484,12 +528,15 @@ __global__ __launch_bounds__(kBlock) void k_tile_count(Src src, int64_t n,
 }
 
 // Tile scan, kernel 1: per-workgroup totals of (gt, eq).
-static __global__ __launch_bounds__(kBlock) void k_tile_sums(const uint32_t* __restrict__ tile_gt,
-                                                      const uint32_t* __restrict__ tile_eq,
-                                                      int64_t n_tiles,
-                                                      uint32_t* __restrict__ blk_gt,
-                                                      uint32_t* __restrict__ blk_eq) {
+static __global__ __launch_bounds__(kBlock) void k_tile_sums(ChainJobs jobs) {
   __shared__ uint32_t s_g[kChunksPerBlock], s_e[kChunksPerBlock];
+  const ChainJob& J = jobs.j[blockIdx.y];
+  const int64_t n_tiles = J.n_tiles;
+  if ((int64_t)blockIdx.x * kTileScanSpan >= n_tiles) return;     // a job with fewer tiles
+  const uint32_t* __restrict__ tile_gt = J.tile_gt;
+  const uint32_t* __restrict__ tile_eq = J.tile_eq;
+  uint32_t* __restrict__ blk_gt = J.blk_gt;
+  uint32_t* __restrict__ blk_eq = J.blk_eq;
   const int64_t base = (int64_t)blockIdx.x * kTileScanSpan + (int64_t)threadIdx.x * kTileScanPer;
   uint32_t g = 0, e = 0;
 #pragma unroll
@@ -526,14 +573,18 @@ __device__ __forceinline__ uint32_t block_excl_scan(uint32_t v, uint32_t* s_w4, 
 // Tile scan, kernel 2: tile_eq[i] <- ties before tile i; tile_gt[i] <- selected
 // coordinates before tile i (ties granted in ascending order until `need`
 // is used up; all of them when tie_all).
-static __global__ __launch_bounds__(kBlock) void k_tile_apply(uint32_t* __restrict__ tile_gt,
-                                                       uint32_t* __restrict__ tile_eq,
-                                                       int64_t n_tiles,
-                                                       const uint32_t* __restrict__ blk_gt,
-                                                       const uint32_t* __restrict__ blk_eq,
-                                                       int n_blocks, int tie_all,
-                                                       SelState* __restrict__ st) {
+static __global__ __launch_bounds__(kBlock) void k_tile_apply(ChainJobs jobs) {
   __shared__ uint32_t s_w4[kChunksPerBlock];
+  const ChainJob& J = jobs.j[blockIdx.y];
+  const int64_t n_tiles = J.n_tiles;
+  const int n_blocks = (int)cdiv64(n_tiles, kTileScanSpan);
+  if ((int)blockIdx.x >= n_blocks) return;                        // a job with fewer tiles
+  uint32_t* __restrict__ tile_gt = J.tile_gt;
+  uint32_t* __restrict__ tile_eq = J.tile_eq;
+  const uint32_t* __restrict__ blk_gt = J.blk_gt;
+  const uint32_t* __restrict__ blk_eq = J.blk_eq;
+  const int tie_all = J.tie_all;
+  SelState* __restrict__ st = J.st;
   const uint32_t need = tie_all ? 0xFFFFFFFFu : st->need;
   // prefixes of the workgroups before this one (n_blocks <= 1024 -> 4 each)
   uint32_t be[4], bg[4];
@@ -599,7 +650,7 @@ static __global__ __launch_bounds__(kBlock) void k_tile_apply(uint32_t* __restri
     }
     sr += scount[j];
   }
-  if (blockIdx.x == gridDim.x - 1 && threadIdx.x == 0) st->n_selected = S0 + blk_tot_s;
+  if ((int)blockIdx.x == n_blocks - 1 && threadIdx.x == 0) st->n_selected = S0 + blk_tot_s;
 }
 
 // Ordered flags for one 256-element slab of a wave's chunk: `sel[e]` says
@@ -641,14 +692,19 @@ __device__ __forceinline__ void slab_select(const uint32_t key[4], const bool va
 }
 
 template <class Src>
-__global__ __launch_bounds__(kBlock) void k_write_mask(Src src, int64_t n, int64_t tile_base,
-                                                       int tie_all,
-                                                       const SelState* __restrict__ st,
-                                                       const uint32_t* __restrict__ tile_sel,
-                                                       const uint32_t* __restrict__ tile_eq,
-                                                       uint8_t* __restrict__ mask, bool mvec,
-                                                       int unless_settled = 0) {
+__global__ __launch_bounds__(kBlock) void k_write_mask(SrcPack<Src> srcs, ChainJobs jobs,
+                                                       int64_t tile_base, int unless_settled,
+                                                       uint8_t* __restrict__ mask_override) {
+  const ChainJob& J = jobs.j[blockIdx.y];
+  const SelState* __restrict__ st = J.st;
   if (unless_settled && st->bracket_ok) return;
+  Src src = srcs.s[blockIdx.y];
+  const int64_t n = J.n;
+  const int tie_all = J.tie_all;
+  const uint32_t* __restrict__ tile_sel = J.tile_gt;
+  const uint32_t* __restrict__ tile_eq = J.tile_eq;
+  uint8_t* __restrict__ mask = mask_override ? mask_override : J.mask;
+  const bool mvec = aligned4(mask, 1);
   const uint32_t T = st->thresh_bits;
   const uint32_t need = tie_all ? 0xFFFFFFFFu : st->need;
   const int64_t n_chunks = cdiv64(n, kChunk);
@@ -683,7 +739,10 @@ __global__ __launch_bounds__(kBlock) void k_write_mask(Src src, int64_t n, int64
   }
 }
 
-static __global__ void k_sel_result(const SelState* st, sga_select_result* out) {
+static __global__ void k_sel_result(ChainJobs jobs) {
+  const SelState* st = jobs.j[blockIdx.y].st;
+  sga_select_result* out = jobs.j[blockIdx.y].result;
+  if (!out) return;
   out->thresh_bits = st->thresh_bits;
   out->need = st->need;
   out->n_gt = st->n_gt;
@@ -704,46 +763,75 @@ static inline dim3 hist_grid(int64_t n) {
   return dim3(stream_grid(n, (int64_t)kBlock * kVec * 4, 256 * 8));
 }
 
-// hist (+ merged scan) of one level for NS states starting at `st`.
-template <class Src, int NS, bool MERGE>
-static inline void launch_level(Src src, int64_t n, const uint32_t* n_dev, int level,
-                                SelState* st, const SelWorkspace& w, hipStream_t s,
-                                unsigned max_blocks = 0) {
-  dim3 grid = hist_grid(n), block(kBlock);
-  if (max_blocks && grid.x > max_blocks) grid.x = max_blocks;
-  if (level == 0) hipLaunchKernelGGL((k_level_hist<Src, 0, NS, MERGE>), grid, block, 0, s, src, n, n_dev, st, w.hist);
-  else if (level == 1) hipLaunchKernelGGL((k_level_hist<Src, 1, NS, MERGE>), grid, block, 0, s, src, n, n_dev, st, w.hist);
-  else hipLaunchKernelGGL((k_level_hist<Src, 2, NS, MERGE>), grid, block, 0, s, src, n, n_dev, st, w.hist);
+// Host side of a batched chain: up to kMaxJobs select problems that go through every short
+// kernel together.  A single select is a batch of one.
+struct SelBatch {
+  int count = 0;
+  ChainJobs jobs;
+  SelWorkspace w[kMaxJobs];
+  int64_t max_n = 0, max_tiles = 0, max_nsv = 0;
+  // true when the job takes the sampled-bracket path (all jobs of one batch must agree)
+  static bool fast_ok(const SelWorkspace& ws, int64_t n) {
+    return n >= kFastMinN && ws.sample != nullptr && n < (1ll << 32);
+  }
+  ChainJob& add(const SelWorkspace& ws, int64_t n, int64_t k, int tie_all) {
+    ChainJob& J = jobs.j[count];
+    w[count++] = ws;
+    J = ChainJob{};
+    J.st = ws.st; J.aux = ws.aux; J.hist = ws.hist;
+    J.tile_gt = ws.tile_gt; J.tile_eq = ws.tile_eq; J.blk_gt = ws.blk_gt; J.blk_eq = ws.blk_eq;
+    J.sample = ws.sample; J.seg_cnt = ws.seg_cnt; J.seg_idx = ws.seg_idx; J.seg_key = ws.seg_key;
+    J.cand_idx = ws.cand_idx; J.cand_key = ws.cand_key;
+    J.n = n; J.n_tiles = cdiv64(n, kChunk);
+    J.n_vec = n / 4;
+    J.n_sv = ws.sample_cap / 4 < J.n_vec ? ws.sample_cap / 4 : J.n_vec;
+    J.k = (uint32_t)k; J.seg_cap = (uint32_t)ws.seg_cap; J.tie_all = tie_all;
+    if (n > max_n) max_n = n;
+    if (J.n_tiles > max_tiles) max_tiles = J.n_tiles;
+    if (J.n_sv > max_nsv) max_nsv = J.n_sv;
+    return J;
+  }
+  dim3 grid(unsigned gx) const { return dim3(gx, (unsigned)count); }
+};
+
+// hist (+ merged scan) of one radix level over the data, for every job of the batch
+template <class Src, bool MERGE>
+static inline void launch_level_data(const SrcPack<Src>& srcs, const SelBatch& B, int level,
+                                     hipStream_t s) {
+  const dim3 grid = B.grid(hist_grid(B.max_n).x), block(kBlock);
+  if (level == 0) hipLaunchKernelGGL((k_level_hist<Src, 0, MERGE>), grid, block, 0, s, srcs, B.jobs);
+  else if (level == 1) hipLaunchKernelGGL((k_level_hist<Src, 1, MERGE>), grid, block, 0, s, srcs, B.jobs);
+  else hipLaunchKernelGGL((k_level_hist<Src, 2, MERGE>), grid, block, 0, s, srcs, B.jobs);
 }
-// piecewise API: histogram only (several views feed one level), then a scan
+// the same over the jobs' sample keys (CAND false) or candidate keys (CAND true)
+template <bool CAND>
+static inline void launch_level_raw(const SelBatch& B, int level, hipStream_t s, unsigned blocks) {
+  const dim3 grid = B.grid(blocks), block(kBlock);
+  if (level == 0) hipLaunchKernelGGL((k_level_hist_raw<0, CAND>), grid, block, 0, s, B.jobs);
+  else if (level == 1) hipLaunchKernelGGL((k_level_hist_raw<1, CAND>), grid, block, 0, s, B.jobs);
+  else hipLaunchKernelGGL((k_level_hist_raw<2, CAND>), grid, block, 0, s, B.jobs);
+}
+static inline void launch_level_scan(int level, const SelBatch& B, hipStream_t s) {
+  if (level == 0) hipLaunchKernelGGL((k_level_scan<0>), B.grid(1), dim3(kBlock), 0, s, B.jobs);
+  else if (level == 1) hipLaunchKernelGGL((k_level_scan<1>), B.grid(1), dim3(kBlock), 0, s, B.jobs);
+  else hipLaunchKernelGGL((k_level_scan<2>), B.grid(1), dim3(kBlock), 0, s, B.jobs);
+}
+
 template <class Src>
-static inline void launch_level_hist(Src src, int64_t n, int level,
-                                     const SelWorkspace& w, hipStream_t s) {
-  launch_level<Src, 1, false>(src, n, (const uint32_t*)nullptr, level, w.st, w, s);
-}
-static inline void launch_level_scan(int level, const SelWorkspace& w, hipStream_t s) {
-  if (level == 0) hipLaunchKernelGGL((k_level_scan<0>), dim3(1), dim3(kBlock), 0, s, w.st, w.hist);
-  else if (level == 1) hipLaunchKernelGGL((k_level_scan<1>), dim3(1), dim3(kBlock), 0, s, w.st, w.hist);
-  else hipLaunchKernelGGL((k_level_scan<2>), dim3(1), dim3(kBlock), 0, s, w.st, w.hist);
+static inline void launch_tile_count(const SrcPack<Src>& srcs, const SelBatch& B, int64_t tile_base,
+                                     hipStream_t s) {
+  hipLaunchKernelGGL((k_tile_count<Src>), B.grid(stream_grid(B.max_tiles, kChunksPerBlock)),
+                     dim3(kBlock), 0, s, srcs, B.jobs, tile_base);
 }
 
-static inline void launch_begin(uint32_t k, const SelWorkspace& w, hipStream_t s) {
-  hipLaunchKernelGGL(k_sel_begin, dim3(1), dim3(kBlock), 0, s, w.st, w.hist, kHistStride * 2, k);
+static inline void launch_tile_scan(const SelBatch& B, hipStream_t s) {
+  const unsigned nb = (unsigned)cdiv64(B.max_tiles, kTileScanSpan);
+  hipLaunchKernelGGL(k_tile_sums, B.grid(nb), dim3(kBlock), 0, s, B.jobs);
+  hipLaunchKernelGGL(k_tile_apply, B.grid(nb), dim3(kBlock), 0, s, B.jobs);
 }
 
-template <class Src>
-static inline void launch_tile_count(Src src, int64_t n, int64_t tile_base,
-                                     const SelWorkspace& w, hipStream_t s) {
-  const int64_t nc = cdiv64(n, kChunk);
-  hipLaunchKernelGGL((k_tile_count<Src>), dim3(stream_grid(nc, kChunksPerBlock)),
-                     dim3(kBlock), 0, s, src, n, tile_base, w.st, w.tile_gt, w.tile_eq);
-}
-
-static inline void launch_tile_scan(int64_t n_tiles, int tie_all,
-                                    const SelWorkspace& w, hipStream_t s) {
-  const int nb = (int)cdiv64(n_tiles, kTileScanSpan);
-  hipLaunchKernelGGL(k_tile_sums, dim3(nb), dim3(kBlock), 0, s, w.tile_gt, w.tile_eq, n_tiles, w.blk_gt, w.blk_eq);
-  hipLaunchKernelGGL(k_tile_apply, dim3(nb), dim3(kBlock), 0, s, w.tile_gt, w.tile_eq, n_tiles, w.blk_gt, w.blk_eq, nb, tie_all, w.st);
+static inline void launch_result(const SelBatch& B, hipStream_t s) {
+  hipLaunchKernelGGL(k_sel_result, B.grid(1), dim3(1), 0, s, B.jobs);
 }
 
 // ===================================================== sampled-bracket path
@@ -766,8 +854,12 @@ __device__ __forceinline__ uint32_t mix32(uint32_t x) {
 // differently from the rest.  `seed` moves the offsets (0: the fixed pattern);
 // the select is exact for any of them.
 template <class Src>
-__global__ __launch_bounds__(kBlock) void k_sample(Src src, int64_t n, int64_t n_sv, int64_t n_vec,
-                                                   uint32_t* __restrict__ keys, uint32_t seed = 0u) {
+__global__ __launch_bounds__(kBlock) void k_sample(SrcPack<Src> srcs, ChainJobs jobs) {
+  const ChainJob& J = jobs.j[blockIdx.y];
+  Src src = srcs.s[blockIdx.y];
+  const int64_t n = J.n, n_sv = J.n_sv, n_vec = J.n_vec;
+  uint32_t* __restrict__ keys = J.sample;
+  const uint32_t seed = J.seed;
   for (int64_t j = (int64_t)blockIdx.x * kBlock + threadIdx.x; j < n_sv;
        j += (int64_t)gridDim.x * kBlock) {
     const int64_t w0 = j * n_vec / n_sv, w1 = (j + 1) * n_vec / n_sv;
@@ -779,28 +871,34 @@ __global__ __launch_bounds__(kBlock) void k_sample(Src src, int64_t n, int64_t n
   }
 }
 
-// Ranks of the two bracket ends inside the sample, r = k*ns/n -/+ (5 sigma + 8):
-// aux[0] descends to the upper end (smaller rank = larger key), aux[1] to the
-// lower end.  Also zeroes both histogram sets.
-static __global__ void k_bracket_ranks(SelState* aux, uint32_t* hist, int nhist, uint32_t k,
-                                       double n, double ns, uint32_t* seg_cnt, uint32_t* hi_part,
-                                       uint32_t* nf_part, double sigmas = 5.0,
-                                       uint32_t* seg_fail = nullptr) {
-  for (int i = threadIdx.x; i < nhist; i += blockDim.x) hist[i] = 0u;
-  if (seg_fail)
-    for (int i = threadIdx.x; i < kSegWaves; i += blockDim.x) seg_fail[i] = 0u;
-  for (int i = threadIdx.x; i <= kSegWaves + 1; i += blockDim.x) seg_cnt[i] = 0u;   // + overflow count
-  for (int i = threadIdx.x; i < kSweepParts; i += blockDim.x) { hi_part[i] = 0u; nf_part[i] = 0u; }
+// First kernel of a select, one workgroup per job: zeroes both histogram sets and the sweep's
+// counters, resets the main state to rank k and, on the sampled-bracket path (`fast`), places
+// the two ends of the bracket inside the sample at ranks r = k*ns/n -/+ (sigmas * sigma + 8):
+// aux[0] descends to the upper end (smaller rank = larger key), aux[1] to the lower end.
+static __global__ __launch_bounds__(kBlock) void k_chain_begin(ChainJobs jobs, int fast, double sigmas) {
+  const ChainJob& J = jobs.j[blockIdx.y];
+  for (int i = threadIdx.x; i < kHistStride * 2; i += blockDim.x) J.hist[i] = 0u;
+  if (fast) {
+    for (int i = threadIdx.x; i <= kSegWaves + 1; i += blockDim.x) J.seg_cnt[i] = 0u;   // + overflow count
+    for (int i = threadIdx.x; i < kSweepParts; i += blockDim.x) { J.blk_gt[i] = 0u; J.blk_eq[i] = 0u; }
+    if (J.seg_fail)
+      for (int i = threadIdx.x; i < kSegWaves; i += blockDim.x) J.seg_fail[i] = 0u;
+  }
   if (threadIdx.x != 0) return;
-  const double frac = (double)k / n;
+  SelState z = {};
+  z.k = J.k;
+  *J.st = z;
+  if (!fast) return;
+  const double n = (double)J.n, ns = (double)(J.n_sv * 4);
+  const double frac = (double)J.k / n;
   const double r = frac * ns;
   const double d = sigmas * sqrt(r * (1.0 - frac) + 1.0) + 8.0;
   SelState hi = {}, lo = {};
   const double rh = floor(r - d), rl = ceil(r + d);
   if (rh < 1.0) hi.skip = 1; else hi.k = (uint32_t)rh;
   if (rl > ns) lo.skip = 1; else lo.k = (uint32_t)rl;
-  aux[0] = hi;
-  aux[1] = lo;
+  J.aux[0] = hi;
+  J.aux[1] = lo;
 }
 
 // The one sweep over the data: a one-shot grid, one 1024-element chunk per
@@ -986,16 +1084,20 @@ __global__ __launch_bounds__(kBlock) void k_bracket_sweep(
 
 // Single workgroup: segment counts -> offsets, validate the bracket, arm the
 // candidate descent (aux) or the radix passes (st->skip == 0).
-static __global__ __launch_bounds__(kBlock) void k_bracket_check(SelState* __restrict__ st,
-                                                                 SelState* __restrict__ aux,
-                                                                 uint32_t* __restrict__ seg_cnt,
-                                                                 uint32_t* __restrict__ hist, int nhist,
-                                                                 uint32_t seg_cap,
-                                                                 const uint32_t* __restrict__ hi_part,
-                                                                 const uint32_t* __restrict__ nf_part,
-                                                                 int spec = 0, uint32_t ovf_cap = 0u,
-                                                                 const uint32_t* __restrict__ seg_fail = nullptr) {
+static __global__ __launch_bounds__(kBlock) void k_bracket_check(ChainJobs jobs) {
   __shared__ uint32_t s_w4[kChunksPerBlock];
+  const ChainJob& J = jobs.j[blockIdx.y];
+  SelState* __restrict__ st = J.st;
+  SelState* __restrict__ aux = J.aux;
+  uint32_t* __restrict__ seg_cnt = J.seg_cnt;
+  uint32_t* __restrict__ hist = J.hist;
+  constexpr int nhist = kHistStride * 2;
+  const uint32_t seg_cap = J.seg_cap;
+  const uint32_t* __restrict__ hi_part = J.blk_gt;
+  const uint32_t* __restrict__ nf_part = J.blk_eq;
+  const int spec = J.spec;
+  const uint32_t ovf_cap = J.ovf_cap;
+  const uint32_t* __restrict__ seg_fail = J.seg_fail;
   constexpr int PER = kSegWaves / kBlock;   // 32
   uint32_t v[PER], mine = 0, over = 0;
 #pragma unroll
@@ -1054,12 +1156,17 @@ static __global__ __launch_bounds__(kBlock) void k_bracket_check(SelState* __res
 }
 
 // Dense candidate list from the per-wave segments (order: wave, then index).
-static __global__ __launch_bounds__(kBlock) void k_cand_compact(
-    const SelState* __restrict__ aux, const uint32_t* __restrict__ seg_off,
-    const uint32_t* __restrict__ seg_idx, const uint32_t* __restrict__ seg_key, uint32_t seg_cap,
-    uint32_t* __restrict__ cand_idx, uint32_t* __restrict__ cand_key,
-    const F4* __restrict__ seg_rec = nullptr, F4* __restrict__ cand_rec = nullptr) {
-  if (aux->skip) return;
+static __global__ __launch_bounds__(kBlock) void k_cand_compact(ChainJobs jobs) {
+  const ChainJob& J = jobs.j[blockIdx.y];
+  if (J.aux->skip) return;
+  const uint32_t* __restrict__ seg_off = J.seg_cnt;
+  const uint32_t* __restrict__ seg_idx = J.seg_idx;
+  const uint32_t* __restrict__ seg_key = J.seg_key;
+  const uint32_t seg_cap = J.seg_cap;
+  uint32_t* __restrict__ cand_idx = J.cand_idx;
+  uint32_t* __restrict__ cand_key = J.cand_key;
+  const F4* __restrict__ seg_rec = J.seg_rec;
+  F4* __restrict__ cand_rec = J.cand_rec;
   for (int w = blockIdx.x * kChunksPerBlock + wave_id(); w < kSegWaves;
        w += gridDim.x * kChunksPerBlock) {
     const uint32_t off = seg_off[w], cnt = seg_off[w + 1] - off;
@@ -1073,11 +1180,15 @@ static __global__ __launch_bounds__(kBlock) void k_cand_compact(
 
 // After the candidate descent: publish the exact threshold and fold each
 // candidate into its chunk's (above, equal) counts.
-static __global__ __launch_bounds__(kBlock) void k_cand_tiles(
-    SelState* __restrict__ st, const SelState* __restrict__ aux,
-    const uint32_t* __restrict__ cand_idx, const uint32_t* __restrict__ cand_key,
-    uint32_t* __restrict__ tile_gt, uint32_t* __restrict__ tile_eq) {
+static __global__ __launch_bounds__(kBlock) void k_cand_tiles(ChainJobs jobs) {
+  const ChainJob& J = jobs.j[blockIdx.y];
+  SelState* __restrict__ st = J.st;
+  const SelState* __restrict__ aux = J.aux;
   if (aux->skip) return;
+  const uint32_t* __restrict__ cand_idx = J.cand_idx;
+  const uint32_t* __restrict__ cand_key = J.cand_key;
+  uint32_t* __restrict__ tile_gt = J.tile_gt;
+  uint32_t* __restrict__ tile_eq = J.tile_eq;
   const uint32_t T = aux->thresh_bits;
   const uint32_t nc = st->cand_count;
   if (blockIdx.x == 0 && threadIdx.x == 0) {
@@ -1140,11 +1251,16 @@ static __global__ __launch_bounds__(kBlock) void k_expand_mask(
 // tile scan tile_eq[c] counts the ties before chunk c, so only the one chunk
 // where the quota runs out has to rank its ties (a chunk's candidates are
 // contiguous and index-ordered in the list).
-static __global__ __launch_bounds__(kBlock) void k_cand_mask(
-    const SelState* __restrict__ st, const uint32_t* __restrict__ cand_idx,
-    const uint32_t* __restrict__ cand_key, const uint32_t* __restrict__ tile_eq,
-    int64_t n_tiles, int tie_all, uint8_t* __restrict__ mask) {
+static __global__ __launch_bounds__(kBlock) void k_cand_mask(ChainJobs jobs) {
+  const ChainJob& J = jobs.j[blockIdx.y];
+  const SelState* __restrict__ st = J.st;
   if (!st->bracket_ok) return;
+  const uint32_t* __restrict__ cand_idx = J.cand_idx;
+  const uint32_t* __restrict__ cand_key = J.cand_key;
+  const uint32_t* __restrict__ tile_eq = J.tile_eq;
+  const int64_t n_tiles = J.n_tiles;
+  const int tie_all = J.tie_all;
+  uint8_t* __restrict__ mask = J.mask;
   const uint32_t T = st->thresh_bits, nc = st->cand_count, n_eq = st->n_eq;
   const uint32_t need = tie_all ? 0xFFFFFFFFu : st->need;
   for (uint32_t j = blockIdx.x * kBlock + threadIdx.x; j < nc; j += gridDim.x * kBlock) {
@@ -1170,11 +1286,16 @@ static __global__ __launch_bounds__(kBlock) void k_cand_mask(
 }
 
 // The same settlement when the mask itself is kept as bit planes.
-static __global__ __launch_bounds__(kBlock) void k_cand_bits(
-    const SelState* __restrict__ st, const uint32_t* __restrict__ cand_idx,
-    const uint32_t* __restrict__ cand_key, const uint32_t* __restrict__ tile_eq,
-    int64_t n_tiles, int tie_all, uint32_t* __restrict__ planes) {
+static __global__ __launch_bounds__(kBlock) void k_cand_bits(ChainJobs jobs) {
+  const ChainJob& J = jobs.j[blockIdx.y];
+  const SelState* __restrict__ st = J.st;
   if (!st->bracket_ok) return;
+  const uint32_t* __restrict__ cand_idx = J.cand_idx;
+  const uint32_t* __restrict__ cand_key = J.cand_key;
+  const uint32_t* __restrict__ tile_eq = J.tile_eq;
+  const int64_t n_tiles = J.n_tiles;
+  const int tie_all = J.tie_all;
+  uint32_t* __restrict__ planes = J.planes;
   const uint32_t T = st->thresh_bits, nc = st->cand_count, n_eq = st->n_eq;
   const uint32_t need = tie_all ? 0xFFFFFFFFu : st->need;
   for (uint32_t j = blockIdx.x * kBlock + threadIdx.x; j < nc; j += gridDim.x * kBlock) {
@@ -1205,12 +1326,16 @@ static __global__ __launch_bounds__(kBlock) void k_cand_bits(
 // Ordered full pass that writes the mask as bit planes (the fallback of
 // k_cand_bits when the sampled bracket failed or was never tried).
 template <class Src>
-__global__ __launch_bounds__(kBlock) void k_write_bits(Src src, int64_t n, int tie_all,
-                                                       const SelState* __restrict__ st,
-                                                       const uint32_t* __restrict__ tile_sel,
-                                                       const uint32_t* __restrict__ tile_eq,
-                                                       uint32_t* __restrict__ planes) {
+__global__ __launch_bounds__(kBlock) void k_write_bits(SrcPack<Src> srcs, ChainJobs jobs) {
+  const ChainJob& J = jobs.j[blockIdx.y];
+  const SelState* __restrict__ st = J.st;
   if (st->bracket_ok) return;
+  Src src = srcs.s[blockIdx.y];
+  const int64_t n = J.n;
+  const int tie_all = J.tie_all;
+  const uint32_t* __restrict__ tile_sel = J.tile_gt;
+  const uint32_t* __restrict__ tile_eq = J.tile_eq;
+  uint32_t* __restrict__ planes = J.planes;
   const uint32_t T = st->thresh_bits;
   const uint32_t need = tie_all ? 0xFFFFFFFFu : st->need;
   const int64_t n_chunks = cdiv64(n, kChunk);
@@ -1259,99 +1384,75 @@ static __global__ __launch_bounds__(kBlock) void k_mask_to_planes(const uint8_t*
   }
 }
 
-// planes (optional): the sweep also records there, as bit planes, which keys
-// lie above the bracket, so a caller that only wants the mask can finish from
-// those bits and the candidates (finish_mask / finish_planes) instead of
-// re-reading the data.
+// The select of every job of a batch: begin -> (sampled-bracket path: sample, dual-rank descent,
+// ONE data sweep per job, check, candidate compaction and descent, per-chunk counts) -> the radix
+// passes (no-ops unless a job's bracket failed) -> chunk scan.  The short kernels run once for
+// the whole batch; only the data sweeps are launched per job.
+// PM: what the sweep leaves behind for a mask-only caller -- 0 nothing, 1 the keys above the
+// bracket as bit planes (job.planes), 2 as mask bytes (job.mask) -- to be finished by
+// finish_planes / finish_mask from those bits and the candidates instead of re-reading the data.
+// All jobs of a batch take the same path (`fast`: SelBatch::fast_ok for every one of them).
 template <class Src>
-static inline void run_select(Src src, int64_t n, int64_t k, int tie_all, bool fast,
-                              const SelWorkspace& w, hipStream_t s, uint32_t* planes = nullptr,
-                              uint8_t* mask_bytes = nullptr) {
-  const bool want_mask = planes != nullptr;
-  const int64_t n_tiles = cdiv64(n, kChunk);
-  launch_begin((uint32_t)k, w, s);
-  if (fast && n >= kFastMinN && w.sample && n < (1ll << 32)) {
-    int64_t n_sv = w.sample_cap / 4;
-    const int64_t n_vec = n / 4;
-    if (n_sv > n_vec) n_sv = n_vec;
-    const int64_t ns = n_sv * 4;
-    hipLaunchKernelGGL((k_sample<Src>), dim3(stream_grid(n_sv, kBlock)), dim3(kBlock), 0, s, src, n,
-                       n_sv, n_vec, w.sample);
-    // the sweep's two totals go through 256 partial counters (blk_gt / blk_eq are free until the
-    // tile scan, which runs after the check has read them)
-    hipLaunchKernelGGL(k_bracket_ranks, dim3(1), dim3(kBlock), 0, s, w.aux, w.hist, kHistStride * 2,
-                       (uint32_t)k, (double)n, (double)ns, w.seg_cnt, w.blk_gt, w.blk_eq);
-    SrcU32 ssrc{w.sample};
-    for (int level = 0; level < 3; ++level)
-      launch_level<SrcU32, 2, true>(ssrc, ns, (const uint32_t*)nullptr, level, w.aux, w, s, kRawKeyBlocks);
-    const unsigned sweep_blocks = (unsigned)cdiv64(n_tiles, kChunksPerBlock);
-    ProfPair* pp = prof_begin(SGA_PROF_SELECT_SWEEP, s);
-    if (mask_bytes)
-      hipLaunchKernelGGL((k_bracket_sweep<Src, 2>), dim3(sweep_blocks), dim3(kBlock), 0, s,
-                         src, n, w.st, w.aux, w.tile_gt, w.tile_eq, w.seg_idx, w.seg_key, w.seg_cnt,
-                         (uint32_t)w.seg_cap, (uint32_t*)nullptr, w.blk_gt, w.blk_eq, mask_bytes,
-                         (reinterpret_cast<uintptr_t>(mask_bytes) & 3) == 0);
-    else if (want_mask)
-      hipLaunchKernelGGL((k_bracket_sweep<Src, 1>), dim3(sweep_blocks), dim3(kBlock), 0, s,
-                         src, n, w.st, w.aux, w.tile_gt, w.tile_eq, w.seg_idx, w.seg_key, w.seg_cnt,
-                         (uint32_t)w.seg_cap, planes, w.blk_gt, w.blk_eq);
-    else
-      hipLaunchKernelGGL((k_bracket_sweep<Src, 0>), dim3(sweep_blocks), dim3(kBlock), 0, s,
-                         src, n, w.st, w.aux, w.tile_gt, w.tile_eq, w.seg_idx, w.seg_key, w.seg_cnt,
-                         (uint32_t)w.seg_cap, (uint32_t*)nullptr, w.blk_gt, w.blk_eq);
-    prof_end(pp, s);
-    hipLaunchKernelGGL(k_bracket_check, dim3(1), dim3(kBlock), 0, s, w.st, w.aux, w.seg_cnt, w.hist,
-                       kHistStride * 2, (uint32_t)w.seg_cap, w.blk_gt, w.blk_eq);
-    hipLaunchKernelGGL(k_cand_compact, dim3(256), dim3(kBlock), 0, s, w.aux, w.seg_cnt, w.seg_idx,
-                       w.seg_key, (uint32_t)w.seg_cap, w.cand_idx, w.cand_key);
-    SrcU32 csrc{w.cand_key};
-    const int64_t cmax = (int64_t)kSegWaves * w.seg_cap;
-    for (int level = 0; level < 3; ++level)
-      launch_level<SrcU32, 1, true>(csrc, cmax, &w.st->cand_count, level, w.aux, w, s, kRawKeyBlocks);
-    hipLaunchKernelGGL(k_cand_tiles, dim3(256), dim3(kBlock), 0, s, w.st, w.aux, w.cand_idx,
-                       w.cand_key, w.tile_gt, w.tile_eq);
+static inline void run_select_batch(const SrcPack<Src>& srcs, const SelBatch& B, bool fast, int pm,
+                                    hipStream_t s, double sigmas = 5.0) {
+  hipLaunchKernelGGL(k_chain_begin, B.grid(1), dim3(kBlock), 0, s, B.jobs, fast ? 1 : 0, sigmas);
+  if (fast) {
+    hipLaunchKernelGGL((k_sample<Src>), B.grid(stream_grid(B.max_nsv, kBlock)), dim3(kBlock), 0, s,
+                       srcs, B.jobs);
+    for (int level = 0; level < 3; ++level) launch_level_raw<false>(B, level, s, kRawKeyBlocks);
+    for (int b = 0; b < B.count; ++b) {
+      const ChainJob& J = B.jobs.j[b];
+      const SelWorkspace& w = B.w[b];
+      const unsigned sweep_blocks = (unsigned)cdiv64(J.n_tiles, kChunksPerBlock);
+      ProfPair* pp = prof_begin(SGA_PROF_SELECT_SWEEP, s);
+      // the sweep's two totals go through 256 partial counters (blk_gt / blk_eq are free until
+      // the tile scan, which runs after the check has read them)
+      if (pm == 2)
+        hipLaunchKernelGGL((k_bracket_sweep<Src, 2>), dim3(sweep_blocks), dim3(kBlock), 0, s,
+                           srcs.s[b], J.n, w.st, w.aux, w.tile_gt, w.tile_eq, w.seg_idx, w.seg_key,
+                           w.seg_cnt, (uint32_t)w.seg_cap, (uint32_t*)nullptr, w.blk_gt, w.blk_eq,
+                           J.mask, (reinterpret_cast<uintptr_t>(J.mask) & 3) == 0);
+      else if (pm == 1)
+        hipLaunchKernelGGL((k_bracket_sweep<Src, 1>), dim3(sweep_blocks), dim3(kBlock), 0, s,
+                           srcs.s[b], J.n, w.st, w.aux, w.tile_gt, w.tile_eq, w.seg_idx, w.seg_key,
+                           w.seg_cnt, (uint32_t)w.seg_cap, J.planes, w.blk_gt, w.blk_eq);
+      else
+        hipLaunchKernelGGL((k_bracket_sweep<Src, 0>), dim3(sweep_blocks), dim3(kBlock), 0, s,
+                           srcs.s[b], J.n, w.st, w.aux, w.tile_gt, w.tile_eq, w.seg_idx, w.seg_key,
+                           w.seg_cnt, (uint32_t)w.seg_cap, (uint32_t*)nullptr, w.blk_gt, w.blk_eq);
+      prof_end(pp, s);
+    }
+    hipLaunchKernelGGL(k_bracket_check, B.grid(1), dim3(kBlock), 0, s, B.jobs);
+    hipLaunchKernelGGL(k_cand_compact, B.grid(256), dim3(kBlock), 0, s, B.jobs);
+    for (int level = 0; level < 3; ++level) launch_level_raw<true>(B, level, s, kRawKeyBlocks);
+    hipLaunchKernelGGL(k_cand_tiles, B.grid(256), dim3(kBlock), 0, s, B.jobs);
     // The radix passes below are no-ops unless the bracket failed
     // (st->skip == 0); k_bracket_check left the histograms zeroed for them.
   }
-  for (int level = 0; level < 3; ++level)
-    launch_level<Src, 1, true>(src, n, (const uint32_t*)nullptr, level, w.st, w, s);
-  launch_tile_count(src, n, 0, w, s);
-  launch_tile_scan(n_tiles, tie_all, w, s);
+  for (int level = 0; level < 3; ++level) launch_level_data<Src, true>(srcs, B, level, s);
+  launch_tile_count(srcs, B, 0, s);
+  launch_tile_scan(B, s);
 }
 
-// Bit-plane mask of the selection after run_select(..., planes): the
-// candidates settle the sweep's planes when the bracket held, else the
-// ordered full pass writes them.
+// Bit-plane masks of the selections after run_select_batch(..., pm = 1): the candidates settle
+// the sweep's planes when the bracket held, else the ordered full pass writes them.
 template <class Src>
-static inline void finish_planes(Src src, int64_t n, int tie_all, const SelWorkspace& w,
-                                 uint32_t* planes, hipStream_t s) {
-  const int64_t nc = cdiv64(n, kChunk);
-  if (w.cand_idx && n >= kFastMinN && n < (1ll << 32))
-    hipLaunchKernelGGL(k_cand_bits, dim3(256), dim3(kBlock), 0, s, w.st, w.cand_idx, w.cand_key,
-                       w.tile_eq, nc, tie_all, planes);
-  hipLaunchKernelGGL((k_write_bits<Src>), dim3(stream_grid(nc, kChunksPerBlock, 1 << 14)),
-                     dim3(kBlock), 0, s, src, n, tie_all, w.st, w.tile_gt, w.tile_eq, planes);
+static inline void finish_planes_batch(const SrcPack<Src>& srcs, const SelBatch& B, bool fast,
+                                       hipStream_t s) {
+  if (fast) hipLaunchKernelGGL(k_cand_bits, B.grid(256), dim3(kBlock), 0, s, B.jobs);
+  hipLaunchKernelGGL((k_write_bits<Src>), B.grid(stream_grid(B.max_tiles, kChunksPerBlock, 1 << 14)),
+                     dim3(kBlock), 0, s, srcs, B.jobs);
 }
 
-// Byte mask of the selection after run_select(..., w.pbits): the bit planes
-// and the candidates settle it when the bracket held, else the ordered full
-// pass writes it.
-// in_bytes: the sweep already wrote the provisional selection as mask bytes (run_select(...,
-// nullptr, mask)); only the candidates are left to settle.
+// Byte masks after run_select_batch(..., pm = 2) (the sweep wrote the provisional selection
+// straight into the caller's mask): the candidates settle it when the bracket held, else the
+// ordered full pass writes it.
 template <class Src>
-static inline void finish_mask(Src src, int64_t n, int tie_all, const SelWorkspace& w,
-                               uint8_t* mask, hipStream_t s, bool in_bytes = false) {
-  const int64_t nc = cdiv64(n, kChunk);
-  if (w.pbits && n >= kFastMinN && n < (1ll << 32)) {
-    if (!in_bytes)
-      hipLaunchKernelGGL(k_expand_mask, dim3(stream_grid(nc, kChunksPerBlock, 1 << 22)), dim3(kBlock),
-                         0, s, w.st, w.pbits, n, mask, (reinterpret_cast<uintptr_t>(mask) & 15) == 0);
-    hipLaunchKernelGGL(k_cand_mask, dim3(256), dim3(kBlock), 0, s, w.st, w.cand_idx, w.cand_key,
-                       w.tile_eq, nc, tie_all, mask);
-  }
-  hipLaunchKernelGGL((k_write_mask<Src>), dim3(stream_grid(nc, kChunksPerBlock, 1 << 14)),
-                     dim3(kBlock), 0, s, src, n, (int64_t)0, tie_all, w.st, w.tile_gt, w.tile_eq,
-                     mask, aligned4(mask, 1), 1);
+static inline void finish_mask_batch(const SrcPack<Src>& srcs, const SelBatch& B, bool fast,
+                                     hipStream_t s) {
+  if (fast) hipLaunchKernelGGL(k_cand_mask, B.grid(256), dim3(kBlock), 0, s, B.jobs);
+  hipLaunchKernelGGL((k_write_mask<Src>), B.grid(stream_grid(B.max_tiles, kChunksPerBlock, 1 << 14)),
+                     dim3(kBlock), 0, s, srcs, B.jobs, (int64_t)0, fast ? 1 : 0, (uint8_t*)nullptr);
 }
 
 #endif  // __HIPCC__

@@ -188,6 +188,53 @@ class FusedSparseStep:
         return read_result(self.result)
 
 
+def fused_step_multi(steppers, grads, resids, ps, ms, vs, step, ks=None, ratio_percent=None,
+                     score="abs_g", factor=1.0, coeff=1.0, fast=True, optimizer="adamw",
+                     fold=False, interval=1.0):
+    """One two-sweep fused step for several buckets in ONE call
+    (``sga_fused_sparse_step_multi``): the per-bucket online path, where every
+    bucket selects its own top-k (``sga/engine.py:822-890``).  ``steppers``:
+    one ``FusedSparseStep`` per bucket (its segment table, workspace, pack
+    buffers, mask and result block are that bucket's); ``grads`` ... ``vs``:
+    the buckets' tensors, same order.  Outputs land where the single-bucket
+    ``step`` puts them; returns [(idx[:k], values[:k])] per bucket.  The
+    buckets share dtypes, score and knobs; the short dependent kernels around
+    their selects run once for up to eight buckets."""
+    nb = len(steppers)
+    if not (nb == len(grads) == len(resids) == len(ps) == len(ms) == len(vs)) or nb == 0:
+        raise ValueError("one gradient / residual / p / m / v per bucket")
+    flags = FusedSparseStep._flags(optimizer, fold, interval, 1.0)
+    if score not in SCORE_MAP:
+        raise ValueError(f"Unknown SGA score '{score}'. Registered: {sorted(SCORE_MAP)}")
+    if ks is None:
+        ks = [k_for(fs.n, ratio_percent) for fs in steppers]
+    table = (L.FusedBucket * nb)()
+    gd, vd = L.dtype_code(grads[0]), L.dtype_code(steppers[0].values)
+    for b, fs in enumerate(steppers):
+        g, r, p, m, v = grads[b], resids[b], ps[b], ms[b], vs[b]
+        for t in (g, r, p, m, v):
+            L.require_dev(t)
+            L.require_contig(t=t)
+            if t.numel() != fs.n:
+                raise ValueError(f"bucket {b}: tensor length does not match the bucket")
+        if L.dtype_code(g) != gd or L.dtype_code(fs.values) != vd:
+            raise ValueError("the buckets of one call share the gradient and value dtypes")
+        if not (1 <= ks[b] <= min(fs.n, fs.max_k)):
+            raise ValueError(f"bucket {b}: k={ks[b]} out of range (n={fs.n}, max_k={fs.max_k})")
+        fs._upload_segments(step)
+        e = table[b]
+        e.g, e.resid, e.p, e.m, e.v = (t.data_ptr() for t in (g, r, p, m, v))
+        e.n, e.k = fs.n, ks[b]
+        e.segs, e.n_segs = fs._seg_dev.data_ptr(), len(fs.segments)
+        e.idx_out, e.values_out = fs.idx.data_ptr(), fs.values.data_ptr()
+        e.mask_out = fs.mask.data_ptr() if fs.mask is not None else None
+        e.result = fs.result.data_ptr()
+        e.ws, e.ws_bytes = fs.ws.data_ptr(), fs.ws_bytes
+    L.call("sga_fused_sparse_step_multi", table, nb, gd, SCORE_MAP[score], vd, L.f32(factor),
+           L.f32(coeff), 1 if fast else 0, flags, L.f32(interval), L.stream())
+    return [(fs.idx[:k], fs.values[:k]) for fs, k in zip(steppers, ks)]
+
+
 class PackedState:
     """resid, p, m, v of one bucket interleaved in 64 KiB records
     ``[resid[4096] | p[4096] | m[4096] | v[4096]]`` (the layout of

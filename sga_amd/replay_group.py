@@ -138,9 +138,12 @@ class ReplayGroup:
         self.qn2 = torch.zeros(G, dtype=torch.float64, device=dev)
         self.coef_d = torch.ones(G, dtype=torch.float64, device=dev)
         self.coef_f = torch.ones(G, dtype=torch.float32, device=dev)
+        # one select workspace and result block per configuration that can re-select in the
+        # same step (allocated on first use)
         self.ws_bytes = int(L.raw("sga_select_workspace_bytes", self.N))
-        self.ws = torch.empty(self.ws_bytes, dtype=torch.uint8, device=dev)
-        self.sel_result = torch.zeros(8, dtype=torch.int32, device=dev)
+        self._ws = []
+        self.sel_results = torch.zeros(G, 8, dtype=torch.int32, device=dev)
+        self._last_result = self.sel_results[0]
         if selection_semantics == "balanced-histogram":
             # every tensor is subsampled on its own param-relative stride-8 grid
             phases = [(-int(e.get("p_off", 0))) % _BAL_STRIDE for e in entries]
@@ -161,6 +164,11 @@ class ReplayGroup:
         # the kernels then skip its traffic (same values either way)
         self.res_zero = [True] * len(configs)
         self.si = 0
+
+    def _select_ws(self, j):
+        while len(self._ws) <= j:
+            self._ws.append(torch.empty(self.ws_bytes, dtype=torch.uint8, device=self.dev))
+        return self._ws[j]
 
     # -- per-step tables ----------------------------------------------------
     def _fill_segments(self, count, lr_of):
@@ -217,25 +225,38 @@ class ReplayGroup:
         L.call("sga_replay_pass1", L.ptr(g), gd, N, L.f32(coef_dense), clip, self._cfg_host, G,
                L.ptr(self.partials), L.ptr(self.qn2), L.ptr(self.coef_d), L.ptr(self.coef_f), st)
         out_sel = {}
-        for ci, c in enumerate(self.configs):        # boundary re-selection
-            if not (bnd[ci] and si > 0 and si + 1 < self.W):
-                continue
-            s = self.state[ci]
-            state_ptrs = [C.c_void_p(s.base(x)) for x in ("res", "w", "m", "v")]
-            tail = [C.c_void_p(self.coef_f.data_ptr() + 4 * ci), L.f32(coef_dense),
-                    int(c.optimizer == "adams"), 1, int(self.res_zero[ci]), L.ptr(s.spare),
-                    L.ptr(self.sel_result)]
+        # boundary re-selections of this step: under the exact-k semantics they go out as ONE
+        # call (configs that rank by the same score share the short kernels of the select)
+        resel = [ci for ci, c in enumerate(self.configs)
+                 if bnd[ci] and si > 0 and si + 1 < self.W]
+        if resel and self.semantics == "topk":
+            jobs = (L.ReselectJob * len(resel))()
+            for j, ci in enumerate(resel):
+                c, s, e = self.configs[ci], self.state[ci], jobs[j]
+                e.res, e.w, e.m, e.v = (s.base(x) for x in ("res", "w", "m", "v"))
+                e.k, e.score_id = self.ks[c.ratio], SCORE_MAP[c.score]
+                e.adams, e.res_zero = int(c.optimizer == "adams"), int(self.res_zero[ci])
+                e.coef_f = self.coef_f.data_ptr() + 4 * ci
+                e.sel_out = s.spare.data_ptr()
+                e.result = self.sel_results[j].data_ptr()
+                ws = self._select_ws(j)
+                e.ws, e.ws_bytes = ws.data_ptr(), self.ws_bytes
+            L.call("sga_replay_reselect_multi", L.ptr(g), gd, N, L.ptr(self._seg_dev),
+                   len(self.entries), L.f32(coef_dense), 1, jobs, len(resel), st)
+            self._last_result = self.sel_results[len(resel) - 1]
+        for ci in resel:
+            c, s = self.configs[ci], self.state[ci]
             if self.semantics == "balanced-histogram":
                 k = self.ks[c.ratio]
                 rank = max(1, round(self._n_sampled * (N - k + 1) / N))   # _histogram.py:122
-                L.call("sga_replay_reselect_balanced", L.ptr(g), gd, *state_ptrs, N, rank,
+                L.call("sga_replay_reselect_balanced", L.ptr(g), gd,
+                       *[C.c_void_p(s.base(x)) for x in ("res", "w", "m", "v")], N, rank,
                        L.ptr(self._seg_dev), len(self.entries), L.ptr(self._seg_phase),
-                       SCORE_MAP[c.score], *tail, L.ptr(self._bal_hist), L.ptr(self.ws),
-                       self.ws_bytes, st)
-            else:
-                L.call("sga_replay_reselect", L.ptr(g), gd, *state_ptrs, N, self.ks[c.ratio],
-                       L.ptr(self._seg_dev), len(self.entries), SCORE_MAP[c.score], *tail,
-                       L.ptr(self.ws), self.ws_bytes, st)
+                       SCORE_MAP[c.score], C.c_void_p(self.coef_f.data_ptr() + 4 * ci),
+                       L.f32(coef_dense), int(c.optimizer == "adams"), 1, int(self.res_zero[ci]),
+                       L.ptr(s.spare), L.ptr(self.sel_results[0]), L.ptr(self._bal_hist),
+                       L.ptr(self._select_ws(0)), self.ws_bytes, st)
+                self._last_result = self.sel_results[0]
             if c.dual_lr != 1.0:
                 out_sel[ci] = s.sel
             s.sel, s.spare = s.spare, s.sel
@@ -254,4 +275,5 @@ class ReplayGroup:
         self.si += 1
 
     def last_select(self):
-        return read_result(self.sel_result)
+        """Result block of the last re-selection launched."""
+        return read_result(self._last_result)

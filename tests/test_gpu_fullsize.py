@@ -145,6 +145,48 @@ def test_qwen06b_set_mask_layout_per_bucket(dev):
         assert torch.equal(dst, torch.where(fs.mask.bool(), buf, torch.zeros((), device=dev)))
 
 
+def test_qwen06b_set_mask_layout_buckets_in_one_call(dev):
+    """Config 2 through `sga_fused_sparse_step_multi`: the eight buckets of the
+    Qwen3-0.6B set stepped by ONE call (their short select kernels batched)
+    give, bucket by bucket, the bits of eight separate calls over two steps."""
+    from sga_amd.fused_step import FusedSparseStep, fused_step_multi, k_for
+    from sga_amd.shapes import qwen3_06b, segments_for
+    segs, n = segments_for(qwen3_06b())
+    grads = [_qwen_log_uniform_grads(dev, segs, n, 5 + i) for i in range(2)]
+    cuts = [0, segs[1]["start"]] + [segs[1 + 11 * j]["start"] for j in range(4, 28, 4)] + [n]
+    spans = list(zip(cuts[:-1], cuts[1:]))
+    gen = torch.Generator(device=dev).manual_seed(5)
+    p0 = torch.randn(n, generator=gen, device=dev) * 0.02
+    state = [[torch.zeros(n, device=dev), p0.clone(), torch.zeros(n, device=dev),
+              torch.zeros(n, device=dev)] for _ in range(2)]                 # r, p, m, v
+    steppers = []
+    for which in range(2):
+        row = []
+        for lo, hi in spans:
+            bsegs = [dict(s, start=s["start"] - lo) for s in segs if lo <= s["start"] < hi]
+            row.append(FusedSparseStep(hi - lo, bsegs, dev, values_dtype=torch.float32,
+                                       max_k=k_for(hi - lo, 1.0), want_mask=True))
+        steppers.append(row)
+    ks = [k_for(hi - lo, 1.0) for lo, hi in spans]
+    for step in (1, 2):
+        g = grads[step - 1]
+        for b, (lo, hi) in enumerate(spans):
+            steppers[0][b].step(g[lo:hi], *[t[lo:hi] for t in state[0]], step, k=ks[b])
+        fused_step_multi(steppers[1], [g[lo:hi] for lo, hi in spans],
+                         *[[state[1][a][lo:hi] for lo, hi in spans] for a in range(4)], step,
+                         ks=ks)
+        for b in range(len(spans)):
+            a, c = steppers[0][b], steppers[1][b]
+            ra, rc = a.read_result(), c.read_result()
+            assert rc.status == 0 and rc.n_selected == ks[b] and rc.path == 1, (step, b, vars(rc))
+            assert vars(ra) == vars(rc), (step, b)
+            assert torch.equal(a.idx[:ks[b]], c.idx[:ks[b]]) and torch.equal(a.mask, c.mask)
+            assert torch.equal(a.values[:ks[b]].view(torch.int32),
+                               c.values[:ks[b]].view(torch.int32))
+        for x, y in zip(state[0], state[1]):
+            assert torch.equal(x.view(torch.int32), y.view(torch.int32)), step
+
+
 def _dev_scalar(x, dev):
     return torch.tensor(x, dtype=torch.float32, device=dev)
 
@@ -157,7 +199,8 @@ def _update_score_torch(segs, p, m, v, q, step):
     dev = q.device
     out = torch.empty_like(q)
     for s in segs:
-        a, b = s["start"], s["start"] + s["n"]
+        a = s["start"] if "start" in s else s["a"]
+        b = a + s["n"]
         b1, b2 = s["b1"], s["b2"]
         sa = (m[a:b] * b1 + q[a:b] * (1.0 - b1)) / _dev_scalar(1.0 - b1 ** step, dev)
         sb = (v[a:b] * b2 + (q[a:b] * (1.0 - b2)) * q[a:b]) / _dev_scalar(1.0 - b2 ** step, dev)
@@ -403,11 +446,12 @@ def test_qwen06b_replay_group_full_window(dev):
     * off a boundary the residual is zero on the mask and the running fp32 sum
       of the recorded gradient since the last boundary elsewhere;
     * the re-selection at si = 16 of the T = 16 arm (15 masked steps of
-      residual behind it) and at si = 28 of a T = 4 `update` arm equal the exact
-      top-k of the score rebuilt from the state just before that step;
+      residual behind it), at si = 28 of a T = 4 `update` arm and at si = 24 of
+      a T = 4 residual-blind arm equal the exact top-k of the score rebuilt,
+      with plain torch ops on the device, from the state just before that step;
     * with clipping off, a T = 1 arm is the dense reference trajectory
       (sga_dense_replay_step) bit for bit."""
-    from sga_amd.replay import score_formula, select_topk_flat
+    from sga_amd.replay import select_topk_flat
     from sga_amd.replay_dense import DenseReplay
     from sga_amd.replay_group import Config, ReplayGroup
     from sga_amd.shapes import qwen3_06b, segments_for
@@ -417,7 +461,7 @@ def test_qwen06b_replay_group_full_window(dev):
     entries = [{"a": s["start"], "n": s["n"], "b1": s["b1"], "b2": s["b2"], "eps": s["eps"],
                 "wd": s["wd"]} for s in segs]
     specs = [("abs_g", 1.0, 1), ("abs_g", 0.1, 4), ("abs_g", 10.0, 16), ("update", 1.0, 4),
-             ("update", 10.0, 1), ("coi", 1.0, 16), ("coi", 0.1, 4), ("update", 0.1, 16)]
+             ("update", 10.0, 1), ("coi", 1.0, 16), ("abs_g_blind", 1.0, 4), ("update", 0.1, 16)]
     cfgs = [Config(*sp) for sp in specs]
     gen = torch.Generator(device=dev).manual_seed(1)
     w0 = torch.randn(n, generator=gen, device=dev) * 0.02
@@ -432,7 +476,7 @@ def test_qwen06b_replay_group_full_window(dev):
     grp = ReplayGroup(entries, w0, m0, v0, sel0, cfgs, t0, W)
     del sel0
     meta = {"clip_grad": 1.0, "grad_norm": float("nan"), "lr": lr}
-    probes = {16: 2, 28: 3}                       # si -> config whose re-selection is rebuilt
+    probes = {16: 2, 24: 6, 28: 3}                # si -> config whose re-selection is rebuilt
     for si in range(W):
         pre = None
         if si in probes:
@@ -445,17 +489,15 @@ def test_qwen06b_replay_group_full_window(dev):
             coef = grp.coef_f[ci:ci + 1]
             assert 0.0 < float(coef) < 1.0                     # the clip is live
             q = (window[si].float() + pre["res"]) * coef       # coef_dense == 1 (no recorded norm)
+            assert float(pre["res"].abs().max()) > 0.0         # a live residual behind the boundary
             if c.score == "abs_g":
                 score = q.abs()
+            elif c.score == "abs_g_blind":
+                score = (window[si].float() * coef).abs()      # the residual takes no part
             else:
-                score = torch.empty_like(q)
-                count = t0 + si + 1
-                for e in entries:
-                    a, b = e["a"], e["a"] + e["n"]
-                    score[a:b] = score_formula(c.score, pre["w"][a:b], pre["m"][a:b],
-                                               pre["v"][a:b], q[a:b], e["b1"], e["b2"], e["eps"],
-                                               e["wd"], 1 - e["b1"] ** count, 1 - e["b2"] ** count,
-                                               "adamw", update_includes_wd=True).abs()
+                assert c.score == "update"
+                score = _update_score_torch(entries, pre["w"], pre["m"], pre["v"], q,
+                                            t0 + si + 1)
             _select_ok(score, grp.state[ci]["sel"].bool(), ks[ci])
             del pre, q, score
     for ci, c in enumerate(cfgs):

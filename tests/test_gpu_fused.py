@@ -274,3 +274,65 @@ def test_randomized_configurations(dev, seed):
         it = torch.int16 if vdtype == torch.bfloat16 else torch.int32
         assert torch.equal(vals.cpu().view(it), val_ref.view(it)), step
         assert same_bits(dr, r) and same_bits(dm, m) and same_bits(dv, v) and same_bits(dp, p), step
+
+
+@pytest.mark.parametrize("score,vdtype,knobs", [("abs_g", torch.float32, {}),
+                                                ("update", torch.bfloat16, {}),
+                                                ("coi", torch.bfloat16, dict(optimizer="adams")),
+                                                ("abs_g", torch.bfloat16,
+                                                 dict(fold=True, interval=3.0, coeff=0.5))])
+def test_multi_bucket_step_equals_the_oracle_bucket_by_bucket(dev, score, vdtype, knobs):
+    """`sga_fused_sparse_step_multi`: eleven buckets in one call -- more than
+    one batch of eight, large ones (the sampled-bracket path, ragged tensors)
+    mixed with buckets below 2^20 elements (the radix passes) and one of a
+    single tensor of three elements -- each with its own k.  Three steps with
+    the device state carried over; every bucket's idx, values, mask, residual,
+    p, m, v and threshold equal the oracle's step of that bucket on its own."""
+    from sga_amd.fused_step import FusedSparseStep, fused_step_multi
+    layouts = [[1 << 20, 130, 37], [300_000, 1024, 100_001], [1_200_000], [3], [700_000, 5, 400_001],
+               [65_536], [1 << 20], [999], [250_000, 250_000], [1_048_577, 7], [40_000, 3, 17]]
+    ratios = [1.0, 10.0, 0.1, 50.0, 1.0, 0.5, 3.0, 1.0, 0.01, 1.0, 25.0]
+    bk = []
+    for b, sizes in enumerate(layouts):
+        segs, n = _segments(sizes, vary=b % 2 == 1)
+        gen = torch.Generator().manual_seed(100 + b)
+        p = torch.randn(n, generator=gen) * 0.02
+        host = [torch.zeros(n), p, torch.zeros(n), torch.zeros(n)]          # r, p, m, v
+        bk.append(dict(segs=segs, n=n, k=SEL.k_for(n, ratios[b]), host=host,
+                       devs=[t.to(dev) for t in host],
+                       fs=FusedSparseStep(n, segs, dev, values_dtype=vdtype, want_mask=True)))
+    it = torch.int16 if vdtype == torch.bfloat16 else torch.int32
+    for step in (1, 2, 3):
+        grads = [student_t(x["n"], 7 * step + b).to(torch.bfloat16) for b, x in enumerate(bk)]
+        outs = fused_step_multi([x["fs"] for x in bk], [g.to(dev) for g in grads],
+                                *[[x["devs"][a] for x in bk] for a in range(4)], step,
+                                ks=[x["k"] for x in bk], score=score, **knobs)
+        for b, x in enumerate(bk):
+            r, p, m, v = x["host"]
+            idx_ref, val_ref, mask_ref, th_ref = OF.fused_sparse_step(
+                grads[b], r, p, m, v, x["segs"], step, k=x["k"], score=score, values_dtype=vdtype,
+                **knobs)
+            res = x["fs"].read_result()
+            what = (step, b, vars(res))
+            assert res.status == 0 and res.n_selected == x["k"] and res.thresh == th_ref, what
+            assert res.path == (1 if x["n"] >= 1 << 20 else 0), what
+            idx, vals = outs[b]
+            assert torch.equal(idx.cpu(), idx_ref), what
+            assert torch.equal(x["fs"].mask.cpu().bool(), mask_ref), what
+            assert torch.equal(vals.cpu().view(it), val_ref.view(it)), what
+            for d, h in zip(x["devs"], x["host"]):
+                assert same_bits(d, h), what
+
+
+def test_multi_bucket_step_refusals(dev):
+    from sga_amd.fused_step import FusedSparseStep, fused_step_multi
+    segs, n = _segments([5000])
+    fs = [FusedSparseStep(n, segs, dev, values_dtype=torch.float32) for _ in range(2)]
+    t = [torch.zeros(n, device=dev) for _ in range(2)]
+    with pytest.raises(ValueError, match="one gradient"):
+        fused_step_multi(fs, t, t, t, t, t[:1], 1, ratio_percent=1.0)
+    with pytest.raises(ValueError, match="out of range"):
+        fused_step_multi(fs, t, t, t, t, t, 1, ks=[10, n + 1])
+    fs[1] = FusedSparseStep(n, segs, dev, values_dtype=torch.bfloat16)
+    with pytest.raises(ValueError, match="share the gradient and value dtypes"):
+        fused_step_multi(fs, t, t, t, t, t, 1, ratio_percent=1.0)
