@@ -570,6 +570,9 @@ def main():
     ap.add_argument("--sweep", action="store_true",
                     help="also time the whole sweep {two-sweep, single-sweep} x {update, abs_g} x "
                          "{0.1, 1, 10 %} x {separate, packed} (24 legs; written to the detail file)")
+    ap.add_argument("--headline-only", action="store_true",
+                    help="time the headline configuration alone: no other step variant, no other "
+                         "layout, no stream-mix copy (what the profiles are taken on)")
     ap.add_argument("--no-rows", action="store_true",
                     help="skip the Qwen3-0.6B mask-layout row and the 1e9 stress row")
     ap.add_argument("--detail", default=os.path.join(ROOT, "gpurun_out", "bench_detail.json"),
@@ -715,7 +718,7 @@ def main():
 
     head = time_leg(args.layout, args.score, args.ratio, args.warmup, args.steps, args.single_sweep)
     stream_mix = None
-    if args.layout == "separate":
+    if args.layout == "separate" and not args.headline_only:
         # What the same five read and four write streams reach WITHOUT the math, on the very
         # tensors the headline ran on: the ceiling this placement of four flat tensors gives a
         # kernel of that stream mix.  (It scribbles over r / p / m / v: they are reset below.)
@@ -729,10 +732,12 @@ def main():
         m.zero_(); v.zero_(); r.zero_()
         state["t"] = 0
     # the other step variant and the other layout of the headline configuration
-    other = time_leg(args.layout, args.score, args.ratio, 2, 5, not args.single_sweep)
-    two = other if args.single_sweep else head
-    packed_leg = time_leg("packed" if args.layout == "separate" else "separate", args.score,
-                          args.ratio, 2, 5, args.single_sweep)
+    other = packed_leg = None
+    if not args.headline_only:
+        other = time_leg(args.layout, args.score, args.ratio, 2, 5, not args.single_sweep)
+        packed_leg = time_leg("packed" if args.layout == "separate" else "separate", args.score,
+                              args.ratio, 2, 5, args.single_sweep)
+    two = head if not args.single_sweep else other
     sweep = []
     if args.sweep:
         for single in (False, True):
@@ -772,16 +777,18 @@ def main():
         "step_roofline": {"bytes_per_elem": head["moved_bytes_per_elem"],
                           "frac": head["step_frac"],
                           "other_kernels_ms": head["other_kernels_ms"]},
-        "two_sweep": {"ms_per_step": two["ms_per_step"], "elem_per_s": two["elem_per_s"],
-                      "bytes_per_elem": two["moved_bytes_per_elem"], "frac": two["step_frac"],
-                      "k_fused_final_ms": two["final_avg_ms"], "k_fused_final_frac": two["final_frac"],
-                      "k_bracket_sweep_ms": two["sweep_avg_ms"],
-                      "k_bracket_sweep_frac": two["sweep_frac"]},
-        ("packed_layout" if args.layout == "separate" else "separate_layout"): {
+    }
+    if two is not None:
+        out["two_sweep"] = {
+            "ms_per_step": two["ms_per_step"], "elem_per_s": two["elem_per_s"],
+            "bytes_per_elem": two["moved_bytes_per_elem"], "frac": two["step_frac"],
+            "k_fused_final_ms": two["final_avg_ms"], "k_fused_final_frac": two["final_frac"],
+            "k_bracket_sweep_ms": two["sweep_avg_ms"], "k_bracket_sweep_frac": two["sweep_frac"]}
+    if packed_leg is not None:
+        out["packed_layout" if args.layout == "separate" else "separate_layout"] = {
             "ms_per_step": packed_leg["ms_per_step"], "elem_per_s": packed_leg["elem_per_s"],
             "frac": packed_leg["step_frac"], "dominant_kernel_ms": packed_leg["final_avg_ms"],
-            "dominant_kernel_frac": packed_leg["final_frac"]},
-    }
+            "dominant_kernel_frac": packed_leg["final_frac"]}
     detail = {"headline_leg": head, "other_variant_leg": other, "other_layout_leg": packed_leg,
               "select": head["select"], "traffic_source": traffic_src,
               "stream_mix_copy": stream_mix}

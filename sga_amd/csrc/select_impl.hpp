@@ -1395,6 +1395,8 @@ static __global__ __launch_bounds__(kBlock) void k_mask_to_planes(const uint8_t*
 template <class Src>
 static inline void run_select_batch(const SrcPack<Src>& srcs, const SelBatch& B, bool fast, int pm,
                                     hipStream_t s, double sigmas = 5.0) {
+  static_assert(sizeof(ChainJobs) + sizeof(SrcPack<Src>) + 64 <= 4096,
+                "the operands of a batched chain kernel travel in its 4 KiB of kernel arguments");
   hipLaunchKernelGGL(k_chain_begin, B.grid(1), dim3(kBlock), 0, s, B.jobs, fast ? 1 : 0, sigmas);
   if (fast) {
     hipLaunchKernelGGL((k_sample<Src>), B.grid(stream_grid(B.max_nsv, kBlock)), dim3(kBlock), 0, s,
