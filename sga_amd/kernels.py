@@ -120,3 +120,44 @@ def masked_norm_sq_contribution(grad, mask, total_norm_sq):
         mk = mk.view(torch.uint8)
     L.call("sga_masked_norm_sq", L.ptr(g), L.ptr(mk), n, L.ptr(_partials(n, g.device)),
            L.ptr(total_norm_sq), L.stream())
+
+
+def _as_int(s):
+    return int(s.item()) if torch.is_tensor(s) else int(s)
+
+
+def _state_step(wrapper, group):
+    """The per-param ``state['step']`` of the first parameter of ``group`` that
+    has one (torch AdamW's counter style), or None."""
+    for p in group['params']:
+        st = wrapper.optimizer.state.get(p)
+        if st is not None and 'step' in st:
+            return _as_int(st['step'])
+    return None
+
+
+def sga_peek_step(wrapper, group):
+    """The step number the NEXT optimizer commit will use, read without
+    touching any counter (``sga/kernels.py:305-326``): the group counter + 1
+    when the optimizer keeps one (TE / apex FusedAdam), else the first
+    per-param state counter + 1 (torch AdamW), else 1."""
+    if 'step' in group:
+        return _as_int(group['step']) + 1
+    s = _state_step(wrapper, group)
+    return 1 if s is None else s + 1
+
+
+def sga_advance_step(wrapper, group):
+    """Advance the shared Adam step counter by one and return the new value as
+    a Python int (``sga/kernels.py:329-367``).  A group without a counter is
+    seeded ONCE per wrapper from the per-param state (0 when there is none);
+    every group then starts from that seed."""
+    if 'step' in group:
+        group['step'] = _as_int(group['step']) + 1
+        return group['step']
+    if not getattr(wrapper, '_sga_step_seeded', False):
+        s = _state_step(wrapper, group)
+        wrapper._sga_step_seeded = True
+        wrapper._sga_step_seed_value = 0 if s is None else s
+    group['step'] = wrapper._sga_step_seed_value + 1
+    return group['step']

@@ -12,6 +12,30 @@ OPTIMIZERS = ("adamw", "adams")
 ADAMS_BIAS_CORRECTION = 1.0
 
 
+# Declared dtypes of a replay run (``sga/replay.py:96-119``): the scans of this build hold their
+# state in fp32; fp64 names the reference's host-side self-check, which is not a scan.
+REPLAY_DTYPES = {"fp32": torch.float32, "fp64": torch.float64}
+
+
+def resolve_replay_dtype(value):
+    try:
+        return REPLAY_DTYPES[value]
+    except (KeyError, TypeError):
+        raise ValueError(f"--replay-dtype must be one of {sorted(REPLAY_DTYPES)}, "
+                         f"got {value!r}") from None
+
+
+def require_scan_dtypes(replay_dtype, norm_dtype):
+    """Scans are fp32-only, as in the reference (``sga/replay.py:109-119``)."""
+    resolve_replay_dtype(replay_dtype)
+    if norm_dtype not in REPLAY_DTYPES:
+        raise ValueError(f"--norm-dtype must be one of {sorted(REPLAY_DTYPES)}, "
+                         f"got {norm_dtype!r}")
+    if replay_dtype != "fp32" or norm_dtype != "fp32":
+        raise ValueError("offline scans require --replay-dtype fp32 and --norm-dtype fp32; "
+                         "fp64 is reserved for --self-check")
+
+
 def _bc_pair(optimizer, count, b1, b2):
     """``sga/replay.py:132-137``"""
     if optimizer == "adamw":

@@ -6,7 +6,7 @@ without the report/ranking diagnostics).
 import torch
 
 from . import _lib as L
-from .replay import _bc_pair, select_topk_flat
+from .replay import _bc_pair, require_scan_dtypes, select_topk_flat
 from .replay_dense import dense_replay_dev
 from .replay_fused import shard_select_balanced
 from .replay_group import SELECTION_SEMANTICS, Config, ReplayGroup
@@ -75,7 +75,7 @@ def _branch_grad(state_path, sp, device):
 
 
 def replay_window(trace_dir, t0, window, configs, horizons, device,
-                  selection_semantics="topk", depth=2):
+                  selection_semantics="topk", depth=2, replay_dtype="fp32", norm_dtype="fp32"):
     """Replays ``configs`` (``replay_group.Config``) over the recorded window
     that starts at branch point ``t0``.  ``selection_semantics`` applies to
     BOTH select sites, the branch-point select and every boundary
@@ -87,6 +87,7 @@ def replay_window(trace_dir, t0, window, configs, horizons, device,
     ``ReplayGroup`` for inspection.
     """
     replay_switches()
+    require_scan_dtypes(replay_dtype, norm_dtype)
     if selection_semantics not in SELECTION_SEMANTICS:
         raise ValueError(f"unknown selection semantics {selection_semantics!r} "
                          f"(expected one of {SELECTION_SEMANTICS})")

@@ -135,3 +135,38 @@ def test_result_block_decoding():
     assert r.path == 1 and r.negative and r.status == 0 and r.nonfinite == 0
     r = read_result(torch.tensor([th, 3, 10, 5, 13, 2, 3, 2], dtype=torch.int32))
     assert r.path == 2 and not r.negative and r.status == 3 and r.nonfinite == 2
+
+
+def test_step_counter_helpers():
+    """``sga_peek_step`` / ``sga_advance_step`` on the two counter styles of
+    ``sga/kernels.py:305-367``: a group counter (int or tensor), and per-param
+    state counters that seed the group counter once per wrapper."""
+    from types import SimpleNamespace
+    from sga_amd.kernels import sga_advance_step, sga_peek_step
+    p1, p2 = object(), object()
+    w = SimpleNamespace(optimizer=SimpleNamespace(state={}))
+    g = {'params': [p1, p2]}
+    assert sga_peek_step(w, g) == 1 and 'step' not in g              # nothing anywhere: first commit
+    g['step'] = torch.tensor(6)
+    assert sga_peek_step(w, g) == 7 and int(g['step']) == 6          # read-only
+    assert sga_advance_step(w, g) == 7 and g['step'] == 7 and isinstance(g['step'], int)
+    # torch-AdamW style: per-param state['step'], seeded once, shared by every group
+    w = SimpleNamespace(optimizer=SimpleNamespace(state={p2: {'step': torch.tensor(41.0)}}))
+    ga, gb = {'params': [p1, p2]}, {'params': [p1]}
+    assert sga_peek_step(w, ga) == 42 and 'step' not in ga
+    assert sga_advance_step(w, ga) == 42 and sga_advance_step(w, ga) == 43
+    assert sga_advance_step(w, gb) == 42                              # the wrapper's one seed
+    w = SimpleNamespace(optimizer=SimpleNamespace(state={}))
+    assert sga_advance_step(w, {'params': [p1]}) == 1                 # fresh moments seed 0
+
+
+def test_replay_dtype_guards():
+    from sga_amd.replay import require_scan_dtypes, resolve_replay_dtype
+    assert resolve_replay_dtype("fp32") is torch.float32
+    with pytest.raises(ValueError, match="--replay-dtype must be one of"):
+        resolve_replay_dtype("bf16")
+    with pytest.raises(ValueError, match="--norm-dtype must be one of"):
+        require_scan_dtypes("fp32", "half")
+    with pytest.raises(ValueError, match="reserved for --self-check"):
+        require_scan_dtypes("fp64", "fp32")
+    require_scan_dtypes("fp32", "fp32")
