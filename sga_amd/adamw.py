@@ -5,12 +5,12 @@ reference's signatures, refusals and step order."""
 import ctypes as C
 import math
 from dataclasses import dataclass, field
-from types import SimpleNamespace
 from typing import Optional
 
 import torch
 
 from . import _lib as L
+from .config import get_args
 from .scores import SCORE_MAP
 
 _BLOCK_SIZE = 1024
@@ -335,11 +335,11 @@ class OptContext:
 
 
 class SgaAdamW:
-    """grad-correct + residual reset (``adamw.py:795-986``).  Constructed from
-    an args namespace carrying the ``sga_*`` flags it reads."""
+    """grad-correct + residual reset (``adamw.py:795-986``).  Reads its
+    ``sga_*`` flags from the args singleton, like the reference (``:798-799``)."""
 
-    def __init__(self, args=None):
-        args = args or SimpleNamespace()
+    def __init__(self):
+        args = get_args()
         self.residual_mean = bool(getattr(args, "sga_optimizer_residual_mean", False))
         self.compact_search = getattr(args, "sga_optimizer_compact_search", "table")
         s = float(getattr(args, "sga_optimizer_full_sync_inactive_lr_scale", 1.0))

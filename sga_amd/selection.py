@@ -13,6 +13,7 @@ from types import SimpleNamespace
 import torch
 
 from . import _lib as L
+from .config import get_args
 
 _HIST_MODES = {"exact": (16, 32769, 1), "balanced": (16, 32769, 8),
                "fast": (19, 4097, 8)}            # _histogram.py:68-72
@@ -330,10 +331,11 @@ class ExactKthvalue:
 
 
 class TopkSelection:
-    """``selection/topk.py:59-167``; ``args`` carries the ``sga_selection_*``
-    flags (the reference reads them from its config singleton)."""
+    """``selection/topk.py:59-167``; reads the ``sga_selection_*`` flags from
+    the args singleton, like the reference (``:59-60``)."""
 
-    def __init__(self, args):
+    def __init__(self):
+        args = get_args()
         self.method = args.sga_selection_method
         self.ratio_percent = float(args.sga_selection_ratio_percent)
         assert 0.0 < self.ratio_percent < 100.0, (

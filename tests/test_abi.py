@@ -170,3 +170,32 @@ def test_replay_dtype_guards():
     with pytest.raises(ValueError, match="reserved for --self-check"):
         require_scan_dtypes("fp64", "fp32")
     require_scan_dtypes("fp32", "fp32")
+
+
+def test_plugins_read_the_args_singleton():
+    """``SgaAdamW()`` / ``TopkSelection()`` take no arguments and read the
+    ``sga_*`` flags from the args singleton (``sga/config/__init__.py:36-51``,
+    ``adamw.py:798-799``, ``topk.py:59-60``); unset, they fail loudly."""
+    from types import SimpleNamespace
+    from sga_amd import config
+    from sga_amd.adams import SgaAdamS
+    from sga_amd.adamw import SgaAdamW
+    from sga_amd.selection import TopkSelection
+    config.set_args(None)
+    with pytest.raises(RuntimeError, match="sga args not set"):
+        SgaAdamW()
+    config.set_args(SimpleNamespace(sga_score="coi", sga_optimizer_residual_mean=True,
+                                    sga_optimizer_compact_search="bisection",
+                                    sga_optimizer_full_sync_inactive_lr_scale=0.25,
+                                    sga_selection_method="histogram",
+                                    sga_selection_ratio_percent=2.5,
+                                    sga_selection_histogram_mode="balanced"))
+    for cls in (SgaAdamW, SgaAdamS):
+        o = cls()
+        assert (o.residual_mean, o.compact_search, o.full_sync_inactive_lr_scale, o.emit_score) == (
+            True, "bisection", 0.25, "coi")
+    s = TopkSelection()
+    assert s.method == "histogram" and s.ratio_percent == 2.5 and s.k_for(1000) == 25
+    config.set_args(SimpleNamespace(sga_score="nope"))
+    with pytest.raises(ValueError, match="no EMIT_MODE branch"):
+        SgaAdamW()

@@ -36,18 +36,20 @@ def _mk(dev, sizes, seed=0):
 @pytest.mark.parametrize("compact", [True, False])
 def test_full_then_sparse_cycle(dev, compact):
     from sga_amd.adamw import OptContext, SgaAdamW, build_dir_table
+    from sga_amd.config import set_args
     from sga_amd.kernels import compact_norm_sq_contribution, pack_selected
     from sga_amd.selection import TopkSelection
     from sga_amd.support import compact_mask_u8
     sizes = [120_000, 1024, 77_777, 128]
     n, w, bucket, recs = _mk(dev, sizes)
-    args = SimpleNamespace(sga_score="abs_g", sga_optimizer_residual_mean=True,
-                           sga_optimizer_compact_search="table",
-                           sga_optimizer_full_sync_inactive_lr_scale=1.0)
-    opt = SgaAdamW(args)
-    sel = TopkSelection(SimpleNamespace(sga_selection_method="histogram",
-                                        sga_selection_ratio_percent=2.0,
-                                        sga_selection_histogram_mode="exact"))
+    # the plugins read their flags from the args singleton, seeded once as the engine does
+    set_args(SimpleNamespace(sga_score="abs_g", sga_optimizer_residual_mean=True,
+                             sga_optimizer_compact_search="table",
+                             sga_optimizer_full_sync_inactive_lr_scale=1.0,
+                             sga_selection_method="histogram", sga_selection_ratio_percent=2.0,
+                             sga_selection_histogram_mode="exact"))
+    opt = SgaAdamW()
+    sel = TopkSelection()
     # oracle-side state
     ow, og = w.clone(), torch.zeros(n)
     om, ov = torch.zeros(n), torch.zeros(n)

@@ -116,9 +116,10 @@ def test_balanced_and_fast_tiers(dev, mode):
     assert t_dev == t_ref
     for a, b in zip(m_dev, m_ref):
         assert torch.equal(a.cpu(), b)
-    sel = TopkSelection(SimpleNamespace(sga_selection_method="histogram",
-                                        sga_selection_ratio_percent=5.0,
-                                        sga_selection_histogram_mode=mode))
+    from sga_amd.config import set_args
+    set_args(SimpleNamespace(sga_selection_method="histogram", sga_selection_ratio_percent=5.0,
+                             sga_selection_histogram_mode=mode))
+    sel = TopkSelection()
     masks = sel.select(SimpleNamespace(grad_views=[v.to(dev) for v in views]))
     assert sel.k_for(n_total) == k and sel.last_threshold == t_ref
     assert all(torch.equal(a.cpu(), b) for a, b in zip(masks, m_ref))
@@ -284,11 +285,12 @@ def test_adaptive_tau_trajectory_matches_oracle(dev):
     from types import SimpleNamespace
 
     from oracle import select as OS
+    from sga_amd.config import set_args
     from sga_amd.selection import TopkSelection
-    args = SimpleNamespace(sga_selection_method="adaptive", sga_selection_ratio_percent=10.0,
-                           sga_selection_adaptive_warmup_syncs=2,
-                           sga_selection_adaptive_warmup_mode="fast")
-    sel = TopkSelection(args)
+    set_args(SimpleNamespace(sga_selection_method="adaptive", sga_selection_ratio_percent=10.0,
+                             sga_selection_adaptive_warmup_syncs=2,
+                             sga_selection_adaptive_warmup_mode="fast"))
+    sel = TopkSelection()
     ref = OS.AdaptiveTau(10.0, 2, "fast")
     assert sel.warmup_sync_target(0, 4) == ref.warmup_sync_target(0, 4) == 1
     gen = torch.Generator().manual_seed(5)
