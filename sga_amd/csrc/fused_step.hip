@@ -1144,7 +1144,7 @@ static int run_fused_spec(const void* g, float* resid, float* p, float* m, float
                      n_segs, w.st, w.aux, w.seg_dir);
   prof_end(pp, s);
   hipLaunchKernelGGL(k_bracket_check, B.grid(1), dim3(kBlock), 0, s, B.jobs);
-  hipLaunchKernelGGL(k_cand_compact, B.grid(512), dim3(kBlock), 0, s, B.jobs);
+  hipLaunchKernelGGL(k_cand_compact, B.grid(kSegWaves / kChunksPerBlock), dim3(kBlock), 0, s, B.jobs);
   hipLaunchKernelGGL(k_spec_ovf_compact, dim3(64), dim3(kBlock), 0, s, w.aux, w.seg_cnt, x.ovf_idx,
                      x.ovf_key, x.ovf_rec, (uint32_t)x.ovf_cap, w.cand_idx, w.cand_key, x.cand_rec,
                      x.tie_cnt);

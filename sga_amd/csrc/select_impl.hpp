@@ -369,7 +369,10 @@ __device__ __forceinline__ void level_hist_body(Src& src, int64_t n,
                                                 SelState* __restrict__ st,
                                                 uint32_t* __restrict__ hist) {
   constexpr int NB = LEVEL == 2 ? kBinsSmall : kBinsBig;
-  __shared__ uint32_t s_h[NS][NB];
+  // Level 0 has no prefix: every state sees the same histogram of all keys, so it is built and
+  // flushed once (set 0) and every state's scan reads that one.
+  constexpr int NH = LEVEL == 0 ? 1 : NS;
+  __shared__ uint32_t s_h[NH][NB];
   __shared__ uint32_t s_suf[kBlock + 1];
   __shared__ uint32_t s_last;
   bool on[NS];
@@ -384,7 +387,7 @@ __device__ __forceinline__ void level_hist_body(Src& src, int64_t n,
   if (!any) return;
   if (n_dev && (int64_t)*n_dev < n) n = (int64_t)*n_dev;
 #pragma unroll
-  for (int q = 0; q < NS; ++q)
+  for (int q = 0; q < NH; ++q)
     for (int b = threadIdx.x; b < NB; b += kBlock) s_h[q][b] = 0u;
   __syncthreads();
   // Raw key buffers (sample, candidates) are short and sit in L2: what their passes cost is load
@@ -413,18 +416,28 @@ __device__ __forceinline__ void level_hist_body(Src& src, int64_t n,
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
 #pragma unroll
-        for (int q = 0; q < NS; ++q) {
+        for (int q = 0; q < NH; ++q) {
           uint32_t bin; bool part;
           level_bin<LEVEL>(key[u][e], prefix[q], full[u] || i + e < n, bin, part);
-          lds_hist_add(s_h[q], bin, part && on[q]);
+          const bool live = NH == NS ? on[q] : any;
+          // Raw key buffers are at most a few million keys for 64 workgroups of one wave per
+          // SIMD: what a pass costs there is the latency of each key's chain, and the folding of
+          // equal bins (two ballots, a cross-lane read and two scalar branches per key) is most of
+          // it.  A plain LDS atomic per lane is shorter; on a plateau (every lane on one bin) it
+          // serialises 64-fold, which for these few keys is a couple of microseconds.
+          if (std::is_same<Src, SrcU32>::value) {
+            if (part && live) atomicAdd(&s_h[q][bin], 1u);
+          } else {
+            lds_hist_add(s_h[q], bin, part && live);
+          }
         }
       }
     }
   }
   __syncthreads();
 #pragma unroll
-  for (int q = 0; q < NS; ++q) {
-    if (!on[q]) continue;
+  for (int q = 0; q < NH; ++q) {
+    if (NH == NS && !on[q]) continue;
     uint32_t* gh = level_hist_of<LEVEL>(hist + q * kHistStride);
     for (int b = threadIdx.x; b < NB; b += kBlock) {
       const uint32_t c = s_h[q][b];
@@ -443,7 +456,8 @@ __device__ __forceinline__ void level_hist_body(Src& src, int64_t n,
   __threadfence();
 #pragma unroll
   for (int q = 0; q < NS; ++q)
-    if (on[q]) level_scan_body<LEVEL>(&st[q], level_hist_of<LEVEL>(hist + q * kHistStride), s_suf);
+    if (on[q])
+      level_scan_body<LEVEL>(&st[q], level_hist_of<LEVEL>(hist + (NH == NS ? q : 0) * kHistStride), s_suf);
   if (threadIdx.x == 0) st[0].done[LEVEL] = 0u;
 }
 // over the data itself (a key source per job): the radix passes, state = st
