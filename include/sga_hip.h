@@ -520,10 +520,11 @@ int sga_replay_reselect(const void* g, int g_dtype, const float* res,
 /* The boundary re-selections of ONE recorded step in one call
  * (replay_fused.py:1752-1825 re-selects up to every configuration of the group
  * at a step): each job is what sga_replay_reselect takes for one
- * configuration, with a workspace of its own (distinct per job).  Jobs that
- * rank by the same score run their short select kernels as one batch (up to 8
- * per batch; the kernels take the job from the grid's second dimension), only
- * the score sweeps are launched per job.  Same outputs, job by job, as
+ * configuration, with a workspace of its own (distinct per job).  Up to 8 jobs
+ * form a batch whose short select kernels run once for all of them (the
+ * kernels take the job from the grid's second dimension); the kernels that
+ * form keys (sample, radix fallback) run once per score among the jobs, the
+ * score sweeps once per job.  Same outputs, job by job, as
  * sga_replay_reselect.  `jobs` is a HOST array, read before the call returns. */
 typedef struct sga_reselect_job {
   const float* res;

@@ -702,50 +702,89 @@ struct ReselJob {
   SelWorkspace ws;
 };
 
-// Exact top-k re-selection of up to kMaxJobs configurations that rank by the same score over
-// the same recorded gradient: their short select kernels run as one batched chain.
-template <bool BF16G, int SCORE>
+// A runtime score id as a compile-time constant for the key source templates.
+template <class F>
+static void with_score(int score_id, F&& f) {
+  switch (score_id) {
+    case 0: f(std::integral_constant<int, 0>{}); break;
+    case 1: f(std::integral_constant<int, 1>{}); break;
+    case 2: f(std::integral_constant<int, 2>{}); break;
+    case 3: f(std::integral_constant<int, 3>{}); break;
+    case 4: f(std::integral_constant<int, 4>{}); break;
+    default: f(std::integral_constant<int, 5>{}); break;
+  }
+}
+
+// Exact top-k re-selection of up to kMaxJobs configurations over the same recorded gradient: the
+// kernels of the select chain that do not form keys run once for all of them, the ones that do
+// (sample, score sweeps, radix fallback, ordered plane pass) once per score among them.
+// score[b]: score id of job b.  All jobs take the same path (sampled bracket or radix passes).
+template <bool BF16G>
 static int run_reselect(const void* g, int64_t n, const sga_segment* segs, int n_segs,
-                        float coef_dense, int packed, const ReselJob* rj, int count, hipStream_t s,
-                        const char* who) {
-  using Src = SrcReplay<BF16G, SCORE>;
+                        float coef_dense, int packed, const ReselJob* rj, const int* score,
+                        int count, hipStream_t s, const char* who) {
   static_assert(kMaxJobs <= 8, "one directory launch per batch");
-  SrcPack<Src> srcs = {};
   SegDirJobs dj = {};
   SelBatch B;
-  bool fast = true;
+  bool fast = true, any_hyper = false;
   for (int b = 0; b < count; ++b) {
     const ReselJob& r = rj[b];
-    const bool vec = aligned4(g, BF16G ? 2 : 4) && aligned4(r.res, 4) && aligned4(r.w, 4) &&
-                     aligned4(r.m, 4) && aligned4(r.v, 4);
-    srcs.s[b] = Src{g, r.res, r.w, r.m, r.v, r.coef_f, coef_dense, r.adams, vec, {},
-                    packed ? kPackExtra : 0, r.res_zero};
-    // only the Adam-normalised scores ever look a tensor up
-    srcs.s[b].sc.init(segs, n_segs, Src::kHyper ? r.ws.seg_dir : nullptr);
     dj.j[b].segs = segs; dj.j[b].dir = r.ws.seg_dir; dj.j[b].n = n; dj.j[b].n_segs = n_segs;
     ChainJob& J = B.add(r.ws, n, r.k, 0);
     J.planes = r.sel_out;
     J.result = r.result;
     fast = fast && SelBatch::fast_ok(r.ws, n);
+    any_hyper = any_hyper || score[b] == SGA_SCORE_UPDATE || score[b] == SGA_SCORE_COI ||
+                score[b] == SGA_SCORE_GR_OVER_SQRT_V;
   }
-  if (Src::kHyper) {
+  if (any_hyper) {                     // only the Adam-normalised scores ever look a tensor up
     const int64_t nb = (n + (1ll << kSegDirLog) - 1) >> kSegDirLog;
     hipLaunchKernelGGL(k_seg_dir_batch, B.grid(stream_grid(nb, kBlock, 128)), dim3(kBlock), 0, s, dj);
   }
-  run_select_batch(srcs, B, fast, 1, s);
-  finish_planes_batch(srcs, B, fast, s);
+  // the jobs of one score, as a sub-batch over the same workspaces, and their key sources
+  auto per_score = [&](auto&& phase) {
+    bool seen[SGA_SCORE_GR_OVER_SQRT_V + 1] = {};
+    for (int a = 0; a < count; ++a) {
+      if (seen[score[a]]) continue;
+      seen[score[a]] = true;
+      with_score(score[a], [&](auto tag) {
+        constexpr int SC = decltype(tag)::value;
+        using Src = SrcReplay<BF16G, SC>;
+        SrcPack<Src> srcs = {};
+        SelBatch sub;
+        for (int b = a; b < count; ++b) {
+          if (score[b] != score[a]) continue;
+          const ReselJob& r = rj[b];
+          const bool vec = aligned4(g, BF16G ? 2 : 4) && aligned4(r.res, 4) && aligned4(r.w, 4) &&
+                           aligned4(r.m, 4) && aligned4(r.v, 4);
+          Src& src = srcs.s[sub.count];
+          src = Src{g, r.res, r.w, r.m, r.v, r.coef_f, coef_dense, r.adams, vec, {},
+                    packed ? kPackExtra : 0, r.res_zero};
+          src.sc.init(segs, n_segs, Src::kHyper ? r.ws.seg_dir : nullptr);
+          ChainJob& J = sub.add(r.ws, n, r.k, 0);
+          J = B.jobs.j[b];
+        }
+        phase(srcs, sub);
+      });
+    }
+  };
+  chain_begin(B, fast, s);
+  if (fast) {
+    per_score([&](auto& srcs, const SelBatch& sub) { chain_sample(srcs, sub, s); });
+    chain_sample_levels(B, s);
+    per_score([&](auto& srcs, const SelBatch& sub) { chain_sweeps(srcs, sub, 1, s); });
+    chain_candidates(B, s);
+  }
+  per_score([&](auto& srcs, const SelBatch& sub) { chain_fallback(srcs, sub, s); });
+  launch_tile_scan(B, s);
+  if (fast) hipLaunchKernelGGL(k_cand_bits, B.grid(256), dim3(kBlock), 0, s, B.jobs);
+  per_score([&](auto& srcs, const SelBatch& sub) {
+    using Src = typename std::remove_reference<decltype(srcs.s[0])>::type;
+    hipLaunchKernelGGL((k_write_bits<Src>), sub.grid(stream_grid(sub.max_tiles, kChunksPerBlock, 1 << 14)),
+                       dim3(kBlock), 0, s, srcs, sub.jobs);
+  });
   launch_result(B, s);
   return check_launch(who);
-}
-
-template <bool BF16G>
-static int run_reselect_score(int score_id, const void* g, int64_t n, const sga_segment* segs,
-                              int n_segs, float coef_dense, int packed, const ReselJob* rj,
-                              int count, hipStream_t s, const char* who) {
-#define SGA_RS(SC) return run_reselect<BF16G, SC>(g, n, segs, n_segs, coef_dense, packed, rj, count, s, who)
-  switch (score_id) { case 0: SGA_RS(0); case 1: SGA_RS(1); case 2: SGA_RS(2);
-                      case 3: SGA_RS(3); case 4: SGA_RS(4); default: SGA_RS(5); }
-#undef SGA_RS
 }
 
 extern "C" int sga_replay_reselect_multi(const void* g, int g_dtype, int64_t n,
@@ -759,8 +798,6 @@ extern "C" int sga_replay_reselect_multi(const void* g, int g_dtype, int64_t n,
     return SGA_ERR_ARG;
   }
   hipStream_t s = (hipStream_t)stream;
-  // configurations that rank by the same score share a batch (the key source is a template
-  // argument of the sweeps); a workspace too small for the sampled bracket gets its own
   bool done[64] = {};
   if (n_jobs > 64) { set_error("%s: at most 64 jobs per call", who); return SGA_ERR_ARG; }
   for (int a = 0; a < n_jobs; ++a) {
@@ -771,13 +808,16 @@ extern "C" int sga_replay_reselect_multi(const void* g, int g_dtype, int64_t n,
       return SGA_ERR_ARG;
     }
   }
+  // batches of up to kMaxJobs jobs that take the same path (a workspace too small for the
+  // sampled bracket sends its job through the radix passes)
   for (int a = 0; a < n_jobs; ++a) {
     if (done[a]) continue;
     ReselJob rj[kMaxJobs];
+    int score[kMaxJobs];
     int cnt = 0;
     bool fast0 = false;
     for (int b = a; b < n_jobs && cnt < kMaxJobs; ++b) {
-      if (done[b] || jobs[b].score_id != jobs[a].score_id) continue;
+      if (done[b]) continue;
       const sga_reselect_job& u = jobs[b];
       SelWorkspace sw;
       if (!sel_ws_carve(u.ws, u.ws_bytes, cdiv64(n, kChunk), &sw)) {
@@ -786,19 +826,20 @@ extern "C" int sga_replay_reselect_multi(const void* g, int g_dtype, int64_t n,
       }
       for (int c = 0; c < cnt; ++c)
         if (rj[c].ws.st == sw.st) {
-          set_error("%s: jobs %d shares its workspace with an earlier job of the call", who, b);
+          set_error("%s: job %d shares its workspace with an earlier job of the call", who, b);
           return SGA_ERR_ARG;
         }
       const bool f = SelBatch::fast_ok(sw, n);
       if (cnt == 0) fast0 = f;
       else if (f != fast0) continue;
+      score[cnt] = u.score_id;
       rj[cnt++] = ReselJob{u.res, u.w, u.m, u.v, u.k, u.coef_f, u.adams, u.res_zero, u.sel_out,
                            u.result, sw};
       done[b] = true;
     }
     const int rc = g_dtype == SGA_BF16
-        ? run_reselect_score<true>(jobs[a].score_id, g, n, segs, n_segs, coef_dense, packed, rj, cnt, s, who)
-        : run_reselect_score<false>(jobs[a].score_id, g, n, segs, n_segs, coef_dense, packed, rj, cnt, s, who);
+        ? run_reselect<true>(g, n, segs, n_segs, coef_dense, packed, rj, score, cnt, s, who)
+        : run_reselect<false>(g, n, segs, n_segs, coef_dense, packed, rj, score, cnt, s, who);
     if (rc != SGA_OK) return rc;
   }
   return SGA_OK;
@@ -824,8 +865,8 @@ extern "C" int sga_replay_reselect(const void* g, int g_dtype, const float* res,
   const ReselJob rj{res, w, m, v, k, coef_f, adams, res_zero, sel_out, result, sw};
   hipStream_t s = (hipStream_t)stream;
   return g_dtype == SGA_BF16
-      ? run_reselect_score<true>(score_id, g, n, segs, n_segs, coef_dense, packed, &rj, 1, s, "sga_replay_reselect")
-      : run_reselect_score<false>(score_id, g, n, segs, n_segs, coef_dense, packed, &rj, 1, s, "sga_replay_reselect");
+      ? run_reselect<true>(g, n, segs, n_segs, coef_dense, packed, &rj, &score_id, 1, s, "sga_replay_reselect")
+      : run_reselect<false>(g, n, segs, n_segs, coef_dense, packed, &rj, &score_id, 1, s, "sga_replay_reselect");
 }
 
 // ------------------------------------------- balanced-histogram re-selection

@@ -1406,47 +1406,75 @@ static __global__ __launch_bounds__(kBlock) void k_mask_to_planes(const uint8_t*
 // bracket as bit planes (job.planes), 2 as mask bytes (job.mask) -- to be finished by
 // finish_planes / finish_mask from those bits and the candidates instead of re-reading the data.
 // All jobs of a batch take the same path (`fast`: SelBatch::fast_ok for every one of them).
+//
+// The chain comes in phases so that a batch whose jobs form their keys differently (the
+// re-selections of a replay step rank by different scores) still shares every kernel that does
+// not form keys: chain_begin, chain_sample_levels, chain_candidates, launch_tile_scan (and the
+// settlement) take the whole batch; chain_sample, chain_sweeps and chain_fallback are templates
+// of the key source and take the jobs of one kind (a sub-batch over the same workspaces).
+static inline void chain_begin(const SelBatch& B, bool fast, hipStream_t s, double sigmas = 5.0) {
+  hipLaunchKernelGGL(k_chain_begin, B.grid(1), dim3(kBlock), 0, s, B.jobs, fast ? 1 : 0, sigmas);
+}
+template <class Src>
+static inline void chain_sample(const SrcPack<Src>& srcs, const SelBatch& B, hipStream_t s) {
+  static_assert(sizeof(ChainJobs) + sizeof(SrcPack<Src>) + 64 <= 4096,
+                "the operands of a batched chain kernel travel in its 4 KiB of kernel arguments");
+  hipLaunchKernelGGL((k_sample<Src>), B.grid(stream_grid(B.max_nsv, kBlock)), dim3(kBlock), 0, s,
+                     srcs, B.jobs);
+}
+static inline void chain_sample_levels(const SelBatch& B, hipStream_t s) {
+  for (int level = 0; level < 3; ++level) launch_level_raw<false>(B, level, s, kRawKeyBlocks);
+}
+template <class Src>
+static inline void chain_sweeps(const SrcPack<Src>& srcs, const SelBatch& B, int pm, hipStream_t s) {
+  for (int b = 0; b < B.count; ++b) {
+    const ChainJob& J = B.jobs.j[b];
+    const SelWorkspace& w = B.w[b];
+    const unsigned sweep_blocks = (unsigned)cdiv64(J.n_tiles, kChunksPerBlock);
+    ProfPair* pp = prof_begin(SGA_PROF_SELECT_SWEEP, s);
+    // the sweep's two totals go through 256 partial counters (blk_gt / blk_eq are free until
+    // the tile scan, which runs after the check has read them)
+    if (pm == 2)
+      hipLaunchKernelGGL((k_bracket_sweep<Src, 2>), dim3(sweep_blocks), dim3(kBlock), 0, s,
+                         srcs.s[b], J.n, w.st, w.aux, w.tile_gt, w.tile_eq, w.seg_idx, w.seg_key,
+                         w.seg_cnt, (uint32_t)w.seg_cap, (uint32_t*)nullptr, w.blk_gt, w.blk_eq,
+                         J.mask, (reinterpret_cast<uintptr_t>(J.mask) & 3) == 0);
+    else if (pm == 1)
+      hipLaunchKernelGGL((k_bracket_sweep<Src, 1>), dim3(sweep_blocks), dim3(kBlock), 0, s,
+                         srcs.s[b], J.n, w.st, w.aux, w.tile_gt, w.tile_eq, w.seg_idx, w.seg_key,
+                         w.seg_cnt, (uint32_t)w.seg_cap, J.planes, w.blk_gt, w.blk_eq);
+    else
+      hipLaunchKernelGGL((k_bracket_sweep<Src, 0>), dim3(sweep_blocks), dim3(kBlock), 0, s,
+                         srcs.s[b], J.n, w.st, w.aux, w.tile_gt, w.tile_eq, w.seg_idx, w.seg_key,
+                         w.seg_cnt, (uint32_t)w.seg_cap, (uint32_t*)nullptr, w.blk_gt, w.blk_eq);
+    prof_end(pp, s);
+  }
+}
+static inline void chain_candidates(const SelBatch& B, hipStream_t s) {
+  hipLaunchKernelGGL(k_bracket_check, B.grid(1), dim3(kBlock), 0, s, B.jobs);
+  hipLaunchKernelGGL(k_cand_compact, B.grid(256), dim3(kBlock), 0, s, B.jobs);
+  for (int level = 0; level < 3; ++level) launch_level_raw<true>(B, level, s, kRawKeyBlocks);
+  hipLaunchKernelGGL(k_cand_tiles, B.grid(256), dim3(kBlock), 0, s, B.jobs);
+}
+// The radix passes and the per-chunk counts over the data: no-ops unless a job's bracket failed
+// (st->skip == 0; k_bracket_check left the histograms zeroed for them) or was never tried.
+template <class Src>
+static inline void chain_fallback(const SrcPack<Src>& srcs, const SelBatch& B, hipStream_t s) {
+  for (int level = 0; level < 3; ++level) launch_level_data<Src, true>(srcs, B, level, s);
+  launch_tile_count(srcs, B, 0, s);
+}
+
 template <class Src>
 static inline void run_select_batch(const SrcPack<Src>& srcs, const SelBatch& B, bool fast, int pm,
                                     hipStream_t s, double sigmas = 5.0) {
-  static_assert(sizeof(ChainJobs) + sizeof(SrcPack<Src>) + 64 <= 4096,
-                "the operands of a batched chain kernel travel in its 4 KiB of kernel arguments");
-  hipLaunchKernelGGL(k_chain_begin, B.grid(1), dim3(kBlock), 0, s, B.jobs, fast ? 1 : 0, sigmas);
+  chain_begin(B, fast, s, sigmas);
   if (fast) {
-    hipLaunchKernelGGL((k_sample<Src>), B.grid(stream_grid(B.max_nsv, kBlock)), dim3(kBlock), 0, s,
-                       srcs, B.jobs);
-    for (int level = 0; level < 3; ++level) launch_level_raw<false>(B, level, s, kRawKeyBlocks);
-    for (int b = 0; b < B.count; ++b) {
-      const ChainJob& J = B.jobs.j[b];
-      const SelWorkspace& w = B.w[b];
-      const unsigned sweep_blocks = (unsigned)cdiv64(J.n_tiles, kChunksPerBlock);
-      ProfPair* pp = prof_begin(SGA_PROF_SELECT_SWEEP, s);
-      // the sweep's two totals go through 256 partial counters (blk_gt / blk_eq are free until
-      // the tile scan, which runs after the check has read them)
-      if (pm == 2)
-        hipLaunchKernelGGL((k_bracket_sweep<Src, 2>), dim3(sweep_blocks), dim3(kBlock), 0, s,
-                           srcs.s[b], J.n, w.st, w.aux, w.tile_gt, w.tile_eq, w.seg_idx, w.seg_key,
-                           w.seg_cnt, (uint32_t)w.seg_cap, (uint32_t*)nullptr, w.blk_gt, w.blk_eq,
-                           J.mask, (reinterpret_cast<uintptr_t>(J.mask) & 3) == 0);
-      else if (pm == 1)
-        hipLaunchKernelGGL((k_bracket_sweep<Src, 1>), dim3(sweep_blocks), dim3(kBlock), 0, s,
-                           srcs.s[b], J.n, w.st, w.aux, w.tile_gt, w.tile_eq, w.seg_idx, w.seg_key,
-                           w.seg_cnt, (uint32_t)w.seg_cap, J.planes, w.blk_gt, w.blk_eq);
-      else
-        hipLaunchKernelGGL((k_bracket_sweep<Src, 0>), dim3(sweep_blocks), dim3(kBlock), 0, s,
-                           srcs.s[b], J.n, w.st, w.aux, w.tile_gt, w.tile_eq, w.seg_idx, w.seg_key,
-                           w.seg_cnt, (uint32_t)w.seg_cap, (uint32_t*)nullptr, w.blk_gt, w.blk_eq);
-      prof_end(pp, s);
-    }
-    hipLaunchKernelGGL(k_bracket_check, B.grid(1), dim3(kBlock), 0, s, B.jobs);
-    hipLaunchKernelGGL(k_cand_compact, B.grid(256), dim3(kBlock), 0, s, B.jobs);
-    for (int level = 0; level < 3; ++level) launch_level_raw<true>(B, level, s, kRawKeyBlocks);
-    hipLaunchKernelGGL(k_cand_tiles, B.grid(256), dim3(kBlock), 0, s, B.jobs);
-    // The radix passes below are no-ops unless the bracket failed
-    // (st->skip == 0); k_bracket_check left the histograms zeroed for them.
+    chain_sample(srcs, B, s);
+    chain_sample_levels(B, s);
+    chain_sweeps(srcs, B, pm, s);
+    chain_candidates(B, s);
   }
-  for (int level = 0; level < 3; ++level) launch_level_data<Src, true>(srcs, B, level, s);
-  launch_tile_count(srcs, B, 0, s);
+  chain_fallback(srcs, B, s);
   launch_tile_scan(B, s);
 }
 
