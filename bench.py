@@ -654,9 +654,11 @@ def main():
     max_steps = max(args.steps, 5)
     results = torch.zeros(max_steps, 8, dtype=torch.int32, device=dev)   # a result block per step
 
-    def time_leg(layout, score, ratio, warmup, steps, single=False):
-        """`warmup` untimed + exactly `steps` timed steps of one configuration."""
+    def time_leg(layout, score, ratio, warmup, steps, single=False, oop=False):
+        """`warmup` untimed + exactly `steps` timed steps of one configuration.  `oop`: the
+        out-of-place single-sweep step on ping-pong state (flat tensors)."""
         k = k_for(n, ratio)
+        sets = [[r, p, m, v], [torch.empty_like(r) for _ in range(4)] if oop else None]
         if layout == "packed" and state["packed"] is None:
             state["packed"] = PackedState(n, dev).pack(r, p, m, v)
         elif layout == "separate" and state["packed"] is not None:
@@ -664,7 +666,11 @@ def main():
             state["packed"] = None
 
         def step_fn(t, res=None):
-            if layout == "packed":
+            if oop:
+                fs.step(grads[t % 2], *sets[0], t + 1, k=k, score=score, single_sweep=True,
+                        check=False, result=res, out=sets[1])
+                sets.reverse()
+            elif layout == "packed":
                 fs.step_packed(grads[t % 2], state["packed"], t + 1, k=k, score=score,
                                single_sweep=single, check=False, result=res)
             else:
@@ -684,6 +690,9 @@ def main():
         fin_ms, fin_n = prof_read(L, PROF_FINAL)
         sw_ms, sw_n = prof_read(L, PROF_SWEEP)
         prof_enable(L, 0)
+        if oop and sets[0][0] is not r:              # leave the current state in r / p / m / v
+            for dst, src in zip((r, p, m, v), sets[0]):
+                dst.copy_(src)
         # every timed step must have ended as an exact top-k step (status word 0, k selected)
         rows = results[:steps].cpu()
         assert bool((rows[:, 6] == 0).all()) and bool((rows[:, 4] == k).all()), rows.tolist()
@@ -700,7 +709,8 @@ def main():
         two_read_bytes = n * step_bytes_per_elem(score) + k * 6.0
         moved = once_bytes if single else two_read_bytes
         fin_avg, sw_avg = fin_ms / max(fin_n, 1), sw_ms / max(sw_n, 1)
-        return {"layout": layout, "single_sweep": single, "score": score, "ratio_percent": ratio,
+        return {"layout": layout, "single_sweep": single, "out_of_place": oop, "score": score,
+                "ratio_percent": ratio,
                 "k": k, "steps": steps, "seconds": dt, "ms_per_step": dt / steps * 1e3,
                 "elem_per_s": n * steps / dt,
                 "moved_bytes_per_elem": moved / n, "moved_bytes_per_step": moved,
@@ -732,9 +742,10 @@ def main():
         m.zero_(); v.zero_(); r.zero_()
         state["t"] = 0
     # the other step variant and the other layout of the headline configuration
-    other = packed_leg = None
+    other = packed_leg = oop_leg = None
     if not args.headline_only:
         other = time_leg(args.layout, args.score, args.ratio, 2, 5, not args.single_sweep)
+        oop_leg = time_leg("separate", args.score, args.ratio, 2, 5, True, oop=True)
         packed_leg = time_leg("packed" if args.layout == "separate" else "separate", args.score,
                               args.ratio, 2, 5, args.single_sweep)
     two = head if not args.single_sweep else other
@@ -789,7 +800,14 @@ def main():
             "ms_per_step": packed_leg["ms_per_step"], "elem_per_s": packed_leg["elem_per_s"],
             "frac": packed_leg["step_frac"], "dominant_kernel_ms": packed_leg["final_avg_ms"],
             "dominant_kernel_frac": packed_leg["final_frac"]}
+    if oop_leg is not None:
+        out["out_of_place"] = {
+            "what": "single-sweep step on ping-pong state (a missed bracket is redone, never lost)",
+            "ms_per_step": oop_leg["ms_per_step"], "elem_per_s": oop_leg["elem_per_s"],
+            "frac": oop_leg["step_frac"], "dominant_kernel_ms": oop_leg["final_avg_ms"],
+            "dominant_kernel_frac": oop_leg["final_frac"]}
     detail = {"headline_leg": head, "other_variant_leg": other, "other_layout_leg": packed_leg,
+              "out_of_place_leg": oop_leg,
               "select": head["select"], "traffic_source": traffic_src,
               "stream_mix_copy": stream_mix}
     if sweep:
@@ -847,7 +865,7 @@ def main():
             out["detail_file"] = f"not written ({e.strerror})"
     # the last line stays compact whatever happens: optional summaries go first if it ever grew
     line = json.dumps(out, separators=(",", ":"))
-    for key in ("cfg5", "cfg2", "packed_layout", "separate_layout", "two_sweep"):
+    for key in ("cfg5", "cfg2", "out_of_place", "packed_layout", "separate_layout", "two_sweep"):
         if len(line) < 6000:
             break
         out.pop(key, None)

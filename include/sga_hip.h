@@ -78,7 +78,8 @@ typedef struct sga_select_result {
   uint32_t status;      /* 0 ok; 1 k out of range; 2 fast path fell back;
                            3 single-sweep bracket missed (step invalid)    */
   uint32_t path;        /* low byte: 0 radix passes, 1 sampled bracket, 2 single
-                           sweep; bit 8: an fp32 score array held a value < 0 */
+                           sweep; bit 8: an fp32 score array held a value < 0;
+                           bit 9: an out-of-place single-sweep step was redone */
 } sga_select_result;
 
 /* ---- scheme-agnostic masked ops (sga/kernels.py) ------------------------ */
@@ -427,6 +428,34 @@ int sga_fused_sparse_step_single_sweep_packed(
     const sga_segment* segs, int n_segs, int score_id, int32_t* idx_out,
     void* values_out, int values_dtype, uint8_t* mask_out, float factor,
     float coeff, int flags, float interval, uint32_t seed,
+    sga_select_result* result, void* ws, size_t ws_bytes, void* ws2,
+    size_t ws2_bytes, void* stream);
+
+/* Out-of-place single-sweep step (no counterpart in the reference): same
+ * sweep, but the new resid / p / m / v go to OTHER arrays (ping-pong state:
+ * swap the two sets after every step) and the inputs are only read.  Nothing
+ * is lost when the bracket misses: the device then redoes the step from the
+ * untouched inputs with the radix passes and the key-forming final sweep of
+ * sga_fused_sparse_step, over whatever the sweep wrote.  result->status is 0
+ * for every input (never 3), outputs equal sga_fused_sparse_step's bit for
+ * bit, and bit 9 (0x200) of result->path says that the step was redone.  The
+ * price is a second copy of the optimizer-side state (16 B per coordinate).
+ * No output array may overlap an input or another output (refused).  The
+ * packed twin takes two packed states (sga_packed_state_elems(n) floats each,
+ * 16-byte aligned). */
+int sga_fused_sparse_step_single_sweep_out(
+    const void* g, int g_dtype, const float* resid, const float* p,
+    const float* m, const float* v, float* resid_out, float* p_out,
+    float* m_out, float* v_out, int64_t n, int64_t k, const sga_segment* segs,
+    int n_segs, int score_id, int32_t* idx_out, void* values_out,
+    int values_dtype, uint8_t* mask_out, float factor, float coeff, int flags,
+    float interval, uint32_t seed, sga_select_result* result, void* ws,
+    size_t ws_bytes, void* ws2, size_t ws2_bytes, void* stream);
+int sga_fused_sparse_step_single_sweep_packed_out(
+    const void* g, int g_dtype, const float* state, float* state_out,
+    int64_t n, int64_t k, const sga_segment* segs, int n_segs, int score_id,
+    int32_t* idx_out, void* values_out, int values_dtype, uint8_t* mask_out,
+    float factor, float coeff, int flags, float interval, uint32_t seed,
     sga_select_result* result, void* ws, size_t ws_bytes, void* ws2,
     size_t ws2_bytes, void* stream);
 

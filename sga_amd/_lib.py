@@ -119,6 +119,12 @@ SIGNATURES = {
     "sga_fused_sparse_step_single_sweep_packed": (I32, [P, I32, P, I64, I64, P, I32, I32, P, P,
                                                         I32, P, F, F, I32, F, U32, P, P, SZ, P,
                                                         SZ, P]),
+    "sga_fused_sparse_step_single_sweep_out": (I32, [P, I32, P, P, P, P, P, P, P, P, I64, I64, P, I32,
+                                                     I32, P, P, I32, P, F, F, I32, F, U32, P, P, SZ,
+                                                     P, SZ, P]),
+    "sga_fused_sparse_step_single_sweep_packed_out": (I32, [P, I32, P, P, I64, I64, P, I32, I32, P, P,
+                                                            I32, P, F, F, I32, F, U32, P, P, SZ, P,
+                                                            SZ, P]),
 }
 
 # include/sga_hip_bench.h: libsga_hip_bench.so, the benchmark-only companion

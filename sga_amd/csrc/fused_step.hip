@@ -126,10 +126,14 @@ struct SrcFused {
 // Everything the final sweep needs besides the chunk index.
 struct FinalArgs {
   const void* g;
-  float* r;
+  float* r;                 // state as the step reads it ...
   float* p;
   float* m;
   float* v;
+  float* ro;                // ... and where it writes the new state (the same arrays for the
+  float* po;                // in-place entry points, other ones for the out-of-place step)
+  float* mo;
+  float* vo;
   int64_t n, k;
   int32_t* idx_out;
   void* values_out;
@@ -156,10 +160,14 @@ __device__ __forceinline__ void final_chunk(const FinalArgs& a, int64_t c, Chunk
                                             SegCursor& sc, SegCursor& lc) {
   const int64_t n = a.n;
   const int64_t sh = pack_shift<true>(c << 10, a.pack_extra);     // c is wave-uniform
-  float* const R = a.r + sh;
-  float* const P = a.p + sh;
-  float* const M = a.m + sh;
-  float* const V = a.v + sh;
+  const float* const R = a.r + sh;
+  const float* const P = a.p + sh;
+  const float* const M = a.m + sh;
+  const float* const V = a.v + sh;
+  float* const RO = a.ro + sh;
+  float* const PO = a.po + sh;
+  float* const MO = a.mo + sh;
+  float* const VO = a.vo + sh;
   float gg[kChunkIters][4], rr[kChunkIters][4], pp[kChunkIters][4], mm[kChunkIters][4],
       vv[kChunkIters][4];
   if (FULL) {
@@ -310,10 +318,10 @@ __device__ __forceinline__ void final_chunk(const FinalArgs& a, int64_t c, Chunk
         rr[it][e] = sel[e] ? 0.0f : q[e];
         if (a.fold) rr[it][e] = __fdiv_rn(rr[it][e], a.interval);
       }
-      st_f32<FULL>(R, i, n, rr[it], a.vec);
-      st_f32<FULL>(M, i, n, mm[it], a.vec);
-      st_f32<FULL>(V, i, n, vv[it], a.vec);
-      st_f32<FULL>(P, i, n, pp[it], a.vec);
+      st_f32<FULL>(RO, i, n, rr[it], a.vec);
+      st_f32<FULL>(MO, i, n, mm[it], a.vec);
+      st_f32<FULL>(VO, i, n, vv[it], a.vec);
+      st_f32<FULL>(PO, i, n, pp[it], a.vec);
       if (a.mask_out) st_u8<FULL>(a.mask_out, i, n, mk, a.mvec);
     }
   }
@@ -381,6 +389,7 @@ struct FusedJob {
   uint8_t* mask_out;
   sga_select_result* result;
   SelWorkspace w;
+  float* out[4];            // resid / p / m / v of the new state; all null: in place
 };
 
 // The two-sweep step for up to kMaxJobs buckets that share dtypes, score and knobs: the short
@@ -407,7 +416,8 @@ static int run_fused(const FusedJob* fj, int count, float factor, float coeff, i
   for (int b = 0; b < count; ++b) {
     const FusedJob& f = fj[b];
     vec[b] = aligned4(f.g, BF16G ? 2 : 4) && aligned4(f.resid, 4) && aligned4(f.p, 4) &&
-             aligned4(f.m, 4) && aligned4(f.v, 4);
+             aligned4(f.m, 4) && aligned4(f.v, 4) && aligned4(f.out[0], 4) &&
+             aligned4(f.out[1], 4) && aligned4(f.out[2], 4) && aligned4(f.out[3], 4);
     srcs.s[b] = Src{f.g, f.resid, f.p, f.m, f.v, vec[b], {}, pack_extra, adams};
     srcs.s[b].sc.init(f.segs, f.n_segs, f.w.seg_dir);
     dj.j[b].segs = f.segs; dj.j[b].dir = f.w.seg_dir; dj.j[b].n = f.n; dj.j[b].n_segs = f.n_segs;
@@ -427,6 +437,8 @@ static int run_fused(const FusedJob* fj, int count, float factor, float coeff, i
     ProfPair* pp = prof_begin(SGA_PROF_FUSED_FINAL, s);
     FinalArgs fa;
     fa.g = f.g; fa.r = f.resid; fa.p = f.p; fa.m = f.m; fa.v = f.v; fa.n = f.n; fa.k = f.k;
+    fa.ro = f.out[0] ? f.out[0] : f.resid; fa.po = f.out[0] ? f.out[1] : f.p;
+    fa.mo = f.out[0] ? f.out[2] : f.m; fa.vo = f.out[0] ? f.out[3] : f.v;
     fa.idx_out = f.idx_out; fa.values_out = f.values_out; fa.mask_out = f.mask_out;
     fa.factor = factor; fa.coeff = coeff; fa.T = 0; fa.need = 0;
     fa.vec = vec[b]; fa.mvec = aligned4(f.mask_out, 1);
@@ -534,7 +546,8 @@ __device__ __forceinline__ void spec_slab(const FinalArgs& a, const SpecArgs& sa
                                           int64_t c, int it, uint32_t T_LO, uint32_t T_MID,
                                           uint32_t T_HI, SegCursor& sc, uint32_t& chi,
                                           uint32_t& s_run, uint32_t& tot_nf, uint32_t& mycnt,
-                                          SpecLds& lds, float* R, float* P, float* M, float* V) {
+                                          SpecLds& lds, const float* R, const float* P,
+                                          const float* M, const float* V, int64_t sh) {
   constexpr bool kHyper = SCORE == SGA_SCORE_UPDATE || SCORE == SGA_SCORE_COI ||
                           SCORE == SGA_SCORE_GR_OVER_SQRT_V;
   const int64_t n = a.n;
@@ -664,10 +677,10 @@ __device__ __forceinline__ void spec_slab(const FinalArgs& a, const SpecArgs& sa
     rr[e] = sel[e] ? 0.0f : q[e];
     if (a.fold) rr[e] = __fdiv_rn(rr[e], a.interval);
   }
-  st_f32<FULL>(R, i, n, rr, a.vec);
-  st_f32<FULL>(M, i, n, mm, a.vec);
-  st_f32<FULL>(V, i, n, vv, a.vec);
-  st_f32<FULL>(P, i, n, pp, a.vec);
+  st_f32<FULL>(a.ro + sh, i, n, rr, a.vec);
+  st_f32<FULL>(a.mo + sh, i, n, mm, a.vec);
+  st_f32<FULL>(a.vo + sh, i, n, vv, a.vec);
+  st_f32<FULL>(a.po + sh, i, n, pp, a.vec);
 }
 
 template <bool BF16G, bool BF16V, int SCORE>
@@ -696,13 +709,13 @@ __global__ __launch_bounds__(kBlock) void k_fused_spec(
     SegCursor sc;
     sc.init(segs, n_segs, seg_dir);
     const int64_t sh = pack_shift<true>(c << 10, a.pack_extra);
-    float* const R = a.r + sh;
-    float* const P = a.p + sh;
-    float* const M = a.m + sh;
-    float* const V = a.v + sh;
+    const float* const R = a.r + sh;
+    const float* const P = a.p + sh;
+    const float* const M = a.m + sh;
+    const float* const V = a.v + sh;
     sc.seek_uniform(uniform_i64(c) * kChunk);
 #define SGA_SPEC_SLAB(FULLP, IT) \
-    spec_slab<BF16G, BF16V, SCORE, FULLP>(a, sa, st, c, IT, T_LO, T_MID, T_HI, sc, chi, s_run, tot_nf, mycnt, lds, R, P, M, V)
+    spec_slab<BF16G, BF16V, SCORE, FULLP>(a, sa, st, c, IT, T_LO, T_MID, T_HI, sc, chi, s_run, tot_nf, mycnt, lds, R, P, M, V, sh)
     if (a.vec && (c + 1) * kChunk <= a.n) {
       SGA_SPEC_SLAB(true, 0); SGA_SPEC_SLAB(true, 1); SGA_SPEC_SLAB(true, 2); SGA_SPEC_SLAB(true, 3);
     } else {
@@ -999,10 +1012,10 @@ __global__ __launch_bounds__(kBlock) void k_spec_repair(
     float rn = on ? 0.0f : rec.x;
     if (a.fold) rn = __fdiv_rn(rn, a.interval);
     const int64_t at = (int64_t)idx + pack_shift<false>((int64_t)idx, a.pack_extra);
-    a.r[at] = rn;
-    a.p[at] = pe;
-    a.m[at] = cm.m_new;
-    a.v[at] = cm.v_new;
+    a.ro[at] = rn;
+    a.po[at] = pe;
+    a.mo[at] = cm.m_new;
+    a.vo[at] = cm.v_new;
     if (on) {
       const uint32_t pos = slab_pos[idx >> 8] + slab_rank_before(fplane, idx);
       if ((int64_t)pos < a.k) {
@@ -1098,9 +1111,14 @@ static int run_fused_spec(const void* g, float* resid, float* p, float* m, float
                           void* values_out, uint8_t* mask_out, float factor, float coeff,
                           int flags, float interval, uint32_t seed, sga_select_result* result,
                           const SelWorkspace& w, const SpecWorkspace& x, hipStream_t s,
-                          int64_t pack_extra) {
+                          int64_t pack_extra, float* const* out = nullptr) {
+  // out: resid / p / m / v of the NEW state when the step runs out of place (the inputs stay
+  // untouched, so a bracket that missed is redone by the radix passes and the key-forming final
+  // sweep like a sweep that stood back); null: in place
   const bool vec = aligned4(g, BF16G ? 2 : 4) && aligned4(resid, 4) && aligned4(p, 4) &&
-                   aligned4(m, 4) && aligned4(v, 4);
+                   aligned4(m, 4) && aligned4(v, 4) &&
+                   (!out || (aligned4(out[0], 4) && aligned4(out[1], 4) && aligned4(out[2], 4) &&
+                             aligned4(out[3], 4)));
   const int adams = (flags & SGA_GC_ADAMS) ? 1 : 0;
   SrcFused<BF16G, SCORE> src{g, resid, p, m, v, vec, {}, pack_extra, adams};
   launch_seg_dir(segs, n_segs, n, w.seg_dir, s);
@@ -1108,6 +1126,8 @@ static int run_fused_spec(const void* g, float* resid, float* p, float* m, float
   const int64_t n_tiles = cdiv64(n, kChunk);
   FinalArgs fa;
   fa.g = g; fa.r = resid; fa.p = p; fa.m = m; fa.v = v; fa.n = n; fa.k = k;
+  fa.ro = out ? out[0] : resid; fa.po = out ? out[1] : p;
+  fa.mo = out ? out[2] : m; fa.vo = out ? out[3] : v;
   fa.idx_out = idx_out; fa.values_out = values_out; fa.mask_out = mask_out;
   fa.factor = factor; fa.coeff = coeff; fa.T = 0; fa.need = 0;
   fa.vec = vec; fa.mvec = aligned4(mask_out, 1);
@@ -1120,7 +1140,7 @@ static int run_fused_spec(const void* g, float* resid, float* p, float* m, float
   srcs.s[0] = src;
   SelBatch B;
   ChainJob& J = B.add(w, n, k, 0);
-  J.seed = seed; J.spec = 1; J.ovf_cap = (uint32_t)x.ovf_cap; J.seg_fail = x.seg_fail;
+  J.seed = seed; J.spec = out ? 2 : 1; J.ovf_cap = (uint32_t)x.ovf_cap; J.seg_fail = x.seg_fail;
   J.seg_rec = x.seg_rec; J.cand_rec = x.cand_rec; J.result = result;
   const int64_t ns = J.n_sv * 4;
   hipLaunchKernelGGL(k_chain_begin, B.grid(1), dim3(kBlock), 0, s, B.jobs, 1, kSpecSigmas);
@@ -1193,7 +1213,8 @@ static int fused_entry(const char* who, const void* g, int g_dtype, float* resid
                        void* values_out, int values_dtype, uint8_t* mask_out, float factor,
                        float coeff, int fast, int flags, float interval, sga_select_result* result,
                        void* ws, size_t ws_bytes, void* stream, bool single = false,
-                       void* ws2 = nullptr, size_t ws2_bytes = 0, uint32_t seed = 0u) {
+                       void* ws2 = nullptr, size_t ws2_bytes = 0, uint32_t seed = 0u,
+                       float* const* out = nullptr) {
   if ((flags & ~(SGA_GC_ADAMS | SGA_GC_FOLD)) != 0) {
     // the dual-lr split belongs to full steps (adamw.py:570-580); HAS_MASK / CLEAR / APPLY_COEFF
     // are what this step does anyway (coeff != 1 applies the coefficient)
@@ -1245,12 +1266,14 @@ static int fused_entry(const char* who, const void* g, int g_dtype, float* resid
     }
     if (!take) { single = false; fast = 1; }
   }
-  const FusedJob job{g, resid, p, m, v, n, k, segs, n_segs, idx_out, values_out, mask_out, result, w};
+  const FusedJob job{g, resid, p, m, v, n, k, segs, n_segs, idx_out, values_out, mask_out, result, w,
+                     {out ? out[0] : nullptr, out ? out[1] : nullptr, out ? out[2] : nullptr,
+                      out ? out[3] : nullptr}};
 #define SGA_RUN(BG, BV, SC)                                                                   \
   if (single)                                                                                 \
     return run_fused_spec<BG, BV, SC>(g, resid, p, m, v, n, k, segs, n_segs, idx_out,        \
                                       values_out, mask_out, factor, coeff, flags, interval,   \
-                                      seed, result, w, x, s, pack_extra);                     \
+                                      seed, result, w, x, s, pack_extra, out);                \
   return run_fused<BG, BV, SC>(&job, 1, factor, coeff, fast, flags, interval, s, pack_extra, who)
 #define SGA_RUN_SC(BG, BV)                    \
   switch (score_id) {                         \
@@ -1325,7 +1348,7 @@ extern "C" int sga_fused_sparse_step_multi(const sga_fused_bucket* buckets, int 
         const bool is_fast = fast != 0 && SelBatch::fast_ok(w, u.n);
         if (is_fast != (pass == 0)) continue;
         jobs[cnt++] = FusedJob{u.g, u.resid, u.p, u.m, u.v, u.n, u.k, u.segs, u.n_segs, u.idx_out,
-                               u.values_out, u.mask_out, u.result, w};
+                               u.values_out, u.mask_out, u.result, w, {nullptr, nullptr, nullptr, nullptr}};
       }
       if (cnt == kMaxJobs || (b == n_buckets && cnt > 0)) {
         int rc;
@@ -1384,6 +1407,67 @@ extern "C" int sga_fused_sparse_step_single_sweep_packed(
                      state ? state + 3 * kPackRun : nullptr, kPackExtra, n, k, segs, n_segs,
                      score_id, idx_out, values_out, values_dtype, mask_out, factor, coeff, 1,
                      flags, interval, result, ws, ws_bytes, stream, true, ws2, ws2_bytes, seed);
+}
+
+// true when [a, a + bytes) and [b, b + bytes) overlap
+static bool ranges_overlap(const void* a, const void* b, size_t bytes) {
+  const uintptr_t x = reinterpret_cast<uintptr_t>(a), y = reinterpret_cast<uintptr_t>(b);
+  return x < y + bytes && y < x + bytes;
+}
+
+extern "C" int sga_fused_sparse_step_single_sweep_out(
+    const void* g, int g_dtype, const float* resid, const float* p, const float* m, const float* v,
+    float* resid_out, float* p_out, float* m_out, float* v_out, int64_t n, int64_t k,
+    const sga_segment* segs, int n_segs, int score_id, int32_t* idx_out, void* values_out,
+    int values_dtype, uint8_t* mask_out, float factor, float coeff, int flags, float interval,
+    uint32_t seed, sga_select_result* result, void* ws, size_t ws_bytes, void* ws2,
+    size_t ws2_bytes, void* stream) {
+  const char* who = "sga_fused_sparse_step_single_sweep_out";
+  float* out[4] = {resid_out, p_out, m_out, v_out};
+  const float* in[4] = {resid, p, m, v};
+  if (!resid_out || !p_out || !m_out || !v_out) {
+    set_error("%s: the four output arrays are required", who);
+    return SGA_ERR_ARG;
+  }
+  if (n > 0)
+    for (int a = 0; a < 4; ++a) {
+      for (int b = 0; b < 4; ++b)
+        if ((in[b] && ranges_overlap(out[a], in[b], (size_t)n * 4)) ||
+            (b != a && ranges_overlap(out[a], out[b], (size_t)n * 4))) {
+          set_error("%s: an output array overlaps an input or another output (the step reads "
+                    "the old state while it writes the new one)", who);
+          return SGA_ERR_ARG;
+        }
+    }
+  return fused_entry(who, g, g_dtype, const_cast<float*>(resid), const_cast<float*>(p),
+                     const_cast<float*>(m), const_cast<float*>(v), 0, n, k, segs, n_segs, score_id,
+                     idx_out, values_out, values_dtype, mask_out, factor, coeff, 1, flags, interval,
+                     result, ws, ws_bytes, stream, true, ws2, ws2_bytes, seed, out);
+}
+
+extern "C" int sga_fused_sparse_step_single_sweep_packed_out(
+    const void* g, int g_dtype, const float* state, float* state_out, int64_t n, int64_t k,
+    const sga_segment* segs, int n_segs, int score_id, int32_t* idx_out, void* values_out,
+    int values_dtype, uint8_t* mask_out, float factor, float coeff, int flags, float interval,
+    uint32_t seed, sga_select_result* result, void* ws, size_t ws_bytes, void* ws2,
+    size_t ws2_bytes, void* stream) {
+  const char* who = "sga_fused_sparse_step_single_sweep_packed_out";
+  if (!state || !state_out || (reinterpret_cast<uintptr_t>(state) & 15) ||
+      (reinterpret_cast<uintptr_t>(state_out) & 15)) {
+    set_error("%s: both packed states are required, 16-byte aligned", who);
+    return SGA_ERR_ARG;
+  }
+  const size_t bytes = (size_t)(n <= 0 ? 0 : cdiv64(n, kPackRun) * 4 * kPackRun) * 4;
+  if (ranges_overlap(state, state_out, bytes)) {
+    set_error("%s: the output state overlaps the input state", who);
+    return SGA_ERR_ARG;
+  }
+  float* out[4] = {state_out, state_out + kPackRun, state_out + 2 * kPackRun, state_out + 3 * kPackRun};
+  float* in = const_cast<float*>(state);
+  return fused_entry(who, g, g_dtype, in, in + kPackRun, in + 2 * kPackRun, in + 3 * kPackRun,
+                     kPackExtra, n, k, segs, n_segs, score_id, idx_out, values_out, values_dtype,
+                     mask_out, factor, coeff, 1, flags, interval, result, ws, ws_bytes, stream, true,
+                     ws2, ws2_bytes, seed, out);
 }
 
 extern "C" int64_t sga_packed_state_elems(int64_t n) {

@@ -45,7 +45,8 @@ struct SelState {
   uint32_t done[3];     // per-level "workgroups finished" tickets (last one scans)
   uint32_t spec;        // 1: the single-sweep step committed on the sampled bracket (no way back)
   uint32_t negative;    // 1: an fp32 score array held a value below zero (magnitudes were ranked)
-  uint32_t pad_[6];
+  uint32_t redone;      // 1: an out-of-place single-sweep step missed its bracket and was redone
+  uint32_t pad_[5];
 };
 static_assert(sizeof(SelState) == 128, "SelState layout");
 
@@ -764,7 +765,7 @@ static __global__ void k_sel_result(ChainJobs jobs) {
   out->n_selected = st->n_selected;
   out->nonfinite = st->nonfinite;
   out->status = st->status;
-  out->path = st->path | (st->negative ? 0x100u : 0u);
+  out->path = st->path | (st->negative ? 0x100u : 0u) | (st->redone ? 0x200u : 0u);
 }
 
 // -------------------------------------------------------------- host drivers
@@ -1154,9 +1155,14 @@ static __global__ __launch_bounds__(kBlock) void k_bracket_check(ChainJobs jobs)
     const bool ok = !st->overflow && !any_over && !ovf_over && n_hi < k && k <= n_hi + total;
     st->n_hi = n_hi;
     st->cand_count = total;
-    // A single-sweep step that went ahead has already committed on the bracket: a miss cannot
-    // be repaired by the radix passes, it is reported (status 3) and nothing further runs.
-    const bool lost = spec && st->spec && !ok;
+    // A single-sweep step that went ahead IN PLACE has already committed on the bracket: a miss
+    // cannot be repaired by the radix passes, it is reported (status 3) and nothing further
+    // runs.  Out of place (spec == 2) the inputs are untouched: the miss is an ordinary failed
+    // bracket, the radix passes and the key-forming final sweep redo the step over what the
+    // sweep wrote, and `redone` says so.
+    const bool missed = spec && st->spec && !ok;
+    const bool lost = missed && spec != 2;
+    if (missed && spec == 2) { st->spec = 0u; st->redone = 1u; }
     st->bracket_ok = ok ? 1u : 0u;
     st->skip = (ok || lost) ? 1u : 0u;   // the radix passes run only when the bracket failed
     st->path = ok ? (spec ? 2u : 1u) : 0u;

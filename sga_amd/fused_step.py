@@ -139,7 +139,7 @@ class FusedSparseStep:
     def step(self, g, resid, p, m, v, step, k=None, ratio_percent=None,
              score="abs_g", factor=1.0, coeff=1.0, fast=True, optimizer="adamw", fold=False,
              interval=1.0, inactive_lr_scale=1.0, single_sweep=False, seed=None, check=True,
-             result=None):
+             result=None, out=None):
         """Run one fused step in place; returns (idx[:k], values[:k]) views.
         ``self.result`` holds the device-side select result (threshold bits,
         counts); nothing is synchronised here.  ``optimizer="adams"`` commits
@@ -158,29 +158,58 @@ class FusedSparseStep:
         waits for the step and raises ``SingleSweepLost`` on status 3 instead
         of handing back a pack that was not written; ``check=False`` leaves
         the status to the caller (``result``: an int32[8] device tensor of the
-        caller's for this step's result block, default ``self.result``)."""
+        caller's for this step's result block, default ``self.result``).
+
+        ``out`` (single sweep only): ``(resid, p, m, v)`` fp32 tensors that
+        receive the new state while the inputs are only read (ping-pong
+        state).  A missed bracket then loses nothing: the device redoes the
+        step from the untouched inputs, the status stays 0 and
+        ``read_result().redone`` is set."""
         for t in (g, resid, p, m, v):
             L.require_dev(t)
             L.require_contig(t=t)
             assert t.numel() == self.n
-        return self._run("sga_fused_sparse_step" + ("_single_sweep" if single_sweep else ""), g,
-                         [L.ptr(resid), L.ptr(p), L.ptr(m), L.ptr(v)], step, k, ratio_percent,
-                         score, factor, coeff, fast, optimizer, fold, interval, inactive_lr_scale,
-                         single_sweep, seed, check, result)
+        state = [L.ptr(resid), L.ptr(p), L.ptr(m), L.ptr(v)]
+        name = "sga_fused_sparse_step" + ("_single_sweep" if single_sweep else "")
+        if out is not None:
+            if not single_sweep:
+                raise ValueError("out=: the out-of-place step is the single-sweep step")
+            if len(out) != 4:
+                raise ValueError("out=: (resid, p, m, v) tensors for the new state")
+            for t in out:
+                L.require_dev(t)
+                L.require_contig(t=t)
+                if t.numel() != self.n or t.dtype != torch.float32:
+                    raise ValueError("out=: flat fp32 tensors of the bucket's length")
+            state += [L.ptr(t) for t in out]
+            name += "_out"
+        return self._run(name, g, state, step, k, ratio_percent, score, factor, coeff, fast,
+                         optimizer, fold, interval, inactive_lr_scale, single_sweep, seed, check,
+                         result)
 
     def step_packed(self, g, state, step, k=None, ratio_percent=None, score="abs_g",
                     factor=1.0, coeff=1.0, fast=True, optimizer="adamw", fold=False,
                     interval=1.0, inactive_lr_scale=1.0, single_sweep=False, seed=None,
-                    check=True, result=None):
+                    check=True, result=None, out=None):
         """Same step on a ``PackedState`` (resid/p/m/v interleaved in 64 KiB
-        records): same arithmetic and outputs."""
+        records): same arithmetic and outputs.  ``out`` (single sweep only):
+        another ``PackedState`` that receives the new state, as in ``step``."""
         L.require_dev(g, state.data)
         L.require_contig(g=g)
         if g.numel() != self.n or state.n != self.n:
             raise ValueError("gradient / packed state length does not match the bucket")
         name = ("sga_fused_sparse_step_single_sweep_packed" if single_sweep else
                 "sga_fused_sparse_step_packed")
-        return self._run(name, g, [L.ptr(state.data)], step, k, ratio_percent, score, factor,
+        args = [L.ptr(state.data)]
+        if out is not None:
+            if not single_sweep:
+                raise ValueError("out=: the out-of-place step is the single-sweep step")
+            if out.n != self.n:
+                raise ValueError("out=: a PackedState of the bucket's length")
+            L.require_dev(out.data)
+            args.append(L.ptr(out.data))
+            name += "_out"
+        return self._run(name, g, args, step, k, ratio_percent, score, factor,
                          coeff, fast, optimizer, fold, interval, inactive_lr_scale, single_sweep,
                          seed, check, result)
 

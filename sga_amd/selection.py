@@ -32,7 +32,7 @@ def read_result(res_t):
     r = res_t.cpu().tolist()
     out = SimpleNamespace(thresh_bits=r[0], need=r[1], n_gt=r[2], n_eq=r[3],
                           n_selected=r[4], nonfinite=r[5], status=r[6], path=r[7] & 0xFF,
-                          negative=bool(r[7] & 0x100))
+                          negative=bool(r[7] & 0x100), redone=bool(r[7] & 0x200))
     out.thresh = torch.tensor([r[0]], dtype=torch.int32).view(torch.float32).item()
     return out
 

@@ -12,7 +12,9 @@ pytestmark = pytest.mark.gpu
 
 
 def _run(dev, sizes, steps, ratio, gdtype, vdtype, score="abs_g", seed0=0, vary=False,
-         expect_path=2, packed=False, grads=None, **knobs):
+         expect_path=2, packed=False, grads=None, out=False, **knobs):
+    """``out``: run the out-of-place step on ping-pong state (the new state
+    lands in the other set, the inputs must come back untouched)."""
     from sga_amd.fused_step import FusedSparseStep, PackedState
     segs, n = _segments(sizes, vary=vary)
     gen = torch.Generator().manual_seed(1234)
@@ -20,13 +22,33 @@ def _run(dev, sizes, steps, ratio, gdtype, vdtype, score="abs_g", seed0=0, vary=
     m, v, r = torch.zeros(n), torch.zeros(n), torch.zeros(n)
     dp, dm, dv, dr = (t.to(dev) for t in (p, m, v, r))
     st = PackedState(n, dev).pack(dr, dp, dm, dv) if packed else None
+    if out:
+        # poisoned, so that a coordinate the step failed to write shows
+        st2 = PackedState(n, dev) if packed else None
+        if packed:
+            st2.data.fill_(float("nan"))
+        other = [torch.full((n,), float("nan"), device=dev) for _ in range(4)]
     fs = FusedSparseStep(n, segs, dev, values_dtype=vdtype, want_mask=True)
     k = SEL.k_for(n, ratio)
     for step in range(1, steps + 1):
         g = (grads(n, seed0 + step - 1) if grads else student_t(n, seed0 + step - 1)).to(gdtype)
         idx_ref, val_ref, mask_ref, th_ref = OF.fused_sparse_step(
             g, r, p, m, v, segs, step, k=k, score=score, values_dtype=vdtype, **knobs)
-        if packed:
+        if out and packed:
+            before = st.data.clone()
+            idx, vals = fs.step_packed(g.to(dev), st, step, k=k, score=score, single_sweep=True,
+                                       out=st2, **knobs)
+            assert same_bits(st.data, before.cpu()), step
+            st, st2 = st2, st
+            st.unpack(dr, dp, dm, dv)
+        elif out:
+            before = [t.clone() for t in (dr, dp, dm, dv)]
+            idx, vals = fs.step(g.to(dev), dr, dp, dm, dv, step, k=k, score=score,
+                                single_sweep=True, out=other, **knobs)
+            for t, b in zip((dr, dp, dm, dv), before):
+                assert same_bits(t, b.cpu()), step
+            (dr, dp, dm, dv), other = other, [dr, dp, dm, dv]
+        elif packed:
             idx, vals = fs.step_packed(g.to(dev), st, step, k=k, score=score, single_sweep=True,
                                        **knobs)
             st.unpack(dr, dp, dm, dv)
@@ -134,6 +156,19 @@ def _mix32(x):
     return x
 
 
+def _adversarial_grad(n, seed):
+    """Magnitudes in [1, 2) in every quad the sample of ``seed`` reads (its
+    offsets restated here), in [3, 4) everywhere else."""
+    n_sv, n_vec = 16384, n // 4
+    gen = torch.Generator().manual_seed(5)
+    g = 3.0 + torch.rand(n, generator=gen)
+    for j in range(n_sv):
+        w0, w1 = j * n_vec // n_sv, (j + 1) * n_vec // n_sv
+        vec = w0 + _mix32(j + seed * 0x9E3779B9) % (w1 - w0)
+        g[4 * vec: 4 * vec + 4] = 1.0 + torch.rand(4, generator=gen)
+    return g
+
+
 def test_a_bracket_that_missed_is_reported(dev):
     """The one outcome the single sweep cannot repair: every quad the sample
     reads (its offsets restated here for the given seed) holds a magnitude in
@@ -143,13 +178,7 @@ def test_a_bracket_that_missed_is_reported(dev):
     sample sees the real population and the same data gives the exact step."""
     from sga_amd.fused_step import FusedSparseStep
     n, seed = 1 << 21, 12345
-    n_sv, n_vec = 16384, n // 4
-    gen = torch.Generator().manual_seed(5)
-    g = 3.0 + torch.rand(n, generator=gen)
-    for j in range(n_sv):
-        w0, w1 = j * n_vec // n_sv, (j + 1) * n_vec // n_sv
-        vec = w0 + _mix32(j + seed * 0x9E3779B9) % (w1 - w0)
-        g[4 * vec: 4 * vec + 4] = 1.0 + torch.rand(4, generator=gen)
+    g = _adversarial_grad(n, seed)
     segs = [dict(start=0, n=n, lr=1e-4, b1=0.9, b2=0.95, eps=1e-8, wd=0.0)]
     k = SEL.k_for(n, 1.0)
 
@@ -172,6 +201,80 @@ def test_a_bracket_that_missed_is_reported(dev):
     ref_mask, th = SEL.select_topk_flat(g.abs(), k)
     assert res.thresh == th and torch.equal(mask, ref_mask)
     assert torch.equal(idx.long(), torch.nonzero(ref_mask).reshape(-1))
+
+
+@pytest.mark.parametrize("packed", [False, True])
+def test_out_of_place_step_on_ping_pong_state(dev, packed):
+    """The out-of-place step: new state in the other set, inputs untouched,
+    every output equal to the oracle's over three steps (ragged tensors, a
+    ragged last chunk), on both layouts; and a small bucket, which the
+    two-sweep step does behind the same call, out of place as well."""
+    sizes = [300_000, 128, 37, 700_000, 3, 1024, 250_001, 130, 5, 60_000]
+    _run(dev, sizes, 3, 1.0, torch.bfloat16, torch.bfloat16, score="update", vary=True,
+         packed=packed, out=True)
+    _run(dev, [200_000, 1024, 100_001], 2, 1.0, torch.float32, torch.float32, packed=packed,
+         out=True, expect_path=None, optimizer="adams", fold=True, interval=3.0)
+
+
+@pytest.mark.parametrize("packed", [False, True])
+def test_out_of_place_step_redoes_a_missed_bracket(dev, packed):
+    """The input of ``test_a_bracket_that_missed_is_reported`` through the
+    out-of-place step: the sweep commits on the wrong bracket into the OUTPUT
+    arrays, the check sees the miss, and the device redoes the step from the
+    untouched inputs.  Status 0, ``redone`` set, every output equal to the
+    oracle's."""
+    from sga_amd.fused_step import FusedSparseStep, PackedState
+    n, seed = 1 << 21, 12345
+    g = _adversarial_grad(n, seed)
+    segs = [dict(start=0, n=n, lr=1e-4, b1=0.9, b2=0.95, eps=1e-8, wd=0.01)]
+    k = SEL.k_for(n, 1.0)
+    gen = torch.Generator().manual_seed(8)
+    p = torch.randn(n, generator=gen) * 0.02
+    r = torch.randn(n, generator=gen) * 1e-3
+    m, v = torch.randn(n, generator=gen) * 1e-3, torch.rand(n, generator=gen) * 1e-6
+    ins = [t.to(dev) for t in (r, p, m, v)]
+    outs = [torch.full((n,), float("nan"), device=dev) for _ in range(4)]
+    fs = FusedSparseStep(n, segs, dev, values_dtype=torch.float32, want_mask=True)
+    if packed:
+        st, st2 = PackedState(n, dev).pack(*ins), PackedState(n, dev)
+        st2.data.fill_(float("nan"))
+        before = st.data.clone()
+        idx, vals = fs.step_packed(g.to(dev), st, 1, k=k, single_sweep=True, seed=seed, out=st2)
+        assert same_bits(st.data, before.cpu())
+        st2.unpack(*outs)
+    else:
+        idx, vals = fs.step(g.to(dev), *ins, 1, k=k, single_sweep=True, seed=seed, out=outs)
+        for t, b in zip(ins, (r, p, m, v)):
+            assert same_bits(t, b)
+    res = fs.read_result()
+    assert res.status == 0 and res.redone and res.path == 0 and res.n_selected == k, vars(res)
+    idx_ref, val_ref, mask_ref, th_ref = OF.fused_sparse_step(
+        g, r, p, m, v, segs, 1, k=k, score="abs_g", values_dtype=torch.float32)
+    assert res.thresh == th_ref
+    assert torch.equal(idx.cpu(), idx_ref) and torch.equal(fs.mask.cpu().bool(), mask_ref)
+    assert torch.equal(vals.cpu().view(torch.int32), val_ref.view(torch.int32))
+    for t, ref in zip(outs, (r, p, m, v)):        # the oracle stepped r / p / m / v in place
+        assert same_bits(t, ref)
+
+
+def test_out_of_place_step_refuses_overlapping_state(dev):
+    from sga_amd.fused_step import FusedSparseStep
+    n = 4096
+    segs = [dict(start=0, n=n, lr=1e-4, b1=0.9, b2=0.95, eps=1e-8, wd=0.0)]
+    fs = FusedSparseStep(n, segs, dev)
+    buf = torch.zeros(9 * n, device=dev)
+    g = torch.randn(n, device=dev)
+    r, p, m, v = (buf[i * n:(i + 1) * n] for i in range(4))
+    ok = [buf[(4 + i) * n:(5 + i) * n] for i in range(4)]
+    with pytest.raises(RuntimeError, match="overlaps"):
+        fs.step(g, r, p, m, v, 1, k=40, single_sweep=True, out=[r, ok[1], ok[2], ok[3]])
+    with pytest.raises(RuntimeError, match="overlaps"):
+        fs.step(g, r, p, m, v, 1, k=40, single_sweep=True,
+                out=[ok[0], ok[1], buf[6 * n - 8:7 * n - 8], ok[3]])
+    with pytest.raises(ValueError, match="single-sweep"):
+        fs.step(g, r, p, m, v, 1, k=40, out=ok)
+    fs.step(g, r, p, m, v, 1, k=40, single_sweep=True, out=ok)
+    assert fs.read_result().status == 0
 
 
 @pytest.mark.parametrize("packed", [False, True])
