@@ -654,9 +654,13 @@ def main():
     max_steps = max(args.steps, 5)
     results = torch.zeros(max_steps, 8, dtype=torch.int32, device=dev)   # a result block per step
 
-    def time_leg(layout, score, ratio, warmup, steps, single=False, oop=False):
+    def time_leg(layout, score, ratio, warmup, steps, single=False, oop=False, no_g=False):
         """`warmup` untimed + exactly `steps` timed steps of one configuration.  `oop`: the
-        out-of-place single-sweep step on ping-pong state (flat tensors)."""
+        out-of-place single-sweep step on ping-pong state (flat tensors).  `no_g`: the
+        reference's own buffer contract, resid already holds g + r and the step takes no
+        separate gradient (backward's accumulation is not part of the step, so the buffer is
+        not refreshed between the timed steps)."""
+        gb = 0.0 if no_g else 2.0
         k = k_for(n, ratio)
         sets = [[r, p, m, v], [torch.empty_like(r) for _ in range(4)] if oop else None]
         if layout == "packed" and state["packed"] is None:
@@ -666,7 +670,10 @@ def main():
             state["packed"] = None
 
         def step_fn(t, res=None):
-            if oop:
+            if no_g:
+                fs.step(None, r, p, m, v, t + 1, k=k, score=score, single_sweep=single,
+                        check=False, result=res)
+            elif oop:
                 fs.step(grads[t % 2], *sets[0], t + 1, k=k, score=score, single_sweep=True,
                         check=False, result=res, out=sets[1])
                 sets.reverse()
@@ -701,15 +708,16 @@ def main():
         # dominant kernel: k_fused_final reads g, r, p, m, v, writes r, p, m, v and the pack
         # (4 + 2 B per selected coordinate); k_fused_spec (single sweep) the same state traffic
         # and one staged 2 B value per coordinate it takes as selected
-        final_bytes = n * ALG_BYTES_FINAL + k * (2.0 if single else 6.0)
-        sweep_bytes = 0.0 if single else n * sweep_bytes_per_elem(score)
+        final_bytes = n * (ALG_BYTES_FINAL - 2.0 + gb) + k * (2.0 if single else 6.0)
+        sweep_bytes = 0.0 if single else n * sweep_bytes_per_elem(score, gb)
         # bytes the step has to move: every array once (34 B per element + the pack) for the
         # single sweep; the score inputs once more for the two-sweep step's select
-        once_bytes = n * ALG_BYTES_FINAL + k * 6.0
-        two_read_bytes = n * step_bytes_per_elem(score) + k * 6.0
+        once_bytes = n * (ALG_BYTES_FINAL - 2.0 + gb) + k * 6.0
+        two_read_bytes = n * step_bytes_per_elem(score, gb) + k * 6.0
         moved = once_bytes if single else two_read_bytes
         fin_avg, sw_avg = fin_ms / max(fin_n, 1), sw_ms / max(sw_n, 1)
-        return {"layout": layout, "single_sweep": single, "out_of_place": oop, "score": score,
+        return {"layout": layout, "single_sweep": single, "out_of_place": oop,
+                "separate_gradient": not no_g, "score": score,
                 "ratio_percent": ratio,
                 "k": k, "steps": steps, "seconds": dt, "ms_per_step": dt / steps * 1e3,
                 "elem_per_s": n * steps / dt,
@@ -742,10 +750,14 @@ def main():
         m.zero_(); v.zero_(); r.zero_()
         state["t"] = 0
     # the other step variant and the other layout of the headline configuration
-    other = packed_leg = oop_leg = None
+    other = packed_leg = oop_leg = nog_leg = None
     if not args.headline_only:
         other = time_leg(args.layout, args.score, args.ratio, 2, 5, not args.single_sweep)
         oop_leg = time_leg("separate", args.score, args.ratio, 2, 5, True, oop=True)
+        if args.score != "abs_g_blind":
+            # the buffer must hold a gradient's worth of values for the first of these steps
+            r.add_(grads[0].float())
+            nog_leg = time_leg("separate", args.score, args.ratio, 2, 5, args.single_sweep, no_g=True)
         packed_leg = time_leg("packed" if args.layout == "separate" else "separate", args.score,
                               args.ratio, 2, 5, args.single_sweep)
     two = head if not args.single_sweep else other
@@ -806,7 +818,16 @@ def main():
             "ms_per_step": oop_leg["ms_per_step"], "elem_per_s": oop_leg["elem_per_s"],
             "frac": oop_leg["step_frac"], "dominant_kernel_ms": oop_leg["final_avg_ms"],
             "dominant_kernel_frac": oop_leg["final_frac"]}
+    if nog_leg is not None:
+        out["single_buffer"] = {
+            "what": "same step, no separate gradient: the fp32 buffer already holds g + r (the "
+                    "reference's own contract)",
+            "ms_per_step": nog_leg["ms_per_step"], "elem_per_s": nog_leg["elem_per_s"],
+            "bytes_per_elem": nog_leg["moved_bytes_per_elem"], "frac": nog_leg["step_frac"],
+            "dominant_kernel_ms": nog_leg["final_avg_ms"],
+            "dominant_kernel_frac": nog_leg["final_frac"]}
     detail = {"headline_leg": head, "other_variant_leg": other, "other_layout_leg": packed_leg,
+              "single_buffer_leg": nog_leg,
               "out_of_place_leg": oop_leg,
               "select": head["select"], "traffic_source": traffic_src,
               "stream_mix_copy": stream_mix}
@@ -865,7 +886,8 @@ def main():
             out["detail_file"] = f"not written ({e.strerror})"
     # the last line stays compact whatever happens: optional summaries go first if it ever grew
     line = json.dumps(out, separators=(",", ":"))
-    for key in ("cfg5", "cfg2", "out_of_place", "packed_layout", "separate_layout", "two_sweep"):
+    for key in ("cfg5", "cfg2", "single_buffer", "out_of_place", "packed_layout", "separate_layout",
+                "two_sweep"):
         if len(line) < 6000:
             break
         out.pop(key, None)

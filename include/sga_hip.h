@@ -346,6 +346,13 @@ int sga_opt_step_inplace(const float* q, float* m, float* v, float* w,
  * zeroed; sparse AdamW commit on p/m/v (engine order: engine.py:416-604,
  * pack kernels.py:166-187, commit adamw.py:637-724).
  * g_dtype / values_dtype: SGA_F32 | SGA_BF16.  mask_out may be NULL.
+ * g may be NULL with g_dtype SGA_F32: resid then ALREADY holds g + r, the
+ * reference's own buffer contract (backward accumulates into the buffer that
+ * keeps the residual and the engine hands that buffer to the pack,
+ * engine.py:453-470); nothing is added, buf = resid bit for bit, and the step
+ * reads 4 B per coordinate less.  Refused for the residual-blind score, which
+ * ranks the step's own gradient.  The same holds for every entry point of
+ * this section (per bucket for sga_fused_sparse_step_multi).
  * idx_out / values_out need room for k entries.  segs is a DEVICE array.
  * flags: SGA_GC_ADAMS commits (and, for update / coi, scores) with the AdamS
  * tail (adams.py:87-213, 507-654: v rebuilt from the pre-commit m, no bias

@@ -26,7 +26,8 @@ def fused_sparse_step(g, resid, p, m, v, segments, step, ratio_percent=None,
                       interval=1.0):
     """One step over a flat bucket.
 
-    g        : flat gradient (bf16 or fp32), read only
+    g        : flat gradient (bf16 or fp32), read only; None: ``resid``
+               already holds g + r
     resid    : flat fp32 residual, updated in place (new residual)
     p, m, v  : flat fp32 state, updated in place
     segments : list of dicts {"start","n","lr","b1","b2","eps","wd"}
@@ -39,8 +40,16 @@ def fused_sparse_step(g, resid, p, m, v, segments, step, ratio_percent=None,
     Returns (idx int32[k], values[k], mask bool[N], thresh).
     """
     n = resid.numel()
-    gf = g.float()
-    resid.add_(gf)                             # buf = r + g (one fp32 add)
+    if g is None:
+        # the reference's own buffer contract: backward has already accumulated
+        # g into the buffer that keeps the residual (engine.py:453-470 hands
+        # ``bs.grad_data`` itself to the pack); nothing is added here
+        if score == "abs_g_blind":
+            raise ValueError("the residual-blind score ranks the step's own gradient")
+        gf = None
+    else:
+        gf = g.float()
+        resid.add_(gf)                         # buf = r + g (one fp32 add)
     buf = resid
     if score == "abs_g":
         sc = buf.abs()
@@ -51,7 +60,8 @@ def fused_sparse_step(g, resid, p, m, v, segments, step, ratio_percent=None,
             bc1 = 1.0 - s["b1"] ** step
             bc2 = 1.0 - s["b2"] ** step
             sc[a:b] = S.step_score(
-                score, p[a:b], m[a:b], v[a:b], buf[a:b], gf[a:b], s["b1"],
+                score, p[a:b], m[a:b], v[a:b], buf[a:b],
+                None if gf is None else gf[a:b], s["b1"],
                 s["b2"], s["eps"], s["wd"], bc1, bc2, optimizer)
     if k is None:
         k = SEL.k_for(n, ratio_percent)

@@ -38,6 +38,9 @@ struct SrcFused {
   static constexpr bool kHyper = SCORE == SGA_SCORE_UPDATE || SCORE == SGA_SCORE_COI ||
                                  SCORE == SGA_SCORE_GR_OVER_SQRT_V;
   static constexpr bool kNeedG = SCORE != SGA_SCORE_ABS_M;
+  // g == nullptr (fp32 instantiations only): the caller's buffer `r` already holds g + r, the
+  // reference's own contract (backward accumulates into the buffer that keeps the residual)
+  __device__ __forceinline__ bool has_g() const { return BF16G || g != nullptr; }
   static constexpr bool kNeedR = kNeedG && SCORE != SGA_SCORE_ABS_G_BLIND;
   static constexpr bool kNeedP = SCORE == SGA_SCORE_UPDATE;
   static constexpr bool kNeedV = kHyper;                       // v, or m in its place under AdamS
@@ -57,7 +60,7 @@ struct SrcFused {
   }
   template <bool FULL>
   __device__ __forceinline__ void fetch(const Chunk& ck, int64_t i, int64_t n, Raw& w) {
-    if (kNeedG) fetch_g<BF16G, FULL>(g, i, n, vec, w.g);
+    if (kNeedG && has_g()) fetch_g<BF16G, FULL>(g, i, n, vec, w.g);
     if (kNeedR) w.r = ldraw_f32<FULL>(r + ck.sh, i, n, vec);
     if (need_m()) w.m = ldraw_f32<FULL>(m + ck.sh, i, n, vec);
     if (kNeedP) w.p = ldraw_f32<FULL>(p + ck.sh, i, n, vec);
@@ -68,11 +71,11 @@ struct SrcFused {
                                        uint32_t key[4]) {
     float q[4] = {0, 0, 0, 0}, rr[4] = {0, 0, 0, 0};
     float pp[4] = {0, 0, 0, 0}, mm[4] = {0, 0, 0, 0}, vv[4] = {0, 0, 0, 0};
-    if (kNeedG) unpack_g<BF16G, FULL>(w.g, q);
+    if (kNeedG && has_g()) unpack_g<BF16G, FULL>(w.g, q);
     if (kNeedR) {
       unpack_f32(w.r, rr);
 #pragma unroll
-      for (int e = 0; e < 4; ++e) q[e] = rr[e] + q[e];
+      for (int e = 0; e < 4; ++e) q[e] = has_g() ? rr[e] + q[e] : rr[e];
     }
     if (need_m()) unpack_f32(w.m, mm);
     if (!kHyper) {
@@ -94,11 +97,11 @@ struct SrcFused {
     const int64_t sh = pack_shift<FULL>(i, pack_extra);
     float q[4] = {0, 0, 0, 0}, rr[4] = {0, 0, 0, 0};
     float pp[4] = {0, 0, 0, 0}, mm[4] = {0, 0, 0, 0}, vv[4] = {0, 0, 0, 0};
-    if (kNeedG) load_g<BF16G, FULL>(g, i, n, q, vec);
+    if (kNeedG && has_g()) load_g<BF16G, FULL>(g, i, n, q, vec);
     if (kNeedR) {
       ld_f32<FULL>(r + sh, i, n, rr, vec);
 #pragma unroll
-      for (int e = 0; e < 4; ++e) q[e] = rr[e] + q[e];
+      for (int e = 0; e < 4; ++e) q[e] = has_g() ? rr[e] + q[e] : rr[e];
     }
     if (need_m()) ld_f32<FULL>(m + sh, i, n, mm, vec);
     if (!kHyper) {
@@ -170,6 +173,7 @@ __device__ __forceinline__ void final_chunk(const FinalArgs& a, int64_t c, Chunk
   float* const VO = a.vo + sh;
   float gg[kChunkIters][4], rr[kChunkIters][4], pp[kChunkIters][4], mm[kChunkIters][4],
       vv[kChunkIters][4];
+  const bool has_g = BF16G || a.g != nullptr;     // no g: the buffer `r` already holds g + r
   if (FULL) {
     // raw loads first (bf16 kept packed), a scheduling fence, then unpacking:
     // the wave has all 20 loads of its chunk in flight before the first wait
@@ -180,7 +184,8 @@ __device__ __forceinline__ void final_chunk(const FinalArgs& a, int64_t c, Chunk
     for (int it = IT0; it < IT0 + NIT; ++it) {
       const int64_t i = c * kChunk + it * (kWave * kVec) + lane_id() * kVec;
       if (BF16G) graw_h[it] = ldh4_nt(reinterpret_cast<const uint16_t*>(a.g) + i);
-      else graw_f[it] = ld4_nt(reinterpret_cast<const float*>(a.g) + i);
+      else if (has_g) graw_f[it] = ld4_nt(reinterpret_cast<const float*>(a.g) + i);
+      else graw_f[it] = F4{0.0f, 0.0f, 0.0f, 0.0f};
       rraw[it] = ld4_nt(R + i);
       praw[it] = ld4_nt(P + i);
       mraw[it] = ld4_nt(M + i);
@@ -207,7 +212,7 @@ __device__ __forceinline__ void final_chunk(const FinalArgs& a, int64_t c, Chunk
 #pragma unroll
       for (int e = 0; e < 4; ++e) gg[it][e] = rr[it][e] = pp[it][e] = mm[it][e] = vv[it][e] = 0.0f;
       if (i < n) {
-        load_g<BF16G, false>(a.g, i, n, gg[it], a.vec);
+        if (has_g) load_g<BF16G, false>(a.g, i, n, gg[it], a.vec);
         load4_f32(R, i, n, rr[it], a.vec);
         load4_f32(P, i, n, pp[it], a.vec);
         load4_f32(M, i, n, mm[it], a.vec);
@@ -231,7 +236,7 @@ __device__ __forceinline__ void final_chunk(const FinalArgs& a, int64_t c, Chunk
       for (int e = 0; e < 4; ++e) {
         const uint64_t mk = pw[e];
         valid[e] = FULL || i + e < n;
-        q[e] = rr[it][e] + gg[it][e];
+        q[e] = has_g ? rr[it][e] + gg[it][e] : rr[it][e];
         sel[e] = __builtin_amdgcn_inverse_ballot_w64(mk);
         below += lanes_below(mk);
         total += (uint32_t)__popcll(mk);
@@ -243,7 +248,7 @@ __device__ __forceinline__ void final_chunk(const FinalArgs& a, int64_t c, Chunk
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         valid[e] = FULL || i + e < n;
-        q[e] = rr[it][e] + gg[it][e];
+        q[e] = has_g ? rr[it][e] + gg[it][e] : rr[it][e];
         if (SCORE == SGA_SCORE_ABS_G) key[e] = abs_key(q[e]);
         else if (SCORE == SGA_SCORE_ABS_G_BLIND) key[e] = abs_key(gg[it][e]);
         else if (SCORE == SGA_SCORE_ABS_M) key[e] = abs_key(mm[it][e]);
@@ -554,17 +559,19 @@ __device__ __forceinline__ void spec_slab(const FinalArgs& a, const SpecArgs& sa
   const int64_t i = c * kChunk + it * (kWave * kVec) + lane_id() * kVec;
   float gg[4] = {0, 0, 0, 0}, rr[4] = {0, 0, 0, 0}, pp[4] = {0, 0, 0, 0}, mm[4] = {0, 0, 0, 0},
         vv[4] = {0, 0, 0, 0};
+  const bool has_g = BF16G || a.g != nullptr;     // no g: the buffer `r` already holds g + r
   if (FULL) {
     H4 gh; F4 gf;
     if (BF16G) gh = ldh4_nt(reinterpret_cast<const uint16_t*>(a.g) + i);
-    else gf = ld4_nt(reinterpret_cast<const float*>(a.g) + i);
+    else if (has_g) gf = ld4_nt(reinterpret_cast<const float*>(a.g) + i);
+    else gf = F4{0.0f, 0.0f, 0.0f, 0.0f};
     const F4 r4 = ld4_nt(R + i), p4 = ld4_nt(P + i), m4 = ld4_nt(M + i), v4 = ld4_nt(V + i);
     __builtin_amdgcn_sched_barrier(0);
     if (BF16G) { gg[0] = bf16_to_f32(gh.x); gg[1] = bf16_to_f32(gh.y); gg[2] = bf16_to_f32(gh.z); gg[3] = bf16_to_f32(gh.w); }
     else { gg[0] = gf.x; gg[1] = gf.y; gg[2] = gf.z; gg[3] = gf.w; }
     unpack_f32(r4, rr); unpack_f32(p4, pp); unpack_f32(m4, mm); unpack_f32(v4, vv);
   } else if (i < n) {
-    load_g<BF16G, false>(a.g, i, n, gg, a.vec);
+    if (has_g) load_g<BF16G, false>(a.g, i, n, gg, a.vec);
     load4_f32(R, i, n, rr, a.vec);
     load4_f32(P, i, n, pp, a.vec);
     load4_f32(M, i, n, mm, a.vec);
@@ -573,7 +580,7 @@ __device__ __forceinline__ void spec_slab(const FinalArgs& a, const SpecArgs& sa
   float q[4];
   uint32_t key[4] = {0u, 0u, 0u, 0u};
 #pragma unroll
-  for (int e = 0; e < 4; ++e) q[e] = rr[e] + gg[e];
+  for (int e = 0; e < 4; ++e) q[e] = has_g ? rr[e] + gg[e] : rr[e];
   if (!kHyper) {
 #pragma unroll
     for (int e = 0; e < 4; ++e)
@@ -1226,7 +1233,13 @@ static int fused_entry(const char* who, const void* g, int g_dtype, float* resid
     set_error("%s: SGA_GC_FOLD needs interval > 0 (got %g)", who, (double)interval);
     return SGA_ERR_ARG;
   }
-  if (!g || !resid || !p || !m || !v || !segs || !idx_out || !values_out || n < 1 ||
+  if (!g && (g_dtype != SGA_F32 || score_id == SGA_SCORE_ABS_G_BLIND)) {
+    // no separate gradient: resid already holds g + r (the reference's own buffer contract)
+    set_error("%s: g may be NULL only with g_dtype SGA_F32 (resid then holds g + r already), and "
+              "not for the residual-blind score, which ranks the step's own gradient", who);
+    return SGA_ERR_ARG;
+  }
+  if (!resid || !p || !m || !v || !segs || !idx_out || !values_out || n < 1 ||
       n >= (1ll << 31) || k < 1 || k > n || n_segs < 1 ||
       (g_dtype != SGA_F32 && g_dtype != SGA_BF16) ||
       (values_dtype != SGA_F32 && values_dtype != SGA_BF16) || score_id < 0 ||
@@ -1333,8 +1346,8 @@ extern "C" int sga_fused_sparse_step_multi(const sga_fused_bucket* buckets, int 
     for (int b = 0; b <= n_buckets; ++b) {
       if (b < n_buckets) {
         const sga_fused_bucket& u = buckets[b];
-        if (!u.g || !u.resid || !u.p || !u.m || !u.v || !u.segs || !u.idx_out || !u.values_out ||
-            u.n < 1 || u.n >= (1ll << 31) || u.k < 1 || u.k > u.n || u.n_segs < 1) {
+        if ((!u.g && (g_dtype != SGA_F32 || score_id == SGA_SCORE_ABS_G_BLIND)) || !u.resid ||
+            !u.p || !u.m || !u.v || !u.segs || !u.idx_out || !u.values_out || u.n < 1 || u.n >= (1ll << 31) || u.k < 1 || u.k > u.n || u.n_segs < 1) {
           set_error("%s: bucket %d: bad argument (n=%lld k=%lld n_segs=%d; need 1 <= k <= n < 2^31)",
                     who, b, (long long)u.n, (long long)u.k, u.n_segs);
           return SGA_ERR_ARG;

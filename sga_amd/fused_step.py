@@ -109,7 +109,10 @@ class FusedSparseStep:
         if score not in SCORE_MAP:
             raise ValueError(f"Unknown SGA score '{score}'. Registered: {sorted(SCORE_MAP)}")
         self._upload_segments(step)
-        head = [L.ptr(g), L.dtype_code(g), *state_args, n, k, L.ptr(self._seg_dev),
+        if g is None and score == "abs_g_blind":
+            raise ValueError("score 'abs_g_blind' ranks the step's own gradient: pass g")
+        head = [L.ptr(g), L.SGA_F32 if g is None else L.dtype_code(g), *state_args, n, k,
+                L.ptr(self._seg_dev),
                 len(self.segments), SCORE_MAP[score], L.ptr(self.idx), L.ptr(self.values),
                 L.dtype_code(self.values), L.ptr(self.mask), L.f32(factor), L.f32(coeff)]
         if result is None:
@@ -142,7 +145,10 @@ class FusedSparseStep:
              result=None, out=None):
         """Run one fused step in place; returns (idx[:k], values[:k]) views.
         ``self.result`` holds the device-side select result (threshold bits,
-        counts); nothing is synchronised here.  ``optimizer="adams"`` commits
+        counts); nothing is synchronised here.  ``g=None``: ``resid`` already
+        holds g + r (the reference's own contract, where backward accumulates
+        into the buffer that keeps the residual); the step then reads 4 B per
+        coordinate less.  ``optimizer="adams"`` commits
         (and scores) with the AdamS tail; ``fold`` divides the new residual by
         ``interval`` (the residual mean taken before a boundary).
 
@@ -166,6 +172,8 @@ class FusedSparseStep:
         step from the untouched inputs, the status stays 0 and
         ``read_result().redone`` is set."""
         for t in (g, resid, p, m, v):
+            if t is None and t is g:
+                continue
             L.require_dev(t)
             L.require_contig(t=t)
             assert t.numel() == self.n
@@ -196,7 +204,7 @@ class FusedSparseStep:
         another ``PackedState`` that receives the new state, as in ``step``."""
         L.require_dev(g, state.data)
         L.require_contig(g=g)
-        if g.numel() != self.n or state.n != self.n:
+        if (g is not None and g.numel() != self.n) or state.n != self.n:
             raise ValueError("gradient / packed state length does not match the bucket")
         name = ("sga_fused_sparse_step_single_sweep_packed" if single_sweep else
                 "sga_fused_sparse_step_packed")
@@ -238,21 +246,27 @@ def fused_step_multi(steppers, grads, resids, ps, ms, vs, step, ks=None, ratio_p
     if ks is None:
         ks = [k_for(fs.n, ratio_percent) for fs in steppers]
     table = (L.FusedBucket * nb)()
-    gd, vd = L.dtype_code(grads[0]), L.dtype_code(steppers[0].values)
+    some_g = next((g for g in grads if g is not None), None)
+    gd = L.SGA_F32 if some_g is None else L.dtype_code(some_g)
+    vd = L.dtype_code(steppers[0].values)
     for b, fs in enumerate(steppers):
         g, r, p, m, v = grads[b], resids[b], ps[b], ms[b], vs[b]
-        for t in (g, r, p, m, v):
+        for t in (r, p, m, v) if g is None else (g, r, p, m, v):
             L.require_dev(t)
             L.require_contig(t=t)
             if t.numel() != fs.n:
                 raise ValueError(f"bucket {b}: tensor length does not match the bucket")
-        if L.dtype_code(g) != gd or L.dtype_code(fs.values) != vd:
+        if g is None and (gd != L.SGA_F32 or score == "abs_g_blind"):
+            raise ValueError(f"bucket {b}: no gradient (resid holds g + r) goes with fp32 "
+                             "gradients in the other buckets, and not with score 'abs_g_blind'")
+        if (g is not None and L.dtype_code(g) != gd) or L.dtype_code(fs.values) != vd:
             raise ValueError("the buckets of one call share the gradient and value dtypes")
         if not (1 <= ks[b] <= min(fs.n, fs.max_k)):
             raise ValueError(f"bucket {b}: k={ks[b]} out of range (n={fs.n}, max_k={fs.max_k})")
         fs._upload_segments(step)
         e = table[b]
-        e.g, e.resid, e.p, e.m, e.v = (t.data_ptr() for t in (g, r, p, m, v))
+        e.g = None if g is None else g.data_ptr()
+        e.resid, e.p, e.m, e.v = (t.data_ptr() for t in (r, p, m, v))
         e.n, e.k = fs.n, ks[b]
         e.segs, e.n_segs = fs._seg_dev.data_ptr(), len(fs.segments)
         e.idx_out, e.values_out = fs.idx.data_ptr(), fs.values.data_ptr()
