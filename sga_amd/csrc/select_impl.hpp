@@ -938,6 +938,7 @@ struct SweepLds {
   uint32_t idx[kWaveCandCap];              // the chunk's candidates, index order
   uint32_t key[kWaveCandCap];
   uint32_t planes[kPlaneWordsPerChunk];    // the chunk's 32 plane words ("key above the bracket")
+  uint32_t mbytes[kChunk / 4];             // the chunk's mask bytes in element order (mask-byte sweeps)
 };
 
 // The flags of a slab live as four wave ballots (element e of every lane), i.e.
@@ -989,7 +990,7 @@ __device__ __forceinline__ void bracket_chunk(Src& src, const typename Src::Chun
                                               uint32_t& mycnt, SweepLds& lds,
                                               uint32_t* __restrict__ pbits,
                                               uint8_t* __restrict__ mask_bytes = nullptr,
-                                              bool mvec = false) {
+                                              bool mvec = false, bool m16 = false) {
   // The loads of kAhead slabs (256 elements each) are issued together, then
   // their keys are formed slab by slab: expensive key sources (Adam-normalised
   // scores) look fewer slabs ahead to stay within their register budget.  The
@@ -1037,7 +1038,10 @@ __device__ __forceinline__ void bracket_chunk(Src& src, const typename Src::Chun
       if (PM == 1) plane_put(above, it, lds.planes);
       if (PM == 2 && (FULL || i < n)) {
         const uint32_t mk[4] = {above.mine(0), above.mine(1), above.mine(2), above.mine(3)};
-        if (FULL && mvec) st_u8<true>(mask_bytes, i, n, mk, true);
+        // a lane's four bytes per slab are parked in LDS in element order, and the chunk's 1024
+        // bytes leave as one 16-byte store per lane (four 4-byte stores per lane otherwise)
+        if (FULL && m16) lds.mbytes[it * kWave + lane_id()] = mk[0] | (mk[1] << 8) | (mk[2] << 16) | (mk[3] << 24);
+        else if (FULL && mvec) st_u8<true>(mask_bytes, i, n, mk, true);
         else store4_u8(mask_bytes, i, n, mk, mvec);
       }
     }
@@ -1045,6 +1049,11 @@ __device__ __forceinline__ void bracket_chunk(Src& src, const typename Src::Chun
   if (PM == 1) {
     __builtin_amdgcn_wave_barrier();
     if (lane_id() < kPlaneWordsPerChunk) pbits[c * kPlaneWordsPerChunk + lane_id()] = lds.planes[lane_id()];
+  }
+  if (PM == 2 && FULL && m16) {
+    __builtin_amdgcn_wave_barrier();
+    const U4 v = reinterpret_cast<const U4*>(lds.mbytes)[lane_id()];
+    *reinterpret_cast<U4*>(mask_bytes + c * kChunk + lane_id() * 16) = v;
   }
 }
 
@@ -1055,6 +1064,7 @@ __global__ __launch_bounds__(kBlock) void k_bracket_sweep(
     uint32_t* __restrict__ seg_key, uint32_t* __restrict__ seg_cnt, uint32_t seg_cap,
     uint32_t* __restrict__ pbits, uint32_t* __restrict__ hi_part, uint32_t* __restrict__ nf_part,
     uint8_t* __restrict__ mask_bytes = nullptr, bool mvec = false) {
+  const bool m16 = PM == 2 && (reinterpret_cast<uintptr_t>(mask_bytes) & 15) == 0;
   __shared__ uint32_t s_hi[kChunksPerBlock], s_nf[kChunksPerBlock];
   __shared__ SweepLds s_lds[kChunksPerBlock];
   // keys equal to the upper sample key stay candidates; a skipped end means
@@ -1072,7 +1082,7 @@ __global__ __launch_bounds__(kBlock) void k_bracket_sweep(
     uint32_t* const my_key = lds.key;
     const typename Src::Chunk ck = src.chunk_begin(c);
     if (src.vec && (c + 1) * kChunk <= n)
-      bracket_chunk<Src, true, PM>(src, ck, n, c, T_LO, T_HI, chi, tot_nf, mycnt, lds, pbits, mask_bytes, mvec);
+      bracket_chunk<Src, true, PM>(src, ck, n, c, T_LO, T_HI, chi, tot_nf, mycnt, lds, pbits, mask_bytes, mvec, m16);
     else
       bracket_chunk<Src, false, PM>(src, ck, n, c, T_LO, T_HI, chi, tot_nf, mycnt, lds, pbits, mask_bytes, mvec);
     if (lane_id() == 0) { tile_gt[c] = chi; tile_eq[c] = 0u; }     // chi / tot_nf are wave totals
