@@ -561,6 +561,10 @@ def main():
     ap.add_argument("--two-sweep", dest="single_sweep", action="store_false",
                     help="headline the two-sweep step (select sweep + final sweep: the score "
                          "inputs are read twice) instead of the single-sweep step")
+    ap.add_argument("--in-place", action="store_true",
+                    help="headline the IN-PLACE single-sweep step (a missed bracket ends in status 3 "
+                         "with the state overwritten) instead of the out-of-place one on ping-pong "
+                         "state, which redoes a missed bracket on the device")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
     ap.add_argument("--cpu-sample", type=int, default=1 << 28)
     ap.add_argument("--calib", action="store_true",
@@ -662,17 +666,25 @@ def main():
         not refreshed between the timed steps)."""
         gb = 0.0 if no_g else 2.0
         k = k_for(n, ratio)
-        sets = [[r, p, m, v], [torch.empty_like(r) for _ in range(4)] if oop else None]
         if layout == "packed" and state["packed"] is None:
             state["packed"] = PackedState(n, dev).pack(r, p, m, v)
         elif layout == "separate" and state["packed"] is not None:
             state["packed"].unpack(r, p, m, v)
             state["packed"] = None
+        if oop and layout == "packed":
+            sets = [state["packed"], PackedState(n, dev)]
+        else:
+            sets = [[r, p, m, v], [torch.empty_like(r) for _ in range(4)] if oop else None]
 
         def step_fn(t, res=None):
             if no_g:
                 fs.step(None, r, p, m, v, t + 1, k=k, score=score, single_sweep=single,
                         check=False, result=res)
+            elif oop and layout == "packed":
+                fs.step_packed(grads[t % 2], sets[0], t + 1, k=k, score=score, single_sweep=True,
+                               check=False, result=res, out=sets[1])
+                sets.reverse()
+                state["packed"] = sets[0]
             elif oop:
                 fs.step(grads[t % 2], *sets[0], t + 1, k=k, score=score, single_sweep=True,
                         check=False, result=res, out=sets[1])
@@ -697,7 +709,7 @@ def main():
         fin_ms, fin_n = prof_read(L, PROF_FINAL)
         sw_ms, sw_n = prof_read(L, PROF_SWEEP)
         prof_enable(L, 0)
-        if oop and sets[0][0] is not r:              # leave the current state in r / p / m / v
+        if oop and layout != "packed" and sets[0][0] is not r:   # leave the current state in r / p / m / v
             for dst, src in zip((r, p, m, v), sets[0]):
                 dst.copy_(src)
         # every timed step must have ended as an exact top-k step (status word 0, k selected)
@@ -734,7 +746,10 @@ def main():
                 "select": {"thresh": res.thresh, "n_gt": res.n_gt, "n_eq": res.n_eq,
                            "path": res.path}}
 
-    head = time_leg(args.layout, args.score, args.ratio, args.warmup, args.steps, args.single_sweep)
+    # the headline single-sweep step runs out of place on ping-pong state unless --in-place
+    head_oop = bool(args.single_sweep and not args.in_place)
+    head = time_leg(args.layout, args.score, args.ratio, args.warmup, args.steps, args.single_sweep,
+                    oop=head_oop)
     stream_mix = None
     if args.layout == "separate" and not args.headline_only:
         # What the same five read and four write streams reach WITHOUT the math, on the very
@@ -753,13 +768,13 @@ def main():
     other = packed_leg = oop_leg = nog_leg = None
     if not args.headline_only:
         other = time_leg(args.layout, args.score, args.ratio, 2, 5, not args.single_sweep)
-        oop_leg = time_leg("separate", args.score, args.ratio, 2, 5, True, oop=True)
+        oop_leg = time_leg(args.layout, args.score, args.ratio, 2, 5, True, oop=not head_oop)
         if args.score != "abs_g_blind":
             # the buffer must hold a gradient's worth of values for the first of these steps
             r.add_(grads[0].float())
             nog_leg = time_leg("separate", args.score, args.ratio, 2, 5, args.single_sweep, no_g=True)
         packed_leg = time_leg("packed" if args.layout == "separate" else "separate", args.score,
-                              args.ratio, 2, 5, args.single_sweep)
+                              args.ratio, 2, 5, args.single_sweep, oop=head_oop)
     two = head if not args.single_sweep else other
     sweep = []
     if args.sweep:
@@ -774,7 +789,8 @@ def main():
     traffic, traffic_src = load_traffic(args.layout, args.score, args.ratio, args.single_sweep)
     k = head["k"]
     value = n * args.steps / head["seconds"]
-    entry = "sga_fused_sparse_step" + ("_single_sweep" if args.single_sweep else "")
+    entry = ("sga_fused_sparse_step" + ("_single_sweep" if args.single_sweep else "")
+             + ("_packed" if args.layout == "packed" else "") + ("_out" if head_oop else ""))
     out = {
         "metric": "grad elems/s (score+top-k+resid AdamW)",
         "value": value, "unit": "elem/s", "n_gpus": 1, "steps": args.steps,
@@ -785,9 +801,11 @@ def main():
                                "146 tensors, bf16 Student-t(3) grads, fp32 p/m/v/residual, score "
                                f"{args.score}, exact top-k {args.ratio}%, index pack int32+bf16, "
                                f"residual-aware AdamW; entry point {entry}"
-                               + ("_packed" if args.layout == "packed" else ""),
+                               + (" (new state written to a second set of arrays: a missed "
+                                  "bracket is redone on the device, never lost)" if head_oop else ""),
                    "ratio_percent": args.ratio, "score": args.score, "k": k,
-                   "single_sweep": bool(args.single_sweep), "state_layout": args.layout},
+                   "single_sweep": bool(args.single_sweep), "out_of_place": head_oop,
+                   "state_layout": args.layout},
         "roofline": {"bound": "hbm",
                      "kernel": "k_fused_spec" if args.single_sweep else "k_fused_final",
                      "avg_ms": head["final_avg_ms"],
@@ -813,8 +831,9 @@ def main():
             "frac": packed_leg["step_frac"], "dominant_kernel_ms": packed_leg["final_avg_ms"],
             "dominant_kernel_frac": packed_leg["final_frac"]}
     if oop_leg is not None:
-        out["out_of_place"] = {
-            "what": "single-sweep step on ping-pong state (a missed bracket is redone, never lost)",
+        out["in_place" if head_oop else "out_of_place"] = {
+            "what": ("single-sweep step in place (a missed bracket ends in status 3)" if head_oop else
+                     "single-sweep step on ping-pong state (a missed bracket is redone, never lost)"),
             "ms_per_step": oop_leg["ms_per_step"], "elem_per_s": oop_leg["elem_per_s"],
             "frac": oop_leg["step_frac"], "dominant_kernel_ms": oop_leg["final_avg_ms"],
             "dominant_kernel_frac": oop_leg["final_frac"]}
@@ -886,7 +905,7 @@ def main():
             out["detail_file"] = f"not written ({e.strerror})"
     # the last line stays compact whatever happens: optional summaries go first if it ever grew
     line = json.dumps(out, separators=(",", ":"))
-    for key in ("cfg5", "cfg2", "single_buffer", "out_of_place", "packed_layout", "separate_layout",
+    for key in ("cfg5", "cfg2", "single_buffer", "out_of_place", "in_place", "packed_layout", "separate_layout",
                 "two_sweep"):
         if len(line) < 6000:
             break
