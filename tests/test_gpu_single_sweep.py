@@ -144,6 +144,10 @@ def test_plateau_inside_the_bracket_stands_back(dev):
         g[flat] = 3e-3
         return g
     _run(dev, [1_300_000], 1, 30.0, torch.float32, torch.float32, expect_path=0, grads=grads)
+    # out of place the key-forming final sweep writes the other set
+    _run(dev, [1_300_000], 1, 30.0, torch.float32, torch.float32, expect_path=0, grads=grads, out=True)
+    _run(dev, [1_300_000], 1, 30.0, torch.float32, torch.bfloat16, expect_path=0, grads=grads, out=True,
+         packed=True)
 
 
 def _mix32(x):
