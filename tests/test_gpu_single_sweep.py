@@ -389,6 +389,43 @@ def test_out_of_place_step_on_row_sparse_gradients(dev, active):
         assert r2.thresh == 0.0
 
 
+@pytest.mark.parametrize("variant", ["two_sweep", "single_sweep", "single_sweep_out"])
+def test_non_finite_gradients_are_counted_and_rank_first(dev, variant):
+    """NaN / Inf in the step's gradient (a loss spike): the reference's exact
+    select refuses such scores after a pass of its own (replay.py:545-547);
+    the fused step reports their number in the result block instead and the
+    caller decides.  What the kernels do with them is defined all the same:
+    a key is the magnitude's bit pattern, so every non-finite coordinate ranks
+    above every finite one and is selected (k permitting), the finite part of
+    the selection is the exact top of the finite scores, and the step ends
+    normally on every route."""
+    from sga_amd.fused_step import FusedSparseStep
+    n = 1_200_003
+    segs = [dict(start=0, n=n, lr=1e-4, b1=0.9, b2=0.95, eps=1e-8, wd=0.0)]
+    g = student_t(n, 5)
+    bad = [0, 1023, 1024, 500_001, 777_777, n - 2, n - 1]
+    vals = [float("nan"), float("inf"), -float("inf"), float("nan"), float("inf"), -float("nan"),
+            float("inf")]
+    for i, x in zip(bad, vals):
+        g[i] = x
+    k = SEL.k_for(n, 1.0)
+    score = g.abs()
+    score[torch.tensor(bad)] = torch.finfo(torch.float32).max     # above every finite score
+    mask_ref, _ = SEL.select_topk_flat(score, k)
+    state = [torch.zeros(n, device=dev) for _ in range(4)]
+    outs = [torch.empty(n, device=dev) for _ in range(4)]
+    fs = FusedSparseStep(n, segs, dev, values_dtype=torch.float32, want_mask=True)
+    idx, _v = fs.step(g.to(dev), *state, 1, k=k, single_sweep=variant != "two_sweep",
+                      out=outs if variant.endswith("out") else None)
+    res = fs.read_result()
+    assert res.status == 0 and res.nonfinite == len(bad) and res.n_selected == k, vars(res)
+    assert torch.equal(fs.mask.cpu().bool(), mask_ref)
+    assert torch.equal(idx.cpu().long(), torch.nonzero(mask_ref).reshape(-1))
+    new_r = (outs if variant.endswith("out") else state)[0].cpu()
+    assert bool((new_r[torch.tensor(bad)] == 0.0).all())           # selected: residual cleared
+    assert bool(torch.isfinite(new_r).all())
+
+
 def test_randomized_single_sweep_equals_two_sweep(dev):
     """Seeded random draws of tensor layouts, hyper-parameters, scores, dtypes,
     ratios, knobs and magnitudes: the single-sweep step and the two-sweep step
