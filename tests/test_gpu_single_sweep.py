@@ -389,6 +389,20 @@ def test_out_of_place_step_on_row_sparse_gradients(dev, active):
         assert r2.thresh == 0.0
 
 
+@pytest.mark.parametrize("ratio", [100.0, 99.9999, 50.0])
+@pytest.mark.parametrize("out", [False, True])
+def test_everything_or_nearly_everything_selected(dev, ratio, out):
+    """k = n, k = n - 1 and k = n / 2: the bracket is open above or below (or
+    too wide for the record lists), so the two-sweep step or the radix passes
+    do the step behind the single-sweep call; against the oracle, two steps.
+    With an all-zero gradient at the second step the buffer is the residual
+    alone: zeros wherever the first step selected."""
+    def grads(n, seed):
+        return student_t(n, seed) if seed == 0 else torch.zeros(n)
+    _run(dev, [1_100_000, 130, 100_001], 2, ratio, torch.float32, torch.float32, expect_path=None,
+         grads=grads, out=out)
+
+
 @pytest.mark.parametrize("variant", ["two_sweep", "single_sweep", "single_sweep_out"])
 def test_non_finite_gradients_are_counted_and_rank_first(dev, variant):
     """NaN / Inf in the step's gradient (a loss spike): the reference's exact
