@@ -873,19 +873,29 @@ __device__ __forceinline__ uint32_t slab_rank_before(const uint32_t* __restrict_
 // instead of 0.3 at 10 %).  Positions of coordinates the repair pass adds
 // (F without S) stay untouched: the window is pre-filled with a sentinel.
 // slab_pos[slab] = pack position of the slab's first selected coordinate.
-constexpr int kPackWindow = 1024;
+constexpr int kPackWindow = 512;
 constexpr int kPackDenseCut = 32;         // k above n / this: a lane per quarter slab
 constexpr int kPackAhead = 8;             // staged values a lane requests before it walks its bits
 template <bool BF16V, int SUB>
-__global__ __launch_bounds__(kWave) void k_spec_pack(
+__global__ __launch_bounds__(kBlock) void k_spec_pack(
     FinalArgs a, const SelState* __restrict__ st, const void* __restrict__ stage,
     const uint32_t* __restrict__ splane, const uint32_t* __restrict__ fplane,
     const uint32_t* __restrict__ tile_sel, uint32_t* __restrict__ slab_pos) {
-  __shared__ uint32_t l_idx[kPackWindow + 4];
-  __shared__ uint32_t l_val[kPackWindow + 4];
+  // Four independent waves per workgroup, each with LDS of its own and no workgroup barrier.
+  // What the kernel costs is memory: both planes (n / 4 bytes), one line per chunk of the
+  // chunk-strided staging array, the pack -- 0.54 GB at 1 % of 1.2e9 elements for 0.16 ms;
+  // a third fewer vector instructions (single-bit extracts on 32-bit halves, staged values
+  // picked from LDS by their running number) and a quarter of the workgroup launches left
+  // that time where it was.
+  __shared__ uint32_t s_idx[kChunksPerBlock][kPackWindow + 4];
+  __shared__ uint32_t s_val[kChunksPerBlock][kPackWindow + 4];
+  __shared__ uint32_t s_ahead[kChunksPerBlock][kPackAhead * kWave];
   if (!st->bracket_ok || !st->spec) return;
+  uint32_t* const l_idx = s_idx[wave_id()];
+  uint32_t* const l_val = s_val[wave_id()];
+  uint32_t* const l_ahead = s_ahead[wave_id()];
   const int64_t n_slabs = cdiv64(a.n, kChunk) * kChunkIters;
-  const int64_t part = (int64_t)blockIdx.x * kWave + threadIdx.x;
+  const int64_t part = (int64_t)blockIdx.x * kBlock + threadIdx.x;
   const int64_t slab = part / SUB;
   const bool live = slab < n_slabs;
   uint64_t S[4] = {0, 0, 0, 0}, F[4] = {0, 0, 0, 0};
@@ -932,47 +942,64 @@ __global__ __launch_bounds__(kWave) void k_spec_pack(
   uint64_t U = S[0] | S[1] | S[2] | S[3] | F[0] | F[1] | F[2] | F[3];
   uint32_t sr = 0, fr = f_start;
   // the lane's first staged values, all requested before the first is used (its run of the
-  // staging array is contiguous); a slab with more entries loads the rest as it goes
-  uint32_t ahead[kPackAhead];
+  // staging array is contiguous) and parked in LDS, where the walk below picks them up by
+  // their running number; a slab with more entries loads the rest as it goes
+  {
+    uint32_t ahead[kPackAhead];
 #pragma unroll
-  for (int t = 0; t < kPackAhead; ++t) {
-    ahead[t] = 0u;
-    if ((uint32_t)t < cntS) {
-      if (BF16V) ahead[t] = reinterpret_cast<const uint16_t*>(stage)[c * kChunk + ps + t];
-      else ahead[t] = reinterpret_cast<const uint32_t*>(stage)[c * kChunk + ps + t];
+    for (int t = 0; t < kPackAhead; ++t) {
+      ahead[t] = 0u;
+      if ((uint32_t)t < cntS) {
+        if (BF16V) ahead[t] = reinterpret_cast<const uint16_t*>(stage)[c * kChunk + ps + t];
+        else ahead[t] = reinterpret_cast<const uint32_t*>(stage)[c * kChunk + ps + t];
+      }
     }
+#pragma unroll
+    for (int t = 0; t < kPackAhead; ++t) l_ahead[t * kWave + lane_id()] = ahead[t];
   }
+  // the planes as 32-bit halves: a lane position's four S bits and four F bits are then eight
+  // single-bit field extracts (lane positions differ from lane to lane, so 64-bit shifts by a
+  // per-lane amount would run on the vector unit, two instructions each)
+  const uint32_t s_lo[4] = {(uint32_t)S[0], (uint32_t)S[1], (uint32_t)S[2], (uint32_t)S[3]};
+  const uint32_t s_hi[4] = {(uint32_t)(S[0] >> 32), (uint32_t)(S[1] >> 32), (uint32_t)(S[2] >> 32),
+                            (uint32_t)(S[3] >> 32)};
+  const uint32_t f_lo[4] = {(uint32_t)F[0], (uint32_t)F[1], (uint32_t)F[2], (uint32_t)F[3]};
+  const uint32_t f_hi[4] = {(uint32_t)(F[0] >> 32), (uint32_t)(F[1] >> 32), (uint32_t)(F[2] >> 32),
+                            (uint32_t)(F[3] >> 32)};
   for (uint32_t w0 = 0; w0 < len; w0 += kPackWindow) {
     const uint32_t wlen = len - w0 < (uint32_t)kPackWindow + 3u ? len - w0 : (uint32_t)kPackWindow + 3u;
     for (uint32_t t = lane_id(); t < wlen; t += kWave) l_idx[t] = 0xFFFFFFFFu;
-    __syncthreads();
+    __builtin_amdgcn_wave_barrier();       // the wave's own LDS: its accesses stay in order
     while (U) {
       const int L = __ffsll((unsigned long long)U) - 1;
       if (fr - F0 >= w0 + (uint32_t)kPackWindow) break;     // belongs to a later window
       U &= U - 1;
+      const bool upper = L >= 32;
+      const uint32_t l = (uint32_t)L & 31u;
+      uint32_t ns = 0, nf = 0;                              // the position's S and F bits, bit e = element e
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        const bool in_s = (S[e] >> L) & 1ull, in_f = (F[e] >> L) & 1ull;
-        if (in_s && in_f) {
-          const uint32_t t = fr - F0 - w0;
-          l_idx[t] = (uint32_t)(slab * (kWave * kVec) + L * kVec + e);
-          uint32_t val;
-          if (sr < (uint32_t)kPackAhead) {
-            val = ahead[0];
-#pragma unroll
-            for (int q = 1; q < kPackAhead; ++q) val = sr == (uint32_t)q ? ahead[q] : val;
-          } else if (BF16V) {
-            val = reinterpret_cast<const uint16_t*>(stage)[c * kChunk + ps + sr];
-          } else {
-            val = reinterpret_cast<const uint32_t*>(stage)[c * kChunk + ps + sr];
-          }
-          l_val[t] = val;
-        }
-        sr += in_s;
-        fr += in_f;
+        ns |= (((upper ? s_hi[e] : s_lo[e]) >> l) & 1u) << e;
+        nf |= (((upper ? f_hi[e] : f_lo[e]) >> l) & 1u) << e;
       }
+      uint32_t both = ns & nf;
+      while (both) {
+        const uint32_t e = (uint32_t)__ffs((int)both) - 1u;
+        both &= both - 1u;
+        const uint32_t lower = (1u << e) - 1u;
+        const uint32_t srq = sr + (uint32_t)__popc(ns & lower);
+        const uint32_t t = fr + (uint32_t)__popc(nf & lower) - F0 - w0;
+        l_idx[t] = (uint32_t)(slab * (kWave * kVec) + L * kVec) + e;
+        uint32_t val;
+        if (srq < (uint32_t)kPackAhead) val = l_ahead[srq * kWave + lane_id()];
+        else if (BF16V) val = reinterpret_cast<const uint16_t*>(stage)[c * kChunk + ps + srq];
+        else val = reinterpret_cast<const uint32_t*>(stage)[c * kChunk + ps + srq];
+        l_val[t] = val;
+      }
+      sr += (uint32_t)__popc(ns);
+      fr += (uint32_t)__popc(nf);
     }
-    __syncthreads();
+    __builtin_amdgcn_wave_barrier();       // the wave's own LDS: its accesses stay in order
     for (uint32_t t = lane_id(); t < wlen; t += kWave) {
       const uint32_t ix = l_idx[t];
       const int64_t pos = (int64_t)F0 + w0 + t;
@@ -982,7 +1009,7 @@ __global__ __launch_bounds__(kWave) void k_spec_pack(
         else reinterpret_cast<uint32_t*>(a.values_out)[pos] = l_val[t];
       }
     }
-    __syncthreads();
+    __builtin_amdgcn_wave_barrier();       // the wave's own LDS: its accesses stay in order
   }
 }
 
@@ -1196,11 +1223,11 @@ static int run_fused_spec(const void* g, float* resid, float* p, float* m, float
   // a lane per slab, or per quarter of one where a slab holds more entries than a lane has
   // staged values in flight
   if (k > n / kPackDenseCut)
-    hipLaunchKernelGGL((k_spec_pack<BF16V, 4>), dim3((unsigned)cdiv64(n_tiles * kChunkIters * 4, kWave)),
-                       dim3(kWave), 0, s, fa, w.st, x.stage, w.pbits, x.dplane, w.tile_gt, x.slab_pos);
+    hipLaunchKernelGGL((k_spec_pack<BF16V, 4>), dim3((unsigned)cdiv64(n_tiles * kChunkIters * 4, kBlock)),
+                       dim3(kBlock), 0, s, fa, w.st, x.stage, w.pbits, x.dplane, w.tile_gt, x.slab_pos);
   else
-    hipLaunchKernelGGL((k_spec_pack<BF16V, 1>), dim3((unsigned)cdiv64(n_tiles * kChunkIters, kWave)),
-                       dim3(kWave), 0, s, fa, w.st, x.stage, w.pbits, x.dplane, w.tile_gt, x.slab_pos);
+    hipLaunchKernelGGL((k_spec_pack<BF16V, 1>), dim3((unsigned)cdiv64(n_tiles * kChunkIters, kBlock)),
+                       dim3(kBlock), 0, s, fa, w.st, x.stage, w.pbits, x.dplane, w.tile_gt, x.slab_pos);
   hipLaunchKernelGGL((k_spec_repair<BF16V>), dim3(1024), dim3(kBlock), 0, s, fa, segs, n_segs,
                      w.seg_dir, w.st, w.cand_idx, w.cand_key, x.cand_rec, x.dplane, x.slab_pos);
   if (mask_out)
