@@ -587,6 +587,9 @@ def main():
                          "back through the pread reader and the dense pass) and print its JSON")
     ap.add_argument("--primitives", action="store_true",
                     help="time the drop-in primitives on their own and print their JSON")
+    ap.add_argument("--only-rows", action="store_true",
+                    help="run just the Qwen3-0.6B mask-layout row and the 1e9 stress row (for "
+                         "profiling) and print their JSON")
     ap.add_argument("--only-replay", action="store_true",
                     help="run just the fused replay leg (for profiling) and print its JSON")
     args = ap.parse_args()
@@ -602,6 +605,11 @@ def main():
     from sga_amd.shapes import llama32_1b, segments_for
 
     L.load()
+    if args.only_rows:
+        torch.cuda.set_device(0)
+        print(json.dumps({"qwen06b_mask_layout": qwen_mask_layout_row(),
+                          "stress_1e9": stress_row()}))
+        return
     if args.only_replay:
         torch.cuda.set_device(0)
         print(json.dumps(replay_bench()[0]))
