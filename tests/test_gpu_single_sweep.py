@@ -442,9 +442,11 @@ def test_non_finite_gradients_are_counted_and_rank_first(dev, variant):
 
 def test_randomized_single_sweep_equals_two_sweep(dev):
     """Seeded random draws of tensor layouts, hyper-parameters, scores, dtypes,
-    ratios, knobs and magnitudes: the single-sweep step and the two-sweep step
-    run from the same state and must agree in every output bit (idx, values,
-    mask, residual, p, m, v, threshold, tie counts) over several steps."""
+    ratios, knobs and magnitudes: the two-sweep step, the single-sweep step in
+    place and the single-sweep step out of place run from the same state and
+    must agree in every output bit (idx, values, mask, residual, p, m, v,
+    threshold, tie counts) over several steps; on half of the fp32-gradient
+    draws the single-sweep arms run without a separate gradient."""
     import random
     from sga_amd.fused_step import FusedSparseStep
     rnd = random.Random(2024)
@@ -461,26 +463,40 @@ def test_randomized_single_sweep_equals_two_sweep(dev):
         scale = 10.0 ** rnd.uniform(-8, 0)
         gen = torch.Generator().manual_seed(draw)
         p0 = (torch.randn(n, generator=gen) * 0.02).to(dev)
-        state = [[p0.clone(), torch.zeros(n, device=dev), torch.zeros(n, device=dev),
-                  torch.zeros(n, device=dev)] for _ in range(2)]
-        fs = [FusedSparseStep(n, segs, dev, values_dtype=vdt, want_mask=True) for _ in range(2)]
+        # arm 0 the two-sweep step, arm 1 the single-sweep step in place, arm 2 the single-sweep
+        # step out of place on ping-pong state; on some draws with fp32 gradients arms 1 and 2 run
+        # on the single-buffer contract (the gradient is added to the buffer beforehand and the
+        # step takes none)
+        no_g = gdt == torch.float32 and score != "abs_g_blind" and rnd.random() < 0.5
+        state = [[torch.zeros(n, device=dev), p0.clone(), torch.zeros(n, device=dev),
+                  torch.zeros(n, device=dev)] for _ in range(3)]                  # r, p, m, v
+        spare = [torch.full((n,), float("nan"), device=dev) for _ in range(4)]
+        fs = [FusedSparseStep(n, segs, dev, values_dtype=vdt, want_mask=True) for _ in range(3)]
         k = SEL.k_for(n, ratio)
         for step in range(1, 4):
             g = (student_t(n, 100 * draw + step) * (scale / 1e-3)).to(gdt).to(dev)
             outs = []
-            for which in range(2):
-                pp, mm, vv, rr = state[which]
-                idx, vals = fs[which].step(g, rr, pp, mm, vv, step, k=k, score=score,
-                                           single_sweep=bool(which), **knobs)
+            for which in range(3):
+                gin = g
+                if which and no_g:
+                    state[which][0].add_(g)
+                    gin = None
+                out = spare if which == 2 else None
+                idx, vals = fs[which].step(gin, *state[which], step, k=k, score=score,
+                                           single_sweep=bool(which), out=out, **knobs)
+                if which == 2:
+                    state[2], spare = spare, state[2]
                 res = fs[which].read_result()
                 assert res.status == 0 and res.n_selected == k, (draw, step, which, vars(res))
                 outs.append((idx, vals, fs[which].mask, res))
-            what = (draw, step, score, ratio, knobs)
-            assert outs[1][3].path in (0, 1, 2), what
-            assert (outs[0][3].thresh_bits, outs[0][3].need, outs[0][3].n_eq) == \
-                   (outs[1][3].thresh_bits, outs[1][3].need, outs[1][3].n_eq), what
-            assert torch.equal(outs[0][0], outs[1][0]) and torch.equal(outs[0][2], outs[1][2]), what
+            what = (draw, step, score, ratio, knobs, no_g)
             it = torch.int16 if vdt == torch.bfloat16 else torch.int32
-            assert torch.equal(outs[0][1].view(it), outs[1][1].view(it)), what
-            for a, b in zip(state[0], state[1]):
-                assert torch.equal(a.view(torch.int32), b.view(torch.int32)), what
+            for which in (1, 2):
+                assert outs[which][3].path in (0, 1, 2), what
+                assert (outs[0][3].thresh_bits, outs[0][3].need, outs[0][3].n_eq) == \
+                       (outs[which][3].thresh_bits, outs[which][3].need, outs[which][3].n_eq), what
+                assert torch.equal(outs[0][0], outs[which][0]), what
+                assert torch.equal(outs[0][2], outs[which][2]), what
+                assert torch.equal(outs[0][1].view(it), outs[which][1].view(it)), what
+                for a, b in zip(state[0], state[which]):
+                    assert torch.equal(a.view(torch.int32), b.view(torch.int32)), what
