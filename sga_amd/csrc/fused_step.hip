@@ -1456,10 +1456,10 @@ extern "C" int sga_fused_sparse_step_single_sweep_packed(
                      flags, interval, result, ws, ws_bytes, stream, true, ws2, ws2_bytes, seed);
 }
 
-// true when [a, a + bytes) and [b, b + bytes) overlap
-static bool ranges_overlap(const void* a, const void* b, size_t bytes) {
+// true when [a, a + a_bytes) and [b, b + b_bytes) overlap
+static bool ranges_overlap(const void* a, size_t a_bytes, const void* b, size_t b_bytes) {
   const uintptr_t x = reinterpret_cast<uintptr_t>(a), y = reinterpret_cast<uintptr_t>(b);
-  return x < y + bytes && y < x + bytes;
+  return x < y + b_bytes && y < x + a_bytes;
 }
 
 extern "C" int sga_fused_sparse_step_single_sweep_out(
@@ -1476,16 +1476,20 @@ extern "C" int sga_fused_sparse_step_single_sweep_out(
     set_error("%s: the four output arrays are required", who);
     return SGA_ERR_ARG;
   }
-  if (n > 0)
+  if (n > 0) {
+    const size_t bytes = (size_t)n * 4, g_bytes = (size_t)n * (g_dtype == SGA_BF16 ? 2 : 4);
     for (int a = 0; a < 4; ++a) {
+      bool bad = g && ranges_overlap(out[a], bytes, g, g_bytes);
       for (int b = 0; b < 4; ++b)
-        if ((in[b] && ranges_overlap(out[a], in[b], (size_t)n * 4)) ||
-            (b != a && ranges_overlap(out[a], out[b], (size_t)n * 4))) {
-          set_error("%s: an output array overlaps an input or another output (the step reads "
-                    "the old state while it writes the new one)", who);
-          return SGA_ERR_ARG;
-        }
+        bad = bad || (in[b] && ranges_overlap(out[a], bytes, in[b], bytes)) ||
+              (b != a && ranges_overlap(out[a], bytes, out[b], bytes));
+      if (bad) {
+        set_error("%s: an output array overlaps an input or another output (the step reads "
+                  "the old state while it writes the new one)", who);
+        return SGA_ERR_ARG;
+      }
     }
+  }
   return fused_entry(who, g, g_dtype, const_cast<float*>(resid), const_cast<float*>(p),
                      const_cast<float*>(m), const_cast<float*>(v), 0, n, k, segs, n_segs, score_id,
                      idx_out, values_out, values_dtype, mask_out, factor, coeff, 1, flags, interval,
@@ -1505,8 +1509,10 @@ extern "C" int sga_fused_sparse_step_single_sweep_packed_out(
     return SGA_ERR_ARG;
   }
   const size_t bytes = (size_t)(n <= 0 ? 0 : cdiv64(n, kPackRun) * 4 * kPackRun) * 4;
-  if (ranges_overlap(state, state_out, bytes)) {
-    set_error("%s: the output state overlaps the input state", who);
+  const size_t g_bytes = (size_t)(n <= 0 ? 0 : n) * (g_dtype == SGA_BF16 ? 2 : 4);
+  if (ranges_overlap(state, bytes, state_out, bytes) ||
+      (g && ranges_overlap(state_out, bytes, g, g_bytes))) {
+    set_error("%s: the output state overlaps the input state or the gradient", who);
     return SGA_ERR_ARG;
   }
   float* out[4] = {state_out, state_out + kPackRun, state_out + 2 * kPackRun, state_out + 3 * kPackRun};

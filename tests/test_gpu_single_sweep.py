@@ -274,7 +274,7 @@ def test_out_of_place_step_refuses_overlapping_state(dev):
     n = 4096
     segs = [dict(start=0, n=n, lr=1e-4, b1=0.9, b2=0.95, eps=1e-8, wd=0.0)]
     fs = FusedSparseStep(n, segs, dev)
-    buf = torch.zeros(9 * n, device=dev)
+    buf = torch.zeros(10 * n, device=dev)
     g = torch.randn(n, device=dev)
     r, p, m, v = (buf[i * n:(i + 1) * n] for i in range(4))
     ok = [buf[(4 + i) * n:(5 + i) * n] for i in range(4)]
@@ -283,6 +283,9 @@ def test_out_of_place_step_refuses_overlapping_state(dev):
     with pytest.raises(RuntimeError, match="overlaps"):
         fs.step(g, r, p, m, v, 1, k=40, single_sweep=True,
                 out=[ok[0], ok[1], buf[6 * n - 8:7 * n - 8], ok[3]])
+    with pytest.raises(RuntimeError, match="overlaps"):          # ... or the gradient
+        fs.step(buf[8 * n:9 * n], r, p, m, v, 1, k=40, single_sweep=True,
+                out=[ok[0], ok[1], ok[2], buf[8 * n + 100:9 * n + 100]])
     with pytest.raises(ValueError, match="single-sweep"):
         fs.step(g, r, p, m, v, 1, k=40, out=ok)
     fs.step(g, r, p, m, v, 1, k=40, single_sweep=True, out=ok)
