@@ -189,28 +189,34 @@ __global__ __launch_bounds__(kBlock) void k_replay_pass1(const void* __restrict_
   }
 }
 
-// One wave per config folds the workgroup partials in a fixed order and
+// One workgroup per config folds the workgroup partials in a fixed order and
 // forms the clip coefficient in double (the host formula of the reference).
+// (One WAVE per config in a single workgroup took 85 us per step for the 8192
+// rows of the table: 128 loads per lane, one after the other.)
 __global__ __launch_bounds__(kBlock) void k_replay_coef(const double* __restrict__ partials,
                                                         int n_blocks, int G, double clip,
                                                         double* __restrict__ qn2,
                                                         double* __restrict__ coef_d,
                                                         float* __restrict__ coef_f, P1Alias al) {
-  for (int c = wave_id(); c < G; c += kChunksPerBlock) {
-    double a = 0.0;
-    const int src = al.src[c];
-    for (int b = lane_id(); b < n_blocks; b += kWave) a += partials[(int64_t)b * kMaxCfg + src];
-    a = wave_sum(a);
-    if (lane_id() == 0) {
-      double coef = 1.0;
-      if (clip > 0.0) {
-        coef = clip / (sqrt(a) + 1.0e-6);
-        if (coef > 1.0) coef = 1.0;
-      }
-      qn2[c] = a;
-      coef_d[c] = coef;
-      coef_f[c] = (float)coef;
+  __shared__ double s_w[kChunksPerBlock];
+  const int c = blockIdx.x;
+  if (c >= G) return;
+  const int src = al.src[c];
+  double a = 0.0;
+  for (int b = threadIdx.x; b < n_blocks; b += kBlock) a += partials[(int64_t)b * kMaxCfg + src];
+  a = wave_sum(a);
+  if (lane_id() == 0) s_w[wave_id()] = a;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    a = ((s_w[0] + s_w[1]) + s_w[2]) + s_w[3];
+    double coef = 1.0;
+    if (clip > 0.0) {
+      coef = clip / (sqrt(a) + 1.0e-6);
+      if (coef > 1.0) coef = 1.0;
     }
+    qn2[c] = a;
+    coef_d[c] = coef;
+    coef_f[c] = (float)coef;
   }
 }
 
@@ -663,7 +669,7 @@ extern "C" int sga_replay_pass1(const void* g, int g_dtype, int64_t n, float coe
   if (bg) launch_pass1<true>(n_b, nb, s, g, n, coef_dense, lst, partials, vec, grp.pack_extra);
   else launch_pass1<false>(n_b, nb, s, g, n, coef_dense, lst, partials, vec, grp.pack_extra);
   prof_end(pp, s);
-  hipLaunchKernelGGL(k_replay_coef, dim3(1), dim3(kBlock), 0, s, partials, (int)nb, G, clip, qn2, coef_d, coef_f, al);
+  hipLaunchKernelGGL(k_replay_coef, dim3((unsigned)G), dim3(kBlock), 0, s, partials, (int)nb, G, clip, qn2, coef_d, coef_f, al);
   return check_launch("sga_replay_pass1");
 }
 
