@@ -1475,7 +1475,11 @@ static inline void chain_sweeps(const SrcPack<Src>& srcs, const SelBatch& B, int
 static inline void chain_candidates(const SelBatch& B, hipStream_t s) {
   hipLaunchKernelGGL(k_bracket_check, B.grid(1), dim3(kBlock), 0, s, B.jobs);
   hipLaunchKernelGGL(k_cand_compact, B.grid(256), dim3(kBlock), 0, s, B.jobs);
-  for (int level = 0; level < 3; ++level) launch_level_raw<true>(B, level, s, kRawKeyBlocks);
+  // a batch's candidate lists are as long as a single select's (millions of keys each at large
+  // sizes and ratios): 256 workgroups for the batch, where the sample's short passes take 64
+  // (four re-selections of the 596 M-element replay set: 97 us for the three levels, 203 with 64)
+  for (int level = 0; level < 3; ++level)
+    launch_level_raw<true>(B, level, s, B.count > 1 ? 4 * kRawKeyBlocks : kRawKeyBlocks);
   hipLaunchKernelGGL(k_cand_tiles, B.grid(256), dim3(kBlock), 0, s, B.jobs);
 }
 // The radix passes and the per-chunk counts over the data: no-ops unless a job's bracket failed
