@@ -1139,11 +1139,14 @@ static inline bool spec_ws_carve(void* ws, size_t bytes, int64_t n, int val_byte
 // Margin of the single-sweep bracket, in standard deviations of the sample rank.
 constexpr double kSpecSigmas = 12.0;
 // Out of place a missed bracket costs a redo (three more sweeps), not the state: the margin only
-// has to make that rare.  At 6 sigma an unbiased sample misses once in 5e8 steps (once in ~400,
-// 0.07 ms per step on average, if the four neighbours of every sampled quad were perfectly
-// correlated), and the sweep records half as many coordinates as at 12: the kernels behind the
-// sweep take 0.62 instead of 0.69 ms on the 1.2e9-element set (0.59 at 5 sigma, 0.57 at 4).
-constexpr double kSpecSigmasOut = 6.0;
+// has to make that rare, and it is the margin of the two-sweep step, which can fall back as
+// well.  Measured on row-sparse gradients (whole rows of 2 K to 16 K coordinates active or
+// zero, so that the four keys of a sampled quad are one draw), 2400 sample seeds per margin:
+// no miss at 3, 4, 5 or 6 sigma, 22 at 2 sigma, each redone to the exact step (the strata of the
+// sample make its rank tighter than the binomial the margin is computed for).  The sweep records
+// 1.25 M coordinates at 1 % of 1.2e9 instead of the 3 M of the in-place step's 12 sigma, and
+// the kernels behind it take 0.59 instead of 0.69 ms.
+constexpr double kSpecSigmasOut = 5.0;
 
 template <bool BF16G, bool BF16V, int SCORE>
 static int run_fused_spec(const void* g, float* resid, float* p, float* m, float* v, int64_t n,
